@@ -1,0 +1,318 @@
+// Elementwise and small reduction kernels around the dense head: optimiser steps, per-model
+// broadcast multiply-add, masks, dropout, and the handful of array ops the bias / ReLU / loss
+// nodes are made of. All are grid-stride loops over flat arrays: consecutive lanes touch
+// consecutive elements, so each wave moves whole 256-byte lines of HBM.
+//
+// Reference semantics: deepity_smat/gradstep.cu:41-72, madd_bcast.cu:41-47, maskout.cu:41-67,
+// dropout.cu:41-109, kangaroo_smat/dropoutord.cu:41-52, smat_cuda/elemwise2.cu:42-77, elemwise3.cu:57-62.
+#include "dbk_common.h"
+
+namespace {
+
+#define GRID_STRIDE(i, n) for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (n); i += (size_t)gridDim.x * blockDim.x)
+
+// Philox4x32-10 counter-based generator (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3").
+// One 128-bit counter value yields four 32-bit words; element i uses word i%4 of counter (offset + i/4).
+__host__ __device__ inline void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1)
+{
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+        uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+        uint32_t n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        uint32_t n3 = (uint32_t)p0;
+        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+// Uniform in [0,1) with 24 bits, for flat element index i.
+__device__ inline float uniform_at(uint64_t seed, uint64_t offset, size_t i)
+{
+    uint64_t ctr = offset + (uint64_t)(i >> 2);
+    uint32_t c[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u};
+    philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
+    return (float)(c[i & 3] >> 8) * (1.0f / 16777216.0f);
+}
+
+template <typename T> __global__ void k_gradstep(T* P, const T* dP, const T* drate, T* mP, const T* mrate, size_t n)
+{
+    GRID_STRIDE(i, n) {
+        T delta = mP[i] * mrate[i] - dP[i] * drate[i];
+        mP[i] = delta;
+        P[i] += delta;
+    }
+}
+template <typename T> __global__ void k_nesterov1(T* P, const T* mP, const T* mrate, size_t n)
+{
+    GRID_STRIDE(i, n) P[i] = P[i] + mrate[i] * mP[i];
+}
+template <typename T> __global__ void k_nesterov2(T* P, const T* dP, const T* drate, T* mP, const T* mrate, size_t n)
+{
+    GRID_STRIDE(i, n) {
+        T delta = dP[i] * drate[i];
+        mP[i] = mP[i] * mrate[i] - delta;
+        P[i] -= delta;
+    }
+}
+template <typename T> __global__ void k_madd_bcast(const T* A, const T* b, T* dst, size_t n, size_t m, size_t k)
+{
+    GRID_STRIDE(i, n) dst[i] += A[i] * b[(i / k) % m];
+}
+template <typename T> __global__ void k_maskout(const uint8_t* M, T* A, size_t n)
+{
+    GRID_STRIDE(i, n) if (!M[i]) A[i] = (T)0;
+}
+template <typename T> __global__ void k_calc_zmask(const T* Z, uint8_t* M, size_t n, size_t m)
+{
+    GRID_STRIDE(i, (n * m) / 2) {
+        size_t row = (i / m) * 2, col = i % m, idx = m * row + col;
+        if (Z[idx] >= Z[idx + m]) M[idx] = 1;
+        else M[idx + m] = 1;
+    }
+}
+// dropout on pooled features; U may be null (then the generator supplies the uniforms)
+template <typename T> __global__ void k_dropout_fp_tr(const T* X, const T* rate, T* Z, uint8_t* M, size_t n, size_t m, size_t k,
+                                                      const float* U, uint64_t seed, uint64_t offset)
+{
+    GRID_STRIDE(i, n) {
+        T p = rate[(i / k) % m];
+        float u = U ? U[i] : uniform_at(seed, offset, i);
+        bool keep = (T)u >= p;
+        M[i] = keep;
+        Z[i] = X[i] * (T)keep;
+    }
+}
+template <typename T> __global__ void k_dropout_fp_tr_match(const T* X, const T* rate, T* Z, uint8_t* M, size_t nrow, size_t ncol,
+                                                            size_t k, const float* U, uint64_t seed, uint64_t offset)
+{
+    GRID_STRIDE(i, nrow * ncol / 2) {
+        size_t row = (i / ncol) * 2, col = i % ncol;
+        T p = rate[col / k];
+        size_t i0 = row * ncol + col, i1 = i0 + ncol;
+        float u = U ? U[i0] : uniform_at(seed, offset, i);
+        bool keep = (T)u >= p;
+        M[i0] = keep; M[i1] = keep;
+        Z[i0] = X[i0] * (T)keep;
+        Z[i1] = X[i1] * (T)keep;
+    }
+}
+template <typename T> __global__ void k_dropout_scale(const T* X, const T* rate, T* Z, size_t n, size_t m, size_t k)
+{
+    GRID_STRIDE(i, n) Z[i] = X[i] * ((T)1 - rate[(i / k) % m]);
+}
+template <typename T> __global__ void k_dropout_bp_tr(const T* dZ, const uint8_t* M, T* dX, size_t n)
+{
+    GRID_STRIDE(i, n) dX[i] = dZ[i] * (T)(M[i] != 0);
+}
+__global__ void k_dropoutord(const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, const float* U, uint64_t seed, uint64_t offset)
+{
+    GRID_STRIDE(i, n) {
+        float u = U ? U[i] : uniform_at(seed, offset, i);
+        bool keep = u >= rate;
+        uint8_t x = X[i];
+        M[i] = keep;
+        Z[i] = (keep || x == 255) ? x : (uint8_t)254;
+    }
+}
+template <typename T> __global__ void k_add_rowvec(const T* X, const T* b, T* Z, size_t n, size_t m)
+{
+    GRID_STRIDE(i, n * m) Z[i] = X[i] + b[i % m];
+}
+// one thread per column, rows in ascending order (fixed summation order)
+template <typename T> __global__ void k_colsum(const T* X, T* out, size_t n, size_t m)
+{
+    GRID_STRIDE(c, m) {
+        T s = (T)0;
+        for (size_t r = 0; r < n; ++r) s += X[r * m + c];
+        out[c] = s;
+    }
+}
+template <typename T> __global__ void k_relu(const T* X, T* Z, size_t n)
+{
+    GRID_STRIDE(i, n) Z[i] = X[i] > (T)0 ? X[i] : (T)0;   // NaN -> 0, as fmax(0, x)
+}
+template <typename T> __global__ void k_mul_sign(const T* dZ, const T* Z, T* dX, size_t n)
+{
+    GRID_STRIDE(i, n) {
+        T z = Z[i];
+        T s = (T)(z > (T)0) - (T)(z < (T)0);
+        dX[i] = dZ[i] * s;
+    }
+}
+template <typename T> __global__ void k_logistic(const T* X, T* Z, size_t n)
+{
+    GRID_STRIDE(i, n) Z[i] = (T)1 / ((T)1 + exp(-X[i]));
+}
+template <typename T> __global__ void k_loss_terms(int kind, const T* Z, const T* Y, T* L, size_t n)
+{
+    GRID_STRIDE(i, n) {
+        T z = Z[i], y = Y[i];
+        if (kind == 0) {
+            T a = z > (T)1e-15 ? z : (T)1e-15;
+            T b = ((T)1 - z) > (T)1e-15 ? ((T)1 - z) : (T)1e-15;
+            L[i] = log(a) * y + log(b) * ((T)1 - y);
+        } else {
+            T d = z - y;
+            L[i] = d * d;
+        }
+    }
+}
+__global__ void k_uniform_fill(float* U, size_t n, uint64_t seed, uint64_t offset)
+{
+    GRID_STRIDE(i, n) U[i] = uniform_at(seed, offset, i);
+}
+template <typename T> __global__ void k_sub_scale(const T* Z, const T* Y, T scale, T* dZ, size_t n)
+{
+    GRID_STRIDE(i, n) dZ[i] = (Z[i] - Y[i]) * scale;
+}
+
+}  // namespace
+
+#define F32(p) ((float*)(p))
+#define CF32(p) ((const float*)(p))
+#define F64(p) ((double*)(p))
+#define CF64(p) ((const double*)(p))
+
+// The typed pointer casts differ per dtype, so each entry point spells out both launches.
+#define EW2(kernel, n, ARGS32, ARGS64)                                                                     \
+    do {                                                                                                   \
+        DBK_DTYPE_OK(dtype);                                                                               \
+        if ((n) == 0) { dbk::clear_error(); return 0; }                                                    \
+        if (dtype == DBK_F32) hipLaunchKernelGGL(kernel<float>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), ARGS32); \
+        else hipLaunchKernelGGL(kernel<double>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), ARGS64);                  \
+        DBK_LAUNCH_OK();                                                                                   \
+    } while (0)
+#define A(...) __VA_ARGS__
+
+extern "C" {
+
+int dbk_gradstep(dbk_stream_t stream, int dtype, size_t n, void* P, const void* dP, const void* drate, void* mP, const void* mrate)
+{
+    EW2(k_gradstep, n, A(F32(P), CF32(dP), CF32(drate), F32(mP), CF32(mrate), n), A(F64(P), CF64(dP), CF64(drate), F64(mP), CF64(mrate), n));
+}
+int dbk_gradstep_nesterov1(dbk_stream_t stream, int dtype, size_t n, void* P, const void* mP, const void* mrate)
+{
+    EW2(k_nesterov1, n, A(F32(P), CF32(mP), CF32(mrate), n), A(F64(P), CF64(mP), CF64(mrate), n));
+}
+int dbk_gradstep_nesterov2(dbk_stream_t stream, int dtype, size_t n, void* P, const void* dP, const void* drate, void* mP, const void* mrate)
+{
+    EW2(k_nesterov2, n, A(F32(P), CF32(dP), CF32(drate), F32(mP), CF32(mrate), n), A(F64(P), CF64(dP), CF64(drate), F64(mP), CF64(mrate), n));
+}
+int dbk_madd_bcast(dbk_stream_t stream, int dtype, const void* A_, const void* b, void* dst, size_t n, size_t m, size_t k)
+{
+    DBK_CHECK(m >= 1 && k >= 1, "ValueError: madd_bcast needs m >= 1 and k >= 1");
+    EW2(k_madd_bcast, n, A(CF32(A_), CF32(b), F32(dst), n, m, k), A(CF64(A_), CF64(b), F64(dst), n, m, k));
+}
+int dbk_maskout(dbk_stream_t stream, int dtype, const uint8_t* M, void* A_, size_t n)
+{
+    EW2(k_maskout, n, A(M, F32(A_), n), A(M, F64(A_), n));
+}
+int dbk_calc_zmask(dbk_stream_t stream, int dtype, const void* Z, uint8_t* M, size_t n, size_t m)
+{
+    size_t half = (n * m) / 2;
+    EW2(k_calc_zmask, half, A(CF32(Z), M, n, m), A(CF64(Z), M, n, m));
+}
+
+static int dropout_fp_tr_impl(dbk_stream_t stream, int dtype, const void* X, const void* rate, void* Z, uint8_t* M,
+                              size_t n, size_t m, size_t k, int matchrows, const float* U, uint64_t seed, uint64_t offset)
+{
+    DBK_CHECK(m >= 1 && k >= 1, "ValueError: dropout needs at least one rate and one column per rate");
+    if (matchrows) {
+        size_t ncol = m * k, nrow = n / ncol, half = n / 2;
+        DBK_CHECK(nrow % 2 == 0, "ValueError: matchrows needs an even number of rows, got %zu", nrow);
+        EW2(k_dropout_fp_tr_match, half, A(CF32(X), CF32(rate), F32(Z), M, nrow, ncol, k, U, seed, offset),
+            A(CF64(X), CF64(rate), F64(Z), M, nrow, ncol, k, U, seed, offset));
+    }
+    EW2(k_dropout_fp_tr, n, A(CF32(X), CF32(rate), F32(Z), M, n, m, k, U, seed, offset),
+        A(CF64(X), CF64(rate), F64(Z), M, n, m, k, U, seed, offset));
+}
+int dbk_dropout_fp_tr(dbk_stream_t stream, int dtype, const void* X, const void* rate, void* Z, uint8_t* M,
+                      size_t n, size_t m, size_t k, int matchrows, uint64_t seed, uint64_t offset)
+{
+    return dropout_fp_tr_impl(stream, dtype, X, rate, Z, M, n, m, k, matchrows, nullptr, seed, offset);
+}
+int dbk_dropout_fp_tr_u(dbk_stream_t stream, int dtype, const void* X, const void* rate, void* Z, uint8_t* M,
+                        size_t n, size_t m, size_t k, int matchrows, const float* U)
+{
+    DBK_CHECK(U != nullptr, "ValueError: U must not be null");
+    return dropout_fp_tr_impl(stream, dtype, X, rate, Z, M, n, m, k, matchrows, U, 0, 0);
+}
+int dbk_dropout_fp_te(dbk_stream_t stream, int dtype, const void* X, const void* rate, void* Z, size_t n, size_t m, size_t k)
+{
+    DBK_CHECK(m >= 1 && k >= 1, "ValueError: dropout needs at least one rate and one column per rate");
+    EW2(k_dropout_scale, n, A(CF32(X), CF32(rate), F32(Z), n, m, k), A(CF64(X), CF64(rate), F64(Z), n, m, k));
+}
+int dbk_dropout_bp_tr(dbk_stream_t stream, int dtype, const void* dZ, const uint8_t* M, void* dX, size_t n)
+{
+    EW2(k_dropout_bp_tr, n, A(CF32(dZ), M, F32(dX), n), A(CF64(dZ), M, F64(dX), n));
+}
+int dbk_dropout_bp_te(dbk_stream_t stream, int dtype, const void* dZ, const void* rate, void* dX, size_t n, size_t m, size_t k)
+{
+    DBK_CHECK(m >= 1 && k >= 1, "ValueError: dropout needs at least one rate and one column per rate");
+    EW2(k_dropout_scale, n, A(CF32(dZ), CF32(rate), F32(dX), n, m, k), A(CF64(dZ), CF64(rate), F64(dX), n, m, k));
+}
+int dbk_dropoutord_fp_tr(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, uint64_t seed, uint64_t offset)
+{
+    if (n == 0) { dbk::clear_error(); return 0; }
+    hipLaunchKernelGGL(k_dropoutord, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), X, Z, M, n, rate, (const float*)nullptr, seed, offset);
+    DBK_LAUNCH_OK();
+}
+int dbk_dropoutord_fp_tr_u(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, const float* U)
+{
+    DBK_CHECK(U != nullptr, "ValueError: U must not be null");
+    if (n == 0) { dbk::clear_error(); return 0; }
+    hipLaunchKernelGGL(k_dropoutord, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), X, Z, M, n, rate, U, (uint64_t)0, (uint64_t)0);
+    DBK_LAUNCH_OK();
+}
+int dbk_add_rowvec(dbk_stream_t stream, int dtype, const void* X, const void* b, void* Z, size_t n, size_t m)
+{
+    size_t total = n * m;
+    EW2(k_add_rowvec, total, A(CF32(X), CF32(b), F32(Z), n, m), A(CF64(X), CF64(b), F64(Z), n, m));
+}
+int dbk_colsum(dbk_stream_t stream, int dtype, const void* X, void* out, size_t n, size_t m)
+{
+    EW2(k_colsum, m, A(CF32(X), F32(out), n, m), A(CF64(X), F64(out), n, m));
+}
+int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
+{
+    EW2(k_relu, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
+}
+int dbk_mul_sign(dbk_stream_t stream, int dtype, const void* dZ, const void* Z, void* dX, size_t n)
+{
+    EW2(k_mul_sign, n, A(CF32(dZ), CF32(Z), F32(dX), n), A(CF64(dZ), CF64(Z), F64(dX), n));
+}
+int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
+{
+    EW2(k_logistic, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
+}
+int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, const void* Y, void* L, size_t n)
+{
+    DBK_CHECK(kind == 0 || kind == 1, "ValueError: loss kind must be 0 (nll) or 1 (mse), got %d", kind);
+    EW2(k_loss_terms, n, A(kind, CF32(Z), CF32(Y), F32(L), n), A(kind, CF64(Z), CF64(Y), F64(L), n));
+}
+int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n)
+{
+    EW2(k_sub_scale, n, A(CF32(Z), CF32(Y), (float)scale, F32(dZ), n), A(CF64(Z), CF64(Y), scale, F64(dZ), n));
+}
+
+int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uint64_t offset)
+{
+    if (n == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(U != nullptr, "ValueError: U must not be null");
+    hipLaunchKernelGGL(k_uniform_fill, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), U, n, seed, offset);
+    DBK_LAUNCH_OK();
+}
+
+// Test hook: the raw Philox block function, so the host can check it against published vectors.
+int dbk_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4])
+{
+    uint32_t c[4] = {ctr[0], ctr[1], ctr[2], ctr[3]};
+    philox4x32_10(c, key[0], key[1]);
+    for (int i = 0; i < 4; ++i) out[i] = c[i];
+    return 0;
+}
+
+}  // extern "C"

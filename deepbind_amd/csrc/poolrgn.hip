@@ -1,0 +1,195 @@
+// Region pooling over the rows of an (N, F) feature map and its gradient.
+//
+// One thread per (region, column): the 64 lanes of a wave take 64 consecutive columns, so every
+// row visit is one coalesced 256-byte read (or read-modify-write) of HBM. Rows are visited in
+// ascending order, which fixes both the argmax tie rule (first strict maximum) and the order of
+// the running sum.
+//
+// Reference semantics: kangaroo_smat/poolrgn.cuh:44-160 (forward), poolrgn_bprop.cuh:45-127 (gradient).
+#include "dbk_common.h"
+
+namespace {
+
+struct region_t { size_t a, b, step, count; };
+
+__device__ __forceinline__ region_t load_region(const uint32_t* __restrict__ R, size_t r, bool per_step)
+{
+    const uint32_t* p = R + r * (per_step ? 3 : 2);
+    region_t g;
+    g.a = p[0];
+    g.b = p[1];
+    g.step = per_step ? p[2] : 1;
+    if (g.step == 0) g.step = 1;
+    g.count = (g.b - g.a + g.step - 1) / g.step;
+    return g;
+}
+
+template <typename T, int PT>
+__global__ __launch_bounds__(256) void poolrgn_kernel(const T* __restrict__ U, size_t F, const uint32_t* __restrict__ R,
+                                                      size_t P, bool per_step, T* __restrict__ pooled,
+                                                      uint32_t* __restrict__ argmax)
+{
+    const size_t f = (size_t)blockIdx.y * 64 + (threadIdx.x & 63);
+    const size_t r = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (f >= F || r >= P) return;
+    const region_t g = load_region(R, r, per_step);
+    size_t xi = g.a * F + f;
+    T x = U[xi];
+    T y = x;
+    for (size_t i = g.a + g.step; i < g.b; i += g.step) {
+        const T v = U[i * F + f];
+        if (PT == DBK_PT_MAX || PT == DBK_PT_ALL) {
+            if (v > x) { x = v; xi = i * F + f; }
+        }
+        if (PT != DBK_PT_MAX) y += v;
+    }
+    const size_t j = r * F + f;
+    if (PT == DBK_PT_MAX) {
+        pooled[j] = x;
+    } else if (PT == DBK_PT_SUM) {
+        pooled[j] = y;
+    } else if (PT == DBK_PT_AVG) {
+        pooled[j] = y / (T)g.count;
+    } else {
+        pooled[2 * j] = x;
+        pooled[2 * j + 1] = y / (T)g.count;
+    }
+    if ((PT == DBK_PT_MAX || PT == DBK_PT_ALL) && argmax) argmax[j] = (uint32_t)xi;
+}
+
+// flag[0] = 1 when regions are sorted, unit-step and non-overlapping (each map element then has a
+// single writer in the gradient kernel), else 0.
+__global__ void regions_disjoint_kernel(const uint32_t* __restrict__ R, size_t P, bool per_step, unsigned* flag)
+{
+    __shared__ unsigned bad;
+    if (threadIdx.x == 0) bad = 0;
+    __syncthreads();
+    unsigned mine = 0;
+    const unsigned rc = per_step ? 3 : 2;
+    for (size_t r = threadIdx.x; r < P; r += blockDim.x) {
+        if (R[r * rc + 1] < R[r * rc]) mine = 1;
+        if (per_step && R[r * rc + 2] != 1) mine = 1;
+        if (r + 1 < P && R[(r + 1) * rc] < R[r * rc + 1]) mine = 1;
+    }
+    if (mine) atomicOr(&bad, 1u);
+    __syncthreads();
+    if (threadIdx.x == 0) flag[0] = bad ? 0u : 1u;
+}
+
+template <bool ATOMIC, typename T>
+__device__ __forceinline__ void accumulate(T* p, T v)
+{
+    if (ATOMIC) atomicAdd(p, v);
+    else *p += v;
+}
+
+// ATOMIC=false runs when flag says "disjoint" (plain read-modify-write, reproducible);
+// ATOMIC=true runs otherwise (overlapping regions: same accumulation races as any scatter-add).
+template <typename T, int PT, bool ATOMIC>
+__global__ __launch_bounds__(256) void poolrgn_bprop_kernel(T* __restrict__ dU, size_t F, size_t nelem_map,
+                                                            const uint32_t* __restrict__ R, size_t P, bool per_step,
+                                                            const T* __restrict__ dP, const uint32_t* __restrict__ argmax,
+                                                            const unsigned* __restrict__ flag)
+{
+    const bool disjoint = flag[0] != 0;
+    if (disjoint == ATOMIC) return;
+    const size_t f = (size_t)blockIdx.y * 64 + (threadIdx.x & 63);
+    const size_t r = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (f >= F || r >= P) return;
+    const region_t g = load_region(R, r, per_step);
+    const size_t j = r * F + f;
+    // the argmax scatter is always atomic: the index is caller data and may point anywhere in the map
+    if (PT == DBK_PT_MAX) {
+        atomicAdd(&dU[argmax[j]], dP[j]);
+        return;
+    }
+    T dy;
+    if (PT == DBK_PT_ALL) dy = dP[2 * j + 1] / (T)g.count;
+    else if (PT == DBK_PT_AVG) dy = dP[j] / (T)g.count;
+    else dy = dP[j];
+    for (size_t i = g.a; i < g.b; i += g.step) accumulate<ATOMIC>(&dU[i * F + f], dy);
+    if (PT == DBK_PT_ALL) atomicAdd(&dU[argmax[j]], dP[2 * j]);
+}
+
+template <typename T>
+int launch_fwd(hipStream_t st, const T* U, size_t F, const uint32_t* R, size_t P, bool per_step, T* pooled,
+               uint32_t* argmax, int ptype)
+{
+    dim3 grid(dbk::divup(P, 4), dbk::divup(F, 64)), block(256);
+    DBK_CHECK(grid.y <= 65535u, "ValueError: too many feature maps (%zu) for one launch", F);
+    switch (ptype) {
+    case DBK_PT_MAX: hipLaunchKernelGGL((poolrgn_kernel<T, DBK_PT_MAX>), grid, block, 0, st, U, F, R, P, per_step, pooled, argmax); break;
+    case DBK_PT_AVG: hipLaunchKernelGGL((poolrgn_kernel<T, DBK_PT_AVG>), grid, block, 0, st, U, F, R, P, per_step, pooled, argmax); break;
+    case DBK_PT_SUM: hipLaunchKernelGGL((poolrgn_kernel<T, DBK_PT_SUM>), grid, block, 0, st, U, F, R, P, per_step, pooled, argmax); break;
+    default:         hipLaunchKernelGGL((poolrgn_kernel<T, DBK_PT_ALL>), grid, block, 0, st, U, F, R, P, per_step, pooled, argmax); break;
+    }
+    DBK_LAUNCH_OK();
+}
+
+template <typename T, int PT>
+void launch_bwd_pt(hipStream_t st, T* dU, size_t F, const uint32_t* R, size_t P, bool per_step, const T* dP,
+                   const uint32_t* argmax, const unsigned* flag)
+{
+    dim3 grid(dbk::divup(P, 4), dbk::divup(F, 64)), block(256);
+    hipLaunchKernelGGL((poolrgn_bprop_kernel<T, PT, false>), grid, block, 0, st, dU, F, (size_t)0, R, P, per_step, dP, argmax, flag);
+    hipLaunchKernelGGL((poolrgn_bprop_kernel<T, PT, true>), grid, block, 0, st, dU, F, (size_t)0, R, P, per_step, dP, argmax, flag);
+}
+
+template <typename T>
+int launch_bwd(hipStream_t st, T* dU, size_t F, const uint32_t* R, size_t P, bool per_step, const T* dP,
+               const uint32_t* argmax, int ptype)
+{
+    DBK_CHECK(dbk::divup(F, 64) <= 65535u, "ValueError: too many feature maps (%zu) for one launch", F);
+    unsigned* flag = (unsigned*)dbk::workspace(256);
+    DBK_CHECK(flag != nullptr, "MemoryError: could not allocate scratch");
+    hipLaunchKernelGGL(regions_disjoint_kernel, dim3(1), dim3(1024), 0, st, R, P, per_step, flag);
+    switch (ptype) {
+    case DBK_PT_MAX: launch_bwd_pt<T, DBK_PT_MAX>(st, dU, F, R, P, per_step, dP, argmax, flag); break;
+    case DBK_PT_AVG: launch_bwd_pt<T, DBK_PT_AVG>(st, dU, F, R, P, per_step, dP, argmax, flag); break;
+    case DBK_PT_SUM: launch_bwd_pt<T, DBK_PT_SUM>(st, dU, F, R, P, per_step, dP, argmax, flag); break;
+    default:         launch_bwd_pt<T, DBK_PT_ALL>(st, dU, F, R, P, per_step, dP, argmax, flag); break;
+    }
+    DBK_LAUNCH_OK();
+}
+
+}  // namespace
+
+extern "C" {
+
+int dbk_poolrgn(dbk_stream_t stream, int dtype, const void* unpooledmaps, size_t nfeaturemap,
+                const uint32_t* regions, size_t nregion, int per_region_step,
+                void* pooledmaps, uint32_t* pooledmaps_argmax, int ptype)
+{
+    DBK_DTYPE_OK(dtype);
+    DBK_CHECK(ptype >= DBK_PT_MAX && ptype <= DBK_PT_ALL, "ValueError: unknown pooling type %d", ptype);
+    DBK_CHECK(!pooledmaps_argmax || ptype == DBK_PT_MAX || ptype == DBK_PT_ALL,
+              "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
+    if (nfeaturemap == 0 || nregion == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(unpooledmaps && regions && pooledmaps, "ValueError: null pointer argument");
+    if (dtype == DBK_F32)
+        return launch_fwd<float>(dbk::as_stream(stream), (const float*)unpooledmaps, nfeaturemap, regions, nregion,
+                                 per_region_step != 0, (float*)pooledmaps, pooledmaps_argmax, ptype);
+    return launch_fwd<double>(dbk::as_stream(stream), (const double*)unpooledmaps, nfeaturemap, regions, nregion,
+                              per_region_step != 0, (double*)pooledmaps, pooledmaps_argmax, ptype);
+}
+
+int dbk_poolrgn_bprop(dbk_stream_t stream, int dtype, void* unpooledmaps, size_t nfeaturemap,
+                      const uint32_t* regions, size_t nregion, int per_region_step,
+                      const void* pooledmaps, const uint32_t* pooledmaps_argmax, int ptype)
+{
+    DBK_DTYPE_OK(dtype);
+    DBK_CHECK(ptype >= DBK_PT_MAX && ptype <= DBK_PT_ALL, "ValueError: unknown pooling type %d", ptype);
+    if (ptype == DBK_PT_MAX || ptype == DBK_PT_ALL)
+        DBK_CHECK(pooledmaps_argmax != nullptr, "ValueError: pooledmaps_argmax must be specified for max pooling.");
+    else
+        DBK_CHECK(pooledmaps_argmax == nullptr, "ValueError: pooledmaps_argmax can only be specified for max pooling.");
+    if (nfeaturemap == 0 || nregion == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(unpooledmaps && regions && pooledmaps, "ValueError: null pointer argument");
+    if (dtype == DBK_F32)
+        return launch_bwd<float>(dbk::as_stream(stream), (float*)unpooledmaps, nfeaturemap, regions, nregion,
+                                 per_region_step != 0, (const float*)pooledmaps, pooledmaps_argmax, ptype);
+    return launch_bwd<double>(dbk::as_stream(stream), (double*)unpooledmaps, nfeaturemap, regions, nregion,
+                              per_region_step != 0, (const double*)pooledmaps, pooledmaps_argmax, ptype);
+}
+
+}  // extern "C"

@@ -1,0 +1,66 @@
+// Error state, version, device count, sync and the scratch workspace.
+#include "dbk_common.h"
+#include <cstring>
+#include <mutex>
+
+namespace dbk {
+
+static thread_local char g_err[512] = {0};
+
+void set_error(const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+void clear_error() { g_err[0] = 0; }
+
+struct ws_t { void* ptr = nullptr; size_t bytes = 0; };
+static ws_t g_ws[64];
+static std::mutex g_ws_mutex;
+
+void* workspace(size_t bytes)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    ws_t& w = g_ws[dev];
+    if (w.bytes >= bytes && w.ptr) return w.ptr;
+    if (w.ptr) {
+        // earlier launches may still be reading the old buffer
+        if (hipDeviceSynchronize() != hipSuccess) return nullptr;
+        (void)hipFree(w.ptr);
+        w.ptr = nullptr;
+        w.bytes = 0;
+    }
+    size_t want = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes + bytes / 4;
+    if (hipMalloc(&w.ptr, want) != hipSuccess) { w.ptr = nullptr; return nullptr; }
+    w.bytes = want;
+    return w.ptr;
+}
+
+}  // namespace dbk
+
+extern "C" {
+
+const char* dbk_last_error(void) { return dbk::g_err; }
+
+int dbk_version(void) { return 1; }
+
+int dbk_device_count(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return -1;
+    return n;
+}
+
+int dbk_sync(dbk_stream_t stream)
+{
+    DBK_HIP(hipStreamSynchronize(dbk::as_stream(stream)));
+    dbk::clear_error();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,150 @@
+"""Sequence operators over device tensors: same names, argument order and in-place conventions
+as the reference's operator shim (reference: code/libs/kangaroo/kangaroo/_ext/kangaroo_smat.py:86-146),
+plus the fused scan+pool entry points. Arrays are torch tensors on the GPU; all arithmetic happens
+in libdeepbind_hip.so on the current HIP stream.
+"""
+import torch
+
+from . import _lib
+from ._lib import DeepbindError, call, dtype_code, ptr, require, str2pooltype, stream
+
+uindex = torch.uint32
+
+_rng_seed = 0
+_rng_offset = 0
+
+
+def set_seed(seed):
+    """Seeds the generator behind dropoutord_fp_train (and resets its stream position)."""
+    global _rng_seed, _rng_offset
+    _rng_seed, _rng_offset = int(seed), 0
+
+
+def _u8(X):
+    require(X.dtype == torch.uint8, "TypeError: X must be uint8, got %s" % X.dtype)
+    return X
+
+
+def _regions(R):
+    require(R.dtype in (torch.uint32, torch.int32), "TypeError: regions must be uint32, got %s" % R.dtype)
+    require(R.dim() == 2 and R.shape[1] in (2, 3), "ValueError: regions array must have 2 or 3 columns.")
+    return R
+
+
+def corr1ord(W, X, Z, nchannel):
+    """Cross-correlates the filter bank W ((M*nchannel) x P) with the ordinal vector X (N uint8,
+    values 0..nchannel-1, 255 = all ordinals, 254 = none) into Z (N x P). The final M-1 rows of Z
+    are left untouched. reference: kangaroo_smat.py:86-99, kangaroo_smat.cpp:98-124"""
+    _u8(X)
+    require(W.shape[0] % nchannel == 0, "ValueError: W rows must be a multiple of nchannel")
+    require(W.dtype == Z.dtype, "TypeError: W dtype must match Z dtype")
+    require(Z.shape[1] == W.shape[1], "ValueError: Z must have one column per filter")
+    require(Z.shape[0] == X.numel(), "ValueError: Z must have one row per element of X")
+    m = W.shape[0] // nchannel
+    n = X.numel() - m + 1
+    if n <= 0:
+        return
+    call("dbk_corr1ord", stream(), dtype_code(Z), ptr(W), m, W.shape[1], ptr(X), n, nchannel, ptr(Z))
+
+
+def corr1ord_bprop_W(dW, X, dZ, nchannel):
+    """Accumulates the filter gradient of corr1ord into dW. reference: kangaroo_smat.py:101-109"""
+    _u8(X)
+    require(dW.shape[0] % nchannel == 0, "ValueError: dW rows must be a multiple of nchannel")
+    require(dW.dtype == dZ.dtype, "TypeError: dW dtype must match dZ dtype")
+    require(dZ.shape[1] == dW.shape[1] and dZ.shape[0] == X.numel(), "ValueError: dZ must be N x P")
+    m = dW.shape[0] // nchannel
+    n = X.numel() - m + 1
+    if n <= 0:
+        return
+    call("dbk_corr1ord_bprop_W", stream(), dtype_code(dZ), ptr(dW), m, dW.shape[1], ptr(X), n, nchannel, ptr(dZ))
+
+
+def corr1ord_bprop_X(dX, W, dZ, nchannel):
+    """Accumulates the input gradient of corr1ord into dX (N x nchannel). reference: kangaroo_smat.py:111-119,
+    kangaroo_smat.cpp:141-168"""
+    require(W.shape[0] % nchannel == 0, "ValueError: W rows must be a multiple of nchannel")
+    require(W.dtype == dZ.dtype and dX.dtype == dZ.dtype, "TypeError: dX, W and dZ must share a dtype")
+    require(dX.shape[1] == nchannel, "ValueError: dX must have nchannel columns")
+    require(dZ.shape[1] == W.shape[1] and dZ.shape[0] == dX.shape[0], "ValueError: dZ must be N x P")
+    m = W.shape[0] // nchannel
+    call("dbk_corr1ord_bprop_X", stream(), dtype_code(dZ), ptr(dX), dX.shape[0], nchannel, ptr(W), m, W.shape[1], ptr(dZ))
+
+
+def poolrgn(unpooledmaps, regions, ptype, want_argmax=False):
+    """Pools rows of unpooledmaps (N x M) per region. Returns (pooled, argmax|None); "all" gives
+    (P x 2M) with (max, avg) at columns (2j, 2j+1). reference: kangaroo_smat.py:121-132"""
+    _regions(regions)
+    noutputs = 2 if ptype == "all" else 1
+    nregion, nfeaturemap = regions.shape[0], unpooledmaps.shape[1]
+    pooledmaps = torch.empty((nregion, nfeaturemap * noutputs), dtype=unpooledmaps.dtype, device=unpooledmaps.device)
+    argmax = None
+    if ptype in ("max", "all") and want_argmax:
+        argmax = torch.empty((nregion, nfeaturemap), dtype=uindex, device=unpooledmaps.device)
+    call("dbk_poolrgn", stream(), dtype_code(unpooledmaps), ptr(unpooledmaps), nfeaturemap, ptr(regions), nregion,
+         int(regions.shape[1] == 3), ptr(pooledmaps), ptr(argmax), str2pooltype[ptype])
+    return pooledmaps, argmax
+
+
+def poolrgn_bprop(unpooledmaps, regions, pooledmaps, pooledmaps_argmax, ptype):
+    """Accumulates the pooling gradient into unpooledmaps. reference: kangaroo_smat.py:134-138"""
+    _regions(regions)
+    nregion, nfeaturemap = regions.shape[0], unpooledmaps.shape[1]
+    noutputs = 2 if ptype == "all" else 1
+    require(unpooledmaps.dtype == pooledmaps.dtype, "TypeError: unpooledmaps dtype must match pooledmaps dtype.")
+    require(tuple(pooledmaps.shape) == (nregion, nfeaturemap * noutputs),
+            "ValueError: pooledmaps must be (regions x feature maps%s)." % (" x 2" if noutputs == 2 else ""))
+    amax = pooledmaps_argmax if (pooledmaps_argmax is not None and ptype in ("max", "all")) else None
+    if amax is not None:
+        require(tuple(amax.shape) == (nregion, nfeaturemap) and amax.dtype in (torch.uint32, torch.int32),
+                "ValueError: pooledmaps_argmax must be a (regions x feature maps) uint32 array.")
+    call("dbk_poolrgn_bprop", stream(), dtype_code(unpooledmaps), ptr(unpooledmaps), nfeaturemap, ptr(regions), nregion,
+         int(regions.shape[1] == 3), ptr(pooledmaps), ptr(amax), str2pooltype[ptype])
+
+
+def dropoutord_fp_train(X, rate, U=None):
+    """Input-base dropout: returns (Z, M) with dropped bases replaced by 254. U (optional, float32,
+    same shape) supplies the uniforms instead of the library's generator. reference: kangaroo_smat.py:140-146"""
+    global _rng_offset
+    _u8(X)
+    Z = torch.empty_like(X)
+    M = torch.empty(X.shape, dtype=torch.bool, device=X.device)
+    n = X.numel()
+    if U is not None:
+        require(U.dtype == torch.float32 and U.numel() == n, "ValueError: U must be float32 with one value per element")
+        call("dbk_dropoutord_fp_tr_u", stream(), ptr(X), ptr(Z), ptr(M), n, float(rate), ptr(U))
+    else:
+        call("dbk_dropoutord_fp_tr", stream(), ptr(X), ptr(Z), ptr(M), n, float(rate), _rng_seed, _rng_offset)
+        _rng_offset += (n + 3) // 4
+    return Z, M
+
+
+# ------------------------------------------------------------------------------------------------
+# fused scan + bias + ReLU + pool
+# ------------------------------------------------------------------------------------------------
+def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, general=False):
+    """pool(relu(corr1ord(W, X) + b)) per region without storing the (N x P) map.
+    Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only."""
+    _u8(X)
+    _regions(regions)
+    require(regions.shape[1] == 2, "ValueError: the fused path takes 2-column regions")
+    require(W.dtype == torch.float32 and b.dtype == torch.float32, "TypeError: the fused path is float32 only")
+    require(W.shape[0] % 4 == 0 and b.numel() == W.shape[1], "ValueError: W must be (4m x P) and b must have P entries")
+    m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
+    pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
+    argmax = torch.empty((P, F), dtype=uindex, device=W.device) if (want_argmax and ptype in ("max", "all")) else None
+    call("dbk_scanpool_fprop_general" if general else "dbk_scanpool_fprop", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(),
+         ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax))
+    return pooled, argmax
+
+
+def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db):
+    """Backward of scanpool_fprop: dW += filter gradient, db[:] = bias gradient."""
+    _u8(X)
+    _regions(regions)
+    require(W.dtype == torch.float32 and dpooled.dtype == torch.float32, "TypeError: the fused path is float32 only")
+    require(dW.shape == W.shape and db.numel() == W.shape[1], "ValueError: dW / db shapes must match W / b")
+    require(dpooled.shape == pooled.shape, "ValueError: dpooled must have pooled's shape")
+    m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
+    call("dbk_scanpool_bprop", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype],
+         ptr(pooled), ptr(argmax), ptr(dpooled), ptr(dW), ptr(db))

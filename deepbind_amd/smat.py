@@ -1,0 +1,98 @@
+"""The few array operations the bias / ReLU / dense / loss nodes call, over device tensors.
+Names follow the reference's array module (reference: code/libs/smat/py/smat/smat.py), but only the
+operations on the motif-scan path exist here, each backed by a kernel in libdeepbind_hip.so.
+torch supplies device memory and the stream; it does no arithmetic on this path.
+"""
+import torch
+
+from ._lib import call, dtype_code, ptr, require, stream
+from . import deepity_smat as _ds
+
+
+def zeros(shape, dtype=torch.float32, device="cuda"):
+    return torch.zeros(shape, dtype=dtype, device=device)
+
+
+def zeros_like(A):
+    return torch.zeros_like(A)
+
+
+def empty(shape, dtype=torch.float32, device="cuda"):
+    return torch.empty(shape, dtype=dtype, device=device)
+
+
+def empty_like(A):
+    return torch.empty_like(A)
+
+
+def asarray(a, dtype=None, device="cuda"):
+    return torch.as_tensor(a, dtype=dtype).to(device).contiguous()
+
+
+def sync():
+    call("dbk_sync", stream())
+
+
+def dot(A, B):
+    """A (n x k) . B (k x m). reference: smat_cuda/dot.cu:50-67"""
+    return _ds.blockwise_dot(A, B, 1)
+
+
+def dot_nt(A, B):
+    """A (n x m) . B (k x m)^T -> (n x k)."""
+    return _ds.blockwise_dot_nt(A, B, 1)
+
+
+def dot_tn(A, B):
+    """A (n x k)^T . B (n x m) -> (k x m)."""
+    W = torch.empty((A.shape[1], B.shape[1]), dtype=A.dtype, device=A.device)
+    return _ds.blockwise_dot_tn(A, B, 1, W)
+
+
+def add_rowvec(X, b):
+    """X + b with the row vector b broadcast down the rows (the bias node's forward)."""
+    require(b.numel() == X.shape[1] and b.dtype == X.dtype, "ValueError: b must have one entry per column of X")
+    Z = torch.empty_like(X)
+    call("dbk_add_rowvec", stream(), dtype_code(X), ptr(X), ptr(b), ptr(Z), X.shape[0], X.shape[1])
+    return Z
+
+
+def sum_axis0(X):
+    """Column sums as a (1 x ncol) row (the bias node's gradient)."""
+    out = torch.empty((1, X.shape[1]), dtype=X.dtype, device=X.device)
+    call("dbk_colsum", stream(), dtype_code(X), ptr(X), ptr(out), X.shape[0], X.shape[1])
+    return out
+
+
+def relu(X):
+    """maximum(0, X)."""
+    Z = torch.empty_like(X)
+    call("dbk_relu", stream(), dtype_code(X), ptr(X), ptr(Z), X.numel())
+    return Z
+
+
+def mul_sign(dZ, Z):
+    """dZ * sign(Z): the ReLU node's gradient."""
+    dX = torch.empty_like(dZ)
+    call("dbk_mul_sign", stream(), dtype_code(dZ), ptr(dZ), ptr(Z), ptr(dX), dZ.numel())
+    return dX
+
+
+def logistic(X):
+    Z = torch.empty_like(X)
+    call("dbk_logistic", stream(), dtype_code(X), ptr(X), ptr(Z), X.numel())
+    return Z
+
+
+def loss_terms(Z, Y, kind):
+    """Elementwise loss terms before masking / averaging; kind is "nll" or "mse"."""
+    L = torch.empty_like(Z)
+    call("dbk_loss_terms", stream(), dtype_code(Z), {"nll": 0, "mse": 1}[kind], ptr(Z), ptr(Y), ptr(L), Z.numel())
+    return L
+
+
+def sub_scale(Z, Y, scale):
+    """(Z - Y) * scale."""
+    dZ = torch.empty_like(Z)
+    call("dbk_sub_scale", stream(), dtype_code(Z), ptr(Z), ptr(Y), float(scale), ptr(dZ), Z.numel())
+    return dZ

@@ -1,0 +1,240 @@
+/* deepbind_hip.h - C ABI of libdeepbind_hip.so (gfx950 / MI355X).
+ *
+ * Every entry point is the raw-pointer form of one of the reference's internal launch
+ * functions (the layer its C++ `api_*` exports dispatch to), with
+ *   - a hipStream_t (passed as void*) where the reference takes a cudaStream_t,
+ *   - an int status return (0 = ok) plus dbk_last_error(), which keeps the reference's
+ *     poll-after-every-call convention (reference: smat/py/smat/smat_dll.py:166-183,
+ *     smat/src/smat/config.h:95-105),
+ *   - device pointers only; no call allocates its outputs (the caller does, as the
+ *     reference's Python wrappers do: kangaroo/_ext/kangaroo_smat.py:121-132).
+ * Matrices are row-major with full stride; "filter fastest" layouts are the reference's.
+ * Calls are asynchronous on `stream`, ordered within it. One process per GPU; a context
+ * (device + scratch workspace) must not be shared between host threads without external
+ * locking, as in the reference (smat/src/smat/vm/context.cpp:71).
+ *
+ * All reference paths below are relative to /root/reference/code/libs.
+ */
+#ifndef DEEPBIND_HIP_H
+#define DEEPBIND_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* dbk_stream_t;                 /* hipStream_t */
+
+/* reference: smat/src/smat/dtypes.h (dtype_t); only the two float types reach these ops */
+enum { DBK_F32 = 0, DBK_F64 = 1 };
+
+/* reference: kangaroo/kangaroo_smat/kangaroo_smat.h:42-47 (pooltype_t) */
+enum { DBK_PT_MAX = 0, DBK_PT_AVG = 1, DBK_PT_SUM = 2, DBK_PT_ALL = 3 };
+
+/* Text of the last failure on the calling thread ("" if none); cleared by the next successful call.
+ * reference: api_get_last_error, smat/py/smat/smat_dll.py:166-183 */
+const char* dbk_last_error(void);
+/* Library/ABI version, bumped when a signature changes. */
+int dbk_version(void);
+/* Number of HIP devices visible; <0 on failure. Touches the runtime only to count devices. */
+int dbk_device_count(void);
+/* Blocks until `stream` has drained. reference: api_sync, smat_cuda/cuda_context.cpp:198-202 */
+int dbk_sync(dbk_stream_t stream);
+
+/* ------------------------------------------------------------------ motif scan (corr1ord) */
+
+/* Z[i,f] = sum_{j<m} w(j, X[i+j], f) for i < n, where w = W[(C*j+k)*F+f] for k<C, 0 for k==254,
+ * and the channel mean for any other code (255 = N / padding). n = number of outputs written
+ * (N-m+1); rows >= n of Z are left untouched. W is (C*m, F), X has n+m-1 bytes, Z is (>=n, F).
+ * reference: launch_corr1ord, kangaroo/kangaroo_smat/kangaroo_smat.cpp:43-46, corr1ord.cu:136-148 */
+int dbk_corr1ord(dbk_stream_t stream, int dtype,
+                 const void* W, size_t m, size_t nfilter,
+                 const uint8_t* X, size_t n, size_t nchannel,
+                 void* Z);
+
+/* dW[(C*j+k),f] += sum_{i<n} dZ[i,f] * [X[i+j]==k]; N/pad codes add dZ/C to all C rows, 254 nothing.
+ * Deterministic: per-workgroup private accumulators and a fixed-order reduction, no float atomics.
+ * reference: launch_corr1ord_bprop_W, kangaroo_smat.cpp:48-51, corr1ord_bprop.cu:97-108 */
+int dbk_corr1ord_bprop_W(dbk_stream_t stream, int dtype,
+                         void* dW, size_t m, size_t nfilter,
+                         const uint8_t* X, size_t n, size_t nchannel,
+                         const void* dZ);
+
+/* dX[i,c] += sum_f sum_{k<m, k<=i} dZ[i-k,f] * W[(C*k+c),f] for i < n; dX is (n, C), dZ is (n, F).
+ * Computed on the device (the reference copies to the host and loops there).
+ * reference: launch_corr1ord_bprop_X, kangaroo_smat.cpp:53-56, corr1ord_bprop.cu:167-224 */
+int dbk_corr1ord_bprop_X(dbk_stream_t stream, int dtype,
+                         void* dX, size_t n, size_t nchannel,
+                         const void* W, size_t m, size_t nfilter,
+                         const void* dZ);
+
+/* ------------------------------------------------------------------ region pooling (poolrgn) */
+
+/* Per region r = [R[r,0], R[r,1]) (optional third column = row step) and column f:
+ * max (first strict maximum, argmax = row*F+f as uint32), avg, sum, or all = (max,avg) interleaved
+ * at columns (2f, 2f+1). pooled is (P, F) or (P, 2F); argmax may be NULL.
+ * reference: launch_poolrgn, kangaroo_smat.cpp:71-74, poolrgn.cu:56-68 */
+int dbk_poolrgn(dbk_stream_t stream, int dtype,
+                const void* unpooledmaps, size_t nfeaturemap,
+                const uint32_t* regions, size_t nregion, int per_region_step,
+                void* pooledmaps, uint32_t* pooledmaps_argmax, int ptype);
+
+/* Accumulates into unpooledmaps (N, F): max adds pooled[r,f] at argmax[r,f]; avg/sum spread
+ * pooled[r,f](/count) over the region's rows; all does both from the interleaved pairs.
+ * Bit-reproducible whenever regions do not overlap (each element then has one writer).
+ * reference: launch_poolrgn_bprop, kangaroo_smat.cpp:76-79, poolrgn_bprop.cu:60-72 */
+int dbk_poolrgn_bprop(dbk_stream_t stream, int dtype,
+                      void* unpooledmaps, size_t nfeaturemap,
+                      const uint32_t* regions, size_t nregion, int per_region_step,
+                      const void* pooledmaps, const uint32_t* pooledmaps_argmax, int ptype);
+
+/* Input-base dropout: Z = keep ? X : 254, except X==255 which always passes; M = keep.
+ * keep = (u >= rate) with u from the library's counter-based generator (seed, offset).
+ * reference: launch_dropoutord_fp_tr, kangaroo_smat.cpp:81-82, dropoutord.cu:41-60 */
+int dbk_dropoutord_fp_tr(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n,
+                         float rate, uint64_t seed, uint64_t offset);
+/* Same with caller-supplied uniforms U (n floats) instead of the generator. */
+int dbk_dropoutord_fp_tr_u(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n,
+                           float rate, const float* U);
+
+/* ------------------------------------------------------------------ fused scan + bias + ReLU + pool */
+
+/* pooled[r, .] = pool_{i in region r} relu(scan(W,X)[i,f] + bias[f]) without materialising the
+ * (N, F) map. Regions have 2 columns. ptype per call (max / avg / all); pooled layout and argmax
+ * (flat row*F+f into the virtual map, may be NULL) exactly as dbk_poolrgn. X has N bytes; windows
+ * reaching past N contribute nothing (the unfused chain leaves those rows at relu(bias)).
+ * float32 only. Replaces the chain corr1ord -> bias -> relu -> poolrgn
+ * (reference: kangaroo/_ext/corr1ord.py:97-117, deepity/std/elemwise.py:71-82,162-180,
+ *  kangaroo/_ext/poolrgn.py:56-76,153-174). */
+int dbk_scanpool_fprop(dbk_stream_t stream,
+                       const float* W, const float* bias, size_t m, size_t nfilter,
+                       const uint8_t* X, size_t N,
+                       const uint32_t* regions, size_t nregion, int ptype,
+                       float* pooled, uint32_t* argmax);
+
+/* Same contract, always through the general kernel (any filter length that fits in LDS, any letter
+ * code); dbk_scanpool_fprop picks a faster kernel when the shape allows and otherwise calls this. */
+int dbk_scanpool_fprop_general(dbk_stream_t stream,
+                               const float* W, const float* bias, size_t m, size_t nfilter,
+                               const uint8_t* X, size_t N,
+                               const uint32_t* regions, size_t nregion, int ptype,
+                               float* pooled, uint32_t* argmax);
+
+/* Backward of the fused chain: given dpooled (same layout as pooled), the forward's pooled and
+ * argmax, accumulates dW (C*m, F) += and writes dbias (1, F) =. Deterministic (no float atomics).
+ * reference chain: poolrgn_bprop -> relu bprop -> bias bprop -> corr1ord_bprop_W
+ * (kangaroo/_ext/poolrgn.py:78-82, deepity/std/elemwise.py:78,172-180, kangaroo/_ext/corr1ord.py:120-138) */
+int dbk_scanpool_bprop(dbk_stream_t stream,
+                       const float* W, const float* bias, size_t m, size_t nfilter,
+                       const uint8_t* X, size_t N,
+                       const uint32_t* regions, size_t nregion, int ptype,
+                       const float* pooled, const uint32_t* argmax, const float* dpooled,
+                       float* dW, float* dbias);
+
+/* ------------------------------------------------------------------ dense head (deepity_smat) */
+
+/* Z[:, b*m:(b+1)*m] = X_b . W[b*k:(b+1)*k, :]; X_b = X[:, b*k:(b+1)*k], or all of X (n x k) when
+ * broadcast_x. X (n, k*nblock | k), W (k*nblock, m), Z (n, m*nblock).
+ * reference: launch_blockwise_dot, deepity/deepity_smat/deepity_smat.cpp:75-77, blockwise_dot.cu:77-105 */
+int dbk_blockwise_dot(dbk_stream_t stream, int dtype, int nblock, int n, int m, int k, int broadcast_x,
+                      const void* X, const void* W, void* Z);
+/* dX[:, b*k:(b+1)*k] = dZ[:, b*m:(b+1)*m] . W[b*k:(b+1)*k, :]^T
+ * reference: launch_blockwise_dot_nt, deepity_smat.cpp:79-81, blockwise_dot.cu:110-130 */
+int dbk_blockwise_dot_nt(dbk_stream_t stream, int dtype, int nblock, int n, int m, int k,
+                         const void* dZ, const void* W, void* dX);
+/* dW[b*k:(b+1)*k, :] = X_b^T . dZ[:, b*m:(b+1)*m]
+ * reference: launch_blockwise_dot_tn, deepity_smat.cpp:83-85, blockwise_dot.cu:132-153 */
+int dbk_blockwise_dot_tn(dbk_stream_t stream, int dtype, int nblock, int n, int m, int k, int broadcast_x,
+                         const void* X, const void* dZ, void* dW);
+/* "combined" forms: W is (p*nblock, m); this input occupies rows [Xoffset, Xoffset+k) of each
+ * model's block of p rows. The forward overwrites Z when Xoffset==0 and adds otherwise.
+ * reference: launch_blockwise_dot_combined / _nt_combined / _tn_combined,
+ * deepity_smat.cpp:87-100, blockwise_dot.cu:156-260 */
+int dbk_blockwise_dot_combined(dbk_stream_t stream, int dtype, int nblock, int Xoffset, int Xbroadcast,
+                               int n, int m, int k, int p, const void* X, const void* W, void* Z);
+int dbk_blockwise_dot_nt_combined(dbk_stream_t stream, int dtype, int nblock, int Xoffset,
+                                  int n, int m, int k, int p, void* dX, const void* W, const void* dZ);
+int dbk_blockwise_dot_tn_combined(dbk_stream_t stream, int dtype, int nblock, int Xoffset, int Xbroadcast,
+                                  int n, int m, int k, int p, const void* X, void* dW, const void* dZ);
+
+/* Momentum / Nesterov updates with per-element rate vectors.
+ * reference: launch_gradstep{,_nesterov1,_nesterov2}, deepity_smat.cpp:42-52, gradstep.cu:41-72 */
+int dbk_gradstep(dbk_stream_t stream, int dtype, size_t n,
+                 void* P, const void* dP, const void* drate, void* mP, const void* mrate);
+int dbk_gradstep_nesterov1(dbk_stream_t stream, int dtype, size_t n,
+                           void* P, const void* mP, const void* mrate);
+int dbk_gradstep_nesterov2(dbk_stream_t stream, int dtype, size_t n,
+                           void* P, const void* dP, const void* drate, void* mP, const void* mrate);
+
+/* dst[i] += A[i] * b[(i/k) % m] for i < n.
+ * reference: launch_madd_bcast, deepity_smat.cpp:54-56, madd_bcast.cu:41-58 */
+int dbk_madd_bcast(dbk_stream_t stream, int dtype, const void* A, const void* b, void* dst,
+                   size_t n, size_t m, size_t k);
+
+/* A[i] = M[i] ? A[i] : 0 (NaN-safe). reference: launch_maskout, deepity_smat.cpp:58, maskout.cu:41-50 */
+int dbk_maskout(dbk_stream_t stream, int dtype, const uint8_t* M, void* A, size_t n);
+/* For each (fwd,rev) row pair of Z (n rows, m cols) set M true at the row holding the larger value
+ * (ties: first row); other entries are left as they are (the caller pre-zeroes M).
+ * reference: launch_calc_zmask, deepity_smat.cpp:60, maskout.cu:52-67 */
+int dbk_calc_zmask(dbk_stream_t stream, int dtype, const void* Z, uint8_t* M, size_t n, size_t m);
+
+/* Dropout on pooled features with one rate per model: column c of an (n/(m*k), m*k) matrix uses
+ * rate[(i/k) % m]. keep = (u >= rate). matchrows gives each (2r, 2r+1) row pair one shared draw.
+ * reference: launch_dropout_fp_tr / _fp_te / _bp_tr / _bp_te, deepity_smat.cpp:62-73, dropout.cu:41-180 */
+int dbk_dropout_fp_tr(dbk_stream_t stream, int dtype, const void* X, const void* rate, void* Z, uint8_t* M,
+                      size_t n, size_t m, size_t k, int matchrows, uint64_t seed, uint64_t offset);
+/* Same with caller-supplied uniforms U (float32, one per element; with matchrows row 2r's are used). */
+int dbk_dropout_fp_tr_u(dbk_stream_t stream, int dtype, const void* X, const void* rate, void* Z, uint8_t* M,
+                        size_t n, size_t m, size_t k, int matchrows, const float* U);
+int dbk_dropout_fp_te(dbk_stream_t stream, int dtype, const void* X, const void* rate, void* Z,
+                      size_t n, size_t m, size_t k);
+int dbk_dropout_bp_tr(dbk_stream_t stream, int dtype, const void* dZ, const uint8_t* M, void* dX, size_t n);
+int dbk_dropout_bp_te(dbk_stream_t stream, int dtype, const void* dZ, const void* rate, void* dX,
+                      size_t n, size_t m, size_t k);
+
+/* The uniforms the dropout entry points draw: U[i] in [0,1) for flat element i (with matchrows,
+ * pair index i). Philox4x32-10, key = seed, counter = offset + i/4, word i%4, top 24 bits.
+ * The reference draws from cuRAND's per-thread XORWOW states (smat_cuda/cuda_context.cpp:210-242),
+ * which cannot be reproduced without the CUDA SDK; this generator is the library's own. */
+int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uint64_t offset);
+/* Host-side block function of that generator, for known-answer tests. */
+int dbk_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+
+/* ------------------------------------------------------------------ the few array ops the bias / relu / loss nodes use */
+
+/* Z = X + b (row vector b broadcast down n rows of m columns).
+ * reference: kernel_elemwise_b_* add, smat/src/smat_cuda/elemwise3.cuh:193-198, elemwise3.cu:57 */
+int dbk_add_rowvec(dbk_stream_t stream, int dtype, const void* X, const void* b, void* Z, size_t n, size_t m);
+/* out[c] = sum_r X[r,c] in row order (bias gradient). reference: smat_cuda/reduce_y.cuh:57-91 */
+int dbk_colsum(dbk_stream_t stream, int dtype, const void* X, void* out, size_t n, size_t m);
+/* Z = max(0, X). reference: smat_cuda/elemwise3.cu:62 */
+int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n);
+/* dX = dZ * sign(Z), sign = (z>0)-(z<0). reference: deepity/std/elemwise.py:78, smat_cuda/elemwise2.cu:42,77 */
+int dbk_mul_sign(dbk_stream_t stream, int dtype, const void* dZ, const void* Z, void* dX, size_t n);
+/* Z = 1/(1+exp(-X)). reference: smat_cuda/elemwise2.cu:46,68 */
+int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n);
+/* Elementwise loss terms L (n rows, m cols): kind 0 = log(max(1e-15,Z))*Y + log(max(1e-15,1-Z))*(1-Y),
+ * kind 1 = (Z-Y)^2. reference: deepity/std/loss.py:131-145 */
+int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, const void* Y, void* L, size_t n);
+/* dZ = (Z - Y) * scale. reference: deepity/std/loss.py:98-112 */
+int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n);
+
+/* ------------------------------------------------------------------ fused dense head for scoring */
+
+/* scores[r, b] = head_b(pooled[r, b*k:(b+1)*k]) for nblock models with k inputs each:
+ * hidden > 0: relu(x.W1_b + b1_b).W2_b + b2_b ; hidden == 0: x.W1_b + b1_b ; then logistic if
+ * apply_logistic. W1 (k*nblock, hidden|1), b1 (1, hidden*nblock | nblock), W2 (hidden*nblock, 1), b2 (1, nblock).
+ * in_scale multiplies the inputs (test-time dropout rescale, one value per model, may be NULL).
+ * Replaces blockwise_dot_combined -> bias -> relu -> blockwise_dot -> bias (-> logistic)
+ * (reference: deepity/std/full.py:78-83,154-160, softmax.py:58-61). float32 only. */
+int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
+                   const float* pooled, const float* in_scale,
+                   const float* W1, const float* b1, const float* W2, const float* b2,
+                   int apply_logistic, float* scores);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEPBIND_HIP_H */

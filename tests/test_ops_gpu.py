@@ -1,0 +1,370 @@
+"""GPU parity: every operator of the C-ABI library, called through the Python surface, against the
+CPU oracle on the same seeded inputs. Tolerances: float32 activations 1e-5 and gradients 1e-4
+relative to the array's scale; indices and masks bit-exact; the unfused scan is bit-exact because it
+accumulates taps in the reference's order."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import deepbind_oracle as orc
+from tests.gpu_util import assert_close, dev, host, random_codes
+
+pytestmark = pytest.mark.gpu
+
+ACT, GRAD = 1e-5, 1e-4
+
+
+@pytest.fixture(scope="module")
+def ks():
+    from deepbind_amd import kangaroo_smat
+    return kangaroo_smat
+
+
+@pytest.fixture(scope="module")
+def ds():
+    from deepbind_amd import deepity_smat
+    return deepity_smat
+
+
+@pytest.fixture(scope="module")
+def sm():
+    from deepbind_amd import smat
+    return smat
+
+
+# ------------------------------------------------------------------------------------------ scan
+@pytest.mark.parametrize("N,m,F", [(300, 24, 16), (1000, 16, 64), (777, 5, 70), (24, 24, 3), (5000, 24, 200), (130, 32, 17)])
+def test_corr1ord_bit_exact(ks, N, m, F):
+    rng = np.random.default_rng(N + m + F)
+    X = random_codes(rng, N, 0.05, 0.03)
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
+    Zr = np.full((N, F), 5.0, np.float32)
+    orc.corr1ord(W, X, Zr)
+    Z = dev(np.full((N, F), 5.0, np.float32))
+    ks.corr1ord(dev(W), dev(X.reshape(-1, 1)), Z, 4)
+    assert np.array_equal(host(Z), Zr)
+
+
+def test_corr1ord_float64_and_short_input(ks):
+    rng = np.random.default_rng(1)
+    X = random_codes(rng, 400, 0.1)
+    W = rng.standard_normal((4 * 7, 33))
+    Zr = np.zeros((400, 33)); orc.corr1ord(W, X, Zr)
+    Z = dev(np.zeros((400, 33)))
+    ks.corr1ord(dev(W), dev(X), Z, 4)
+    assert np.array_equal(host(Z), Zr)
+    # fewer symbols than taps: nothing is written
+    Z2 = dev(np.ones((3, 33)))
+    ks.corr1ord(dev(W), dev(X[:3]), Z2, 4)
+    assert np.all(host(Z2) == 1.0)
+
+
+def test_corr1ord_rejects_bad_arguments(ks):
+    from deepbind_amd._lib import DeepbindError
+    W = dev(np.zeros((12, 4), np.float32))
+    X = dev(np.zeros(20, np.uint8))
+    with pytest.raises(DeepbindError):
+        ks.corr1ord(W, X, dev(np.zeros((20, 5), np.float32)), 4)       # wrong number of columns
+    with pytest.raises(DeepbindError):
+        ks.corr1ord(W, X, dev(np.zeros((20, 4), np.float32)), 3)       # no kernel for 3 channels
+    with pytest.raises(DeepbindError):
+        ks.corr1ord(W, dev(np.zeros(20, np.float32)), dev(np.zeros((20, 4), np.float32)), 4)
+
+
+@pytest.mark.parametrize("N,m,F,dense", [(400, 24, 16, True), (3000, 16, 100, True), (2000, 24, 64, False), (50, 7, 5, True)])
+def test_corr1ord_bprop_W(ks, N, m, F, dense):
+    rng = np.random.default_rng(N + F)
+    X = random_codes(rng, N, 0.05, 0.02)
+    dZ = rng.standard_normal((N, F)).astype(np.float32)
+    if not dense:
+        dZ[rng.random((N, F)) < 0.98] = 0                              # 1-sparse-like, as after max pooling
+    ref = np.zeros((4 * m, F), np.float64)
+    orc.corr1ord_bprop_W(ref, X, dZ.astype(np.float64))
+    dW = dev(np.ones((4 * m, F), np.float32))                          # accumulates onto existing content
+    ks.corr1ord_bprop_W(dW, dev(X), dev(dZ), 4)
+    assert_close(host(dW), ref + 1.0, GRAD, "dW")
+    # run-to-run bit stability (no float atomics)
+    dW2 = dev(np.ones((4 * m, F), np.float32))
+    ks.corr1ord_bprop_W(dW2, dev(X), dev(dZ), 4)
+    assert np.array_equal(host(dW), host(dW2))
+
+
+def test_corr1ord_bprop_X(ks):
+    rng = np.random.default_rng(5)
+    n, m, F = 300, 24, 48
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
+    dZ = rng.standard_normal((n, F)).astype(np.float32)
+    ref = np.ones((n, 4)); orc.corr1ord_bprop_X(ref, W.astype(np.float64), dZ.astype(np.float64))
+    dX = dev(np.ones((n, 4), np.float32))
+    ks.corr1ord_bprop_X(dX, dev(W), dev(dZ), 4)
+    assert_close(host(dX), ref, GRAD, "dX")
+
+
+# ------------------------------------------------------------------------------------------ pooling
+def _regions(rng, P, lo, hi, gap=0):
+    lens = rng.integers(lo, hi + 1, size=P)
+    edges = np.concatenate([[0], np.cumsum(lens + gap)])
+    return np.stack([edges[:-1], edges[:-1] + lens], axis=1).astype(np.uint32), int(edges[-1])
+
+
+@pytest.mark.parametrize("ptype", ["max", "avg", "sum", "all"])
+@pytest.mark.parametrize("F", [16, 100])
+def test_poolrgn_forward_and_backward(ks, ptype, F):
+    rng = np.random.default_rng(F)
+    R, N = _regions(rng, 37, 1, 60)
+    U = rng.standard_normal((N, F)).astype(np.float32)
+    U[3] = U[1]                                                        # exact tie: first row must win
+    Zr, Ir = orc.poolrgn(U, R, ptype, want_argmax=True)
+    Z, I = ks.poolrgn(dev(U), dev(R), ptype, want_argmax=True)
+    if ptype in ("max", "all"):
+        assert np.array_equal(host(I), Ir)
+        got = host(Z)
+        assert np.array_equal(got if ptype == "max" else got[:, 0::2], Zr if ptype == "max" else Zr[:, 0::2])
+    else:
+        assert I is None
+    assert_close(host(Z), Zr, ACT, "pooled")
+    Z0, I0 = ks.poolrgn(dev(U), dev(R), ptype, want_argmax=False)
+    assert I0 is None and np.array_equal(host(Z0), host(Z))
+    dP = rng.standard_normal(Zr.shape).astype(np.float32)
+    ref = np.ones((N, F), np.float32); orc.poolrgn_bprop(ref, R, dP, Ir, ptype)
+    dU = dev(np.ones((N, F), np.float32))
+    ks.poolrgn_bprop(dU, dev(R), dev(dP), I, ptype)
+    assert_close(host(dU), ref, ACT, "dU")
+
+
+def test_poolrgn_step_and_overlapping_regions(ks):
+    rng = np.random.default_rng(9)
+    U = rng.standard_normal((64, 8)).astype(np.float32)
+    R = np.array([[0, 20, 3], [10, 40, 2], [5, 64, 7]], np.uint32)      # strided and overlapping
+    for ptype in ("max", "avg", "all"):
+        Zr, Ir = orc.poolrgn(U, R, ptype, want_argmax=True)
+        Z, I = ks.poolrgn(dev(U), dev(R), ptype, want_argmax=True)
+        assert_close(host(Z), Zr, ACT, ptype)
+        if Ir is not None:
+            assert np.array_equal(host(I), Ir)
+        dP = rng.standard_normal(Zr.shape).astype(np.float32)
+        ref = np.zeros_like(U); orc.poolrgn_bprop(ref, R, dP, Ir, ptype)
+        dU = dev(np.zeros_like(U))
+        ks.poolrgn_bprop(dU, dev(R), dev(dP), I, ptype)
+        assert_close(host(dU), ref, GRAD, "dU " + ptype)
+
+
+# ------------------------------------------------------------------------------------------ fused scan + pool
+def _chain_oracle(W, b, X, R, ptype):
+    Z = np.zeros((X.size, W.shape[1]), W.dtype)
+    orc.corr1ord(W, X, Z)
+    A = orc.relu_fprop(orc.bias_fprop(Z, b))
+    P, I = orc.poolrgn(A, R, ptype, want_argmax=True)
+    return A, P, I
+
+
+def _fused_case(seed, B, lo, hi, m, F, pn=0.03, p254=0.0):
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(lo, hi + 1, size=B)
+    ords = [random_codes(rng, int(n), pn, p254) for n in lens]
+    from deepbind_amd import data
+    X, R = data.pack_ordinals(ords, m - 1)
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
+    b = (rng.standard_normal((1, F)) * 0.05).astype(np.float32)
+    return rng, W, b, X, R
+
+
+@pytest.mark.parametrize("general", [True, False])
+@pytest.mark.parametrize("ptype", ["max", "avg", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (40, 20, 40, 24, 144), (9, 1, 300, 11, 70)])
+def test_scanpool_fprop(ks, general, ptype, B, lo, hi, m, F):
+    rng, W, b, X, R = _fused_case(B + m + F, B, lo, hi, m, F, p254=0.01)
+    A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
+    P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=True, general=general)
+    assert_close(host(P), Pr, ACT, "pooled")
+    if Ir is not None:
+        got = host(I)
+        same = got == Ir
+        if not same.all():
+            # only an exact or round-off tie may move the argmax: the map values must agree to tolerance
+            va, vb = A.ravel()[got[~same]], A.ravel()[Ir[~same]]
+            assert np.all(np.abs(va - vb) <= ACT * np.abs(A).max()), "argmax differs off a tie"
+            assert (~same).mean() < 0.01
+        # each index addresses the right column and a row of its own region
+        rows, cols = got // F, got % F
+        assert np.array_equal(cols, np.tile(np.arange(F), (len(R), 1)))
+        assert np.all(rows >= R[:, :1]) and np.all(rows < R[:, 1:2])
+
+
+def test_scanpool_regions_past_the_end_and_gaps(ks):
+    """Arbitrary (non-packed) regions, including rows the scan does not define (relu(bias) there)."""
+    rng = np.random.default_rng(77)
+    m, F, N = 8, 20, 120
+    X = random_codes(rng, N, 0.1)
+    W = rng.standard_normal((4 * m, F)).astype(np.float32)
+    b = rng.standard_normal((1, F)).astype(np.float32)
+    R = np.array([[0, 10], [50, 51], [30, 90], [100, 120], [5, 6]], np.uint32)
+    for ptype in ("max", "avg", "all"):
+        A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
+        P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=True)
+        assert_close(host(P), Pr, ACT, ptype)
+        if Ir is not None:
+            assert np.array_equal(host(I), Ir)
+
+
+@pytest.mark.parametrize("ptype", ["max", "avg", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (30, 20, 40, 24, 144)])
+def test_scanpool_bprop(ks, ptype, B, lo, hi, m, F):
+    rng, W, b, X, R = _fused_case(B + F, B, lo, hi, m, F)
+    A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
+    dP = rng.standard_normal(Pr.shape).astype(np.float32)
+    dA = np.zeros_like(A)
+    orc.poolrgn_bprop(dA, R, dP.astype(np.float64), Ir, ptype)
+    dZ = orc.relu_bprop(dA, A)
+    dbr = orc.bias_bprop(dZ)[1]
+    dWr = np.zeros(W.shape); orc.corr1ord_bprop_W(dWr, X, dZ)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True)
+    if Ir is not None and not np.array_equal(host(I), Ir):
+        pytest.skip("argmax moved on a round-off tie; gradient comparison needs identical argmax")
+    dW = dev(np.ones(W.shape, np.float32)); db = dev(np.full((1, F), 7.0, np.float32))
+    ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P, I, dev(dP), dW, db)
+    assert_close(host(dW), dWr + 1.0, GRAD, "dW")
+    assert_close(host(db), dbr, GRAD, "db")                            # written, not accumulated
+    dW2 = dev(np.ones(W.shape, np.float32)); db2 = dev(np.zeros((1, F), np.float32))
+    ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P, I, dev(dP), dW2, db2)
+    assert np.array_equal(host(dW), host(dW2)) and np.array_equal(host(db), host(db2))
+
+
+# ------------------------------------------------------------------------------------------ dense head
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_blockwise_dot_family(ds, dtype):
+    rng = np.random.default_rng(3)
+    n, k, m, nb = 50, 16, 32, 7
+    tol = ACT if dtype == np.float32 else 1e-12
+    X = rng.standard_normal((n, k * nb)).astype(dtype)
+    W = rng.standard_normal((k * nb, m)).astype(dtype)
+    Zr = orc.blockwise_dot(X, W, nb)
+    assert_close(host(ds.blockwise_dot(dev(X), dev(W), nb)), Zr, tol, "Z")
+    dZ = rng.standard_normal(Zr.shape).astype(dtype)
+    assert_close(host(ds.blockwise_dot_nt(dev(dZ), dev(W), nb)), orc.blockwise_dot_nt(dZ, W, nb), tol * 10, "dX")
+    assert_close(host(ds.blockwise_dot_tn(dev(X), dev(dZ), nb, dev(W))), orc.blockwise_dot_tn(X, dZ, nb, W), tol * 10, "dW")
+    Xs = rng.standard_normal((n, k)).astype(dtype)                     # one input shared by all models
+    assert_close(host(ds.blockwise_dot(dev(Xs), dev(W), nb)), orc.blockwise_dot(Xs, W, nb), tol, "Z shared")
+    assert_close(host(ds.blockwise_dot_tn(dev(Xs), dev(dZ), nb, dev(W))), orc.blockwise_dot_tn(Xs, dZ, nb, W), tol * 10, "dW shared")
+    # nblock == 1 is a plain matrix product
+    assert_close(host(ds.blockwise_dot(dev(X), dev(W), 1)), X @ W, tol, "dot")
+    # combined: conv features + a shared feature block, as the sequence model's combiner uses them
+    k2 = 5
+    X2 = rng.standard_normal((n, k2)).astype(dtype)
+    Wc = rng.standard_normal(((k + k2) * nb, m)).astype(dtype)
+    Xl, bc = [X, X2], [False, True]
+    Zc = orc.blockwise_dot_combined(Xl, Wc, nb, bc)
+    assert_close(host(ds.blockwise_dot_combined([dev(X), dev(X2)], dev(Wc), nb, bc)), Zc, tol, "Zc")
+    dZc = rng.standard_normal(Zc.shape).astype(dtype)
+    got = ds.blockwise_dot_nt_combined([dev(X), dev(X2)], dev(dZc), dev(Wc), nb, bc)
+    ref = orc.blockwise_dot_nt_combined(Xl, dZc, Wc, nb, bc)
+    assert got[1] is None and ref[1] is None
+    assert_close(host(got[0]), ref[0], tol * 10, "dXc")
+    assert_close(host(ds.blockwise_dot_tn_combined([dev(X), dev(X2)], dev(dZc), dev(Wc), nb, bc)),
+                 orc.blockwise_dot_tn_combined(Xl, dZc, Wc, nb, bc), tol * 10, "dWc")
+    assert_close(host(ds.blockwise_dot_tn_combined([dev(X), dev(X2)], dev(dZc), dev(Wc), nb, bc, dWmask=[True, False])),
+                 orc.blockwise_dot_tn_combined(Xl, dZc, Wc, nb, bc, dWmask=[True, False]), tol * 10, "dWc masked")
+
+
+def test_head_fprop(ds):
+    rng = np.random.default_rng(4)
+    n, k, nb, h = 300, 16, 9, 32
+    Pl = np.abs(rng.standard_normal((n, k * nb))).astype(np.float32)
+    W1 = (rng.standard_normal((k * nb, h)) * 0.3).astype(np.float32); b1 = (rng.standard_normal((1, h * nb)) * 0.1).astype(np.float32)
+    W2 = (rng.standard_normal((h * nb, 1)) * 0.3).astype(np.float32); b2 = (rng.standard_normal((1, nb)) * 0.1).astype(np.float32)
+    H = orc.relu_fprop(orc.bias_fprop(orc.blockwise_dot(Pl, W1, nb), b1))
+    ref = orc.bias_fprop(orc.blockwise_dot(H, W2, nb), b2)
+    got = ds.head_fprop(dev(Pl), dev(W1), dev(b1), dev(W2), dev(b2), nblock=nb)
+    assert_close(host(got), ref, ACT, "scores")
+    got = ds.head_fprop(dev(Pl), dev(W1), dev(b1), dev(W2), dev(b2), nblock=nb, apply_logistic=True)
+    assert_close(host(got), orc.logistic(ref), ACT, "probabilities")
+    # no hidden layer, with the test-time dropout rescale
+    W0 = (rng.standard_normal((k * nb, 1)) * 0.3).astype(np.float32); b0 = (rng.standard_normal((1, nb)) * 0.1).astype(np.float32)
+    rate = rng.choice([0.0, 0.25, 0.5], size=nb).astype(np.float32)
+    ref0 = orc.bias_fprop(orc.blockwise_dot(orc.dropout_fp_test(Pl, rate), W0, nb), b0)
+    got0 = ds.head_fprop(dev(Pl), dev(W0), dev(b0), nblock=nb, in_scale=1 - rate)
+    assert_close(host(got0), ref0, ACT, "scores (no hidden)")
+
+
+# ------------------------------------------------------------------------------------------ elementwise / optimiser
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_gradstep_and_madd_bcast(ds, dtype):
+    rng = np.random.default_rng(6)
+    n = 5000
+    P0, dP, mP0 = (rng.standard_normal(n).astype(dtype) for _ in range(3))
+    drate = (rng.random(n) * 0.1).astype(dtype); mrate = (0.9 + rng.random(n) * 0.09).astype(dtype)
+    for nesterov in (False, True):
+        Pr, mPr = P0.copy(), mP0.copy()
+        if nesterov:
+            orc.gradstep_nesterov1(Pr, mPr, mrate); orc.gradstep_nesterov2(Pr, dP, drate, mPr, mrate)
+        else:
+            orc.gradstep(Pr, dP, drate, mPr, mrate)
+        P, mP, called = dev(P0.reshape(-1, 1)), dev(mP0.reshape(-1, 1)), []
+        ds.gradstep(P, dev(dP.reshape(-1, 1)), dev(drate.reshape(-1, 1)), mP, dev(mrate.reshape(-1, 1)),
+                    grad=lambda: called.append(1), nesterov=nesterov)
+        assert called == [1]
+        assert np.array_equal(host(P).ravel(), Pr) and np.array_equal(host(mP).ravel(), mPr)
+    A = rng.standard_normal((24, 10)).astype(dtype); b = rng.standard_normal(3).astype(dtype)
+    dst = rng.standard_normal((24, 10)).astype(dtype)
+    ref = dst.copy(); orc.madd_bcast(A, b, 16, ref)
+    d = dev(dst); ds.madd_bcast(dev(A), b, 16, d)
+    assert np.array_equal(host(d), ref)
+    d = dev(dst); ds.madd_bcast(dev(A), 0.5, 1, d)
+    assert np.array_equal(host(d), dst + A * dtype(0.5))
+
+
+def test_masks_dropout_and_loss_ops(ds, sm, ks):
+    rng = np.random.default_rng(8)
+    n, nb, k = 64, 5, 16
+    X = rng.standard_normal((n, nb * k)).astype(np.float32)
+    rate = np.array([0.0, 0.25, 0.5, 0.5, 0.1], np.float32)
+    U = rng.random((n, nb * k)).astype(np.float32)
+    for match in (False, True):
+        Zr, Mr = orc.dropout_fp_train(X, rate, U, matchrows=match)
+        Z, M = ds.dropout_fp_train(dev(X), rate, match, U=dev(U))
+        assert np.array_equal(host(M), Mr) and np.array_equal(host(Z), Zr)
+    assert np.array_equal(host(ds.dropout_bp_tr(dev(X), M)), orc.dropout_bp_tr(X, Mr))
+    assert np.array_equal(host(ds.dropout_fp_test(dev(X), rate)), orc.dropout_fp_test(X, rate))
+    assert np.array_equal(host(ds.dropout_bp_te(dev(X), rate)), orc.dropout_bp_te(X, rate))
+    # the library's own generator: uniforms in [0,1), keep fraction ~ 1-rate, identical to uniform_like
+    ds.set_seed(123)
+    Z, M = ds.dropout_fp_train(dev(X), rate, False)
+    Ug = host(ds.uniform_like(dev(X), 123, 0))
+    assert Ug.min() >= 0.0 and Ug.max() < 1.0 and abs(Ug.mean() - 0.5) < 0.02
+    assert np.array_equal(host(M), orc.dropout_fp_train(X, rate, Ug)[1])
+    Z2, M2 = ds.dropout_fp_train(dev(X), rate, False)
+    assert not np.array_equal(host(M2), host(M))                       # the stream advances
+    # input-base dropout
+    Xo = random_codes(rng, 500, 0.1)
+    Uo = rng.random(500).astype(np.float32)
+    Zo, Mo = ks.dropoutord_fp_train(dev(Xo), 0.3, U=dev(Uo))
+    Zor, Mor = orc.dropoutord_fp_train(Xo, np.float32(0.3), Uo)
+    assert np.array_equal(host(Zo), Zor) and np.array_equal(host(Mo), Mor)
+    # maskout / zmask
+    A = rng.standard_normal((n, nb)).astype(np.float32); A[3, 2] = np.nan
+    Mk = rng.random((n, nb)) < 0.7; Mk[3, 2] = False
+    ref = A.copy(); orc.maskout(Mk, ref)
+    a = dev(A); ds.maskout(dev(Mk), a)
+    assert np.array_equal(host(a), ref)
+    Zp = rng.standard_normal((n, nb)).astype(np.float32); Zp[4] = Zp[5]
+    zm = torch.zeros((n, nb), dtype=torch.bool, device="cuda")
+    ds.calc_Zmask(dev(Zp), zm)
+    assert np.array_equal(host(zm), orc.calc_zmask(Zp))
+    # bias / relu / logistic / loss pieces
+    b = rng.standard_normal((1, nb * k)).astype(np.float32)
+    assert np.array_equal(host(sm.add_rowvec(dev(X), dev(b))), orc.bias_fprop(X, b))
+    assert np.array_equal(host(sm.relu(dev(X))), orc.relu_fprop(X))
+    assert np.array_equal(host(sm.mul_sign(dev(U), dev(X))), orc.relu_bprop(U, X))
+    assert_close(host(sm.sum_axis0(dev(X))), orc.bias_bprop(X.astype(np.float64))[1], ACT, "colsum")
+    assert_close(host(sm.logistic(dev(X))), orc.logistic(X), ACT, "logistic")
+    Zl = orc.logistic(A := rng.standard_normal((n, nb)).astype(np.float32))
+    Y = (rng.random((n, nb)) < 0.5).astype(np.float32)
+    eps = np.float32(1e-15)
+    ref = np.log(np.maximum(eps, Zl)) * Y + np.log(np.maximum(eps, 1 - Zl)) * (1 - Y)
+    assert_close(host(sm.loss_terms(dev(Zl), dev(Y), "nll")), ref, ACT, "nll terms")
+    assert_close(host(sm.loss_terms(dev(A), dev(Y), "mse")), (A - Y) ** 2, ACT, "mse terms")
+    assert_close(host(sm.sub_scale(dev(Zl), dev(Y), 1.0 / n)), orc.loss_bprop(Zl, Y), ACT, "dZ")
+    assert_close(host(sm.dot(dev(X), dev(X.T.copy()))), X.astype(np.float64) @ X.T.astype(np.float64), ACT, "dot")
+    assert_close(host(sm.dot_nt(dev(X), dev(X))), X.astype(np.float64) @ X.T.astype(np.float64), ACT, "dot_nt")
+    assert_close(host(sm.dot_tn(dev(X), dev(X))), X.T.astype(np.float64) @ X.astype(np.float64), ACT, "dot_tn")
