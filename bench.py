@@ -1,0 +1,147 @@
+"""Benchmark of the motif-scan hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config5|config5_small]
+
+One step = one pass of the fused forward (scan + bias + ReLU + max pool over every region, then the
+dense head) over the whole synthetic batch of the bulk-scoring configuration: 64 models x 16 motif
+detectors of width 24 over 100 000 DNA sequences of length 500 (1 % N), producing the 100000 x 64
+score matrix. Inputs are resident in HBM before the timed region. Prints ONE JSON line.
+
+Units: a "position" is one row of the (virtual) feature map, sum over sequences of (len + m - 1);
+the scan's algorithmic work is positions * filters * m gather-adds (1 FLOP each).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published FP32 vector peak (FMA = 2 FLOP)
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(cfg, nseq_c, nseq_np):
+    """Times the CPU restatement (the checker's plain-C port, OpenMP over all host cores) and the
+    NumPy float32 formulation on a bounded subsample of the same workload; returns positions/s."""
+    from oracle import oracle_c, deepbind_oracle as orc
+    spec, p = cfg["spec"], cfg["params"]
+    m = spec.m
+
+    def sample(nseq):
+        R = cfg["R"][:nseq]
+        end = int(R[-1, 1])
+        X = np.ascontiguousarray(cfg["X"][:end + m - 1])
+        return X, np.ascontiguousarray(R), end
+
+    cores = len(os.sched_getaffinity(0))
+    X, R, pos = sample(nseq_c)
+    oracle_c.scanpool(p["Wc"], p["bc"], X[:2000 + m], R[:2], 0)       # warm-up (thread pool, page-in)
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        oracle_c.scanpool(p["Wc"], p["bc"], X, R, 0)
+        best = min(best, time.perf_counter() - t0)
+    c_rate = pos / best
+    Xn, Rn, posn = sample(nseq_np)
+    t0 = time.perf_counter()
+    Z = np.zeros((Xn.size, spec.F), np.float32)
+    orc.corr1ord(p["Wc"], Xn, Z)
+    A = np.maximum(Z + p["bc"], 0)
+    np.maximum.reduceat(A, Rn[:, 0].astype(np.int64), axis=0)
+    np_rate = posn / (time.perf_counter() - t0)
+    return {
+        "value": c_rate, "unit": "positions/s", "cores": cores, "kind": "port",
+        "sample": "plain-C port of the reference scan+bias+relu+maxpool (OpenMP, %d threads), %d of the %d sequences x all %d filters, best of 3"
+                  % (cores, nseq_c, len(cfg["R"]), spec.F),
+        "numpy_f32_positions_per_s": np_rate,
+        "numpy_sample": "NumPy float32 LUT-gather formulation, single process, %d sequences x all %d filters, 1 run" % (nseq_np, spec.F),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="config5", choices=["config5", "config5_small"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the path shards over models or sequences with no exchange step, "
+                 "and this build runs on a single MI355X (got --gpus %d)" % args.gpus)
+
+    import torch
+    from deepbind_amd import kangaroo_smat as ks, deepity_smat as ds, synth
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    nseq = 100000 if args.workload == "config5" else 5000
+    cfg = synth.config5(seed=4, nseq=nseq)
+    spec, p = cfg["spec"], cfg["params"]
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    W, b, X, R = dev(p["Wc"]), dev(p["bc"]), dev(cfg["X"]), dev(cfg["R"])
+    W1, b1, W2, b2 = dev(p["W1"]), dev(p["b1"]), dev(p["W2"]), dev(p["b2"])
+    positions = synth.positions(cfg["R"])
+    adds = float(positions) * spec.F * spec.m
+
+    def step():
+        pooled, _ = ks.scanpool_fprop(W, b, X, R, "max")
+        return ds.head_fprop(pooled, W1, b1, W2, b2, nblock=spec.nmodel)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        # events bracket the scan+pool launches only (recorded on the stream they run on)
+        ev[k][0].record()
+        pooled, _ = ks.scanpool_fprop(W, b, X, R, "max")
+        ev[k][1].record()
+        scores = ds.head_fprop(pooled, W1, b1, W2, b2, nblock=spec.nmodel)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    scan_ms = float(np.mean([a.elapsed_time(c) for a, c in ev]))
+    assert tuple(scores.shape) == (nseq, spec.nmodel) and bool(torch.isfinite(scores).all())
+
+    ms_per_step = elapsed / args.steps * 1e3
+    adds_per_s = adds / (scan_ms * 1e-3)
+    # algorithmic HBM bytes of the scan+pool launch: sequence bytes in, filters in, pooled features out
+    hbm_bytes = cfg["X"].size + p["Wc"].nbytes + p["bc"].nbytes + positions * 0 + nseq * spec.F * 4
+    out = {
+        "metric": "seq_positions_per_sec_fwd_scan_pool",
+        "value": positions * args.steps / elapsed,
+        "unit": "positions/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: bulk forward scoring, %d models x %d motifs x width %d, %d DNA sequences x %d nt (1%% N), "
+                               "fused scan+bias+relu+maxpool then dense 16->32->1; output %d x %d scores"
+                               % (args.workload, spec.nmodel, spec.nfilter, spec.m, nseq, 500, nseq, spec.nmodel),
+                   "positions_per_step": positions, "filters": spec.F, "motif_width": spec.m},
+        "sequences_per_s": nseq * args.steps / elapsed,
+        "model_sequences_per_s": nseq * spec.nmodel * args.steps / elapsed,
+        "roofline": {
+            "bound": "valu_fp32", "achieved": adds_per_s / 1e12, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": adds_per_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS, "traffic": None,
+            "kernel": "fused scan+bias+relu+maxpool (dbk_scanpool_fprop launches)", "kernel_ms": scan_ms,
+            "algorithmic_adds_per_launch": adds,
+            "frac_of_unpacked_add_issue_rate": adds_per_s / (256 * 64 * 2.4e9),
+            "hbm": {"algorithmic_bytes_per_launch": hbm_bytes, "achieved_GBs": hbm_bytes / (scan_ms * 1e-3) / 1e9,
+                    "peak_GBs": HBM_PEAK_GBS, "frac": hbm_bytes / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, nseq_c=min(nseq, 1000), nseq_np=min(nseq, 100))
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

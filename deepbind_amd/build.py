@@ -24,9 +24,14 @@ FLAGS = [
 ]
 
 
+# The running max of the k-mer kernel must compile to bare v_max / v_max3 instructions; with NaNs
+# honoured every fmaxf gets two extra canonicalising ops. Infinities stay honoured (-inf seeds the max).
+EXTRA = {"scanpool_kmer.hip": ["-fno-honor-nans"]}
+
+
 def _compile(src):
     obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    cmd = [HIPCC] + FLAGS + EXTRA.get(os.path.basename(src), []) + ["-c", src, "-o", obj]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines() if "is not a recognized feature for this target" not in l)
     if res.returncode != 0:

@@ -51,9 +51,12 @@ template <int PT, bool WANT_ARGMAX>
 __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __restrict__ W, const float* __restrict__ bias,
                                                              unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
                                                              const uint32_t* __restrict__ R, size_t P,
-                                                             float* __restrict__ pooled, uint32_t* __restrict__ argmax)
+                                                             float* __restrict__ pooled, uint32_t* __restrict__ argmax,
+                                                             const unsigned* __restrict__ run_if_flag)
 {
     extern __shared__ __align__(16) unsigned char smem[];
+    // when given, the launch only does work if the device flag is set (fallback behind the k-mer kernel)
+    if (run_if_flag && run_if_flag[0] == 0) return;
     const unsigned nw = blockDim.x >> 6;
     const unsigned chunk = nw * XCH_SUBS * PSUB;
     float* lut = reinterpret_cast<float*>(smem);
@@ -109,6 +112,7 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
             }
             const size_t j = r * F + f;
             const float cnt = (float)(b - a);
+            bm = bm > 0.0f ? bm : 0.0f;                          // only an empty region gets here with bm < 0
             if (PT == DBK_PT_MAX) pooled[j] = bm;
             else if (PT == DBK_PT_AVG) pooled[j] = bs / cnt;
             else { pooled[2 * j] = bm; pooled[2 * j + 1] = bs / cnt; }
@@ -239,7 +243,7 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dst, const float* __rest
 
 template <int PT>
 int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
-                    const uint32_t* R, size_t P, float* pooled, uint32_t* argmax)
+                    const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, const unsigned* run_if_flag)
 {
     const unsigned nw = 4;
     const unsigned chunk = nw * XCH_SUBS * PSUB;
@@ -253,11 +257,11 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     if (argmax) {
         auto kern = scanpool_fprop_kernel<PT, true>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
     } else {
         auto kern = scanpool_fprop_kernel<PT, false>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
     }
     DBK_LAUNCH_OK();
 }
@@ -292,12 +296,12 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
 }
 
 int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
-          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax)
+          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, const unsigned* run_if_flag)
 {
     switch (ptype) {
-    case DBK_PT_MAX: return launch_fprop_pt<DBK_PT_MAX>(st, W, bias, m, F, X, N, R, P, pooled, argmax);
-    case DBK_PT_AVG: return launch_fprop_pt<DBK_PT_AVG>(st, W, bias, m, F, X, N, R, P, pooled, nullptr);
-    default:         return launch_fprop_pt<DBK_PT_ALL>(st, W, bias, m, F, X, N, R, P, pooled, argmax);
+    case DBK_PT_MAX: return launch_fprop_pt<DBK_PT_MAX>(st, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag);
+    case DBK_PT_AVG: return launch_fprop_pt<DBK_PT_AVG>(st, W, bias, m, F, X, N, R, P, pooled, nullptr, run_if_flag);
+    default:         return launch_fprop_pt<DBK_PT_ALL>(st, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag);
     }
 }
 
@@ -320,7 +324,7 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream, const float* W, const float*
     DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
-    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax);
+    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr);
 }
 
 int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
@@ -334,7 +338,7 @@ int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, s
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
     int rc = dbk_scanpool_kmer::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax);
     if (rc >= 0) return rc;
-    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax);
+    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr);
 }
 
 int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,

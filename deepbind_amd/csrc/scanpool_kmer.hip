@@ -1,13 +1,352 @@
-// Fast path of the fused scan + pool forward (k-mer lookup table in LDS). Placeholder: declines
-// every shape so the general kernel runs.
+// Fast path of the fused scan + bias + ReLU + max-pool forward: a 3-mer lookup table in LDS.
+//
+// The scan is a gather-add: Z[p,f] = sum_j w(j, X[p+j], f). Grouping taps three at a time turns
+// it into G = ceil(m/3) adds per (position, filter): Z[p,f] = sum_g L_g[kmer(p+3g)][f], where
+// kmer(t) indexes the 5-letter triple (X[t], X[t+1], X[t+2]) (A,C,G,T and "mean of the four" for
+// N / padding: 125 triples) and L_g holds the three taps' weights pre-summed (bias folded into
+// L_0). That cuts executed VALU adds and LDS bytes per algorithmic add by 3.
+//
+// Mapping to the hardware:
+//  * A workgroup owns 32 filters. Its table lut[kmer][row][32 filters] (125 x (G+1) rows of 128 B,
+//    144 KB for m = 24) fills the CU's LDS; one workgroup per CU.
+//  * ds_read_b128 only reaches the LDS's full rate when each group of 16 lanes reads 256
+//    contiguous bytes. So a "stream" is 16 lanes walking one region: lanes 0-7 (half A) read row
+//    2i+par, lanes 8-15 (half B) the next row, 4 filters per lane. Half A owns the positions whose
+//    group-of-three index is even, half B the odd ones; "par" alternates every three steps so that
+//    each half meets each tap group of its positions exactly once. Row G repeats row 0 so half B
+//    can start a position on odd steps.
+//  * Each lane keeps a ring of 3 x G/2 float4 accumulators in VGPRs: at text position t the G/2
+//    reads add into the positions t-3g the lane owns; a position is complete 3(G-1) steps after it
+//    starts, is folded into the running max and its slot is reused. The step loop is unrolled over
+//    3G positions so every ring index is a compile-time register.
+//  * The sequence is pre-translated once into one byte per position (the triple index). A stream's
+//    16 lanes fetch a block's 3G indices cooperatively (one or two bytes per lane, one block ahead)
+//    and each step takes its index from the owning lane with a DPP row_share folded into the add
+//    that forms the LDS address: one VALU instruction of addressing per step.
+//
+//  * Positions outside a region never need a test. At a region's start every ring slot is reset to
+//    a large negative "poison" (-1e30), so the partial sums in flight from before the region finish
+//    far below any real value; and the steps a region's last block runs past its final useful
+//    position read a 126th table entry whose rows are all poison, which sinks exactly the positions
+//    that lie beyond the region. The running max ignores both, and ReLU follows the max.
+//
+// Shapes this path declines (filter length > 24, average pooling, argmax, code 254 present, regions
+// reaching past the last row the scan defines) go through the general kernel in scanpool.hip.
+//
+// Reference chain being fused: kangaroo/_ext/corr1ord.py:97-117 -> deepity/std/elemwise.py:162-180,71-82
+// -> kangaroo/_ext/poolrgn.py:56-76 (kernels corr1ord.cuh:139-157, poolrgn.cuh:44-79).
 #include "dbk_common.h"
+#include "scan_common.h"
+#include <cmath>
+
+namespace dbk_scanpool_general {
+int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, const unsigned* run_if_flag);
+}
 
 namespace dbk_scanpool_kmer {
 
-int fprop(hipStream_t, const float*, const float*, size_t, size_t, const uint8_t*, size_t,
-          const uint32_t*, size_t, int, float*, uint32_t*)
+constexpr int FTILE = 32;            // filters per workgroup
+constexpr int ROWB = FTILE * 4;      // bytes per table row
+constexpr int NKMER = 125;          // real triples; entry 125 is the poison entry
+constexpr float POISON = -1.0e30f;
+constexpr int KPAD = 128;            // index bytes readable past the end of the sequence
+
+__device__ __forceinline__ unsigned letter5(unsigned code) { return code < 4u ? code : 4u; }
+
+// flag[0] = 1 if a region is reversed or reaches past row ndef, the last row the scan defines
+// (the fast kernel then stands down)
+__global__ void check_regions_kernel(const uint32_t* __restrict__ R, size_t P, size_t ndef, unsigned* flag)
 {
-    return -1;
+    __shared__ unsigned bad;
+    if (threadIdx.x == 0) bad = 0;
+    __syncthreads();
+    unsigned mine = 0;
+    for (size_t r = threadIdx.x; r < P; r += blockDim.x)
+        if (R[2 * r + 1] < R[2 * r] || R[2 * r + 1] > ndef) mine = 1;
+    if (mine) atomicOr(&bad, 1u);
+    __syncthreads();
+    if (threadIdx.x == 0) flag[0] = bad;
+}
+
+// K[t] = 25*l(X[t]) + 5*l(X[t+1]) + l(X[t+2]) for t < N + KPAD, reading past the end as N (letter 4).
+// Sets flag[0] when a code 254 ("contributes nothing") is present: the table has no letter for it.
+__global__ __launch_bounds__(256) void kmer_index_kernel(const uint8_t* __restrict__ X, size_t N, uint8_t* __restrict__ K, unsigned* flag)
+{
+    const size_t total = N + KPAD;
+    unsigned saw = 0;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (size_t)gridDim.x * blockDim.x) {
+        unsigned c0 = t < N ? X[t] : 255u, c1 = t + 1 < N ? X[t + 1] : 255u, c2 = t + 2 < N ? X[t + 2] : 255u;
+        saw |= (c0 == 254u);
+        K[t] = (uint8_t)(25u * letter5(c0) + 5u * letter5(c1) + letter5(c2));
+    }
+    if (saw) atomicOr(flag, 1u);
+}
+
+__device__ __forceinline__ void add4(float4& a, const float4& v) { a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w; }
+__device__ __forceinline__ void fma4(float4& a, float s, const float4& v)
+{
+    a.x = __builtin_fmaf(a.x, s, v.x); a.y = __builtin_fmaf(a.y, s, v.y);
+    a.z = __builtin_fmaf(a.z, s, v.z); a.w = __builtin_fmaf(a.w, s, v.w);
+}
+__device__ __forceinline__ void max4(float4& m, const float4& v)
+{
+    m.x = fmaxf(m.x, v.x); m.y = fmaxf(m.y, v.y); m.z = fmaxf(m.z, v.z); m.w = fmaxf(m.w, v.w);
+}
+__device__ __forceinline__ void max4x2(float4& m, const float4& u, const float4& v)
+{
+    m.x = fmaxf(fmaxf(m.x, u.x), v.x); m.y = fmaxf(fmaxf(m.y, u.y), v.y);
+    m.z = fmaxf(fmaxf(m.z, u.z), v.z); m.w = fmaxf(fmaxf(m.w, u.w), v.w);
+}
+
+// Value of `v` held by lane `src` of the caller's row of 16 lanes (DPP row_share, folded by the
+// compiler into the consuming VALU instruction).
+template <int SRC>
+__device__ __forceinline__ unsigned row_share(unsigned v)
+{
+    return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + SRC, 0xf, 0xf, false);
+}
+
+// One unrolled block of 3G text positions for one lane.
+//   k0, k1    table byte offsets (triple index * bytes per triple) of this block's positions, spread
+//             over the stream's 16 lanes: lane i holds position i in k0 and position 16+i in k1
+//   acc       ring of partial sums, mx the running max
+template <int G>
+__device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigned k0, unsigned k1,
+                                           float4 (&acc)[3][G / 2], float4& mx, unsigned lanebase, bool isA,
+                                           float mulA, float mulB)
+{
+    constexpr int H = G / 2;
+#pragma unroll
+    for (int q = 0; q < G; ++q) {
+        const int par = q & 1, sb = q >> 1;
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            const int t = 3 * q + c;
+            unsigned koff;
+            switch (t) {
+#define DBK_CASE(T) case T: koff = (T < 16) ? row_share<(T < 16 ? T : 0)>(k0) : row_share<(T < 16 ? 0 : T - 16)>(k1); break;
+                DBK_CASE(0) DBK_CASE(1) DBK_CASE(2) DBK_CASE(3) DBK_CASE(4) DBK_CASE(5) DBK_CASE(6) DBK_CASE(7)
+                DBK_CASE(8) DBK_CASE(9) DBK_CASE(10) DBK_CASE(11) DBK_CASE(12) DBK_CASE(13) DBK_CASE(14) DBK_CASE(15)
+                DBK_CASE(16) DBK_CASE(17) DBK_CASE(18) DBK_CASE(19) DBK_CASE(20) DBK_CASE(21) DBK_CASE(22) DBK_CASE(23)
+#undef DBK_CASE
+                default: koff = 0; break;
+            }
+            const unsigned addr = koff + lanebase;
+#pragma unroll
+            for (int i = 0; i < H; ++i) {
+                const int slot = (((sb - i) % H) + H) % H;
+                const float4 v = *reinterpret_cast<const float4*>(lds + addr + (2 * i + par) * ROWB);
+                if (par == 0 && i == 0) fma4(acc[c][slot], mulB, v);            // half A starts a position here
+                else if (par == 1 && i == H - 1) fma4(acc[c][slot], mulA, v);   // half B starts a position here
+                else add4(acc[c][slot], v);
+            }
+        }
+        // the half that just read its last tap group (B on even q, A on odd q) has three finished positions
+        const int cs = (((sb - (H - 1)) % H) + H) % H;
+        const bool mine = (par == 0) ? !isA : isA;
+        if (mine) {
+            max4x2(mx, acc[0][cs], acc[1][cs]);
+            max4(mx, acc[2][cs]);
+        }
+    }
+}
+
+template <int G>
+__global__ __launch_bounds__(512) void scanpool_kmer_kernel(const float* __restrict__ W, const float* __restrict__ bias,
+                                                            unsigned m, unsigned F, const uint8_t* __restrict__ K, size_t N,
+                                                            const uint32_t* __restrict__ R, unsigned P, unsigned nsplit,
+                                                            const unsigned* __restrict__ flag, float* __restrict__ pooled)
+{
+    constexpr int H = G / 2, STEPS = 3 * G;
+    constexpr unsigned KSTRIDE = (G + 1) * ROWB;
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (flag[0] != 0) return;                                   // the general kernel takes this call
+    float* lut = reinterpret_cast<float*>(smem);
+    float* w5 = lut + (size_t)(NKMER + 1) * (G + 1) * FTILE;   // [3G taps][5 letters][32 filters]
+
+    const unsigned split = blockIdx.x % nsplit, tile = blockIdx.x / nsplit;
+    const unsigned f0 = tile * FTILE;
+
+    // ---- per-tap, per-letter weights for this filter tile (taps >= m are zero)
+    for (unsigned e = threadIdx.x; e < (unsigned)STEPS * FTILE; e += blockDim.x) {
+        const unsigned j = e / FTILE, fl = e % FTILE, f = f0 + fl;
+        float w0 = 0.f, w1 = 0.f, w2 = 0.f, w3 = 0.f;
+        if (j < m && f < F) {
+            w0 = W[(size_t)(4 * j + 0) * F + f];
+            w1 = W[(size_t)(4 * j + 1) * F + f];
+            w2 = W[(size_t)(4 * j + 2) * F + f];
+            w3 = W[(size_t)(4 * j + 3) * F + f];
+        }
+        float z = w0; z += w1; z += w2; z += w3;
+        float* row = w5 + (size_t)j * 5 * FTILE + fl;
+        row[0 * FTILE] = w0; row[1 * FTILE] = w1; row[2 * FTILE] = w2; row[3 * FTILE] = w3; row[4 * FTILE] = z * 0.25f;
+    }
+    __syncthreads();
+    // ---- the 3-mer table: taps in ascending order, bias first for group 0; row G repeats row 0;
+    //      entry 125 is all poison
+    for (unsigned e = threadIdx.x; e < (unsigned)(NKMER + 1) * (G + 1) * FTILE; e += blockDim.x) {
+        const unsigned fl = e % FTILE, row = (e / FTILE) % (G + 1), km = e / (FTILE * (G + 1));
+        const unsigned g = row == (unsigned)G ? 0u : row;
+        const unsigned l0 = km / 25u, l1 = (km / 5u) % 5u, l2 = km % 5u;
+        float s = POISON;
+        if (km < (unsigned)NKMER) {
+            s = (g == 0 && f0 + fl < F) ? bias[f0 + fl] : 0.0f;
+            s += w5[((size_t)(3 * g + 0) * 5 + l0) * FTILE + fl];
+            s += w5[((size_t)(3 * g + 1) * 5 + l1) * FTILE + fl];
+            s += w5[((size_t)(3 * g + 2) * 5 + l2) * FTILE + fl];
+        }
+        lut[e] = s;
+    }
+    __syncthreads();
+
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = blockDim.x >> 6;
+    const unsigned q8 = lane & 7, sidx = lane >> 4;
+    const bool isA = ((lane >> 3) & 1) == 0;
+    const unsigned lanebase = (isA ? 0u : (unsigned)ROWB) + q8 * 16u;
+    const float mulA = isA ? 1.0f : 0.0f, mulB = isA ? 0.0f : 1.0f;
+    const unsigned nstream = nsplit * nwave * 4u;
+    constexpr unsigned TAIL = 3 * (G - 1);                       // steps between a position's start and its completion
+
+    unsigned r = (split * nwave + wave) * 4u + sidx;
+    unsigned a = 0, rows = 0, a_next = 0, rows_next = 0;
+    if (r < P) { a = R[2 * (size_t)r]; rows = R[2 * (size_t)r + 1] - a; }
+    if (r < P && r + nstream < P) { a_next = R[2 * (size_t)(r + nstream)]; rows_next = R[2 * (size_t)(r + nstream) + 1] - a_next; }
+    unsigned nblk = (rows + TAIL + STEPS - 1) / STEPS;
+    if (nblk < 1) nblk = 1;
+
+    // lane i of a stream fetches the triple index of block positions i and 16+i; positions at or
+    // past rows+TAIL (nothing valid completes there any more) read the poison entry instead
+    const unsigned q16 = lane & 15;
+    const unsigned q16b = 16u + (STEPS > 16 ? (q16 < (unsigned)(STEPS - 16) ? q16 : (unsigned)(STEPS - 17)) : 0u);
+    auto fetch = [&](unsigned base, unsigned limit, unsigned pos0, unsigned& o0, unsigned& o1) {
+        // base: absolute text position of the block's first step, pos0: its region-relative position,
+        // limit: rows + TAIL of the block's region
+        unsigned v0 = K[(size_t)base + q16];
+        unsigned v1 = STEPS > 16 ? (unsigned)K[(size_t)base + q16b] : 0u;
+        o0 = (pos0 + q16 < limit ? v0 : (unsigned)NKMER) * KSTRIDE;
+        o1 = (pos0 + q16b < limit ? v1 : (unsigned)NKMER) * KSTRIDE;
+    };
+    unsigned k0, k1;
+    fetch(a, r < P ? rows + TAIL : 0u, 0u, k0, k1);
+
+    float4 acc[3][H];
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+        for (int s = 0; s < H; ++s) acc[c][s] = make_float4(POISON, POISON, POISON, POISON);
+    float4 mx = make_float4(POISON, POISON, POISON, POISON);
+    unsigned blk = 0;
+    const char* lds = reinterpret_cast<const char*>(smem);
+
+    while (true) {
+        const bool active = r < P;
+        if (!__any(active)) break;
+        const bool last = blk + 1 >= nblk;
+        // the next block's indices travel while this block computes
+        unsigned n0, n1;
+        if (last) fetch(a_next, (r < P && r + nstream < P) ? rows_next + TAIL : 0u, 0u, n0, n1);
+        else fetch(a + (blk + 1) * STEPS, rows + TAIL, (blk + 1) * STEPS, n0, n1);
+        scan_block<G>(lds, k0, k1, acc, mx, lanebase, isA, mulA, mulB);
+        k0 = n0;
+        k1 = n1;
+        if (last) {
+            // fold the two halves, ReLU, store this region's 32 pooled features
+            float4 o;
+            o.x = fmaxf(mx.x, __shfl_xor(mx.x, 8, 64)); o.y = fmaxf(mx.y, __shfl_xor(mx.y, 8, 64));
+            o.z = fmaxf(mx.z, __shfl_xor(mx.z, 8, 64)); o.w = fmaxf(mx.w, __shfl_xor(mx.w, 8, 64));
+            if (active && isA) {
+                const unsigned f = f0 + q8 * 4;
+                float* out = pooled + (size_t)r * F + f;
+                if (f + 0 < F) out[0] = fmaxf(o.x, 0.f);
+                if (f + 1 < F) out[1] = fmaxf(o.y, 0.f);
+                if (f + 2 < F) out[2] = fmaxf(o.z, 0.f);
+                if (f + 3 < F) out[3] = fmaxf(o.w, 0.f);
+            }
+            // new region: everything still in the ring belongs to the old one
+            mx = make_float4(POISON, POISON, POISON, POISON);
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+#pragma unroll
+                for (int s = 0; s < H; ++s) acc[c][s] = make_float4(POISON, POISON, POISON, POISON);
+            r = r < P ? r + nstream : r;
+            a = a_next; rows = rows_next; blk = 0;
+            nblk = (rows + TAIL + STEPS - 1) / STEPS;
+            if (nblk < 1) nblk = 1;
+            a_next = 0; rows_next = 0;
+            if (r < P && r + nstream < P) { a_next = R[2 * (size_t)(r + nstream)]; rows_next = R[2 * (size_t)(r + nstream) + 1] - a_next; }
+        } else {
+            ++blk;
+        }
+    }
+}
+
+template <int G>
+int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* K, size_t N,
+           const uint32_t* R, size_t P, const unsigned* flag, float* pooled)
+{
+    size_t smem = ((size_t)(NKMER + 1) * (G + 1) * FTILE + (size_t)3 * G * 5 * FTILE) * sizeof(float);
+    if (smem > dbk_scan::lds_limit()) return -1;
+    const unsigned ntile = dbk::divup(F, FTILE);
+    unsigned nsplit = 256u / ntile;
+    if (nsplit < 1) nsplit = 1;
+    const unsigned nwave = 8;
+    while (nsplit > 1 && (size_t)(nsplit - 1) * nwave * 4 >= P) --nsplit;       // no more streams than regions
+    auto kern = scanpool_kmer_kernel<G>;
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3(ntile * nsplit), dim3(nwave * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, K, N, R,
+                       (unsigned)P, nsplit, flag, pooled);
+    return 0;
+}
+
+// force: take the fast path whenever the shape allows, regardless of problem size
+int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+               const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, bool force)
+{
+    if (ptype != DBK_PT_MAX || argmax != nullptr) return -1;
+    if (m > 24 || N == 0 || N > 0x7fffff00u || P > 0x7fff0000u) return -1;
+    // a filter tile's table costs ~0.1 M position-equivalents to build: only worth it for bulk work
+    if (!force && (double)N * dbk::divup(F, FTILE) < 2.0e6) return -1;
+    const size_t kbytes = (N + KPAD + 255) & ~(size_t)255;
+    unsigned char* ws = (unsigned char*)dbk::workspace(256 + kbytes);
+    if (!ws) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", 256 + kbytes); return 1; }
+    unsigned* flag = (unsigned*)ws;
+    uint8_t* K = ws + 256;
+    const size_t ndef = N + 1 >= m + 1 ? N - m + 1 : 0;          // rows the scan defines
+    hipLaunchKernelGGL(check_regions_kernel, dim3(1), dim3(1024), 0, st, R, P, ndef, flag);
+    hipLaunchKernelGGL(kmer_index_kernel, dim3(dbk::ew_grid(N + KPAD)), dim3(256), 0, st, X, N, K, flag);
+    int G = (int)((m + 2) / 3);
+    G += G & 1;
+    int rc;
+    switch (G) {
+    case 2: rc = launch<2>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
+    case 4: rc = launch<4>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
+    case 6: rc = launch<6>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
+    default: rc = launch<8>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
+    }
+    if (rc != 0) return rc;
+    // inputs the table cannot express (code 254, regions outside the sequence): the general kernel
+    // runs instead, gated on the same device flag so that no host synchronisation is needed
+    rc = dbk_scanpool_general::fprop(st, W, bias, m, F, X, N, R, P, ptype, pooled, argmax, flag);
+    return rc;
+}
+
+int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax)
+{
+    return fprop_impl(st, W, bias, m, F, X, N, R, P, ptype, pooled, argmax, false);
 }
 
 }  // namespace dbk_scanpool_kmer
+
+extern "C" int dbk_scanpool_fprop_kmer(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
+                                       const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
+                                       float* pooled, uint32_t* argmax)
+{
+    DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
+    if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
+    int rc = dbk_scanpool_kmer::fprop_impl(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, true);
+    DBK_CHECK(rc >= 0, "NotImplementedError: the k-mer table path takes max pooling without argmax and filter length <= 24");
+    return rc;
+}

@@ -122,9 +122,10 @@ def dropoutord_fp_train(X, rate, U=None):
 # ------------------------------------------------------------------------------------------------
 # fused scan + bias + ReLU + pool
 # ------------------------------------------------------------------------------------------------
-def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, general=False):
+def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto"):
     """pool(relu(corr1ord(W, X) + b)) per region without storing the (N x P) map.
-    Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only."""
+    Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only.
+    path: "auto" lets the library choose, "general" / "kmer" force one kernel."""
     _u8(X)
     _regions(regions)
     require(regions.shape[1] == 2, "ValueError: the fused path takes 2-column regions")
@@ -133,7 +134,8 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, general=False):
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
     pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
     argmax = torch.empty((P, F), dtype=uindex, device=W.device) if (want_argmax and ptype in ("max", "all")) else None
-    call("dbk_scanpool_fprop_general" if general else "dbk_scanpool_fprop", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(),
+    entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "kmer": "dbk_scanpool_fprop_kmer"}[path]
+    call(entry, stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(),
          ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax))
     return pooled, argmax
 

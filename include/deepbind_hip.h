@@ -122,6 +122,16 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream,
                                const uint32_t* regions, size_t nregion, int ptype,
                                float* pooled, uint32_t* argmax);
 
+/* Same contract through the 3-mer lookup-table kernel regardless of problem size; fails with
+ * NotImplementedError for shapes that kernel does not take (filter length > 24, avg/all pooling,
+ * argmax requested). Inputs it cannot express (code 254, regions outside the sequence) are detected
+ * on the device and computed by the general kernel inside the same call. */
+int dbk_scanpool_fprop_kmer(dbk_stream_t stream,
+                            const float* W, const float* bias, size_t m, size_t nfilter,
+                            const uint8_t* X, size_t N,
+                            const uint32_t* regions, size_t nregion, int ptype,
+                            float* pooled, uint32_t* argmax);
+
 /* Backward of the fused chain: given dpooled (same layout as pooled), the forward's pooled and
  * argmax, accumulates dW (C*m, F) += and writes dbias (1, F) =. Deterministic (no float atomics).
  * reference chain: poolrgn_bprop -> relu bprop -> bias bprop -> corr1ord_bprop_W

@@ -173,9 +173,10 @@ def _fused_case(seed, B, lo, hi, m, F, pn=0.03, p254=0.0):
 @pytest.mark.parametrize("ptype", ["max", "avg", "all"])
 @pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (40, 20, 40, 24, 144), (9, 1, 300, 11, 70)])
 def test_scanpool_fprop(ks, general, ptype, B, lo, hi, m, F):
+    path = "general" if general else "auto"
     rng, W, b, X, R = _fused_case(B + m + F, B, lo, hi, m, F, p254=0.01)
     A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
-    P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=True, general=general)
+    P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=True, path=path)
     assert_close(host(P), Pr, ACT, "pooled")
     if Ir is not None:
         got = host(I)
@@ -368,3 +369,46 @@ def test_masks_dropout_and_loss_ops(ds, sm, ks):
     assert_close(host(sm.dot(dev(X), dev(X.T.copy()))), X.astype(np.float64) @ X.T.astype(np.float64), ACT, "dot")
     assert_close(host(sm.dot_nt(dev(X), dev(X))), X.astype(np.float64) @ X.T.astype(np.float64), ACT, "dot_nt")
     assert_close(host(sm.dot_tn(dev(X), dev(X))), X.T.astype(np.float64) @ X.astype(np.float64), ACT, "dot_tn")
+
+
+# ------------------------------------------------------------------------------------------ k-mer table fast path
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (300, 20, 40, 24, 144), (33, 1, 300, 11, 70),
+                                          (50, 500, 500, 24, 64), (17, 0, 9, 5, 33), (700, 30, 60, 20, 40), (40, 90, 110, 2, 8)])
+def test_scanpool_kmer_path_matches_oracle(ks, B, lo, hi, m, F):
+    rng, W, b, X, R = _fused_case(1000 + B + m + F, B, lo, hi, m, F, pn=0.04)
+    A, Pr, Ir = _chain_oracle(W, b, X, R, "max")
+    P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max", path="kmer")
+    assert I is None
+    assert_close(host(P), Pr, ACT, "pooled (kmer path)")
+    # and it agrees with the general kernel to the same tolerance
+    Pg, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max", path="general")
+    assert_close(host(P), host(Pg), ACT, "kmer vs general")
+
+
+def test_scanpool_kmer_path_device_side_fallbacks(ks):
+    """Code 254 and regions past the scan's last row cannot be expressed in the table: the call must
+    still return the right answer (the general kernel runs behind a device flag)."""
+    rng, W, b, X, R = _fused_case(4242, 60, 30, 50, 24, 48, pn=0.03, p254=0.02)
+    assert (X == 254).any()
+    A, Pr, _ = _chain_oracle(W, b, X, R, "max")
+    P, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max", path="kmer")
+    assert_close(host(P), Pr, ACT, "pooled with code 254")
+    rng, W, b, X, R = _fused_case(4243, 20, 30, 50, 24, 48)
+    R2 = R.copy(); R2[-1, 1] = X.size                                   # last region runs into rows >= n
+    A, Pr, _ = _chain_oracle(W, b, X, R2, "max")
+    P, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R2), "max", path="kmer")
+    assert_close(host(P), Pr, ACT, "pooled with a region past the last scan row")
+    from deepbind_amd._lib import DeepbindError
+    with pytest.raises(DeepbindError):
+        ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "all", path="kmer")
+
+
+def test_scanpool_auto_path_bulk(ks):
+    """A batch large enough for the library to pick the table kernel by itself."""
+    rng, W, b, X, R = _fused_case(99, 2500, 100, 100, 24, 256, pn=0.01)
+    P, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max")
+    Pg, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max", path="general")
+    assert_close(host(P), host(Pg), ACT, "auto vs general")
+    from oracle import oracle_c
+    Pr, _ = oracle_c.scanpool(W, b, X, R, 0)
+    assert_close(host(P), Pr, ACT, "auto vs C oracle")
