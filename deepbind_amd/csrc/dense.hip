@@ -74,38 +74,55 @@ __global__ __launch_bounds__(256) void k_bdot_tn(int nblock, size_t n, int m, in
     }
 }
 
-// Scoring head: one thread per (row, model).
+// Scoring head: a workgroup owns one model and a tile of 256 rows. The model's weights (a few KB)
+// are staged in LDS once and read back as wave-wide broadcasts; each thread keeps its row's k inputs
+// in registers (one contiguous k*4-byte read of HBM per thread) and writes one score.
+constexpr int HEAD_MAXK = 64;
+template <int KMAX>
 __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int hidden, const float* __restrict__ pooled,
                                               const float* __restrict__ in_scale, const float* __restrict__ W1,
                                               const float* __restrict__ b1, const float* __restrict__ W2,
                                               const float* __restrict__ b2, bool apply_logistic, float* __restrict__ scores)
 {
-    const size_t total = n * (size_t)nblock;
-    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
-        const size_t r = e / nblock;
-        const unsigned b = (unsigned)(e % nblock);
+    extern __shared__ float hsm[];
+    const unsigned b = blockIdx.y;
+    const int h1 = hidden > 0 ? hidden : 1;
+    float* w1s = hsm;                       // [k][h1]
+    float* b1s = w1s + (size_t)k * h1;      // [h1]
+    float* w2s = b1s + h1;                  // [hidden]
+    for (int e = threadIdx.x; e < k * h1; e += blockDim.x) w1s[e] = W1[(size_t)b * k * h1 + e];
+    for (int e = threadIdx.x; e < h1; e += blockDim.x) b1s[e] = b1[(size_t)b * h1 + e];
+    for (int e = threadIdx.x; e < hidden; e += blockDim.x) w2s[e] = W2[(size_t)b * hidden + e];
+    __syncthreads();
+    const float sc = in_scale ? in_scale[b] : 1.0f;
+    const float bias2 = hidden > 0 ? b2[b] : 0.0f;
+    for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n; r += (size_t)gridDim.x * blockDim.x) {
         const float* x = pooled + r * (size_t)k * nblock + (size_t)b * k;
-        const float sc = in_scale ? in_scale[b] : 1.0f;
+        float xr[KMAX];
+#pragma unroll
+        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = kk < k ? x[kk] * sc : 0.0f;
         float out;
         if (hidden > 0) {
             out = 0.0f;
-            const float* w1 = W1 + (size_t)b * k * hidden;
             for (int h = 0; h < hidden; ++h) {
                 float a = 0.0f;
-                for (int kk = 0; kk < k; ++kk) a += (x[kk] * sc) * w1[(size_t)kk * hidden + h];
-                a += b1[(size_t)b * hidden + h];
+#pragma unroll
+                for (int kk = 0; kk < KMAX; ++kk)
+                    if (kk < k) a += xr[kk] * w1s[kk * hidden + h];
+                a += b1s[h];
                 a = a > 0.0f ? a : 0.0f;
-                out += a * W2[(size_t)b * hidden + h];
+                out += a * w2s[h];
             }
-            out += b2[b];
+            out += bias2;
         } else {
             out = 0.0f;
-            const float* w1 = W1 + (size_t)b * k;
-            for (int kk = 0; kk < k; ++kk) out += (x[kk] * sc) * w1[kk];
-            out += b1[b];
+#pragma unroll
+            for (int kk = 0; kk < KMAX; ++kk)
+                if (kk < k) out += xr[kk] * w1s[kk];
+            out += b1s[0];
         }
         if (apply_logistic) out = 1.0f / (1.0f + expf(-out));
-        scores[e] = out;
+        scores[r * (size_t)nblock + b] = out;
     }
 }
 
@@ -118,15 +135,6 @@ int check_dims(int nblock, int n, int m, int k, int p, int off)
 }
 
 }  // namespace
-
-#define DISPATCH(kernel, total, ...)                                                                                   \
-    do {                                                                                                               \
-        if (dtype == DBK_F32) hipLaunchKernelGGL(kernel<float>, dim3(dbk::ew_grid(total)), dim3(256), 0, dbk::as_stream(stream), __VA_ARGS__); \
-        else hipLaunchKernelGGL(kernel<double>, dim3(dbk::ew_grid(total)), dim3(256), 0, dbk::as_stream(stream), __VA_ARGS__);                  \
-        DBK_LAUNCH_OK();                                                                                               \
-    } while (0)
-
-template <typename T> static const T* cp(const void* p) { return (const T*)p; }
 
 extern "C" {
 
@@ -210,8 +218,15 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(pooled && W1 && b1 && scores, "ValueError: null pointer argument");
     DBK_CHECK(hidden == 0 || (W2 && b2), "ValueError: hidden layer requested but W2/b2 are null");
-    size_t total = n * (size_t)nblock;
-    hipLaunchKernelGGL(k_head, dim3(dbk::ew_grid(total)), dim3(256), 0, dbk::as_stream(stream), n, nblock, k, hidden, pooled, in_scale,
+    DBK_CHECK(k <= HEAD_MAXK, "ValueError: the fused head takes at most %d inputs per model (got %d)", HEAD_MAXK, k);
+    DBK_CHECK(nblock <= 65535, "ValueError: too many models (%d) for one launch", nblock);
+    const int h1 = hidden > 0 ? hidden : 1;
+    size_t smem = ((size_t)k * h1 + h1 + hidden) * sizeof(float);
+    DBK_CHECK(smem <= 65536, "ValueError: head weights (%zu bytes per model) do not fit in LDS", smem);
+    unsigned gx = dbk::divup(n, 256);
+    if (gx > 2048u) gx = 2048u;
+    auto kern = k <= 16 ? k_head<16> : (k <= 32 ? k_head<32> : k_head<64>);
+    hipLaunchKernelGGL(kern, dim3(gx, nblock), dim3(256), smem, dbk::as_stream(stream), n, nblock, k, hidden, pooled, in_scale,
                        W1, b1, W2, b2, apply_logistic != 0, scores);
     DBK_LAUNCH_OK();
 }

@@ -7,28 +7,28 @@
 // L_0). That cuts executed VALU adds and LDS bytes per algorithmic add by 3.
 //
 // Mapping to the hardware:
-//  * A workgroup owns 32 filters. Its table lut[kmer][row][32 filters] (125 x (G+1) rows of 128 B,
-//    144 KB for m = 24) fills the CU's LDS; one workgroup per CU.
-//  * ds_read_b128 only reaches the LDS's full rate when each group of 16 lanes reads 256
-//    contiguous bytes. So a "stream" is 16 lanes walking one region: lanes 0-7 (half A) read row
-//    2i+par, lanes 8-15 (half B) the next row, 4 filters per lane. Half A owns the positions whose
-//    group-of-three index is even, half B the odd ones; "par" alternates every three steps so that
-//    each half meets each tap group of its positions exactly once. Row G repeats row 0 so half B
-//    can start a position on odd steps.
-//  * Each lane keeps a ring of 3 x G/2 float4 accumulators in VGPRs: at text position t the G/2
-//    reads add into the positions t-3g the lane owns; a position is complete 3(G-1) steps after it
-//    starts, is folded into the running max and its slot is reused. The step loop is unrolled over
-//    3G positions so every ring index is a compile-time register.
+//  * A workgroup owns 32 filters. Its table fills the CU's LDS (126 KB for m = 24), one workgroup
+//    per CU: lut[triple][line i][lane l][4 floats] with line i holding tap groups 2i and 2i+1 and the
+//    lane's 16 bytes holding (group 2i, filters 2l and 2l+1 | group 2i+1, filters 2l and 2l+1).
+//  * ds_read_b128 only reaches the LDS's full rate (~210 B/clk/CU measured, against ~155 otherwise)
+//    when each group of 16 lanes reads one 256-byte-ALIGNED line. So a "stream" is 16 lanes walking
+//    one region, 2 filters per lane, and a step's G/2 reads are the G/2 lines of the step's triple:
+//    always aligned, never conflicting. A wave carries 4 streams (4 regions at once).
+//  * Each lane keeps a ring of 3 x G float2 accumulators in VGPRs: at text position t the read of
+//    line i adds group 2i into position t-6i and group 2i+1 into position t-6i-3; group 0 starts a
+//    position (plain assignment), group G-1 completes it, it is folded into the running max and
+//    its slot is reused. The step loop is unrolled over 3G positions so every ring index is a
+//    compile-time register; per (position, 2 filters) that is 2(G-1) adds and ~1.3 max
+//    instructions for 2*3G algorithmic adds.
 //  * The sequence is pre-translated once into one byte per position (the triple index). A stream's
 //    16 lanes fetch a block's 3G indices cooperatively (one or two bytes per lane, one block ahead)
 //    and each step takes its index from the owning lane with a DPP row_share folded into the add
 //    that forms the LDS address: one VALU instruction of addressing per step.
-//
 //  * Positions outside a region never need a test. At a region's start every ring slot is reset to
 //    a large negative "poison" (-1e30), so the partial sums in flight from before the region finish
 //    far below any real value; and the steps a region's last block runs past its final useful
-//    position read a 126th table entry whose rows are all poison, which sinks exactly the positions
-//    that lie beyond the region. The running max ignores both, and ReLU follows the max.
+//    position read a 126th table entry that is all poison, which sinks exactly the positions that
+//    lie beyond the region. The running max ignores both, and ReLU follows the max.
 //
 // Shapes this path declines (filter length > 24, average pooling, argmax, code 254 present, regions
 // reaching past the last row the scan defines) go through the general kernel in scanpool.hip.
@@ -38,6 +38,7 @@
 #include "dbk_common.h"
 #include "scan_common.h"
 #include <cmath>
+#include <cstdlib>
 
 namespace dbk_scanpool_general {
 int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
@@ -83,22 +84,6 @@ __global__ __launch_bounds__(256) void kmer_index_kernel(const uint8_t* __restri
     if (saw) atomicOr(flag, 1u);
 }
 
-__device__ __forceinline__ void add4(float4& a, const float4& v) { a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w; }
-__device__ __forceinline__ void fma4(float4& a, float s, const float4& v)
-{
-    a.x = __builtin_fmaf(a.x, s, v.x); a.y = __builtin_fmaf(a.y, s, v.y);
-    a.z = __builtin_fmaf(a.z, s, v.z); a.w = __builtin_fmaf(a.w, s, v.w);
-}
-__device__ __forceinline__ void max4(float4& m, const float4& v)
-{
-    m.x = fmaxf(m.x, v.x); m.y = fmaxf(m.y, v.y); m.z = fmaxf(m.z, v.z); m.w = fmaxf(m.w, v.w);
-}
-__device__ __forceinline__ void max4x2(float4& m, const float4& u, const float4& v)
-{
-    m.x = fmaxf(fmaxf(m.x, u.x), v.x); m.y = fmaxf(fmaxf(m.y, u.y), v.y);
-    m.z = fmaxf(fmaxf(m.z, u.z), v.z); m.w = fmaxf(fmaxf(m.w, u.w), v.w);
-}
-
 // Value of `v` held by lane `src` of the caller's row of 16 lanes (DPP row_share, folded by the
 // compiler into the consuming VALU instruction).
 template <int SRC>
@@ -110,16 +95,14 @@ __device__ __forceinline__ unsigned row_share(unsigned v)
 // One unrolled block of 3G text positions for one lane.
 //   k0, k1    table byte offsets (triple index * bytes per triple) of this block's positions, spread
 //             over the stream's 16 lanes: lane i holds position i in k0 and position 16+i in k1
-//   acc       ring of partial sums, mx the running max
+//   acc       ring of partial sums (2 filters per lane), mx the running max
 template <int G>
 __device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigned k0, unsigned k1,
-                                           float4 (&acc)[3][G / 2], float4& mx, unsigned lanebase, bool isA,
-                                           float mulA, float mulB)
+                                           float2 (&acc)[3][G], float2& mx, unsigned lanebase)
 {
     constexpr int H = G / 2;
 #pragma unroll
     for (int q = 0; q < G; ++q) {
-        const int par = q & 1, sb = q >> 1;
 #pragma unroll
         for (int c = 0; c < 3; ++c) {
             const int t = 3 * q + c;
@@ -135,35 +118,33 @@ __device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigne
             const unsigned addr = koff + lanebase;
 #pragma unroll
             for (int i = 0; i < H; ++i) {
-                const int slot = (((sb - i) % H) + H) % H;
-                const float4 v = *reinterpret_cast<const float4*>(lds + addr + (2 * i + par) * ROWB);
-                if (par == 0 && i == 0) fma4(acc[c][slot], mulB, v);            // half A starts a position here
-                else if (par == 1 && i == H - 1) fma4(acc[c][slot], mulA, v);   // half B starts a position here
-                else add4(acc[c][slot], v);
+                const float4 v = *reinterpret_cast<const float4*>(lds + addr + i * 256);
+                const int s0 = (((q - 2 * i) % G) + G) % G;          // position t - 6i   takes group 2i
+                const int s1 = (((q - 2 * i - 1) % G) + G) % G;      // position t - 6i-3 takes group 2i+1
+                if (i == 0) { acc[c][s0].x = v.x; acc[c][s0].y = v.y; }     // group 0 starts a position
+                else { acc[c][s0].x += v.x; acc[c][s0].y += v.y; }
+                acc[c][s1].x += v.z; acc[c][s1].y += v.w;
             }
         }
-        // the half that just read its last tap group (B on even q, A on odd q) has three finished positions
-        const int cs = (((sb - (H - 1)) % H) + H) % H;
-        const bool mine = (par == 0) ? !isA : isA;
-        if (mine) {
-            max4x2(mx, acc[0][cs], acc[1][cs]);
-            max4(mx, acc[2][cs]);
-        }
+        // group G-1 just landed in slot (q+1) mod G of each class: three finished positions
+        const int cs = (q + 1) % G;
+        mx.x = fmaxf(fmaxf(mx.x, acc[0][cs].x), acc[1][cs].x); mx.y = fmaxf(fmaxf(mx.y, acc[0][cs].y), acc[1][cs].y);
+        mx.x = fmaxf(mx.x, acc[2][cs].x); mx.y = fmaxf(mx.y, acc[2][cs].y);
     }
 }
 
-template <int G>
-__global__ __launch_bounds__(512) void scanpool_kmer_kernel(const float* __restrict__ W, const float* __restrict__ bias,
+template <int G, int MAXT>
+__global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __restrict__ W, const float* __restrict__ bias,
                                                             unsigned m, unsigned F, const uint8_t* __restrict__ K, size_t N,
                                                             const uint32_t* __restrict__ R, unsigned P, unsigned nsplit,
                                                             const unsigned* __restrict__ flag, float* __restrict__ pooled)
 {
-    constexpr int H = G / 2, STEPS = 3 * G;
-    constexpr unsigned KSTRIDE = (G + 1) * ROWB;
+    constexpr int STEPS = 3 * G;
+    constexpr unsigned KSTRIDE = G * ROWB;                     // bytes per triple: G/2 lines of 256 B
     extern __shared__ __align__(16) unsigned char smem[];
     if (flag[0] != 0) return;                                   // the general kernel takes this call
     float* lut = reinterpret_cast<float*>(smem);
-    float* w5 = lut + (size_t)(NKMER + 1) * (G + 1) * FTILE;   // [3G taps][5 letters][32 filters]
+    float* w5 = lut + (size_t)(NKMER + 1) * G * FTILE;         // [3G taps][5 letters][32 filters]
 
     const unsigned split = blockIdx.x % nsplit, tile = blockIdx.x / nsplit;
     const unsigned f0 = tile * FTILE;
@@ -183,11 +164,11 @@ __global__ __launch_bounds__(512) void scanpool_kmer_kernel(const float* __restr
         row[0 * FTILE] = w0; row[1 * FTILE] = w1; row[2 * FTILE] = w2; row[3 * FTILE] = w3; row[4 * FTILE] = z * 0.25f;
     }
     __syncthreads();
-    // ---- the 3-mer table: taps in ascending order, bias first for group 0; row G repeats row 0;
-    //      entry 125 is all poison
-    for (unsigned e = threadIdx.x; e < (unsigned)(NKMER + 1) * (G + 1) * FTILE; e += blockDim.x) {
-        const unsigned fl = e % FTILE, row = (e / FTILE) % (G + 1), km = e / (FTILE * (G + 1));
-        const unsigned g = row == (unsigned)G ? 0u : row;
+    // ---- the 3-mer table: taps in ascending order, bias first for group 0; entry 125 is all poison.
+    //      element e -> (triple, line i, lane l, j): group 2i + j/2, filter 2l + j%2
+    for (unsigned e = threadIdx.x; e < (unsigned)(NKMER + 1) * G * FTILE; e += blockDim.x) {
+        const unsigned j = e & 3u, l = (e >> 2) & 15u, i = (e >> 6) % (unsigned)(G / 2), km = e / (unsigned)(G * FTILE);
+        const unsigned g = 2 * i + (j >> 1), fl = 2 * l + (j & 1u);
         const unsigned l0 = km / 25u, l1 = (km / 5u) % 5u, l2 = km % 5u;
         float s = POISON;
         if (km < (unsigned)NKMER) {
@@ -201,10 +182,8 @@ __global__ __launch_bounds__(512) void scanpool_kmer_kernel(const float* __restr
     __syncthreads();
 
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = blockDim.x >> 6;
-    const unsigned q8 = lane & 7, sidx = lane >> 4;
-    const bool isA = ((lane >> 3) & 1) == 0;
-    const unsigned lanebase = (isA ? 0u : (unsigned)ROWB) + q8 * 16u;
-    const float mulA = isA ? 1.0f : 0.0f, mulB = isA ? 0.0f : 1.0f;
+    const unsigned sidx = lane >> 4;
+    const unsigned lanebase = (lane & 15u) * 16u;
     const unsigned nstream = nsplit * nwave * 4u;
     constexpr unsigned TAIL = 3 * (G - 1);                       // steps between a position's start and its completion
 
@@ -230,12 +209,12 @@ __global__ __launch_bounds__(512) void scanpool_kmer_kernel(const float* __restr
     unsigned k0, k1;
     fetch(a, r < P ? rows + TAIL : 0u, 0u, k0, k1);
 
-    float4 acc[3][H];
+    float2 acc[3][G];
 #pragma unroll
     for (int c = 0; c < 3; ++c)
 #pragma unroll
-        for (int s = 0; s < H; ++s) acc[c][s] = make_float4(POISON, POISON, POISON, POISON);
-    float4 mx = make_float4(POISON, POISON, POISON, POISON);
+        for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
+    float2 mx = make_float2(POISON, POISON);
     unsigned blk = 0;
     const char* lds = reinterpret_cast<const char*>(smem);
 
@@ -247,28 +226,23 @@ __global__ __launch_bounds__(512) void scanpool_kmer_kernel(const float* __restr
         unsigned n0, n1;
         if (last) fetch(a_next, (r < P && r + nstream < P) ? rows_next + TAIL : 0u, 0u, n0, n1);
         else fetch(a + (blk + 1) * STEPS, rows + TAIL, (blk + 1) * STEPS, n0, n1);
-        scan_block<G>(lds, k0, k1, acc, mx, lanebase, isA, mulA, mulB);
+        scan_block<G>(lds, k0, k1, acc, mx, lanebase);
         k0 = n0;
         k1 = n1;
         if (last) {
-            // fold the two halves, ReLU, store this region's 32 pooled features
-            float4 o;
-            o.x = fmaxf(mx.x, __shfl_xor(mx.x, 8, 64)); o.y = fmaxf(mx.y, __shfl_xor(mx.y, 8, 64));
-            o.z = fmaxf(mx.z, __shfl_xor(mx.z, 8, 64)); o.w = fmaxf(mx.w, __shfl_xor(mx.w, 8, 64));
-            if (active && isA) {
-                const unsigned f = f0 + q8 * 4;
+            // ReLU and store this lane's two of the region's 32 pooled features
+            if (active) {
+                const unsigned f = f0 + (lane & 15u) * 2;
                 float* out = pooled + (size_t)r * F + f;
-                if (f + 0 < F) out[0] = fmaxf(o.x, 0.f);
-                if (f + 1 < F) out[1] = fmaxf(o.y, 0.f);
-                if (f + 2 < F) out[2] = fmaxf(o.z, 0.f);
-                if (f + 3 < F) out[3] = fmaxf(o.w, 0.f);
+                if (f + 0 < F) out[0] = fmaxf(mx.x, 0.f);
+                if (f + 1 < F) out[1] = fmaxf(mx.y, 0.f);
             }
             // new region: everything still in the ring belongs to the old one
-            mx = make_float4(POISON, POISON, POISON, POISON);
+            mx = make_float2(POISON, POISON);
 #pragma unroll
             for (int c = 0; c < 3; ++c)
 #pragma unroll
-                for (int s = 0; s < H; ++s) acc[c][s] = make_float4(POISON, POISON, POISON, POISON);
+                for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
             r = r < P ? r + nstream : r;
             a = a_next; rows = rows_next; blk = 0;
             nblk = (rows + TAIL + STEPS - 1) / STEPS;
@@ -285,14 +259,17 @@ template <int G>
 int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* K, size_t N,
            const uint32_t* R, size_t P, const unsigned* flag, float* pooled)
 {
-    size_t smem = ((size_t)(NKMER + 1) * (G + 1) * FTILE + (size_t)3 * G * 5 * FTILE) * sizeof(float);
+    size_t smem = ((size_t)(NKMER + 1) * G * FTILE + (size_t)3 * G * 5 * FTILE) * sizeof(float);
     if (smem > dbk_scan::lds_limit()) return -1;
     const unsigned ntile = dbk::divup(F, FTILE);
     unsigned nsplit = 256u / ntile;
     if (nsplit < 1) nsplit = 1;
-    const unsigned nwave = 8;
+    // 12 waves (3 per SIMD) measured fastest on MI355X: 8 leave LDS latency exposed, 16 add nothing.
+    unsigned nwave = 12;
+    if (const char* e = getenv("DBK_KMER_WAVES")) nwave = (unsigned)atoi(e);     // tuning knob
+    if (nwave != 8 && nwave != 12 && nwave != 16) nwave = 12;
     while (nsplit > 1 && (size_t)(nsplit - 1) * nwave * 4 >= P) --nsplit;       // no more streams than regions
-    auto kern = scanpool_kmer_kernel<G>;
+    auto kern = nwave == 8 ? scanpool_kmer_kernel<G, 512> : (nwave == 12 ? scanpool_kmer_kernel<G, 768> : scanpool_kmer_kernel<G, 1024>);
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3(ntile * nsplit), dim3(nwave * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, K, N, R,
                        (unsigned)P, nsplit, flag, pooled);
