@@ -71,6 +71,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="config5", choices=["config5", "config5_small"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain copy kernel over 1 GiB (reference point for the HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path shards over models or sequences with no exchange step, "
@@ -94,6 +96,14 @@ def main():
         pooled, _ = ks.scanpool_fprop(W, b, X, R, "max")
         return ds.head_fprop(pooled, W1, b1, W2, b2, nblock=spec.nmodel)
 
+    if args.calibrate_copy:
+        # elementwise kernel that reads 1 GiB and writes 1 GiB (larger than every cache level)
+        src = torch.ones(256 << 20, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        torch.mul(src, 2.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
