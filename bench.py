@@ -64,6 +64,22 @@ def cpu_baseline(cfg, nseq_c, nseq_np):
     }
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch of the dominant kernel as measured offline with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known size) for the full-size workload;
+    None when no measurement is on file for this workload."""
+    if workload != "config5":
+        return None
+    path = os.path.join(ROOT, "profiles", "scanpool_kmer_config5_counters.md")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -123,7 +139,7 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     adds_per_s = adds / (scan_ms * 1e-3)
     # algorithmic HBM bytes of the scan+pool launch: sequence bytes in, filters in, pooled features out
-    hbm_bytes = cfg["X"].size + p["Wc"].nbytes + p["bc"].nbytes + positions * 0 + nseq * spec.F * 4
+    hbm_bytes = cfg["X"].size + p["Wc"].nbytes + p["bc"].nbytes + nseq * spec.F * 4
     out = {
         "metric": "seq_positions_per_sec_fwd_scan_pool",
         "value": positions * args.steps / elapsed,
@@ -140,7 +156,7 @@ def main():
         "model_sequences_per_s": nseq * spec.nmodel * args.steps / elapsed,
         "roofline": {
             "bound": "valu_fp32", "achieved": adds_per_s / 1e12, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": adds_per_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS, "traffic": None,
+            "frac": adds_per_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS, "traffic": measured_traffic(args.workload),
             "kernel": "fused scan+bias+relu+maxpool (dbk_scanpool_fprop launches)", "kernel_ms": scan_ms,
             "algorithmic_adds_per_launch": adds,
             "frac_of_unpacked_add_issue_rate": adds_per_s / (256 * 64 * 2.4e9),

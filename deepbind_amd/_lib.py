@@ -63,6 +63,7 @@ _SIGNATURES = {
     "dbk_colsum": [_P, _I, _P, _P, _Z, _Z],
     "dbk_relu": [_P, _I, _P, _P, _Z],
     "dbk_mul_sign": [_P, _I, _P, _P, _P, _Z],
+    "dbk_sign": [_P, _I, _P, _P, _Z],
     "dbk_logistic": [_P, _I, _P, _P, _Z],
     "dbk_loss_terms": [_P, _I, _I, _P, _P, _P, _Z],
     "dbk_sub_scale": [_P, _I, _P, _P, _D, _P, _Z],

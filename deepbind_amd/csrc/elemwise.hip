@@ -142,6 +142,10 @@ template <typename T> __global__ void k_mul_sign(const T* dZ, const T* Z, T* dX,
         dX[i] = dZ[i] * s;
     }
 }
+template <typename T> __global__ void k_sign(const T* X, T* Z, size_t n)
+{
+    GRID_STRIDE(i, n) Z[i] = (T)(X[i] > (T)0) - (T)(X[i] < (T)0);
+}
 template <typename T> __global__ void k_logistic(const T* X, T* Z, size_t n)
 {
     GRID_STRIDE(i, n) Z[i] = (T)1 / ((T)1 + exp(-X[i]));
@@ -283,6 +287,10 @@ int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
 int dbk_mul_sign(dbk_stream_t stream, int dtype, const void* dZ, const void* Z, void* dX, size_t n)
 {
     EW2(k_mul_sign, n, A(CF32(dZ), CF32(Z), F32(dX), n), A(CF64(dZ), CF64(Z), F64(dX), n));
+}
+int dbk_sign(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
+{
+    EW2(k_sign, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
 }
 int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
 {

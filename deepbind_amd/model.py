@@ -1,0 +1,230 @@
+"""A batch of independent sequence models on the model axis, and one SGD step on all of them.
+
+Host-side mirror of what the reference's node graph and trainer do for this path, built on the
+operators of this package:
+
+  layer order   motif scan -> bias -> ReLU -> max / max+avg pool -> dropout -> dense [-> bias -> ReLU -> dense]
+                -> bias -> (logistic) -> nll / mse
+                (reference: code/libs/kangaroo/kangaroo/model.py:45-132, code/libs/deepity/deepity/_io_/load.py:51-72,
+                 code/cfg/classification/M1.cfg, M2.cfg)
+  parameters    one flat vector P with its gradient dP, momentum mP and per-element learning / momentum
+                rates; every layer's weights are a view into it. Scan filters put the models side by
+                side in columns, dense weights stack them in row blocks
+                (reference: code/libs/deepity/deepity/sgd.py:287-354, std/full.py:57, kangaroo/_ext/corr1ord.py:57-58)
+  step          Nesterov: P += mu*mP; g = grad(P); mP = mu*mP - eta*g; P -= eta*g
+                (reference: code/libs/deepity/deepity/_ext/deepity_smat.py:77-117, sgd.py:121-147)
+  L1 decay      sign(W)*decay per model added to the weight gradients once step >= weight_decay_start
+                (reference: kangaroo/_ext/corr1ord.py:120-127, deepity/std/full.py:111-119)
+  loss          dA = (Z - Y)/nrow, masked by Ymask (reference: deepity/std/loss.py:98-112)
+
+Two execution modes give the same numbers: "fused" runs the scan, bias, ReLU and pooling as one kernel
+forward and one backward; "unfused" calls the drop-in operators one by one, as the reference's graph does.
+All models of one SequenceNet share pool type and hidden size; a calibration batch that mixes
+architectures is run as one SequenceNet per architecture (see ModelGroup).
+"""
+import numpy as np
+import torch
+
+from . import deepity_smat as ds
+from . import kangaroo_smat as ks
+from . import smat as sm
+
+
+class SequenceNet(object):
+    def __init__(self, nmodel, nfilter, m, pool="max", hidden=32, loss="nll", dtype=torch.float32,
+                 rate=0.01, momentum=0.9, decay_conv=0.0, decay_full=0.0, dropout=0.0,
+                 weight_decay_start=100, nesterov=True, mode="fused", device="cuda"):
+        assert pool in ("max", "avg", "all") and loss in ("nll", "mse", None)
+        self.ninst, self.nfilter, self.m = int(nmodel), int(nfilter), int(m)
+        self.pool, self.hidden, self.loss = pool, int(hidden), loss
+        self.dtype, self.device, self.mode, self.nesterov = dtype, device, mode, nesterov
+        self.weight_decay_start = weight_decay_start
+        self.step_count = 0
+        ni, nf = self.ninst, self.nfilter
+        self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
+        h = self.hidden
+        # (name, shape, axis along which models are laid out)
+        layout = [("Wc", (4 * m, nf * ni), 1), ("bc", (1, nf * ni), 1)]
+        if h > 0:
+            layout += [("W1", (self.k * ni, h), 0), ("b1", (1, h * ni), 1), ("W2", (h * ni, 1), 0), ("b2", (1, ni), 1)]
+        else:
+            layout += [("W1", (self.k * ni, 1), 0), ("b1", (1, ni), 1)]
+        self.layout = layout
+        sizes = [int(np.prod(shape)) for _, shape, _ in layout]
+        self.offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        n = int(self.offsets[-1])
+        z = lambda: torch.zeros((n, 1), dtype=dtype, device=device)
+        self.P, self.dP, self.mP, self.drate, self.mrate = z(), z(), z(), z(), z()
+        self.p, self.g = {}, {}
+        for (name, shape, _), a, b in zip(layout, self.offsets[:-1], self.offsets[1:]):
+            self.p[name] = self.P[a:b].view(shape)
+            self.g[name] = self.dP[a:b].view(shape)
+        self._per_model = {}
+        self.set_rates(rate, momentum)
+        self.decay_conv = self._vec(decay_conv)
+        self.decay_full = self._vec(decay_full)
+        self.dropout = self._vec(dropout)
+        self.use_dropout = bool(np.any(np.asarray(dropout) > 0))
+
+    # ------------------------------------------------------------------ parameters
+    def _vec(self, v):
+        v = np.broadcast_to(np.asarray(v, dtype=np.float64), (self.ninst,)).copy()
+        return torch.as_tensor(v, dtype=self.dtype, device=self.device)
+
+    def _k_of(self, name):
+        """Elements per model along the flat layout, as the reference computes it for madd_bcast
+        (reference: code/libs/deepity/deepity/sgd.py:318-323)."""
+        _, shape, axis = [l for l in self.layout if l[0] == name][0]
+        per_model = (shape[0] // self.ninst, shape[1]) if axis == 0 else (shape[0], shape[1] // self.ninst)
+        return per_model[0] * per_model[1] if axis == 0 else per_model[1]
+
+    def set_rates(self, rate, momentum):
+        """Per-model learning and momentum rates spread over the flat vectors."""
+        self.drate.zero_()
+        self.mrate.zero_()
+        ones = torch.ones_like(self.P)
+        for (name, _, _), a, b in zip(self.layout, self.offsets[:-1], self.offsets[1:]):
+            ds.madd_bcast(ones[a:b], self._vec(rate), self._k_of(name), self.drate[a:b])
+            ds.madd_bcast(ones[a:b], self._vec(momentum), self._k_of(name), self.mrate[a:b])
+
+    def set_params(self, params):
+        """Copies a dict of NumPy arrays shaped like the layout into the flat parameter vector."""
+        for name, shape, _ in self.layout:
+            src = np.asarray(params[name])
+            assert tuple(src.shape) == tuple(shape), "%s: expected %s, got %s" % (name, shape, src.shape)
+            self.p[name].copy_(torch.as_tensor(src, dtype=self.dtype))
+
+    def get_params(self):
+        torch.cuda.synchronize()
+        return {name: self.p[name].cpu().numpy().copy() for name, _, _ in self.layout}
+
+    def get_grads(self):
+        torch.cuda.synchronize()
+        return {name: self.g[name].cpu().numpy().copy() for name, _, _ in self.layout}
+
+    # ------------------------------------------------------------------ forward
+    def _conv_forward(self, X, R, want_argmax):
+        p = self.p
+        if self.mode == "fused":
+            pooled, amax = ks.scanpool_fprop(p["Wc"], p["bc"], X, R, self.pool, want_argmax=want_argmax)
+            return pooled, amax, None
+        Z = sm.zeros((X.numel(), p["Wc"].shape[1]), dtype=self.dtype, device=self.device)
+        ks.corr1ord(p["Wc"], X, Z, 4)
+        A = sm.relu(sm.add_rowvec(Z, p["bc"]))
+        pooled, amax = ks.poolrgn(A, R, self.pool, want_argmax=want_argmax)
+        return pooled, amax, A
+
+    def forward(self, X, R, train=False, U=None, want_argmax=False):
+        """Returns the state dict of one forward pass; st["Z"] are the predictions (n x ninst)."""
+        p, ni = self.p, self.ninst
+        st = {}
+        st["pooled"], st["argmax"], st["A0"] = self._conv_forward(X, R, want_argmax)
+        H0 = st["pooled"]
+        if self.use_dropout:
+            if train:
+                H0, st["M"] = ds.dropout_fp_train(H0, self.dropout, False, U=U)
+            else:
+                H0 = ds.dropout_fp_test(H0, self.dropout)
+        st["H0"] = H0
+        A1 = sm.add_rowvec(ds.blockwise_dot(H0, p["W1"], ni), p["b1"])
+        if self.hidden > 0:
+            st["H1"] = sm.relu(A1)
+            A2 = sm.add_rowvec(ds.blockwise_dot(st["H1"], p["W2"], ni), p["b2"])
+        else:
+            A2 = A1
+        st["A"] = A2
+        st["Z"] = sm.logistic(A2) if self.loss == "nll" else A2
+        return st
+
+    def predict(self, X, R):
+        """Test-mode predictions through the fused scoring head (dropout rescale folded in)."""
+        p = self.p
+        pooled, _, _ = self._conv_forward(X, R, False)
+        if self.dtype != torch.float32:
+            return self.forward(X, R)["Z"]
+        scale = (1.0 - self.dropout) if self.use_dropout else None
+        return ds.head_fprop(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), nblock=self.ninst,
+                             in_scale=scale, apply_logistic=(self.loss == "nll"))
+
+    def loss_value(self, st, Y, Ymask=None):
+        """Per-model mean loss (1 x ninst), on the host (reference: deepity/std/loss.py:52-82)."""
+        L = sm.loss_terms(st["Z"], Y, self.loss)
+        if Ymask is not None:
+            ds.maskout(Ymask, L)
+        L = sm.sum_axis0(L)
+        torch.cuda.synchronize()
+        L = L.cpu().numpy() / st["Z"].shape[0]
+        return -L if self.loss == "nll" else 0.5 * L
+
+    # ------------------------------------------------------------------ backward
+    def backward(self, X, R, st, Y, Ymask=None):
+        """Fills dP with the gradient of the summed per-model losses (plus L1 decay when active)."""
+        p, g, ni = self.p, self.g, self.ninst
+        dA = sm.sub_scale(st["Z"], Y, 1.0 / st["Z"].shape[0])
+        if Ymask is not None:
+            ds.maskout(Ymask, dA)
+        if self.hidden > 0:
+            g["b2"].copy_(sm.sum_axis0(dA))
+            g["W2"].copy_(ds.blockwise_dot_tn(st["H1"], dA, ni, p["W2"]))
+            dA1 = sm.mul_sign(ds.blockwise_dot_nt(dA, p["W2"], ni), st["H1"])
+        else:
+            dA1 = dA
+        g["b1"].copy_(sm.sum_axis0(dA1))
+        g["W1"].copy_(ds.blockwise_dot_tn(st["H0"], dA1, ni, p["W1"]))
+        dH0 = ds.blockwise_dot_nt(dA1, p["W1"], ni)
+        if self.use_dropout:
+            dH0 = ds.dropout_bp_tr(dH0, st["M"]) if "M" in st else ds.dropout_bp_te(dH0, self.dropout)
+        g["Wc"].zero_()
+        if self.mode == "fused":
+            ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, st["pooled"], st["argmax"], dH0, g["Wc"], g["bc"])
+        else:
+            dA0 = sm.zeros_like(st["A0"])
+            ks.poolrgn_bprop(dA0, R, dH0, st["argmax"], self.pool)
+            dZ0 = sm.mul_sign(dA0, st["A0"])
+            g["bc"].copy_(sm.sum_axis0(dZ0))
+            ks.corr1ord_bprop_W(g["Wc"], X, dZ0, 4)
+        if self.weight_decay_start <= self.step_count:
+            # the reference passes rows/ninst as the block length for the scan filters although their
+            # models lie along columns (kangaroo/_ext/corr1ord.py:126); kept as is for step parity
+            kq = max(1, p["Wc"].shape[0] // ni)
+            ds.madd_bcast(sm.sign(p["Wc"]), self.decay_conv, kq, g["Wc"])
+            ds.madd_bcast(sm.sign(p["W1"]), self.decay_full, p["W1"].numel() // ni, g["W1"])
+            if self.hidden > 0:
+                ds.madd_bcast(sm.sign(p["W2"]), self.decay_full, p["W2"].numel() // ni, g["W2"])
+
+    # ------------------------------------------------------------------ one optimiser step
+    def train_step(self, X, R, Y, Ymask=None, U=None):
+        def grad():
+            st = self.forward(X, R, train=True, U=U, want_argmax=True)
+            self.backward(X, R, st, Y, Ymask)
+        ds.gradstep(self.P, self.dP, self.drate, self.mP, self.mrate, grad, nesterov=self.nesterov)
+        self.step_count += 1
+
+
+class ModelGroup(object):
+    """A calibration batch whose models differ in pool type / hidden size: one SequenceNet per
+    architecture, all stepped on the same shared batch. Column j of the outputs is model j of the
+    original ordering."""
+
+    def __init__(self, pools, hiddens, nfilter, m, loss="nll", **per_model):
+        self.nmodel = len(pools)
+        keys = sorted(set(zip(pools, hiddens)))
+        self.groups = []
+        for key in keys:
+            idx = [j for j in range(self.nmodel) if (pools[j], hiddens[j]) == key]
+            kw = {k: (np.asarray(v)[idx] if np.ndim(v) else v) for k, v in per_model.items()}
+            self.groups.append((idx, SequenceNet(len(idx), nfilter, m, pool=key[0], hidden=key[1], loss=loss, **kw)))
+
+    def train_step(self, X, R, Y, Ymask=None, U=None):
+        """U, when given, is a list with one uniforms tensor per architecture group (see self.groups)."""
+        for gi, (idx, net) in enumerate(self.groups):
+            ii = torch.as_tensor(idx, device=Y.device)
+            Yg = Y.index_select(1, ii).contiguous()
+            Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
+            net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
+
+    def predict(self, X, R):
+        out = torch.empty((R.shape[0], self.nmodel), dtype=torch.float32, device=X.device)
+        for idx, net in self.groups:
+            out[:, torch.as_tensor(idx, device=X.device)] = net.predict(X, R)
+        return out

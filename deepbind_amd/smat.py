@@ -78,6 +78,13 @@ def mul_sign(dZ, Z):
     return dX
 
 
+def sign(X):
+    """(x > 0) - (x < 0)."""
+    Z = torch.empty_like(X)
+    call("dbk_sign", stream(), dtype_code(X), ptr(X), ptr(Z), X.numel())
+    return Z
+
+
 def logistic(X):
     Z = torch.empty_like(X)
     call("dbk_logistic", stream(), dtype_code(X), ptr(X), ptr(Z), X.numel())

@@ -223,6 +223,8 @@ int dbk_colsum(dbk_stream_t stream, int dtype, const void* X, void* out, size_t 
 int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n);
 /* dX = dZ * sign(Z), sign = (z>0)-(z<0). reference: deepity/std/elemwise.py:78, smat_cuda/elemwise2.cu:42,77 */
 int dbk_mul_sign(dbk_stream_t stream, int dtype, const void* dZ, const void* Z, void* dX, size_t n);
+/* Z = (x>0)-(x<0) (L1 weight-decay gradient). reference: smat_cuda/elemwise2.cu:42,77 */
+int dbk_sign(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n);
 /* Z = 1/(1+exp(-X)). reference: smat_cuda/elemwise2.cu:46,68 */
 int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n);
 /* Elementwise loss terms L (n rows, m cols): kind 0 = log(max(1e-15,Z))*Y + log(max(1e-15,1-Z))*(1-Y),

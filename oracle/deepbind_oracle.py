@@ -506,3 +506,51 @@ def model_backward(params, X, R, st, dA, nmodel, pool, hidden, dropout=None, tra
     g["Wc"] = np.zeros_like(params["Wc"])
     corr1ord_bprop_W(g["Wc"], X, dZ0)
     return g
+
+
+# ----------------------------------------------------------------------------------------------
+# one optimiser step on a homogeneous batch of models
+# deepity/deepity/sgd.py:121-147,287-354 ; deepity/_ext/deepity_smat.py:77-117 ;
+# kangaroo/_ext/corr1ord.py:120-138 ; deepity/std/full.py:111-119
+# ----------------------------------------------------------------------------------------------
+def _per_element(values, shape, nmodel, axis):
+    """Spread one value per model over a parameter whose models lie along `axis`."""
+    values = np.broadcast_to(np.asarray(values, dtype=np.float64), (nmodel,))
+    out = np.empty(shape)
+    per = shape[axis] // nmodel
+    for b in range(nmodel):
+        if axis == 0:
+            out[b * per:(b + 1) * per, :] = values[b]
+        else:
+            out[:, b * per:(b + 1) * per] = values[b]
+    return out
+
+
+PARAM_AXIS = {"Wc": 1, "bc": 1, "W1": 0, "b1": 1, "W2": 0, "b2": 1}
+
+
+def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum, Ymask=None, dropout=None,
+               decay_conv=0.0, decay_full=0.0, step=0, weight_decay_start=100):
+    """Nesterov step in place on params / mom (dicts of arrays). dropout = (rates, U) or None."""
+    names = [n for n in ("Wc", "bc", "W1", "b1", "W2", "b2") if n in params]
+    eta = {n: _per_element(rate, params[n].shape, nmodel, PARAM_AXIS[n]).astype(params[n].dtype) for n in names}
+    mu = {n: _per_element(momentum, params[n].shape, nmodel, PARAM_AXIS[n]).astype(params[n].dtype) for n in names}
+    for n in names:
+        gradstep_nesterov1(params[n], mom[n], mu[n])
+    out = "logistic" if loss == "nll" else "linear"
+    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=True)
+    dA = loss_bprop(st["Zout"], Y, Ymask=Ymask)
+    g = model_backward(params, X, R, st, dA, nmodel, pool, hidden, dropout=dropout, train=True)
+    if weight_decay_start <= step:
+        # scan filters: the reference indexes its per-model decay with block length rows/ninst over the
+        # flattened (4m, F) matrix (kangaroo/_ext/corr1ord.py:126), kept literally
+        W = params["Wc"]
+        kq = max(1, W.shape[0] // nmodel)
+        madd_bcast(sign(W), np.broadcast_to(np.asarray(decay_conv, dtype=W.dtype), (nmodel,)), kq, g["Wc"])
+        for n in ("W1", "W2"):
+            if n in params:
+                Wn = params[n]
+                madd_bcast(sign(Wn), np.broadcast_to(np.asarray(decay_full, dtype=Wn.dtype), (nmodel,)), Wn.size // nmodel, g[n])
+    for n in names:
+        gradstep_nesterov2(params[n], g[n].astype(params[n].dtype), eta[n], mom[n], mu[n])
+    return st, g

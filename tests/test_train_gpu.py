@@ -1,0 +1,122 @@
+"""GPU parity of whole training steps (forward + backward + Nesterov update) on the benchmark's
+training configurations against the float64 CPU oracle, in both execution modes, plus bit-stability."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import deepbind_oracle as orc
+from tests.gpu_util import assert_close, dev, host
+
+pytestmark = pytest.mark.gpu
+
+ACT, GRAD = 1e-5, 1e-4
+
+
+def _f64(d):
+    return {k: np.asarray(v, dtype=np.float64).copy() for k, v in d.items()}
+
+
+def _run_config(cfg, mode, nsteps, dropout_rate=0.0, decay=(0.0, 0.0), weight_decay_start=100, bias_jitter=0.01):
+    from deepbind_amd.model import SequenceNet
+    spec = cfg["spec"]
+    rng = np.random.default_rng(99)
+    params = {k: v.copy() for k, v in cfg["params"].items()}
+    for k in params:                                   # non-zero biases so every gradient path is exercised
+        if k.startswith("b"):
+            params[k] = (rng.standard_normal(params[k].shape) * bias_jitter).astype(np.float32)
+    net = SequenceNet(spec.nmodel, spec.nfilter, spec.m, pool=spec.pool[0], hidden=spec.hidden[0], loss=spec.loss,
+                      rate=cfg.get("rate", 0.01), momentum=cfg.get("momentum", 0.9), dropout=dropout_rate,
+                      decay_conv=decay[0], decay_full=decay[1], weight_decay_start=weight_decay_start, mode=mode)
+    net.set_params(params)
+    X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
+    U = cfg.get("U")
+    Ud = dev(U) if (U is not None and dropout_rate > 0) else None
+    ref_p, ref_m = _f64(params), {k: np.zeros(v.shape) for k, v in params.items()}
+    drop = (np.full(spec.nmodel, dropout_rate), U) if dropout_rate > 0 else None
+    for step in range(nsteps):
+        net.train_step(X, R, Y, U=Ud)
+        st, g = orc.train_step(ref_p, ref_m, cfg["X"], cfg["R"], cfg["Y"].astype(np.float64), spec.nmodel, spec.pool[0],
+                               spec.hidden[0], spec.loss, cfg.get("rate", 0.01), cfg.get("momentum", 0.9), dropout=drop,
+                               decay_conv=decay[0], decay_full=decay[1], step=step, weight_decay_start=weight_decay_start)
+        got_g = net.get_grads()
+        for k in g:
+            assert_close(got_g[k], g[k], GRAD, "step %d grad %s (%s)" % (step, k, mode))
+    got = net.get_params()
+    for k in ref_p:
+        assert_close(got[k], ref_p[k], GRAD, "params %s after %d steps (%s)" % (k, nsteps, mode))
+    return net, got
+
+
+@pytest.mark.parametrize("mode", ["fused", "unfused"])
+def test_config2_rna_regression_train_steps(mode):
+    from deepbind_amd import synth
+    _run_config(synth.config2(), mode, nsteps=3)
+
+
+@pytest.mark.parametrize("mode", ["fused", "unfused"])
+def test_config3_classification_train_steps_with_dropout_and_decay(mode):
+    from deepbind_amd import synth
+    cfg = synth.config3()
+    _run_config(cfg, mode, nsteps=3, dropout_rate=0.5, decay=(1e-4, 1e-3), weight_decay_start=1)
+
+
+def test_train_step_is_bit_stable_and_modes_agree():
+    from deepbind_amd import synth
+    cfg = synth.config3()
+    _, a = _run_config(cfg, "fused", nsteps=2, dropout_rate=0.5)
+    _, b = _run_config(cfg, "fused", nsteps=2, dropout_rate=0.5)
+    for k in a:
+        assert np.array_equal(a[k], b[k]), "run-to-run difference in %s" % k
+    _, c = _run_config(cfg, "unfused", nsteps=2, dropout_rate=0.5)
+    for k in a:
+        assert_close(a[k], c[k], GRAD, "fused vs unfused %s" % k)
+
+
+def test_config1_forward_scores():
+    from deepbind_amd import synth
+    from deepbind_amd.model import SequenceNet
+    cfg = synth.config1()
+    spec = cfg["spec"]
+    net = SequenceNet(1, spec.nfilter, spec.m, pool="max", hidden=32, loss=None)
+    net.set_params(cfg["params"])
+    st = orc.model_forward(_f64(cfg["params"]), cfg["X"], cfg["R"], 1, "max", 32)
+    got = host(net.predict(dev(cfg["X"]), dev(cfg["R"])))
+    assert got.shape == (64, 1)
+    assert_close(got, st["A"], ACT, "config 1 scores")
+    assert_close(host(net.forward(dev(cfg["X"]), dev(cfg["R"]))["Z"]), st["A"], ACT, "config 1 scores (layer by layer)")
+
+
+def test_config4_calibration_batch_mixed_architectures():
+    """90 models (30 hyper-parameter draws x 3 folds), pool and hidden size chosen per model, shared batch."""
+    from deepbind_amd import synth
+    from deepbind_amd.model import ModelGroup
+    cfg = synth.config4()
+    spec, hp = cfg["spec"], cfg["hp"]
+    grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
+                     decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=0.0, weight_decay_start=0)
+    assert len(grp.groups) <= 4 and sum(len(i) for i, _ in grp.groups) == 90
+    for idx, net in grp.groups:
+        stacked = {}
+        for name, shape, axis in net.layout:
+            parts = [cfg["models"][j][name] for j in idx]
+            stacked[name] = np.concatenate(parts, axis=axis)
+        net.set_params(stacked)
+    X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
+    nsteps = 2
+    for _ in range(nsteps):
+        grp.train_step(X, R, Y, M)
+    # the oracle steps each architecture group with the same model-axis layout (the reference's
+    # scan-filter decay indexing depends on the number of models sharing a graph, so the grouping is part of the semantics)
+    for idx, net in grp.groups:
+        pool, hid = net.pool, net.hidden
+        p = {name: np.concatenate([cfg["models"][j][name] for j in idx], axis=axis).astype(np.float64) for name, _, axis in net.layout}
+        mom = {k: np.zeros(v.shape) for k, v in p.items()}
+        for step in range(nsteps):
+            orc.train_step(p, mom, cfg["X"], cfg["R"], cfg["Y"][:, idx].astype(np.float64), len(idx), pool, hid, "nll",
+                           hp["rate"][idx], hp["momentum"][idx], Ymask=cfg["Ymask"][:, idx],
+                           decay_conv=hp["decay_conv"][idx], decay_full=hp["decay_full"][idx], step=step, weight_decay_start=0)
+        got = net.get_params()
+        for k in p:
+            assert_close(got[k], p[k], GRAD, "%s/%d group %s" % (pool, hid, k))
+    scores = host(grp.predict(X, R))
+    assert scores.shape == (256, 90) and np.isfinite(scores).all() and scores.min() >= 0 and scores.max() <= 1
