@@ -80,6 +80,44 @@ def measured_traffic(workload):
     return None
 
 
+def train_throughput(steps=30, warmup=5):
+    """Secondary figures: whole train steps (forward + backward + Nesterov update) per second on the
+    three training configurations, fused mode. sequences/s = batch rows * steps / wall time."""
+    import torch
+    from deepbind_amd import synth
+    from deepbind_amd.model import ModelGroup, SequenceNet
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    out = {}
+
+    def timed(fn, nseq, nmodel):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        return {"ms_per_step": dt * 1e3, "sequences_per_s": nseq / dt, "model_sequences_per_s": nseq * nmodel / dt}
+
+    for name, cfg, drop in (("config2_rna_regression", synth.config2(), 0.0), ("config3_classification", synth.config3(), 0.5)):
+        spec = cfg["spec"]
+        net = SequenceNet(1, spec.nfilter, spec.m, pool=spec.pool[0], hidden=spec.hidden[0], loss=spec.loss,
+                          rate=cfg["rate"], momentum=cfg["momentum"], dropout=drop)
+        net.set_params(cfg["params"])
+        X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
+        out[name] = timed(lambda: net.train_step(X, R, Y), len(cfg["R"]), 1)
+    cfg = synth.config4()
+    spec, hp = cfg["spec"], cfg["hp"]
+    grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
+                     decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"])
+    for idx, net in grp.groups:
+        net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
+    X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
+    out["config4_calibration_90_models"] = timed(lambda: grp.train_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -87,6 +125,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="config5", choices=["config5", "config5_small"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-train", action="store_true", help="skip the secondary train-step throughput figures")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain copy kernel over 1 GiB (reference point for the HBM byte counters)")
     args = ap.parse_args()
@@ -164,6 +203,8 @@ def main():
                     "peak_GBs": HBM_PEAK_GBS, "frac": hbm_bytes / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         },
     }
+    if not args.no_train:
+        out["train"] = train_throughput()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, nseq_c=min(nseq, 1000), nseq_np=min(nseq, 100))
     print(json.dumps(out))
