@@ -52,6 +52,7 @@ _SIGNATURES = {
     "dbk_madd_bcast": [_P, _I, _P, _P, _P, _Z, _Z, _Z],
     "dbk_maskout": [_P, _I, _P, _P, _Z],
     "dbk_calc_zmask": [_P, _I, _P, _P, _Z, _Z],
+    "dbk_pair_max": [_P, _I, _P, _P, _Z, _Z],
     "dbk_dropout_fp_tr": [_P, _I, _P, _P, _P, _P, _Z, _Z, _Z, _I, _U64, _U64],
     "dbk_dropout_fp_tr_u": [_P, _I, _P, _P, _P, _P, _Z, _Z, _Z, _I, _P],
     "dbk_dropout_fp_te": [_P, _I, _P, _P, _P, _Z, _Z, _Z],

@@ -117,6 +117,14 @@ __global__ void k_dropoutord(const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n,
         Z[i] = (keep || x == 255) ? x : (uint8_t)254;
     }
 }
+template <typename T> __global__ void k_pair_max(const T* Z, T* out, size_t npair, size_t m)
+{
+    GRID_STRIDE(i, npair * m) {
+        size_t r = i / m, c = i % m;
+        T a = Z[(2 * r) * m + c], b = Z[(2 * r + 1) * m + c];
+        out[i] = a >= b ? a : b;
+    }
+}
 template <typename T> __global__ void k_add_rowvec(const T* X, const T* b, T* Z, size_t n, size_t m)
 {
     GRID_STRIDE(i, n * m) Z[i] = X[i] + b[i % m];
@@ -270,6 +278,12 @@ int dbk_dropoutord_fp_tr_u(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, ui
     if (n == 0) { dbk::clear_error(); return 0; }
     hipLaunchKernelGGL(k_dropoutord, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), X, Z, M, n, rate, U, (uint64_t)0, (uint64_t)0);
     DBK_LAUNCH_OK();
+}
+int dbk_pair_max(dbk_stream_t stream, int dtype, const void* Z, void* out, size_t n, size_t m)
+{
+    DBK_CHECK(n % 2 == 0, "ValueError: pair_max needs an even number of rows, got %zu", n);
+    size_t total = (n / 2) * m;
+    EW2(k_pair_max, total, A(CF32(Z), F32(out), n / 2, m), A(CF64(Z), F64(out), n / 2, m));
 }
 int dbk_add_rowvec(dbk_stream_t stream, int dtype, const void* X, const void* b, void* Z, size_t n, size_t m)
 {

@@ -68,6 +68,13 @@ def calc_Zmask(Z, Zmask):
     call("dbk_calc_zmask", stream(), dtype_code(Z), ptr(Z), ptr(Zmask), Z.shape[0], Z.shape[1])
 
 
+def pair_max(Z):
+    """Row-pair maximum: the score kept from each (forward, reverse-complement) pair; (n/2 x ncol)."""
+    out = torch.empty((Z.shape[0] // 2, Z.shape[1]), dtype=Z.dtype, device=Z.device)
+    call("dbk_pair_max", stream(), dtype_code(Z), ptr(Z), ptr(out), Z.shape[0], Z.shape[1])
+    return out
+
+
 def dropout_fp_train(X, rate, matchrows, U=None):
     """Z = X*M with M = (u >= rate[model of the column]); matchrows shares the draw inside each
     (fwd, rev) row pair. U (optional float32, X's shape) supplies the uniforms. Returns (Z, M).

@@ -33,12 +33,16 @@ from . import smat as sm
 class SequenceNet(object):
     def __init__(self, nmodel, nfilter, m, pool="max", hidden=32, loss="nll", dtype=torch.float32,
                  rate=0.01, momentum=0.9, decay_conv=0.0, decay_full=0.0, dropout=0.0,
-                 weight_decay_start=100, nesterov=True, mode="fused", device="cuda"):
+                 weight_decay_start=100, nesterov=True, mode="fused", reverse_complement=False, device="cuda"):
         assert pool in ("max", "avg", "all") and loss in ("nll", "mse", None)
         self.ninst, self.nfilter, self.m = int(nmodel), int(nfilter), int(m)
         self.pool, self.hidden, self.loss = pool, int(hidden), loss
         self.dtype, self.device, self.mode, self.nesterov = dtype, device, mode, nesterov
         self.weight_decay_start = weight_decay_start
+        # rows interleaved fwd,rev,fwd,rev,...: each pair shares its dropout draw and only the larger
+        # prediction of a pair contributes to loss and gradient
+        # (reference: kangaroo/kangaroo/data.py:274-306, deepity/std/loss.py:114-119, deepity_smat/dropout.cu:57-77)
+        self.reverse_complement = bool(reverse_complement)
         self.step_count = 0
         ni, nf = self.ninst, self.nfilter
         self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
@@ -122,7 +126,7 @@ class SequenceNet(object):
         H0 = st["pooled"]
         if self.use_dropout:
             if train:
-                H0, st["M"] = ds.dropout_fp_train(H0, self.dropout, False, U=U)
+                H0, st["M"] = ds.dropout_fp_train(H0, self.dropout, self.reverse_complement, U=U)
             else:
                 H0 = ds.dropout_fp_test(H0, self.dropout)
         st["H0"] = H0
@@ -134,6 +138,9 @@ class SequenceNet(object):
             A2 = A1
         st["A"] = A2
         st["Z"] = sm.logistic(A2) if self.loss == "nll" else A2
+        if self.reverse_complement:
+            st["Zmask"] = torch.zeros(st["Z"].shape, dtype=torch.bool, device=self.device)
+            ds.calc_Zmask(st["Z"], st["Zmask"])
         return st
 
     def predict(self, X, R):
@@ -141,16 +148,20 @@ class SequenceNet(object):
         p = self.p
         pooled, _, _ = self._conv_forward(X, R, False)
         if self.dtype != torch.float32:
-            return self.forward(X, R)["Z"]
+            Z = self.forward(X, R)["Z"]
+            return ds.pair_max(Z) if self.reverse_complement else Z
         scale = (1.0 - self.dropout) if self.use_dropout else None
-        return ds.head_fprop(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), nblock=self.ninst,
-                             in_scale=scale, apply_logistic=(self.loss == "nll"))
+        Z = ds.head_fprop(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), nblock=self.ninst,
+                          in_scale=scale, apply_logistic=(self.loss == "nll"))
+        return ds.pair_max(Z) if self.reverse_complement else Z
 
     def loss_value(self, st, Y, Ymask=None):
         """Per-model mean loss (1 x ninst), on the host (reference: deepity/std/loss.py:52-82)."""
         L = sm.loss_terms(st["Z"], Y, self.loss)
         if Ymask is not None:
             ds.maskout(Ymask, L)
+        if "Zmask" in st:
+            ds.maskout(st["Zmask"], L)
         L = sm.sum_axis0(L)
         torch.cuda.synchronize()
         L = L.cpu().numpy() / st["Z"].shape[0]
@@ -163,6 +174,8 @@ class SequenceNet(object):
         dA = sm.sub_scale(st["Z"], Y, 1.0 / st["Z"].shape[0])
         if Ymask is not None:
             ds.maskout(Ymask, dA)
+        if "Zmask" in st:
+            ds.maskout(st["Zmask"], dA)
         if self.hidden > 0:
             g["b2"].copy_(sm.sum_axis0(dA))
             g["W2"].copy_(ds.blockwise_dot_tn(st["H1"], dA, ni, p["W2"]))

@@ -190,6 +190,10 @@ int dbk_maskout(dbk_stream_t stream, int dtype, const uint8_t* M, void* A, size_
  * reference: launch_calc_zmask, deepity_smat.cpp:60, maskout.cu:52-67 */
 int dbk_calc_zmask(dbk_stream_t stream, int dtype, const void* Z, uint8_t* M, size_t n, size_t m);
 
+/* out[i,c] = max(Z[2i,c], Z[2i+1,c]): the prediction kept from each (fwd, rev) row pair; out is (n/2, m).
+ * reference: maskout_revcomp, kangaroo/kangaroo/predict.py:145-164 (done there on the host) */
+int dbk_pair_max(dbk_stream_t stream, int dtype, const void* Z, void* out, size_t n, size_t m);
+
 /* Dropout on pooled features with one rate per model: column c of an (n/(m*k), m*k) matrix uses
  * rate[(i/k) % m]. keep = (u >= rate). matchrows gives each (2r, 2r+1) row pair one shared draw.
  * reference: launch_dropout_fp_tr / _fp_te / _bp_tr / _bp_te, deepity_smat.cpp:62-73, dropout.cu:41-180 */

@@ -456,7 +456,7 @@ def madd_bcast(A, b, k, dst):
 # whole-model forward / backward for a homogeneous batch of models on the model axis
 # layer order: kangaroo/kangaroo/model.py:45-132 ; deepity/_io_/load.py:51-72 ; cfg/*/M{1,2}.cfg
 # ----------------------------------------------------------------------------------------------
-def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None, train=False, keep=None):
+def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None, train=False, matchrows=False):
     """scan -> bias -> relu -> pool -> dropout -> dense(+bias[,relu,dense,bias]) -> (logistic)."""
     m = params["Wc"].shape[0] // 4
     N = np.asarray(X).size
@@ -469,7 +469,7 @@ def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None
     if dropout is not None:
         rate, U = dropout
         if train:
-            H, st["M"] = dropout_fp_train(H, rate, U)
+            H, st["M"] = dropout_fp_train(H, rate, U, matchrows=matchrows)
         else:
             H = dropout_fp_test(H, rate)
     st["H0"] = H
@@ -530,7 +530,7 @@ PARAM_AXIS = {"Wc": 1, "bc": 1, "W1": 0, "b1": 1, "W2": 0, "b2": 1}
 
 
 def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum, Ymask=None, dropout=None,
-               decay_conv=0.0, decay_full=0.0, step=0, weight_decay_start=100):
+               decay_conv=0.0, decay_full=0.0, step=0, weight_decay_start=100, reverse_complement=False):
     """Nesterov step in place on params / mom (dicts of arrays). dropout = (rates, U) or None."""
     names = [n for n in ("Wc", "bc", "W1", "b1", "W2", "b2") if n in params]
     eta = {n: _per_element(rate, params[n].shape, nmodel, PARAM_AXIS[n]).astype(params[n].dtype) for n in names}
@@ -538,8 +538,9 @@ def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum,
     for n in names:
         gradstep_nesterov1(params[n], mom[n], mu[n])
     out = "logistic" if loss == "nll" else "linear"
-    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=True)
-    dA = loss_bprop(st["Zout"], Y, Ymask=Ymask)
+    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=True, matchrows=reverse_complement)
+    Zmask = calc_zmask(st["Zout"]) if reverse_complement else None      # deepity/std/loss.py:114-119
+    dA = loss_bprop(st["Zout"], Y, Ymask=Ymask, Zmask=Zmask)
     g = model_backward(params, X, R, st, dA, nmodel, pool, hidden, dropout=dropout, train=True)
     if weight_decay_start <= step:
         # scan filters: the reference indexes its per-model decay with block length rows/ninst over the

@@ -120,3 +120,39 @@ def test_config4_calibration_batch_mixed_architectures():
             assert_close(got[k], p[k], GRAD, "%s/%d group %s" % (pool, hid, k))
     scores = host(grp.predict(X, R))
     assert scores.shape == (256, 90) and np.isfinite(scores).all() and scores.min() >= 0 and scores.max() <= 1
+
+
+def test_reverse_complement_mode_train_and_predict():
+    """Interleaved fwd/rev rows: shared dropout draw per pair, only the larger prediction of a pair
+    trains, and prediction keeps the pair maximum."""
+    from deepbind_amd import data
+    from deepbind_amd.model import SequenceNet
+    rng = np.random.default_rng(5)
+    nm, nf, m, hid, B = 2, 16, 11, 8, 24
+    seqs = ["".join(rng.choice(list("ACGTN"), p=[.24, .24, .24, .24, .04], size=int(rng.integers(15, 40)))) for _ in range(B)]
+    X, R = data.pack_sequences(seqs, m - 1, reverse_complement=True)
+    assert len(R) == 2 * B
+    p = {"Wc": rng.standard_normal((4 * m, nf * nm)) * 0.2, "bc": rng.standard_normal((1, nf * nm)) * 0.05,
+         "W1": rng.standard_normal((nf * nm, hid)) * 0.3, "b1": rng.standard_normal((1, hid * nm)) * 0.1,
+         "W2": rng.standard_normal((hid * nm, 1)) * 0.5, "b2": rng.standard_normal((1, nm)) * 0.1}
+    p = {k: v.astype(np.float32) for k, v in p.items()}
+    Y = np.repeat((rng.random((B, nm)) < 0.5).astype(np.float32), 2, axis=0)
+    U = rng.random((2 * B, nf * nm)).astype(np.float32)
+    rate = np.array([0.25, 0.5])
+    net = SequenceNet(nm, nf, m, pool="max", hidden=hid, loss="nll", rate=0.05, momentum=0.9, dropout=rate,
+                      reverse_complement=True)
+    net.set_params(p)
+    q = _f64(p); mom = {k: np.zeros(v.shape) for k, v in q.items()}
+    Xd, Rd, Yd, Ud = dev(X), dev(R), dev(Y), dev(U)
+    for step in range(2):
+        net.train_step(Xd, Rd, Yd, U=Ud)
+        orc.train_step(q, mom, X, R, Y.astype(np.float64), nm, "max", hid, "nll", 0.05, 0.9, dropout=(rate, U), step=step,
+                       reverse_complement=True)
+    got = net.get_params()
+    for k in q:
+        assert_close(got[k], q[k], GRAD, "revcomp params %s" % k)
+    st = orc.model_forward(q, X, R, nm, "max", hid, out="logistic", dropout=(rate, None), train=False)
+    ref = np.maximum(st["Zout"][0::2], st["Zout"][1::2])
+    pred = host(net.predict(Xd, Rd))
+    assert pred.shape == (B, nm)
+    assert_close(pred, ref, 1e-4, "revcomp predictions")
