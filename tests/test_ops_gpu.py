@@ -412,3 +412,16 @@ def test_scanpool_auto_path_bulk(ks):
     from oracle import oracle_c
     Pr, _ = oracle_c.scanpool(W, b, X, R, 0)
     assert_close(host(P), Pr, ACT, "auto vs C oracle")
+
+
+@pytest.mark.parametrize("B,lo,hi,m,F", [(200, 101, 101, 24, 64), (150, 30, 60, 16, 40), (77, 24, 24, 24, 16), (500, 1, 5, 24, 32)])
+def test_scanpool_kmer_regions_in_any_order(ks, B, lo, hi, m, F):
+    """Regions need not be sorted or contiguous for the table kernel: shuffling the region table
+    permutes the output rows and nothing else."""
+    rng, W, b, X, R = _fused_case(31 + B + m, B, lo, hi, m, F, pn=0.03)
+    A, Pr, _ = _chain_oracle(W, b, X, R, "max")
+    P, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max", path="kmer")
+    assert_close(host(P), Pr, ACT, "packed order")
+    perm = rng.permutation(B)
+    P2, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R[perm]), "max", path="kmer")
+    assert_close(host(P2), Pr[perm], ACT, "shuffled order")
