@@ -6,36 +6,14 @@
 // Reference semantics: deepity_smat/gradstep.cu:41-72, madd_bcast.cu:41-47, maskout.cu:41-67,
 // dropout.cu:41-109, kangaroo_smat/dropoutord.cu:41-52, smat_cuda/elemwise2.cu:42-77, elemwise3.cu:57-62.
 #include "dbk_common.h"
+#include "rng.h"
 
 namespace {
 
+using dbk_rng::philox4x32_10;
+using dbk_rng::uniform_at;
+
 #define GRID_STRIDE(i, n) for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (n); i += (size_t)gridDim.x * blockDim.x)
-
-// Philox4x32-10 counter-based generator (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3").
-// One 128-bit counter value yields four 32-bit words; element i uses word i%4 of counter (offset + i/4).
-__host__ __device__ inline void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1)
-{
-    for (int r = 0; r < 10; ++r) {
-        uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
-        uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
-        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
-        uint32_t n1 = (uint32_t)p1;
-        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
-        uint32_t n3 = (uint32_t)p0;
-        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
-        k0 += 0x9E3779B9u;
-        k1 += 0xBB67AE85u;
-    }
-}
-
-// Uniform in [0,1) with 24 bits, for flat element index i.
-__device__ inline float uniform_at(uint64_t seed, uint64_t offset, size_t i)
-{
-    uint64_t ctr = offset + (uint64_t)(i >> 2);
-    uint32_t c[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u};
-    philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
-    return (float)(c[i & 3] >> 8) * (1.0f / 16777216.0f);
-}
 
 template <typename T> __global__ void k_gradstep(T* P, const T* dP, const T* drate, T* mP, const T* mrate, size_t n)
 {
@@ -129,14 +107,19 @@ template <typename T> __global__ void k_add_rowvec(const T* X, const T* b, T* Z,
 {
     GRID_STRIDE(i, n * m) Z[i] = X[i] + b[i % m];
 }
-// one thread per column, rows in ascending order (fixed summation order)
-template <typename T> __global__ void k_colsum(const T* X, T* out, size_t n, size_t m)
+// 64 columns per workgroup; wave w sums rows w, w+4, ... in ascending order and the four partial
+// sums are combined in wave order: a fixed summation order, independent of the launch
+template <typename T> __global__ __launch_bounds__(256) void k_colsum(const T* X, T* out, size_t n, size_t m)
 {
-    GRID_STRIDE(c, m) {
-        T s = (T)0;
-        for (size_t r = 0; r < n; ++r) s += X[r * m + c];
-        out[c] = s;
-    }
+    __shared__ T part[4][64];
+    const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const size_t c = (size_t)blockIdx.x * 64 + lane;
+    T s = (T)0;
+    if (c < m)
+        for (size_t r = w; r < n; r += 4) s += X[r * m + c];
+    part[w][lane] = s;
+    __syncthreads();
+    if (w == 0 && c < m) out[c] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
 }
 template <typename T> __global__ void k_relu(const T* X, T* Z, size_t n)
 {
@@ -176,6 +159,7 @@ __global__ void k_uniform_fill(float* U, size_t n, uint64_t seed, uint64_t offse
 {
     GRID_STRIDE(i, n) U[i] = uniform_at(seed, offset, i);
 }
+__global__ void k_counter_add(unsigned long long* ctr, unsigned long long delta) { if (threadIdx.x == 0 && blockIdx.x == 0) ctr[0] += delta; }
 template <typename T> __global__ void k_sub_scale(const T* Z, const T* Y, T scale, T* dZ, size_t n)
 {
     GRID_STRIDE(i, n) dZ[i] = (Z[i] - Y[i]) * scale;
@@ -292,7 +276,12 @@ int dbk_add_rowvec(dbk_stream_t stream, int dtype, const void* X, const void* b,
 }
 int dbk_colsum(dbk_stream_t stream, int dtype, const void* X, void* out, size_t n, size_t m)
 {
-    EW2(k_colsum, m, A(CF32(X), F32(out), n, m), A(CF64(X), F64(out), n, m));
+    DBK_DTYPE_OK(dtype);
+    if (m == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(dbk::divup(m, 64) <= 0x7fffffffu, "ValueError: too many columns");
+    if (dtype == DBK_F32) hipLaunchKernelGGL(k_colsum<float>, dim3(dbk::divup(m, 64)), dim3(256), 0, dbk::as_stream(stream), CF32(X), F32(out), n, m);
+    else hipLaunchKernelGGL(k_colsum<double>, dim3(dbk::divup(m, 64)), dim3(256), 0, dbk::as_stream(stream), CF64(X), F64(out), n, m);
+    DBK_LAUNCH_OK();
 }
 int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
 {
@@ -325,6 +314,13 @@ int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uin
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(U != nullptr, "ValueError: U must not be null");
     hipLaunchKernelGGL(k_uniform_fill, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), U, n, seed, offset);
+    DBK_LAUNCH_OK();
+}
+
+int dbk_counter_add(dbk_stream_t stream, uint64_t* counter, uint64_t delta)
+{
+    DBK_CHECK(counter != nullptr, "ValueError: counter must not be null");
+    hipLaunchKernelGGL(k_counter_add, dim3(1), dim3(64), 0, dbk::as_stream(stream), (unsigned long long*)counter, (unsigned long long)delta);
     DBK_LAUNCH_OK();
 }
 

@@ -236,3 +236,26 @@ def head_fprop(pooled, W1, b1, W2=None, b2=None, nblock=1, in_scale=None, apply_
     call("dbk_head_fprop", stream(), n, nblock, k, hidden, ptr(pooled), ptr(sc), ptr(W1), ptr(b1), ptr(W2), ptr(b2),
          int(bool(apply_logistic)), ptr(scores))
     return scores
+
+
+def head_train(pooled, W1, b1, W2, b2, Y, nblock, loss, dW1, db1, dW2=None, db2=None, Ymask=None, rate=None, U=None,
+               seed=0, offset=0, counter=None, reverse_complement=False, want_loss=False):
+    """Forward and backward of nblock dense heads in one launch. Returns (Z, dpooled, loss|None);
+    the weight gradients are written into dW1, db1, dW2, db2. float32 only."""
+    require(pooled.dtype == torch.float32, "TypeError: the fused head is float32 only")
+    n = pooled.shape[0]
+    k = pooled.shape[1] // nblock
+    hidden = 0 if W2 is None else W1.shape[1]
+    Z = torch.empty((n, nblock), dtype=torch.float32, device=pooled.device)
+    dpooled = torch.empty_like(pooled)
+    L = torch.empty((1, nblock), dtype=torch.float32, device=pooled.device) if want_loss else None
+    r = None if rate is None else _vec(rate, pooled)
+    call("dbk_head_train", stream(), n, nblock, k, hidden, {"nll": 0, "mse": 1}[loss], int(bool(reverse_complement)),
+         ptr(pooled), ptr(r), ptr(U), int(seed), int(offset), ptr(counter), ptr(W1), ptr(b1), ptr(W2), ptr(b2), ptr(Y), ptr(Ymask),
+         ptr(Z), ptr(dpooled), ptr(dW1), ptr(db1), ptr(dW2), ptr(db2), ptr(L))
+    return Z, dpooled, L
+
+
+def counter_add(counter, delta):
+    """counter[0] += delta on the device (int64 tensor of one element)."""
+    call("dbk_counter_add", stream(), ptr(counter), int(delta))

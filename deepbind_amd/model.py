@@ -69,6 +69,10 @@ class SequenceNet(object):
         self.decay_full = self._vec(decay_full)
         self.dropout = self._vec(dropout)
         self.use_dropout = bool(np.any(np.asarray(dropout) > 0))
+        # position of the dropout generator, kept on the device so that a captured graph advances it
+        self.rng_seed = 0
+        self.rng_counter = torch.zeros(1, dtype=torch.int64, device=device)
+        self._rng_offset = 0                 # host mirror of rng_counter (layer-by-layer mode draws from it)
 
     # ------------------------------------------------------------------ parameters
     def _vec(self, v):
@@ -126,6 +130,11 @@ class SequenceNet(object):
         H0 = st["pooled"]
         if self.use_dropout:
             if train:
+                if U is None and not self.reverse_complement:
+                    # same stream position as the fused head would use
+                    U = ds.uniform_like(H0, self.rng_seed, self._rng_offset)
+                    self._rng_offset += (H0.numel() + 3) // 4
+                    ds.counter_add(self.rng_counter, (H0.numel() + 3) // 4)
                 H0, st["M"] = ds.dropout_fp_train(H0, self.dropout, self.reverse_complement, U=U)
             else:
                 H0 = ds.dropout_fp_test(H0, self.dropout)
@@ -197,19 +206,47 @@ class SequenceNet(object):
             g["bc"].copy_(sm.sum_axis0(dZ0))
             ks.corr1ord_bprop_W(g["Wc"], X, dZ0, 4)
         if self.weight_decay_start <= self.step_count:
-            # the reference passes rows/ninst as the block length for the scan filters although their
-            # models lie along columns (kangaroo/_ext/corr1ord.py:126); kept as is for step parity
-            kq = max(1, p["Wc"].shape[0] // ni)
-            ds.madd_bcast(sm.sign(p["Wc"]), self.decay_conv, kq, g["Wc"])
-            ds.madd_bcast(sm.sign(p["W1"]), self.decay_full, p["W1"].numel() // ni, g["W1"])
-            if self.hidden > 0:
-                ds.madd_bcast(sm.sign(p["W2"]), self.decay_full, p["W2"].numel() // ni, g["W2"])
+            self._add_decay()
+
+    def _add_decay(self):
+        p, g, ni = self.p, self.g, self.ninst
+        # the reference passes rows/ninst as the block length for the scan filters although their
+        # models lie along columns (kangaroo/_ext/corr1ord.py:126); kept as is for step parity
+        kq = max(1, p["Wc"].shape[0] // ni)
+        ds.madd_bcast(sm.sign(p["Wc"]), self.decay_conv, kq, g["Wc"])
+        ds.madd_bcast(sm.sign(p["W1"]), self.decay_full, p["W1"].numel() // ni, g["W1"])
+        if self.hidden > 0:
+            ds.madd_bcast(sm.sign(p["W2"]), self.decay_full, p["W2"].numel() // ni, g["W2"])
+
+    def _grad_fused(self, X, R, Y, Ymask, U):
+        """Gradient of one batch in four launches: fused scan+pool forward, the whole dense head
+        forward+backward, fused scan+pool backward (+ its two slab reductions)."""
+        p, g = self.p, self.g
+        pooled, amax = ks.scanpool_fprop(p["Wc"], p["bc"], X, R, self.pool, want_argmax=True)
+        rate = self.dropout if self.use_dropout else None
+        Z, dpooled, _ = ds.head_train(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), Y, self.ninst, self.loss,
+                                      g["W1"], g["b1"], g.get("W2"), g.get("b2"), Ymask=Ymask, rate=rate, U=U,
+                                      seed=self.rng_seed, counter=self.rng_counter,
+                                      reverse_complement=self.reverse_complement)
+        if rate is not None and U is None:
+            ds.counter_add(self.rng_counter, (pooled.numel() + 3) // 4)
+            self._rng_offset += (pooled.numel() + 3) // 4
+        g["Wc"].zero_()
+        ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, pooled, amax, dpooled, g["Wc"], g["bc"])
+        if self.weight_decay_start <= self.step_count:
+            self._add_decay()
+        return Z
 
     # ------------------------------------------------------------------ one optimiser step
     def train_step(self, X, R, Y, Ymask=None, U=None):
+        fused = self.mode == "fused" and self.dtype == torch.float32 and self.k <= 64 and self.loss is not None
+
         def grad():
-            st = self.forward(X, R, train=True, U=U, want_argmax=True)
-            self.backward(X, R, st, Y, Ymask)
+            if fused:
+                self._grad_fused(X, R, Y, Ymask, U)
+            else:
+                st = self.forward(X, R, train=True, U=U, want_argmax=True)
+                self.backward(X, R, st, Y, Ymask)
         ds.gradstep(self.P, self.dP, self.drate, self.mP, self.mrate, grad, nesterov=self.nesterov)
         self.step_count += 1
 

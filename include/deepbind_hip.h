@@ -250,6 +250,26 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
                    const float* W1, const float* b1, const float* W2, const float* b2,
                    int apply_logistic, float* scores);
 
+/* Forward AND backward of the dense head for nblock models in one launch (one workgroup per model):
+ * dropout (rate per model, NULL = none; uniforms from U when given, else from the generator at
+ * (seed, offset), or at (seed, *counter) when counter is a device pointer) -> dense (+bias, ReLU, dense
+ * when hidden > 0) -> bias -> logistic (loss_kind 0) or identity (loss_kind 1) -> dA = (Z-Y)/n masked by
+ * Ymask (may be NULL) and, with reverse_complement, by the pair rule of dbk_calc_zmask -> all gradients.
+ * Writes Z (n, nblock), dpooled (n, k*nblock), dW1, db1, dW2, db2 (overwritten, not accumulated) and,
+ * if loss is not NULL, the per-model mean loss (nblock). Masks drawn here equal those of
+ * dbk_dropout_fp_tr for the same (seed, offset). float32; k <= 64. Deterministic.
+ * Replaces the reference's layer-by-layer head in a training step (deepity/std/elemwise.py:71-180,
+ * full.py:78-119, softmax.py:58-77, loss.py:98-119). */
+int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden, int loss_kind, int reverse_complement,
+                   const float* pooled, const float* rate, const float* U, uint64_t seed, uint64_t offset,
+                   const uint64_t* counter,
+                   const float* W1, const float* b1, const float* W2, const float* b2,
+                   const float* Y, const uint8_t* Ymask,
+                   float* Z, float* dpooled, float* dW1, float* db1, float* dW2, float* db2, float* loss);
+/* counter[0] += delta on the device (advances a generator position kept in device memory, so that a
+ * captured HIP graph draws fresh masks on every replay). */
+int dbk_counter_add(dbk_stream_t stream, uint64_t* counter, uint64_t delta);
+
 #ifdef __cplusplus
 }
 #endif

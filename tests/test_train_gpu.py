@@ -156,3 +156,54 @@ def test_reverse_complement_mode_train_and_predict():
     pred = host(net.predict(Xd, Rd))
     assert pred.shape == (B, nm)
     assert_close(pred, ref, 1e-4, "revcomp predictions")
+
+
+def test_fused_and_layerwise_steps_draw_the_same_dropout_masks():
+    """With no uniforms supplied both modes draw from the library's generator at the same stream
+    position, so three steps with dropout end in the same parameters."""
+    from deepbind_amd import synth
+    from deepbind_amd.model import SequenceNet
+    cfg = synth.config3()
+    spec = cfg["spec"]
+    out = {}
+    for mode in ("fused", "unfused"):
+        net = SequenceNet(1, spec.nfilter, spec.m, pool="max", hidden=32, loss="nll", rate=0.05, momentum=0.9, dropout=0.5, mode=mode)
+        net.rng_seed = 77
+        params = {k: v.copy() for k, v in cfg["params"].items()}
+        jit = np.random.default_rng(1)
+        for k in params:                                 # non-zero biases: a sum that cancels to ~0 has no scale to compare against
+            if k.startswith("b"):
+                params[k] = (jit.standard_normal(params[k].shape) * 0.01).astype(np.float32)
+        net.set_params(params)
+        X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
+        for _ in range(3):
+            net.train_step(X, R, Y)
+        out[mode] = net.get_params()
+        assert int(net.rng_counter.item()) == net._rng_offset == 3 * ((128 * 16 + 3) // 4)
+    for k in out["fused"]:
+        assert_close(out["fused"][k], out["unfused"][k], GRAD, "fused vs layer-by-layer %s" % k)
+
+
+def test_head_train_loss_output():
+    from deepbind_amd import deepity_smat as ds
+    rng = np.random.default_rng(3)
+    n, nb, k, h = 300, 5, 16, 32
+    Pl = np.abs(rng.standard_normal((n, k * nb))).astype(np.float32)
+    W1 = (rng.standard_normal((k * nb, h)) * 0.3).astype(np.float32); b1 = (rng.standard_normal((1, h * nb)) * 0.1).astype(np.float32)
+    W2 = (rng.standard_normal((h * nb, 1)) * 0.3).astype(np.float32); b2 = (rng.standard_normal((1, nb)) * 0.1).astype(np.float32)
+    Y = (rng.random((n, nb)) < 0.5).astype(np.float32)
+    M = rng.random((n, nb)) < 0.8
+    g = [torch.empty_like(dev(a)) for a in (W1, b1, W2, b2)]
+    Z, dP, L = ds.head_train(dev(Pl), dev(W1), dev(b1), dev(W2), dev(b2), dev(Y), nb, "nll", g[0], g[1], g[2], g[3],
+                             Ymask=dev(M), want_loss=True)
+    H = orc.relu_fprop(orc.bias_fprop(orc.blockwise_dot(Pl.astype(np.float64), W1.astype(np.float64), nb), b1))
+    A = orc.bias_fprop(orc.blockwise_dot(H, W2.astype(np.float64), nb), b2)
+    Zr = orc.logistic(A)
+    assert_close(host(Z), Zr, ACT, "Z")
+    assert_close(host(L), orc.loss_fprop(Zr, Y.astype(np.float64), "nll", nb, Ymask=M), 1e-4, "loss")
+    dA = orc.loss_bprop(Zr, Y.astype(np.float64), Ymask=M)
+    assert_close(host(g[3]), orc.bias_bprop(dA)[1], GRAD, "db2")
+    assert_close(host(g[2]), orc.blockwise_dot_tn(H, dA, nb, W2), GRAD, "dW2")
+    dA1 = orc.relu_bprop(orc.blockwise_dot_nt(dA, W2.astype(np.float64), nb), H)
+    assert_close(host(g[0]), orc.blockwise_dot_tn(Pl.astype(np.float64), dA1, nb, W1), GRAD, "dW1")
+    assert_close(host(dP), orc.blockwise_dot_nt(dA1, W1.astype(np.float64), nb), GRAD, "dpooled")
