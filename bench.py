@@ -82,7 +82,8 @@ def measured_traffic(workload):
 
 def train_throughput(steps=30, warmup=5):
     """Secondary figures: whole train steps (forward + backward + Nesterov update) per second on the
-    three training configurations, fused mode. sequences/s = batch rows * steps / wall time."""
+    three training configurations, fused mode, launched kernel by kernel ("eager") and as one
+    captured HIP graph per step ("graphed"). sequences/s = batch rows * steps / wall time."""
     import torch
     from deepbind_amd import synth
     from deepbind_amd.model import ModelGroup, SequenceNet
@@ -107,6 +108,7 @@ def train_throughput(steps=30, warmup=5):
         net.set_params(cfg["params"])
         X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
         out[name] = timed(lambda: net.train_step(X, R, Y), len(cfg["R"]), 1)
+        out[name]["graphed"] = timed(net.make_graphed_step(X, R, Y), len(cfg["R"]), 1)
     cfg = synth.config4()
     spec, hp = cfg["spec"], cfg["hp"]
     grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
@@ -115,6 +117,7 @@ def train_throughput(steps=30, warmup=5):
         net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
     X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
     out["config4_calibration_90_models"] = timed(lambda: grp.train_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
+    out["config4_calibration_90_models"]["graphed"] = timed(grp.make_graphed_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
     return out
 
 

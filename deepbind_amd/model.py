@@ -238,6 +238,14 @@ class SequenceNet(object):
         return Z
 
     # ------------------------------------------------------------------ one optimiser step
+    def make_graphed_step(self, X, R, Y, Ymask=None):
+        """Captures one fused training step on the given (static) batch tensors into a HIP graph and
+        returns a function that replays it: for launch-bound batch sizes the step then costs one
+        graph launch instead of ~10 kernel launches. Dropout masks stay fresh on every replay because
+        the generator position lives in device memory. The graph bakes in whether L1 decay is
+        active, so it is re-captured when the step counter crosses weight_decay_start."""
+        return _graphed_step([(self, X, R, Y, Ymask)])
+
     def train_step(self, X, R, Y, Ymask=None, U=None):
         fused = self.mode == "fused" and self.dtype == torch.float32 and self.k <= 64 and self.loss is not None
 
@@ -249,6 +257,51 @@ class SequenceNet(object):
                 self.backward(X, R, st, Y, Ymask)
         ds.gradstep(self.P, self.dP, self.drate, self.mP, self.mrate, grad, nesterov=self.nesterov)
         self.step_count += 1
+
+
+def _graphed_step(jobs):
+    """jobs: list of (net, X, R, Y, Ymask) with static device tensors. Returns step(): one replay of a
+    HIP graph holding one fused training step of every net, in list order."""
+    for net, *_ in jobs:
+        assert net.mode == "fused" and net.dtype == torch.float32 and net.loss is not None
+    state = {"graph": None, "decay": None}
+
+    def decay_flags():
+        return tuple(net.weight_decay_start <= net.step_count for net, *_ in jobs)
+
+    def body():
+        for net, X, R, Y, Ymask in jobs:
+            ds.gradstep(net.P, net.dP, net.drate, net.mP, net.mrate,
+                        lambda: net._grad_fused(X, R, Y, Ymask, None), nesterov=net.nesterov)
+
+    def capture():
+        # one eager run first so that every scratch buffer already has its final size; state is restored after it
+        live = [t for net, *_ in jobs for t in (net.P, net.mP, net.dP, net.rng_counter)]
+        saved = [t.clone() for t in live]
+        host_off = [net._rng_offset for net, *_ in jobs]
+        body()
+        torch.cuda.synchronize()
+        for t, s_ in zip(live, saved):
+            t.copy_(s_)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            body()
+        # capturing executes nothing on the device; only the host mirrors of the generator position moved
+        for (net, *_), off in zip(jobs, host_off):
+            net._rng_offset = off
+        state["graph"], state["decay"] = g, decay_flags()
+
+    def step():
+        if state["graph"] is None or state["decay"] != decay_flags():
+            capture()
+        state["graph"].replay()
+        for net, X, R, Y, Ymask in jobs:
+            if net.use_dropout:
+                net._rng_offset += (R.shape[0] * net.k * net.ninst + 3) // 4
+            net.step_count += 1
+
+    return step
 
 
 class ModelGroup(object):
@@ -272,6 +325,15 @@ class ModelGroup(object):
             Yg = Y.index_select(1, ii).contiguous()
             Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
             net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
+
+    def make_graphed_step(self, X, R, Y, Ymask=None):
+        """One HIP graph holding the fused training step of every architecture group on a static batch."""
+        jobs = []
+        for idx, net in self.groups:
+            ii = torch.as_tensor(idx, device=Y.device)
+            jobs.append((net, X, R, Y.index_select(1, ii).contiguous(),
+                         Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
+        return _graphed_step(jobs)
 
     def predict(self, X, R):
         out = torch.empty((R.shape[0], self.nmodel), dtype=torch.float32, device=X.device)

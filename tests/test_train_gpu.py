@@ -207,3 +207,62 @@ def test_head_train_loss_output():
     dA1 = orc.relu_bprop(orc.blockwise_dot_nt(dA, W2.astype(np.float64), nb), H)
     assert_close(host(g[0]), orc.blockwise_dot_tn(Pl.astype(np.float64), dA1, nb, W1), GRAD, "dW1")
     assert_close(host(dP), orc.blockwise_dot_nt(dA1, W1.astype(np.float64), nb), GRAD, "dpooled")
+
+
+def test_graphed_step_replays_match_eager_steps():
+    """A captured step must give the eager result on EVERY replay (fresh dropout masks included), with
+    other work and synchronisations between the replays, and across the L1-decay switch-on."""
+    from deepbind_amd import synth
+    from deepbind_amd.model import SequenceNet
+    cfg = synth.config3()
+    spec = cfg["spec"]
+    jit = np.random.default_rng(2)
+    params = {k: (v if not k.startswith("b") else (jit.standard_normal(v.shape) * 0.01).astype(np.float32)) for k, v in cfg["params"].items()}
+
+    def make():
+        net = SequenceNet(1, spec.nfilter, spec.m, pool="max", hidden=32, loss="nll", rate=0.05, momentum=0.9, dropout=0.5,
+                          decay_conv=1e-4, decay_full=1e-3, weight_decay_start=3)
+        net.rng_seed = 5
+        net.set_params(params)
+        return net
+
+    eager, graphed = make(), make()
+    X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
+    step = graphed.make_graphed_step(X, R, Y)
+    for i in range(6):
+        eager.train_step(X, R, Y)
+        step()
+        junk = torch.rand(1000, device="cuda").sum().item()          # unrelated eager work + a sync between replays
+        a, b = eager.get_params(), graphed.get_params()
+        for k in a:
+            assert np.array_equal(a[k], b[k]), "replay %d differs from the eager step in %s" % (i, k)
+    assert graphed.step_count == 6 and graphed._rng_offset == eager._rng_offset
+    assert int(graphed.rng_counter.item()) == int(eager.rng_counter.item())
+
+
+def test_graphed_group_step_matches_eager_group_step():
+    """All architecture groups of the calibration batch in one captured graph, dropout on."""
+    from deepbind_amd import synth
+    from deepbind_amd.model import ModelGroup
+    cfg = synth.config4()
+    spec, hp = cfg["spec"], cfg["hp"]
+
+    def make():
+        grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
+                         decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"], weight_decay_start=2)
+        for gi, (idx, net) in enumerate(grp.groups):
+            net.rng_seed = 100 + gi
+            net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
+        return grp
+
+    eager, graphed = make(), make()
+    X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
+    step = graphed.make_graphed_step(X, R, Y, M)
+    for i in range(4):
+        eager.train_step(X, R, Y, M)
+        step()
+        torch.cuda.synchronize()
+        for (_, a), (_, b) in zip(eager.groups, graphed.groups):
+            pa, pb = a.get_params(), b.get_params()
+            for k in pa:
+                assert np.array_equal(pa[k], pb[k]), "replay %d, %s/%d group, %s" % (i, a.pool, a.hidden, k)
