@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void scanpool_bprop_kernel(const float* __rest
                                                              const uint32_t* __restrict__ R, size_t P,
                                                              const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
                                                              const float* __restrict__ dpooled,
-                                                             float* __restrict__ slabW, float* __restrict__ slabB)
+                                                             float* __restrict__ slabs, size_t stride)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const unsigned nw = blockDim.x >> 6;
@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256) void scanpool_bprop_kernel(const float* __rest
     }
     dbacc[wave * FT + lane] = db;
     __syncthreads();
-    float* outW = slabW + (size_t)blockIdx.x * (4 * m) * F;
+    float* outW = slabs + (size_t)blockIdx.x * stride;
     for (unsigned e = threadIdx.x; e < tab; e += blockDim.x) {
         float s = acc_tab[e];
         for (unsigned w = 1; w < nw; ++w) s += acc_tab[(size_t)w * tab + e];
@@ -222,14 +222,203 @@ __global__ __launch_bounds__(256) void scanpool_bprop_kernel(const float* __rest
     if (wave == 0 && f < F) {
         float s = dbacc[lane];
         for (unsigned w = 1; w < nw; ++w) s += dbacc[w * FT + lane];
-        slabB[(size_t)blockIdx.x * F + f] = s;
+        outW[(size_t)4 * m * F + f] = s;
     }
 }
 
-// dst[e] (+)= fixed-shape tree sum over slabs
-template <bool ACCUMULATE>
-__global__ void reduce_slabs_kernel(float* __restrict__ dst, const float* __restrict__ slabs, size_t nelem, unsigned nslab)
+// Adds g at (tap j, letter of X[i+j]) for j < m into this lane's column of a [tap][channel][FT] table.
+// Taps are handled eight at a time with all LDS reads issued before the writes (distinct taps are
+// distinct cells), so a position costs two LDS round trips per eight taps instead of sixteen.
+__device__ __forceinline__ void add_position(float* mine, const uint8_t* __restrict__ xs, unsigned m, float g)
 {
+    const float gq = g * 0.25f;
+    for (unsigned j0 = 0; j0 < m; j0 += 8) {
+        unsigned l[8];
+        float v[8];
+#pragma unroll
+        for (unsigned t = 0; t < 8; ++t) l[t] = j0 + t < m ? letter_of(xs[j0 + t]) : 5u;
+#pragma unroll
+        for (unsigned t = 0; t < 8; ++t) v[t] = l[t] < 4u ? mine[((j0 + t) * 4 + l[t]) * FT] : 0.0f;
+#pragma unroll
+        for (unsigned t = 0; t < 8; ++t)
+            if (l[t] < 4u) mine[((j0 + t) * 4 + l[t]) * FT] = v[t] + g;
+#pragma unroll
+        for (unsigned t = 0; t < 8; ++t)
+            if (l[t] == 4u) {
+                float* cell = mine + (size_t)(j0 + t) * 4 * FT;
+                cell[0 * FT] += gq;
+                cell[1 * FT] += gq;
+                cell[2 * FT] += gq;
+                cell[3 * FT] += gq;
+            }
+    }
+}
+
+// Sparse half of the backward pass (max and max+avg pooling): one position per (region, filter)
+// receives the pooled gradient. One wave per workgroup, one lane per filter, a private
+// [tap][channel][FT] table in LDS that the wave writes out as its slab; regions are taken four at a
+// time so that their pooled / gradient / argmax loads are in flight together. Slab s of the launch
+// lives at slabs + s*stride: 4m*F gradient entries followed by F bias-gradient entries.
+template <int PT>
+__global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                   size_t P, const float* __restrict__ pooled,
+                                                                   const uint32_t* __restrict__ argmax, const float* __restrict__ dpooled,
+                                                                   float* __restrict__ slabs, size_t stride)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* table = reinterpret_cast<float*>(smem);
+    const unsigned lane = threadIdx.x;
+    const unsigned f = blockIdx.y * FT + lane;
+    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
+    float* mine = table + lane;                                   // a lane only ever touches its own column: no barriers needed
+    for (unsigned row = 0; row < 4 * m; ++row) mine[row * FT] = 0.0f;
+    float db = 0.0f;
+    if (f < F) {
+        const size_t gx = gridDim.x;
+        for (size_t r = blockIdx.x; r < P; r += 4 * gx) {
+            float g[4];
+            size_t pos[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const size_t ru = r + u * gx;
+                g[u] = 0.0f;
+                pos[u] = 0;
+                if (ru < P) {
+                    const size_t j0 = ru * F + f;
+                    const float pv = PT == DBK_PT_MAX ? pooled[j0] : pooled[2 * j0];
+                    const float gd = PT == DBK_PT_MAX ? dpooled[j0] : dpooled[2 * j0];
+                    pos[u] = argmax[j0] / F;
+                    g[u] = pv > 0.0f ? gd : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (g[u] != 0.0f) {
+                    db += g[u];
+                    if (pos[u] < n) add_position(mine, X + pos[u], m, g[u]);
+                }
+            }
+        }
+        float* out = slabs + (size_t)blockIdx.x * stride;
+        for (unsigned row = 0; row < 4 * m; ++row) out[(size_t)row * F + f] = mine[row * FT];
+        out[(size_t)4 * m * F + f] = db;
+    }
+}
+
+// Dense half of the backward pass (avg and max+avg pooling), filters of at most MT taps: every
+// position of a region receives davg/count where the recomputed activation is positive. A lane keeps
+// its filter's whole [tap][channel] gradient column in registers: the letter at a position is the
+// same for all 64 lanes (lanes are filters), so it is read once into scalar registers, turned into
+// four scalar weights (1 for the matching channel, 1/4 each for N, else 0) and applied as fused
+// multiply-adds whose products are exact, i.e. one rounding per addition as in the reference's add.
+template <int PT, int MT>
+__global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* __restrict__ W, const float* __restrict__ bias,
+                                                                   unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                   const uint32_t* __restrict__ R, size_t P,
+                                                                   const float* __restrict__ dpooled,
+                                                                   float* __restrict__ slabs, size_t stride)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const unsigned nw = blockDim.x >> 6;
+    const unsigned chunk = nw * XCH_SUBS * PSUB;
+    float* lut = reinterpret_cast<float*>(smem);                   // [m][NL][FT]; reused for the cross-wave fold at the end
+    float* dbacc = lut + (size_t)m * NL * FT;                      // [nw][FT]
+    uint8_t* xl = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT);   // 4-byte aligned: everything before it is float
+
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
+    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
+    build_letter_table(lut, W, m, F, f0);
+    const float bf = f < F ? bias[f] : 0.0f;
+    float db = 0.0f;
+    float aw[MT][4];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) aw[j][0] = aw[j][1] = aw[j][2] = aw[j][3] = 0.0f;
+
+    for (size_t r = blockIdx.x; r < P; r += gridDim.x) {
+        const size_t a = R[2 * r], b = R[2 * r + 1];
+        const size_t j0 = r * F + f;
+        const float gavg = f < F ? (PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1]) / (float)(b - a) : 0.0f;
+        for (size_t c0 = a; c0 < b; c0 += chunk) {
+            const unsigned rows = (unsigned)((b - c0) < chunk ? (b - c0) : chunk);
+            __syncthreads();
+            stage(xl, X, N, c0, rows + m - 1);
+            __syncthreads();
+            for (unsigned s = 0; s < XCH_SUBS; ++s) {
+                const unsigned p0 = (s * nw + wave) * PSUB;
+                if (p0 >= rows) break;
+                float g[PSUB];
+                scan16(lut, xl, m, p0, lane, g);
+#pragma unroll
+                for (int p = 0; p < PSUB; ++p) {
+                    const size_t i = c0 + p0 + p;
+                    const float z = (i < n ? g[p] : 0.0f) + bf;
+                    const float gg = (p0 + p < rows && z > 0.0f) ? gavg : 0.0f;
+                    db += gg;
+                    g[p] = i < n ? gg : 0.0f;                   // rows past the scan's end carry bias only
+                }
+                // letters of this sub-chunk's window, four per scalar register (bytes past the staged
+                // window are stale but only ever meet g == 0 or taps >= m)
+                constexpr int NWORD = (PSUB + MT - 1 + 3) / 4;
+                unsigned wq[NWORD];
+                const unsigned* xw = reinterpret_cast<const unsigned*>(xl + p0);
+#pragma unroll
+                for (int t = 0; t < NWORD; ++t) wq[t] = (unsigned)__builtin_amdgcn_readfirstlane((int)xw[t]);
+#pragma unroll
+                for (int q = 0; q < PSUB + MT - 1; ++q) {
+                    const unsigned l = (wq[q >> 2] >> ((q & 3) * 8)) & 0xffu;
+                    const float base = l == 4u ? 0.25f : 0.0f;
+                    const float m0 = l == 0u ? 1.0f : base, m1 = l == 1u ? 1.0f : base;
+                    const float m2 = l == 2u ? 1.0f : base, m3 = l == 3u ? 1.0f : base;
+#pragma unroll
+                    for (int p = 0; p < PSUB; ++p) {
+                        const int j = q - p;
+                        if (j >= 0 && j < MT) {
+                            aw[j][0] = __builtin_fmaf(g[p], m0, aw[j][0]);
+                            aw[j][1] = __builtin_fmaf(g[p], m1, aw[j][1]);
+                            aw[j][2] = __builtin_fmaf(g[p], m2, aw[j][2]);
+                            aw[j][3] = __builtin_fmaf(g[p], m3, aw[j][3]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    // fold the waves in wave order through the (now unused) letter table's memory
+    dbacc[wave * FT + lane] = db;
+    float* fold = lut + lane;
+    for (unsigned w = 0; w < nw; ++w) {
+        __syncthreads();
+        if (wave == w) {
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                if ((unsigned)j < m) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float* cell = fold + (j * 4 + c) * FT;
+                        *cell = w == 0 ? aw[j][c] : *cell + aw[j][c];
+                    }
+                }
+        }
+    }
+    __syncthreads();
+    float* out = slabs + (size_t)blockIdx.x * stride;
+    for (unsigned e = threadIdx.x; e < m * 4 * FT; e += blockDim.x) {
+        const unsigned row = e / FT, fl = e % FT;
+        if (f0 + fl < F) out[(size_t)row * F + f0 + fl] = lut[e];
+    }
+    if (wave == 0 && f < F) {
+        float s = dbacc[lane];
+        for (unsigned w = 1; w < nw; ++w) s += dbacc[w * FT + lane];
+        out[(size_t)4 * m * F + f] = s;
+    }
+}
+
+// Fixed-shape tree sum over slabs of nW + nB entries each: dW[e] += total for e < nW, dbias[e - nW] = total after that.
+__global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ dbias, const float* __restrict__ slabs,
+                                    size_t nW, size_t nB, unsigned nslab)
+{
+    const size_t nelem = nW + nB;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < nelem; e += (size_t)gridDim.x * blockDim.x) {
         float total = 0.0f;
         for (unsigned base = 0; base < nslab; base += 8) {
@@ -237,7 +426,8 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dst, const float* __rest
             for (unsigned s = 0; s < 8; ++s) buf[s] = base + s < nslab ? slabs[(size_t)(base + s) * nelem + e] : 0.0f;
             total += ((buf[0] + buf[1]) + (buf[2] + buf[3])) + ((buf[4] + buf[5]) + (buf[6] + buf[7]));
         }
-        dst[e] = ACCUMULATE ? dst[e] + total : total;
+        if (e < nW) dW[e] += total;
+        else dbias[e - nW] = total;
     }
 }
 
@@ -266,32 +456,75 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     DBK_LAUNCH_OK();
 }
 
+template <int PT, int MT>
+void launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, const float* W, const float* bias, size_t m, size_t F,
+                  const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* dpooled, float* slabs, size_t stride)
+{
+    auto kern = scanpool_bprop_dense_kernel<PT, MT>;
+    hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, dpooled, slabs, stride);
+}
+
 template <int PT>
 int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                     const uint32_t* R, size_t P, const float* pooled, const uint32_t* argmax, const float* dpooled,
                     float* dW, float* dbias)
 {
-    unsigned nw = 4;
-    const size_t lutb = PT == DBK_PT_MAX ? 0 : m * NL * FT * sizeof(float);
-    auto need = [&](unsigned w) { return lutb + (size_t)w * (m * 4 * FT + FT) * sizeof(float) + w * XCH_SUBS * PSUB + m - 1; };
-    while (nw > 1 && need(nw) > lds_limit()) nw >>= 1;
-    size_t smem = need(nw);
-    DBK_CHECK(smem <= lds_limit(), "ValueError: filter length %zu needs %zu bytes of LDS (limit %zu)", m, smem, lds_limit());
-    unsigned ftiles = dbk::divup(F, FT);
+    const unsigned ftiles = dbk::divup(F, FT);
     DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
-    unsigned gx = 1024u / ftiles;
-    if (gx < 1) gx = 1;
-    if (gx > P) gx = (unsigned)P;
-    const size_t nW = 4 * m * F;
-    float* slabW = (float*)dbk::workspace((nW + F) * gx * sizeof(float));
-    DBK_CHECK(slabW != nullptr, "MemoryError: could not allocate %zu bytes of scratch", (nW + F) * gx * sizeof(float));
-    float* slabB = slabW + nW * gx;
-    auto kern = scanpool_bprop_kernel<PT>;
-    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P,
-                       pooled, argmax, dpooled, slabW, slabB);
-    hipLaunchKernelGGL(reduce_slabs_kernel<true>, dim3(dbk::ew_grid(nW)), dim3(256), 0, st, dW, (const float*)slabW, nW, gx);
-    hipLaunchKernelGGL(reduce_slabs_kernel<false>, dim3(dbk::ew_grid(F)), dim3(256), 0, st, dbias, (const float*)slabB, F, gx);
+    const size_t nW = 4 * m * F, stride = nW + F;
+    const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 24 ? 24 : 0));    // the register budget of the dense kernel ends at 24 taps
+    if (mt == 0) {
+        // any filter length: one kernel does both halves through per-wave LDS tables
+        unsigned nw = 4;
+        const size_t lutb = PT == DBK_PT_MAX ? 0 : m * NL * FT * sizeof(float);
+        auto need = [&](unsigned w) { return lutb + (size_t)w * (m * 4 * FT + FT) * sizeof(float) + w * XCH_SUBS * PSUB + m - 1; };
+        while (nw > 1 && need(nw) > lds_limit()) nw >>= 1;
+        const size_t smem = need(nw);
+        DBK_CHECK(smem <= lds_limit(), "ValueError: filter length %zu needs %zu bytes of LDS (limit %zu)", m, smem, lds_limit());
+        unsigned gx = 1024u / ftiles;
+        if (gx < 1) gx = 1;
+        if (gx > P) gx = (unsigned)P;
+        float* slabs = (float*)dbk::workspace(stride * gx * sizeof(float));
+        DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * gx * sizeof(float));
+        auto kern = scanpool_bprop_kernel<PT>;
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P,
+                           pooled, argmax, dpooled, slabs, stride);
+        hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gx);
+        DBK_LAUNCH_OK();
+    }
+    // sparse half: ~2048 single-wave workgroups, at least four regions each
+    unsigned gxs = 0, gxd = 0;
+    if (PT != DBK_PT_AVG) {
+        gxs = 2048u / ftiles;
+        if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);
+        if (gxs < 1) gxs = 1;
+    }
+    // dense half: ~1024 four-wave workgroups
+    if (PT != DBK_PT_MAX) {
+        gxd = 1024u / ftiles;
+        if (gxd < 1) gxd = 1;
+        if (gxd > P) gxd = (unsigned)P;
+    }
+    const size_t smem_s = m * 4 * FT * sizeof(float);
+    const size_t smem_d = (m * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 3) & ~(size_t)3);
+    DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
+    float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float));
+    DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * (gxs + gxd) * sizeof(float));
+    if (gxs) {
+        auto kern = scanpool_bprop_sparse_kernel<PT == DBK_PT_AVG ? DBK_PT_MAX : PT>;
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_s));
+        hipLaunchKernelGGL(kern, dim3(gxs, ftiles), dim3(64), smem_s, st, (unsigned)m, (unsigned)F, X, N, P, pooled, argmax, dpooled, slabs, stride);
+    }
+    if (gxd) {
+        constexpr int PD = PT == DBK_PT_MAX ? DBK_PT_AVG : PT;
+        float* sd = slabs + stride * gxs;
+        if (mt == 8) launch_dense<PD, 8>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
+        else if (mt == 16) launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
+        else launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
+    }
+    hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd);
     DBK_LAUNCH_OK();
 }
 

@@ -209,7 +209,8 @@ def test_scanpool_regions_past_the_end_and_gaps(ks):
 
 
 @pytest.mark.parametrize("ptype", ["max", "avg", "all"])
-@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (30, 20, 40, 24, 144)])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (30, 20, 40, 24, 144), (33, 1, 300, 11, 70),
+                                          (17, 0, 9, 5, 33), (25, 200, 300, 7, 64), (12, 480, 520, 30, 40), (40, 90, 110, 2, 8)])
 def test_scanpool_bprop(ks, ptype, B, lo, hi, m, F):
     rng, W, b, X, R = _fused_case(B + F, B, lo, hi, m, F)
     A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
