@@ -14,14 +14,16 @@ __device__ __forceinline__ unsigned letter_of(unsigned code)
 }
 
 // Builds lut[(j*NL + l)*FT + fl] for filters [f0, f0+FT) from W (4m, F); missing filters read as 0.
+// With mpad > m the table gets all-zero rows for taps m..mpad-1.
 template <typename T>
-__device__ void build_letter_table(T* lut, const T* __restrict__ W, unsigned m, unsigned F, unsigned f0)
+__device__ void build_letter_table(T* lut, const T* __restrict__ W, unsigned m, unsigned F, unsigned f0, unsigned mpad = 0)
 {
-    for (unsigned e = threadIdx.x; e < m * FT; e += blockDim.x) {
+    if (mpad < m) mpad = m;
+    for (unsigned e = threadIdx.x; e < mpad * FT; e += blockDim.x) {
         unsigned j = e / FT, fl = e % FT;
         unsigned f = f0 + fl;
         T w0 = 0, w1 = 0, w2 = 0, w3 = 0;
-        if (f < F) {
+        if (f < F && j < m) {
             w0 = W[(4 * j + 0) * (size_t)F + f];
             w1 = W[(4 * j + 1) * (size_t)F + f];
             w2 = W[(4 * j + 2) * (size_t)F + f];

@@ -38,6 +38,54 @@ __device__ __forceinline__ void scan16(const float* __restrict__ lut, const uint
     }
 }
 
+// Number of 4-letter words covering the window of PSUB positions and MT taps.
+template <int MT> struct window { static constexpr int words = (PSUB + MT - 1 + 3) / 4; };
+
+// Reads the letters of the window starting at 4-byte aligned xl+p0 into scalar registers (all lanes of
+// a wave look at the same positions).
+template <int MT>
+__device__ __forceinline__ void load_window(const uint8_t* xl, unsigned p0, unsigned (&wq)[window<MT>::words])
+{
+    const unsigned* xw = reinterpret_cast<const unsigned*>(xl + p0);
+#pragma unroll
+    for (int t = 0; t < window<MT>::words; ++t) wq[t] = (unsigned)__builtin_amdgcn_readfirstlane((int)xw[t]);
+}
+
+// Bytes to stage so that every window word of a chunk with `rows` positions holds valid letters.
+template <int MT>
+__device__ __forceinline__ unsigned window_span(unsigned rows) { return ((rows + PSUB - 1) & ~(unsigned)(PSUB - 1)) + 4 * window<MT>::words - PSUB; }
+
+__device__ __forceinline__ unsigned window_letter(const unsigned* wq, int q) { return (wq[q >> 2] >> ((q & 3) * 8)) & 0xffu; }
+
+// scan16 for filters of at most MT taps with the letters in scalar registers: one address add per
+// letter, then every (position, tap) pair is a single LDS read with an immediate offset. The table
+// must have been built with MT taps (zero rows past m). Taps are added in ascending order per
+// position, exactly as scan16 does.
+template <int MT>
+__device__ __forceinline__ void scan16_window(const float* __restrict__ lut, const unsigned (&wq)[window<MT>::words], unsigned lane,
+                                              float acc[PSUB])
+{
+#pragma unroll
+    for (int p = 0; p < PSUB; ++p) acc[p] = 0.0f;
+#pragma unroll
+    for (int q = 0; q < PSUB + MT - 1; ++q) {
+        const float* col = lut + window_letter(wq, q) * FT + lane;
+#pragma unroll
+        for (int p = 0; p < PSUB; ++p) {
+            const int j = q - p;
+            if (j >= 0 && j < MT) acc[p] += col[j * NL * FT];
+        }
+        // pin the running sums every fourth letter: otherwise the scheduler issues the whole window's reads
+        // first and finishes one position's chain at a time, holding ~400 loaded values in registers
+        if ((q & 3) == 3) {
+            static_assert(PSUB == 16, "the pin below lists 16 accumulators");
+            asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]),
+                         "+v"(acc[7]), "+v"(acc[8]), "+v"(acc[9]), "+v"(acc[10]), "+v"(acc[11]), "+v"(acc[12]), "+v"(acc[13]),
+                         "+v"(acc[14]), "+v"(acc[15]));
+        }
+    }
+}
+
 // Stages letters for absolute positions [c0, c0+cnt) into xl; past the end of X -> "nothing".
 __device__ __forceinline__ void stage(uint8_t* xl, const uint8_t* __restrict__ X, size_t N, size_t c0, unsigned cnt)
 {
@@ -47,7 +95,8 @@ __device__ __forceinline__ void stage(uint8_t* xl, const uint8_t* __restrict__ X
     }
 }
 
-template <int PT, bool WANT_ARGMAX>
+// MT > 0: filters of at most MT taps, letters held in scalar registers (scan16_window); MT == 0: any length.
+template <int PT, bool WANT_ARGMAX, int MT>
 __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __restrict__ W, const float* __restrict__ bias,
                                                              unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
                                                              const uint32_t* __restrict__ R, size_t P,
@@ -60,13 +109,13 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
     const unsigned nw = blockDim.x >> 6;
     const unsigned chunk = nw * XCH_SUBS * PSUB;
     float* lut = reinterpret_cast<float*>(smem);
-    float* red = lut + (size_t)m * NL * FT;                       // [nw][3][FT]: max, index, sum
+    float* red = lut + (size_t)(MT ? MT : m) * NL * FT;           // [nw][3][FT]: max, index, sum
     uint8_t* xl = reinterpret_cast<uint8_t*>(red + (size_t)nw * 3 * FT);
 
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;    // rows the scan defines; later rows are relu(bias)
-    build_letter_table(lut, W, m, F, f0);
+    build_letter_table(lut, W, m, F, f0, MT);
     const float bf = f < F ? bias[f] : 0.0f;
 
     for (size_t r = blockIdx.x; r < P; r += gridDim.x) {
@@ -76,13 +125,20 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
         for (size_t c0 = a; c0 < b; c0 += chunk) {
             const unsigned rows = (unsigned)((b - c0) < chunk ? (b - c0) : chunk);
             __syncthreads();
-            stage(xl, X, N, c0, rows + m - 1);
+            stage(xl, X, N, c0, MT ? window_span<MT ? MT : 1>(rows) : rows + m - 1);
             __syncthreads();
+#pragma unroll 1
             for (unsigned s = 0; s < XCH_SUBS; ++s) {
                 const unsigned p0 = (s * nw + wave) * PSUB;
                 if (p0 >= rows) break;
                 float acc[PSUB];
-                scan16(lut, xl, m, p0, lane, acc);
+                if (MT) {
+                    unsigned wq[window<MT ? MT : 1>::words];
+                    load_window<MT ? MT : 1>(xl, p0, wq);
+                    scan16_window<MT ? MT : 1>(lut, wq, lane, acc);
+                } else {
+                    scan16(lut, xl, m, p0, lane, acc);
+                }
 #pragma unroll
                 for (int p = 0; p < PSUB; ++p) {
                     const size_t i = c0 + p0 + p;
@@ -188,7 +244,8 @@ __global__ __launch_bounds__(256) void scanpool_bprop_kernel(const float* __rest
                 __syncthreads();
                 stage(xl, X, N, c0, rows + m - 1);
                 __syncthreads();
-                for (unsigned s = 0; s < XCH_SUBS; ++s) {
+    #pragma unroll 1
+            for (unsigned s = 0; s < XCH_SUBS; ++s) {
                     const unsigned p0 = (s * nw + wave) * PSUB;
                     if (p0 >= rows) break;
                     float acc[PSUB];
@@ -321,14 +378,14 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
     extern __shared__ __align__(16) unsigned char smem[];
     const unsigned nw = blockDim.x >> 6;
     const unsigned chunk = nw * XCH_SUBS * PSUB;
-    float* lut = reinterpret_cast<float*>(smem);                   // [m][NL][FT]; reused for the cross-wave fold at the end
-    float* dbacc = lut + (size_t)m * NL * FT;                      // [nw][FT]
+    float* lut = reinterpret_cast<float*>(smem);                   // [MT][NL][FT]; reused for the cross-wave fold at the end
+    float* dbacc = lut + (size_t)MT * NL * FT;                     // [nw][FT]
     uint8_t* xl = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT);   // 4-byte aligned: everything before it is float
 
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
-    build_letter_table(lut, W, m, F, f0);
+    build_letter_table(lut, W, m, F, f0, MT);
     const float bf = f < F ? bias[f] : 0.0f;
     float db = 0.0f;
     float aw[MT][4];
@@ -342,13 +399,18 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
         for (size_t c0 = a; c0 < b; c0 += chunk) {
             const unsigned rows = (unsigned)((b - c0) < chunk ? (b - c0) : chunk);
             __syncthreads();
-            stage(xl, X, N, c0, rows + m - 1);
+            stage(xl, X, N, c0, window_span<MT>(rows));
             __syncthreads();
+#pragma unroll 1
             for (unsigned s = 0; s < XCH_SUBS; ++s) {
                 const unsigned p0 = (s * nw + wave) * PSUB;
                 if (p0 >= rows) break;
+                // letters of this sub-chunk's window, four per scalar register (letters past the region's
+                // own window only ever meet zero table rows, g == 0 or taps >= m)
+                unsigned wq[window<MT>::words];
+                load_window<MT>(xl, p0, wq);
                 float g[PSUB];
-                scan16(lut, xl, m, p0, lane, g);
+                scan16_window<MT>(lut, wq, lane, g);
 #pragma unroll
                 for (int p = 0; p < PSUB; ++p) {
                     const size_t i = c0 + p0 + p;
@@ -357,16 +419,9 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
                     db += gg;
                     g[p] = i < n ? gg : 0.0f;                   // rows past the scan's end carry bias only
                 }
-                // letters of this sub-chunk's window, four per scalar register (bytes past the staged
-                // window are stale but only ever meet g == 0 or taps >= m)
-                constexpr int NWORD = (PSUB + MT - 1 + 3) / 4;
-                unsigned wq[NWORD];
-                const unsigned* xw = reinterpret_cast<const unsigned*>(xl + p0);
-#pragma unroll
-                for (int t = 0; t < NWORD; ++t) wq[t] = (unsigned)__builtin_amdgcn_readfirstlane((int)xw[t]);
 #pragma unroll
                 for (int q = 0; q < PSUB + MT - 1; ++q) {
-                    const unsigned l = (wq[q >> 2] >> ((q & 3) * 8)) & 0xffu;
+                    const unsigned l = window_letter(wq, q);
                     const float base = l == 4u ? 0.25f : 0.0f;
                     const float m0 = l == 0u ? 1.0f : base, m1 = l == 1u ? 1.0f : base;
                     const float m2 = l == 2u ? 1.0f : base, m3 = l == 3u ? 1.0f : base;
@@ -431,27 +486,44 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
     }
 }
 
+template <int PT, int MT>
+void launch_fprop_mt(hipStream_t st, unsigned gx, unsigned ftiles, unsigned nw, size_t smem, const float* W, const float* bias, size_t m,
+                     size_t F, const uint8_t* X, size_t N, const uint32_t* R, size_t P, float* pooled, uint32_t* argmax,
+                     const unsigned* run_if_flag)
+{
+    if (argmax) {
+        auto kern = scanpool_fprop_kernel<PT, true, MT>;
+        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
+    } else {
+        auto kern = scanpool_fprop_kernel<PT, false, MT>;
+        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
+    }
+}
+
 template <int PT>
 int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                     const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, const unsigned* run_if_flag)
 {
     const unsigned nw = 4;
     const unsigned chunk = nw * XCH_SUBS * PSUB;
-    size_t smem = m * NL * FT * sizeof(float) + nw * 3 * FT * sizeof(float) + chunk + m - 1;
+    const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 24 ? 24 : (m <= 32 ? 32 : 0)));    // 0: any-length kernel
+    const size_t taps = mt ? mt : m;
+    size_t smem = taps * NL * FT * sizeof(float) + nw * 3 * FT * sizeof(float) + ((chunk + taps - 1 + 7) & ~(size_t)3);
     DBK_CHECK(smem <= lds_limit(), "ValueError: filter length %zu needs %zu bytes of LDS (limit %zu)", m, smem, lds_limit());
     unsigned ftiles = dbk::divup(F, FT);
     DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
-    unsigned gx = 4096u / ftiles;
+    // three workgroups fit a CU; each builds its letter table once and then walks its share of the regions
+    unsigned gx = 768u / ftiles;
     if (gx < 1) gx = 1;
     if (gx > P) gx = (unsigned)P;
-    if (argmax) {
-        auto kern = scanpool_fprop_kernel<PT, true>;
-        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
-    } else {
-        auto kern = scanpool_fprop_kernel<PT, false>;
-        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
+    switch (mt) {
+    case 8:  launch_fprop_mt<PT, 8>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
+    case 16: launch_fprop_mt<PT, 16>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
+    case 24: launch_fprop_mt<PT, 24>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
+    case 32: launch_fprop_mt<PT, 32>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
+    default: launch_fprop_mt<PT, 0>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
     }
     DBK_LAUNCH_OK();
 }
@@ -501,14 +573,14 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);
         if (gxs < 1) gxs = 1;
     }
-    // dense half: ~1024 four-wave workgroups
+    // dense half: ~768 four-wave workgroups (three resident per CU)
     if (PT != DBK_PT_MAX) {
-        gxd = 1024u / ftiles;
+        gxd = 768u / ftiles;
         if (gxd < 1) gxd = 1;
         if (gxd > P) gxd = (unsigned)P;
     }
     const size_t smem_s = m * 4 * FT * sizeof(float);
-    const size_t smem_d = (m * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 3) & ~(size_t)3);
+    const size_t smem_d = ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3);
     DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
     float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float));
     DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * (gxs + gxd) * sizeof(float));
