@@ -217,7 +217,7 @@ int launch_bprop_W(hipStream_t st, T* dW, size_t m, size_t F, const uint8_t* X, 
     if (gy < 1) gy = 1;
     if (gy > nchunk) gy = nchunk;
     size_t nelem = 4 * m * F;
-    T* partial = (T*)dbk::workspace(nelem * gy * sizeof(T));
+    T* partial = (T*)dbk::workspace(nelem * gy * sizeof(T), st);
     DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", nelem * gy * sizeof(T));
     auto kern = corr1ord_bprop_W_partial_kernel<T>;
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));

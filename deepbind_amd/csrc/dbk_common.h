@@ -14,9 +14,11 @@ namespace dbk {
 void set_error(const char* fmt, ...);
 void clear_error();
 
-// Device scratch that grows on demand and lives until the process ends. One buffer per device;
-// kernels launched on different streams of one device must not use it concurrently.
-void* workspace(size_t bytes);
+// Device scratch that grows on demand and lives until the process ends. One buffer per (device, stream):
+// launches are ordered within a stream, so consecutive calls on it can share the buffer, and calls on
+// different streams never do. At most 64 distinct streams per device; null when that is exceeded or
+// when memory runs out. Growing a buffer synchronises the device (and so cannot happen under capture).
+void* workspace(size_t bytes, hipStream_t stream);
 
 inline hipStream_t as_stream(dbk_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -234,7 +234,7 @@ extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, 
     a.nchunk = (unsigned)nchunk;
     a.pstride = (unsigned)(k * h1 + 2 * h1 + 2);
     const size_t pbytes = nchunk * (size_t)nblock * a.pstride * sizeof(float);
-    a.partial = (float*)dbk::workspace(pbytes);
+    a.partial = (float*)dbk::workspace(pbytes, dbk::as_stream(stream));
     DBK_CHECK(a.partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", pbytes);
     DBK_HIP(hipFuncSetAttribute((const void*)k_head_train, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(k_head_train, dim3(nblock, (unsigned)nchunk), dim3(NT), smem, dbk::as_stream(stream), a);

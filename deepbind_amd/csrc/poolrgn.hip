@@ -140,7 +140,7 @@ int launch_bwd(hipStream_t st, T* dU, size_t F, const uint32_t* R, size_t P, boo
                const uint32_t* argmax, int ptype)
 {
     DBK_CHECK(dbk::divup(F, 64) <= 65535u, "ValueError: too many feature maps (%zu) for one launch", F);
-    unsigned* flag = (unsigned*)dbk::workspace(256);
+    unsigned* flag = (unsigned*)dbk::workspace(256, st);
     DBK_CHECK(flag != nullptr, "MemoryError: could not allocate scratch");
     hipLaunchKernelGGL(regions_disjoint_kernel, dim3(1), dim3(1024), 0, st, R, P, per_step, flag);
     switch (ptype) {

@@ -17,28 +17,36 @@ void set_error(const char* fmt, ...)
 
 void clear_error() { g_err[0] = 0; }
 
-struct ws_t { void* ptr = nullptr; size_t bytes = 0; };
-static ws_t g_ws[64];
+struct ws_t { hipStream_t stream = nullptr; void* ptr = nullptr; size_t bytes = 0; bool used = false; };
+constexpr int WS_DEVICES = 64, WS_STREAMS = 64;
+static ws_t g_ws[WS_DEVICES][WS_STREAMS];
 static std::mutex g_ws_mutex;
 
-void* workspace(size_t bytes)
+void* workspace(size_t bytes, hipStream_t stream)
 {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= WS_DEVICES) return nullptr;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    ws_t& w = g_ws[dev];
-    if (w.bytes >= bytes && w.ptr) return w.ptr;
-    if (w.ptr) {
+    ws_t* w = nullptr;
+    for (int i = 0; i < WS_STREAMS && !w; ++i) {
+        ws_t& c = g_ws[dev][i];
+        if (c.used ? c.stream == stream : true) w = &c;        // this stream's slot, or the first free one
+    }
+    if (!w) return nullptr;
+    w->used = true;
+    w->stream = stream;
+    if (w->bytes >= bytes && w->ptr) return w->ptr;
+    if (w->ptr) {
         // earlier launches may still be reading the old buffer
         if (hipDeviceSynchronize() != hipSuccess) return nullptr;
-        (void)hipFree(w.ptr);
-        w.ptr = nullptr;
-        w.bytes = 0;
+        (void)hipFree(w->ptr);
+        w->ptr = nullptr;
+        w->bytes = 0;
     }
     size_t want = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes + bytes / 4;
-    if (hipMalloc(&w.ptr, want) != hipSuccess) { w.ptr = nullptr; return nullptr; }
-    w.bytes = want;
-    return w.ptr;
+    if (hipMalloc(&w->ptr, want) != hipSuccess) { w->ptr = nullptr; return nullptr; }
+    w->bytes = want;
+    return w->ptr;
 }
 
 }  // namespace dbk

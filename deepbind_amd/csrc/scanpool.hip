@@ -557,7 +557,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         unsigned gx = 1024u / ftiles;
         if (gx < 1) gx = 1;
         if (gx > P) gx = (unsigned)P;
-        float* slabs = (float*)dbk::workspace(stride * gx * sizeof(float));
+        float* slabs = (float*)dbk::workspace(stride * gx * sizeof(float), st);
         DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * gx * sizeof(float));
         auto kern = scanpool_bprop_kernel<PT>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -582,7 +582,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     const size_t smem_s = m * 4 * FT * sizeof(float);
     const size_t smem_d = ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3);
     DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
-    float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float));
+    float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float), st);
     DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * (gxs + gxd) * sizeof(float));
     if (gxs) {
         auto kern = scanpool_bprop_sparse_kernel<PT == DBK_PT_AVG ? DBK_PT_MAX : PT>;

@@ -285,7 +285,7 @@ int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size
     // a filter tile's table costs ~0.1 M position-equivalents to build: only worth it for bulk work
     if (!force && (double)N * dbk::divup(F, FTILE) < 2.0e6) return -1;
     const size_t kbytes = (N + KPAD + 255) & ~(size_t)255;
-    unsigned char* ws = (unsigned char*)dbk::workspace(256 + kbytes);
+    unsigned char* ws = (unsigned char*)dbk::workspace(256 + kbytes, st);
     if (!ws) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", 256 + kbytes); return 1; }
     unsigned* flag = (unsigned*)ws;
     uint8_t* K = ws + 256;

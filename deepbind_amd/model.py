@@ -259,9 +259,22 @@ class SequenceNet(object):
         self.step_count += 1
 
 
-def _graphed_step(jobs):
+def _side_by_side(streams, jobs):
+    """Runs job i on streams[i], all forked from the current stream and joined back into it. The nets of
+    a group share nothing but read-only inputs, so their small kernels can fill the GPU together.
+    (All streams have the default priority; the library keeps its scratch memory per stream.)"""
+    cur = torch.cuda.current_stream()
+    for s, job in zip(streams, jobs):
+        s.wait_stream(cur)
+        with torch.cuda.stream(s):
+            job()
+    for s in streams[:len(jobs)]:
+        cur.wait_stream(s)
+
+
+def _graphed_step(jobs, streams=None):
     """jobs: list of (net, X, R, Y, Ymask) with static device tensors. Returns step(): one replay of a
-    HIP graph holding one fused training step of every net, in list order."""
+    HIP graph holding one fused training step of every net (as parallel branches when streams are given)."""
     for net, *_ in jobs:
         assert net.mode == "fused" and net.dtype == torch.float32 and net.loss is not None
     state = {"graph": None, "decay": None}
@@ -269,23 +282,35 @@ def _graphed_step(jobs):
     def decay_flags():
         return tuple(net.weight_decay_start <= net.step_count for net, *_ in jobs)
 
+    def one(net, X, R, Y, Ymask):
+        return lambda: ds.gradstep(net.P, net.dP, net.drate, net.mP, net.mrate,
+                                   lambda: net._grad_fused(X, R, Y, Ymask, None), nesterov=net.nesterov)
+
     def body():
-        for net, X, R, Y, Ymask in jobs:
-            ds.gradstep(net.P, net.dP, net.drate, net.mP, net.mrate,
-                        lambda: net._grad_fused(X, R, Y, Ymask, None), nesterov=net.nesterov)
+        if streams is None:
+            for job in jobs:
+                one(*job)()
+        else:
+            _side_by_side(streams, [one(*job) for job in jobs])
 
     def capture():
-        # one eager run first so that every scratch buffer already has its final size; state is restored after it
+        # The library's scratch buffers belong to a stream and cannot grow under capture: run the step
+        # once eagerly on the stream the capture will use (state is restored after it), then capture there.
+        if "stream" not in state:
+            state["stream"] = torch.cuda.Stream()
+        cap = state["stream"]
         live = [t for net, *_ in jobs for t in (net.P, net.mP, net.dP, net.rng_counter)]
         saved = [t.clone() for t in live]
         host_off = [net._rng_offset for net, *_ in jobs]
-        body()
+        cap.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(cap):
+            body()
         torch.cuda.synchronize()
         for t, s_ in zip(live, saved):
             t.copy_(s_)
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+        with torch.cuda.graph(g, stream=cap):
             body()
         # capturing executes nothing on the device; only the host mirrors of the generator position moved
         for (net, *_), off in zip(jobs, host_off):
@@ -317,14 +342,23 @@ class ModelGroup(object):
             idx = [j for j in range(self.nmodel) if (pools[j], hiddens[j]) == key]
             kw = {k: (np.asarray(v)[idx] if np.ndim(v) else v) for k, v in per_model.items()}
             self.groups.append((idx, SequenceNet(len(idx), nfilter, m, pool=key[0], hidden=key[1], loss=loss, **kw)))
+        self.streams = None
+
+    def _streams(self):
+        if self.streams is None:
+            self.streams = [torch.cuda.Stream() for _ in self.groups]
+        return self.streams
 
     def train_step(self, X, R, Y, Ymask=None, U=None):
         """U, when given, is a list with one uniforms tensor per architecture group (see self.groups)."""
-        for gi, (idx, net) in enumerate(self.groups):
-            ii = torch.as_tensor(idx, device=Y.device)
-            Yg = Y.index_select(1, ii).contiguous()
-            Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
-            net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
+        def one(gi, idx, net):
+            def run():
+                ii = torch.as_tensor(idx, device=Y.device)
+                Yg = Y.index_select(1, ii).contiguous()
+                Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
+                net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
+            return run
+        _side_by_side(self._streams(), [one(gi, idx, net) for gi, (idx, net) in enumerate(self.groups)])
 
     def make_graphed_step(self, X, R, Y, Ymask=None):
         """One HIP graph holding the fused training step of every architecture group on a static batch."""
@@ -333,7 +367,7 @@ class ModelGroup(object):
             ii = torch.as_tensor(idx, device=Y.device)
             jobs.append((net, X, R, Y.index_select(1, ii).contiguous(),
                          Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
-        return _graphed_step(jobs)
+        return _graphed_step(jobs, self._streams())
 
     def predict(self, X, R):
         out = torch.empty((R.shape[0], self.nmodel), dtype=torch.float32, device=X.device)
