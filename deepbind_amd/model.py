@@ -164,6 +164,45 @@ class SequenceNet(object):
                           in_scale=scale, apply_logistic=(self.loss == "nll"))
         return ds.pair_max(Z) if self.reverse_complement else Z
 
+    def input_gradients(self, X, R):
+        """Test-mode predictions plus the gradient map used for sequence logos / mutation maps:
+        returns (Z (rows, ninst), dX (N, 4)) where dX is the back-propagated gradient w.r.t. the
+        one-hot inputs of dA = Z (targets 0, no batch mean, output column 0 only, and with
+        reverse complements only each pair's larger prediction). Runs layer by layer because the
+        backward pass needs the full (N, F) activation map.
+        (reference: deepity/deepity/node.py:298-341, kangaroo/kangaroo/predict.py:168-193,
+        kangaroo/_ext/corr1ord.py:129-133, deepity/std/elemwise.py:148-157)"""
+        p, ni = self.p, self.ninst
+        Z0 = sm.zeros((X.numel(), p["Wc"].shape[1]), dtype=self.dtype, device=self.device)
+        ks.corr1ord(p["Wc"], X, Z0, 4)
+        A0 = sm.relu(sm.add_rowvec(Z0, p["bc"]))
+        pooled, amax = ks.poolrgn(A0, R, self.pool, want_argmax=True)
+        H0 = ds.dropout_fp_test(pooled, self.dropout) if self.use_dropout else pooled
+        A1 = sm.add_rowvec(ds.blockwise_dot(H0, p["W1"], ni), p["b1"])
+        if self.hidden > 0:
+            H1 = sm.relu(A1)
+            A2 = sm.add_rowvec(ds.blockwise_dot(H1, p["W2"], ni), p["b2"])
+        else:
+            A2 = A1
+        Z = sm.logistic(A2) if self.loss == "nll" else A2
+        dA = Z.clone()
+        if self.reverse_complement:
+            Zmask = torch.zeros(Z.shape, dtype=torch.bool, device=self.device)
+            ds.calc_Zmask(Z, Zmask)
+            ds.maskout(Zmask, dA)
+        if dA.shape[1] > 1:
+            dA[:, 1:] = 0
+        dA1 = sm.mul_sign(ds.blockwise_dot_nt(dA, p["W2"], ni), H1) if self.hidden > 0 else dA
+        dH0 = ds.blockwise_dot_nt(dA1, p["W1"], ni)
+        if self.use_dropout:
+            dH0 = ds.dropout_bp_te(dH0, self.dropout)
+        dA0 = sm.zeros_like(A0)
+        ks.poolrgn_bprop(dA0, R, dH0, amax, self.pool)
+        dZ0 = sm.mul_sign(dA0, A0)
+        dX = sm.zeros((X.numel(), 4), dtype=self.dtype, device=self.device)
+        ks.corr1ord_bprop_X(dX, p["Wc"], dZ0, 4)
+        return Z, dX
+
     def loss_value(self, st, Y, Ymask=None):
         """Per-model mean loss (1 x ninst), on the host (reference: deepity/std/loss.py:52-82)."""
         L = sm.loss_terms(st["Z"], Y, self.loss)

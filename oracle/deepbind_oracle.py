@@ -24,6 +24,11 @@ checks live in tests/test_oracle_pins.py):
                         CUDA SDK): masks are INPUTS here (uniforms U supplied by the caller);
                         the random stream itself is PARITY UNPINNED
   pack (asbatches)    - worked example "AC","G", m=3 from the reference's packing code
+  eval_with_input_gradients - central finite differences of softplus(A) (nll) / Z^2/2 (mse) w.r.t. a
+                        real-valued 4-channel input, through a dense-correlation restatement
+  gen_predictions / gen_predictionmaps - glue loops restated from predict.py; the finite-difference
+                        map is checked against brute-force single-mutant rescoring, the window
+                        scan against scoring each window by hand
 All paths in the comments are relative to /root/reference/code/libs.
 """
 import numpy as np
@@ -555,3 +560,142 @@ def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum,
     for n in names:
         gradstep_nesterov2(params[n], g[n].astype(params[n].dtype), eta[n], mom[n], mu[n])
     return st, g
+
+
+# ----------------------------------------------------------------------------------------------
+# prediction-time callers of the path: kangaroo/kangaroo/predict.py:145-345 ;
+# deepity/deepity/node.py:298-341 (eval with want_bprop_inputs) ; kangaroo/_ext/corr1ord.py:129-133
+# The loops below are the reference's loops, one forward pass per mutated (position, base).
+# ----------------------------------------------------------------------------------------------
+_COMPLEMENT = {"A": "T", "C": "G", "G": "C", "T": "A", "U": "A", "N": "N"}
+
+
+def revcomp_string(s):
+    """kangaroo/kangaroo/util.py:29-37,76-80: complement of the reversed string; unknown letters -> N."""
+    return "".join(_COMPLEMENT.get(ch.upper(), "N") for ch in reversed(s))
+
+
+def insert_reverse_complements(seqs):
+    """kangaroo/kangaroo/data.py:274-284: rows become fwd0, rev0, fwd1, rev1, ..."""
+    out = []
+    for s in seqs:
+        out += [s, revcomp_string(s)]
+    return out
+
+
+def ord2acgt(x):
+    return "".join("ACGT"[v] if v < 4 else "N" for v in np.asarray(x).ravel())
+
+
+def maskout_revcomp(Z, reverse_complement):
+    """predict.py:145-164: of each (fwd, rev) pair of rows keep the larger prediction (ties: fwd)."""
+    if not reverse_complement:
+        return Z, None
+    Zc = Z.reshape((-1, 2))
+    Zmask = np.zeros_like(Zc, dtype=bool)
+    Zmask[:, 0] = Zc[:, 0] >= Zc[:, 1]
+    Zmask[:, 1] = Zc[:, 0] < Zc[:, 1]
+    Zmask = Zmask.reshape((-1, 1))
+    return Z[Zmask.ravel()], Zmask
+
+
+def eval_with_input_gradients(params, X, R, nmodel, pool, hidden, out, dropout_rate=None, reverse_complement=False):
+    """Test-mode forward pass, then back-propagation of dA = Z (targets 0, no batch mean, only
+    output column 0, reverse-complement losers masked) down to the one-hot inputs: dX (N, 4).
+    node.py:317-339, loss.py:98-109, elemwise.py:148-157 (test-mode dropout bprop), corr1ord.py:129-133."""
+    dropout = None if dropout_rate is None else (np.asarray(dropout_rate, dtype=params["Wc"].dtype), None)
+    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=False)
+    Z = st["Zout"]
+    dA = Z.copy()
+    if reverse_complement:
+        maskout(calc_zmask(Z), dA)
+    if dA.shape[1] > 1:
+        dA[:, 1:] = 0
+    if hidden:
+        dA1 = relu_bprop(blockwise_dot_nt(dA, params["W2"], nmodel), st["H1"])
+    else:
+        dA1 = dA
+    dH0 = blockwise_dot_nt(dA1, params["W1"], nmodel)
+    if dropout is not None:
+        dH0 = dropout_bp_te(dH0, dropout[0])
+    dA0 = np.zeros_like(st["A0"])
+    poolrgn_bprop(dA0, R, dH0, st["I"], pool)
+    dZ0 = relu_bprop(dA0, st["A0"])
+    dX = np.zeros((np.asarray(X).size, 4), dtype=params["Wc"].dtype)
+    corr1ord_bprop_X(dX, params["Wc"], dZ0)
+    return Z, dX
+
+
+def gen_predictions(params, seqs, pool, hidden, out, dropout_rate=None, reverse_complement=False, want_gmaps=False):
+    """predict.py:168-260 for one model and one batch. Returns (predictions (nseq, 1), gmaps) where
+    gmaps is None, or a list of (sequence string, (len, 4) map): the back-propagated input gradient
+    (want_gmaps=True; with reverse complements only the winning strand's entry is kept), or the
+    finite-difference mutation map (want_gmaps="finite_diff"; forward strands only)."""
+    m = params["Wc"].shape[0] // 4
+    pad = m - 1
+    rows = insert_reverse_complements(seqs) if reverse_complement else list(seqs)
+    X, R = pack(rows, pad)
+    X = X.ravel()
+    R = R.astype(np.int64)
+
+    def predict(Xb):
+        dropout = None if dropout_rate is None else (np.asarray(dropout_rate, dtype=params["Wc"].dtype), None)
+        return model_forward(params, Xb, R, 1, pool, hidden, out=out, dropout=dropout, train=False)["Zout"]
+
+    if not want_gmaps:
+        Z, _ = maskout_revcomp(predict(X), reverse_complement)
+        return Z, None
+    Zall, dX = eval_with_input_gradients(params, X, R, 1, pool, hidden, out, dropout_rate, reverse_complement)
+    Z, Zmask = maskout_revcomp(Zall, reverse_complement)
+    if want_gmaps == "finite_diff":
+        rcindex = [3, 2, 1, 0]
+        Xlen = R[:, 1] - R[:, 0]
+        for i in range(int(Xlen.max())):
+            for j in range(4):
+                mtX = X.copy()
+                for k in range(len(R)):
+                    a, b = R[k]
+                    if i < b - a:
+                        if (k % 2 == 0) or not reverse_complement:
+                            mtX[pad + a + i] = j
+                        else:
+                            mtX[b - i - 1] = rcindex[j]
+                mtZ, _ = maskout_revcomp(predict(mtX), reverse_complement)
+                dZ = mtZ - Z
+                dZ = dZ * np.maximum(0, np.sign(np.maximum(Z, mtZ)))
+                for k in range(len(R)):
+                    if (k % 2 == 0) or not reverse_complement:
+                        a, b = R[k]
+                        if i < b - a:
+                            dX[pad + a + i, j] = dZ[(k // 2) if reverse_complement else k, 0]
+        fwd = R[np.arange(0, len(R), 2)] if reverse_complement else R
+        return Z, [(ord2acgt(X[a + pad:b]), dX[a + pad:b].copy()) for a, b in fwd]
+    maps = [(ord2acgt(X[a + pad:b]), dX[a + pad:b].copy()) for a, b in R]
+    if Zmask is not None:
+        maps = [maps[i] for i in range(len(maps)) if Zmask[i]]
+    return Z, maps
+
+
+def gen_predictionmaps(params, seqs, pool, hidden, out, dropout_rate=None, reverse_complement=False, stride=1, windowsize=20,
+                       want_gmaps=False):
+    """predict.py:263-345: every sequence is N-padded by windowsize-1 on both sides and cut into windows
+    of `windowsize` every `stride` letters; each window is scored as a sequence of its own. Returns
+    (list of per-sequence prediction maps, list of (len+windowsize-1, 4) averaged gradient maps | None)."""
+    pmaps, gmaps = [], []
+    for raw in seqs:
+        padseq = "N" * (windowsize - 1) + raw + "N" * (windowsize - 1)
+        windows = [padseq[i:i + windowsize] for i in range(0, max(1, len(padseq) - windowsize + 1), stride)]
+        Z, wmaps = gen_predictions(params, windows, pool, hidden, out, dropout_rate, reverse_complement, want_gmaps=want_gmaps)
+        pmaps.append(Z.ravel().copy())
+        if want_gmaps:
+            gmap = np.zeros((len(raw) + windowsize - 1, 4), Z.dtype)
+            denom = np.zeros_like(gmap)
+            nwin = len(windows)
+            for j in range(nwin):
+                dXj = wmaps[j][1][:min(windowsize, (nwin - j) * stride)]
+                gmap[j * stride:j * stride + windowsize] += dXj
+                denom[j * stride:j * stride + windowsize] += np.ones_like(dXj)
+            with np.errstate(invalid="ignore", divide="ignore"):
+                gmap /= denom
+            gmaps.append(np.nan_to_num(gmap))
+    return pmaps, (gmaps if want_gmaps else None)
