@@ -34,7 +34,8 @@ _SIGNATURES = {
     "dbk_corr1ord_bprop_X": [_P, _I, _P, _Z, _Z, _P, _Z, _Z, _P],
     "dbk_poolrgn": [_P, _I, _P, _Z, _P, _Z, _I, _P, _P, _I],
     "dbk_poolrgn_bprop": [_P, _I, _P, _Z, _P, _Z, _I, _P, _P, _I],
-    "dbk_dropoutord_fp_tr": [_P, _P, _P, _P, _Z, _F, _U64, _U64],
+    "dbk_dropoutord_fp_tr": [_P, _P, _P, _P, _Z, _F, _U64, _U64, _P],
+    "dbk_dropoutord_mirror": [_P, _P, _P, _P, _P, _Z, _Z],
     "dbk_dropoutord_fp_tr_u": [_P, _P, _P, _P, _Z, _F, _P],
     "dbk_scanpool_fprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
     "dbk_scanpool_fprop_general": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],

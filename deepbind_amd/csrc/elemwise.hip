@@ -85,14 +85,33 @@ template <typename T> __global__ void k_dropout_bp_tr(const T* dZ, const uint8_t
 {
     GRID_STRIDE(i, n) dX[i] = dZ[i] * (T)(M[i] != 0);
 }
-__global__ void k_dropoutord(const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, const float* U, uint64_t seed, uint64_t offset)
+__global__ void k_dropoutord(const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, const float* U, uint64_t seed, uint64_t offset,
+                             const unsigned long long* counter)
 {
+    if (counter) offset = counter[0];
     GRID_STRIDE(i, n) {
         float u = U ? U[i] : uniform_at(seed, offset, i);
-        bool keep = u >= rate;
         uint8_t x = X[i];
-        M[i] = keep;
-        Z[i] = (keep || x == 255) ? x : (uint8_t)254;
+        bool mask = x == 255 || u >= rate;                  // padding always passes (and reports "kept")
+        M[i] = mask;
+        Z[i] = mask ? x : (uint8_t)254;
+    }
+}
+// One workgroup per (fwd, rev) pair of regions: the reverse strand drops the mirrored letters of the
+// forward strand. Regions are [leading pad | sequence]; letter t of the forward sequence pairs with
+// letter len-1-t of the reverse one.
+__global__ void k_dropoutord_mirror(const uint8_t* X, uint8_t* Z, uint8_t* M, const uint32_t* R, size_t npair, unsigned pad)
+{
+    for (size_t p = blockIdx.x; p < npair; p += gridDim.x) {
+        const size_t a = R[4 * p], b = R[4 * p + 1], c = R[4 * p + 2], d = R[4 * p + 3];
+        const size_t lf = b - a, lr = d - c;
+        const size_t len = (lf < lr ? lf : lr);
+        for (size_t t = threadIdx.x; t + pad < len; t += blockDim.x) {
+            const size_t src = a + pad + t, dst = d - 1 - t;
+            const uint8_t mk = M[src];
+            M[dst] = mk;
+            Z[dst] = mk ? X[dst] : (uint8_t)254;
+        }
     }
 }
 template <typename T> __global__ void k_pair_max(const T* Z, T* out, size_t npair, size_t m)
@@ -250,17 +269,30 @@ int dbk_dropout_bp_te(dbk_stream_t stream, int dtype, const void* dZ, const void
     DBK_CHECK(m >= 1 && k >= 1, "ValueError: dropout needs at least one rate and one column per rate");
     EW2(k_dropout_scale, n, A(CF32(dZ), CF32(rate), F32(dX), n, m, k), A(CF64(dZ), CF64(rate), F64(dX), n, m, k));
 }
-int dbk_dropoutord_fp_tr(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, uint64_t seed, uint64_t offset)
+int dbk_dropoutord_fp_tr(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, uint64_t seed, uint64_t offset,
+                         const uint64_t* counter)
 {
     if (n == 0) { dbk::clear_error(); return 0; }
-    hipLaunchKernelGGL(k_dropoutord, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), X, Z, M, n, rate, (const float*)nullptr, seed, offset);
+    hipLaunchKernelGGL(k_dropoutord, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), X, Z, M, n, rate, (const float*)nullptr, seed, offset,
+                       (const unsigned long long*)counter);
+    DBK_LAUNCH_OK();
+}
+int dbk_dropoutord_mirror(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, const uint32_t* regions, size_t nregion, size_t padding)
+{
+    DBK_CHECK(nregion % 2 == 0, "ValueError: reverse-complement regions come in pairs, got %zu", nregion);
+    if (nregion == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(X && Z && M && regions, "ValueError: null pointer argument");
+    const size_t npair = nregion / 2;
+    hipLaunchKernelGGL(k_dropoutord_mirror, dim3(npair < 4096 ? (unsigned)npair : 4096u), dim3(64), 0, dbk::as_stream(stream), X, Z, M, regions, npair,
+                       (unsigned)padding);
     DBK_LAUNCH_OK();
 }
 int dbk_dropoutord_fp_tr_u(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n, float rate, const float* U)
 {
     DBK_CHECK(U != nullptr, "ValueError: U must not be null");
     if (n == 0) { dbk::clear_error(); return 0; }
-    hipLaunchKernelGGL(k_dropoutord, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), X, Z, M, n, rate, U, (uint64_t)0, (uint64_t)0);
+    hipLaunchKernelGGL(k_dropoutord, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), X, Z, M, n, rate, U, (uint64_t)0, (uint64_t)0,
+                       (const unsigned long long*)nullptr);
     DBK_LAUNCH_OK();
 }
 int dbk_pair_max(dbk_stream_t stream, int dtype, const void* Z, void* out, size_t n, size_t m)

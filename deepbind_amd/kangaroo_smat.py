@@ -102,9 +102,13 @@ def poolrgn_bprop(unpooledmaps, regions, pooledmaps, pooledmaps_argmax, ptype):
          int(regions.shape[1] == 3), ptr(pooledmaps), ptr(amax), str2pooltype[ptype])
 
 
-def dropoutord_fp_train(X, rate, U=None):
-    """Input-base dropout: returns (Z, M) with dropped bases replaced by 254. U (optional, float32,
-    same shape) supplies the uniforms instead of the library's generator. reference: kangaroo_smat.py:140-146"""
+def dropoutord_fp_train(X, rate, U=None, regions=None, padding=None, seed=None, offset=None, counter=None):
+    """Input-base dropout: returns (Z, M) with dropped bases replaced by 254 (padding always passes and
+    reports True in M). U (optional, float32, same shape) supplies the uniforms instead of the
+    library's generator; `offset` / `counter` (device int64 tensor) supply the generator position
+    instead of the module's host-side one. With `regions` (pairs of fwd/rev rows) and `padding` the reverse
+    strand's mask is the forward strand's mirrored, as in reverse-complement training.
+    reference: kangaroo_smat.py:140-146, kangaroo/_ext/dropoutord.py:50-70"""
     global _rng_offset
     _u8(X)
     Z = torch.empty_like(X)
@@ -113,9 +117,17 @@ def dropoutord_fp_train(X, rate, U=None):
     if U is not None:
         require(U.dtype == torch.float32 and U.numel() == n, "ValueError: U must be float32 with one value per element")
         call("dbk_dropoutord_fp_tr_u", stream(), ptr(X), ptr(Z), ptr(M), n, float(rate), ptr(U))
+    elif counter is not None:
+        call("dbk_dropoutord_fp_tr", stream(), ptr(X), ptr(Z), ptr(M), n, float(rate), _rng_seed if seed is None else int(seed), 0, ptr(counter))
+    elif offset is not None:
+        call("dbk_dropoutord_fp_tr", stream(), ptr(X), ptr(Z), ptr(M), n, float(rate), _rng_seed if seed is None else int(seed), int(offset), None)
     else:
-        call("dbk_dropoutord_fp_tr", stream(), ptr(X), ptr(Z), ptr(M), n, float(rate), _rng_seed, _rng_offset)
+        call("dbk_dropoutord_fp_tr", stream(), ptr(X), ptr(Z), ptr(M), n, float(rate), _rng_seed if seed is None else int(seed), _rng_offset, None)
         _rng_offset += (n + 3) // 4
+    if regions is not None:
+        _regions(regions)
+        require(regions.shape[1] == 2 and padding is not None, "ValueError: mirroring needs 2-column regions and the padding length")
+        call("dbk_dropoutord_mirror", stream(), ptr(X), ptr(Z), ptr(M), ptr(regions), regions.shape[0], int(padding))
     return Z, M
 
 

@@ -33,7 +33,8 @@ from . import smat as sm
 class SequenceNet(object):
     def __init__(self, nmodel, nfilter, m, pool="max", hidden=32, loss="nll", dtype=torch.float32,
                  rate=0.01, momentum=0.9, decay_conv=0.0, decay_full=0.0, dropout=0.0,
-                 weight_decay_start=100, nesterov=True, mode="fused", reverse_complement=False, device="cuda"):
+                 weight_decay_start=100, nesterov=True, mode="fused", reverse_complement=False, input_dropout=0.0,
+                 device="cuda"):
         assert pool in ("max", "avg", "all") and loss in ("nll", "mse", None)
         self.ninst, self.nfilter, self.m = int(nmodel), int(nfilter), int(m)
         self.pool, self.hidden, self.loss = pool, int(hidden), loss
@@ -43,6 +44,10 @@ class SequenceNet(object):
         # prediction of a pair contributes to loss and gradient
         # (reference: kangaroo/kangaroo/data.py:274-306, deepity/std/loss.py:114-119, deepity_smat/dropout.cu:57-77)
         self.reverse_complement = bool(reverse_complement)
+        # input-base dropout: while training each letter is replaced by the "contributes nothing" code with
+        # this probability; at test time the scan output is scaled by (1 - rate) instead
+        # (reference: kangaroo/_ext/dropoutord.py:42-74, kangaroo/_ext/corr1ord.py:104-109)
+        self.input_dropout = float(input_dropout)
         self.step_count = 0
         ni, nf = self.ninst, self.nfilter
         self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
@@ -111,13 +116,35 @@ class SequenceNet(object):
         return {name: self.g[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
     # ------------------------------------------------------------------ forward
-    def _conv_forward(self, X, R, want_argmax):
-        p = self.p
+    def _drop_inputs(self, X, R, U_input=None):
+        """Training-time input dropout; draws come from this net's generator position (device counter in
+        fused mode, its host mirror layer by layer) unless uniforms are supplied."""
+        if self.input_dropout <= 0:
+            return X
+        kw = dict(regions=R if self.reverse_complement else None, padding=self.m - 1, seed=self.rng_seed)
+        if U_input is not None:
+            return ks.dropoutord_fp_train(X, self.input_dropout, U=U_input, **kw)[0]
+        draws = (X.numel() + 3) // 4
         if self.mode == "fused":
-            pooled, amax = ks.scanpool_fprop(p["Wc"], p["bc"], X, R, self.pool, want_argmax=want_argmax)
+            Z = ks.dropoutord_fp_train(X, self.input_dropout, counter=self.rng_counter, **kw)[0]
+        else:
+            Z = ks.dropoutord_fp_train(X, self.input_dropout, offset=self._rng_offset, **kw)[0]
+        ds.counter_add(self.rng_counter, draws)
+        self._rng_offset += draws
+        return Z
+
+    def _conv_forward(self, X, R, want_argmax, train=False):
+        p = self.p
+        keep = 1.0 if (train or self.input_dropout <= 0) else 1.0 - self.input_dropout
+        if self.mode == "fused":
+            # test-time rescale folded into the filters (sum of scaled taps instead of scaled sum)
+            Wc = p["Wc"] if keep == 1.0 else p["Wc"] * keep
+            pooled, amax = ks.scanpool_fprop(Wc, p["bc"], X, R, self.pool, want_argmax=want_argmax)
             return pooled, amax, None
         Z = sm.zeros((X.numel(), p["Wc"].shape[1]), dtype=self.dtype, device=self.device)
         ks.corr1ord(p["Wc"], X, Z, 4)
+        if keep != 1.0:
+            Z *= keep
         A = sm.relu(sm.add_rowvec(Z, p["bc"]))
         pooled, amax = ks.poolrgn(A, R, self.pool, want_argmax=want_argmax)
         return pooled, amax, A
@@ -126,7 +153,7 @@ class SequenceNet(object):
         """Returns the state dict of one forward pass; st["Z"] are the predictions (n x ninst)."""
         p, ni = self.p, self.ninst
         st = {}
-        st["pooled"], st["argmax"], st["A0"] = self._conv_forward(X, R, want_argmax)
+        st["pooled"], st["argmax"], st["A0"] = self._conv_forward(X, R, want_argmax, train=train)
         H0 = st["pooled"]
         if self.use_dropout:
             if train:
@@ -175,6 +202,8 @@ class SequenceNet(object):
         p, ni = self.p, self.ninst
         Z0 = sm.zeros((X.numel(), p["Wc"].shape[1]), dtype=self.dtype, device=self.device)
         ks.corr1ord(p["Wc"], X, Z0, 4)
+        if self.input_dropout > 0:
+            Z0 *= 1.0 - self.input_dropout           # forward only: the reference's backward pass ignores this factor too
         A0 = sm.relu(sm.add_rowvec(Z0, p["bc"]))
         pooled, amax = ks.poolrgn(A0, R, self.pool, want_argmax=True)
         H0 = ds.dropout_fp_test(pooled, self.dropout) if self.use_dropout else pooled
@@ -257,10 +286,11 @@ class SequenceNet(object):
         if self.hidden > 0:
             ds.madd_bcast(sm.sign(p["W2"]), self.decay_full, p["W2"].numel() // ni, g["W2"])
 
-    def _grad_fused(self, X, R, Y, Ymask, U):
-        """Gradient of one batch in four launches: fused scan+pool forward, the whole dense head
-        forward+backward, fused scan+pool backward (+ its two slab reductions)."""
+    def _grad_fused(self, X, R, Y, Ymask, U, U_input=None):
+        """Gradient of one batch in a handful of launches: fused scan+pool forward, the whole dense head
+        forward+backward (+ chunk reduction), fused scan+pool backward (+ slab reduction)."""
         p, g = self.p, self.g
+        X = self._drop_inputs(X, R, U_input)
         pooled, amax = ks.scanpool_fprop(p["Wc"], p["bc"], X, R, self.pool, want_argmax=True)
         rate = self.dropout if self.use_dropout else None
         Z, dpooled, _ = ds.head_train(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), Y, self.ninst, self.loss,
@@ -285,15 +315,18 @@ class SequenceNet(object):
         active, so it is re-captured when the step counter crosses weight_decay_start."""
         return _graphed_step([(self, X, R, Y, Ymask)])
 
-    def train_step(self, X, R, Y, Ymask=None, U=None):
-        fused = self.mode == "fused" and self.dtype == torch.float32 and self.k <= 64 and self.loss is not None
+    def train_step(self, X, R, Y, Ymask=None, U=None, U_input=None):
+        """One optimiser step. U / U_input optionally supply the uniforms of the pooled-feature and the
+        input dropout (otherwise the library's generator draws them)."""
+        fused = self.mode == "fused" and self.dtype == torch.float32 and self.loss is not None
 
         def grad():
             if fused:
-                self._grad_fused(X, R, Y, Ymask, U)
+                self._grad_fused(X, R, Y, Ymask, U, U_input)
             else:
-                st = self.forward(X, R, train=True, U=U, want_argmax=True)
-                self.backward(X, R, st, Y, Ymask)
+                Xd = self._drop_inputs(X, R, U_input)
+                st = self.forward(Xd, R, train=True, U=U, want_argmax=True)
+                self.backward(Xd, R, st, Y, Ymask)
         ds.gradstep(self.P, self.dP, self.drate, self.mP, self.mrate, grad, nesterov=self.nesterov)
         self.step_count += 1
 
@@ -361,6 +394,8 @@ def _graphed_step(jobs, streams=None):
             capture()
         state["graph"].replay()
         for net, X, R, Y, Ymask in jobs:
+            if net.input_dropout > 0:
+                net._rng_offset += (X.numel() + 3) // 4
             if net.use_dropout:
                 net._rng_offset += (R.shape[0] * net.k * net.ninst + 3) // 4
             net.step_count += 1

@@ -90,14 +90,21 @@ int dbk_poolrgn_bprop(dbk_stream_t stream, int dtype,
                       const uint32_t* regions, size_t nregion, int per_region_step,
                       const void* pooledmaps, const uint32_t* pooledmaps_argmax, int ptype);
 
-/* Input-base dropout: Z = keep ? X : 254, except X==255 which always passes; M = keep.
- * keep = (u >= rate) with u from the library's counter-based generator (seed, offset).
+/* Input-base dropout: M = (X == 255) || (u >= rate); Z = M ? X : 254 (padding always passes).
+ * u comes from the library's counter-based generator at (seed, offset); when `counter` is not null
+ * the offset is read from that device word instead (see dbk_counter_add).
  * reference: launch_dropoutord_fp_tr, kangaroo_smat.cpp:81-82, dropoutord.cu:41-60 */
 int dbk_dropoutord_fp_tr(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n,
-                         float rate, uint64_t seed, uint64_t offset);
+                         float rate, uint64_t seed, uint64_t offset, const uint64_t* counter);
 /* Same with caller-supplied uniforms U (n floats) instead of the generator. */
 int dbk_dropoutord_fp_tr_u(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n,
                            float rate, const float* U);
+/* Reverse-complement mode of the input dropout: regions come in (fwd, rev) pairs of equal length,
+ * each [padding | sequence]; the reverse strand's mask becomes the forward strand's mask mirrored
+ * (letter t <-> letter len-1-t) and Z is rewritten there as M ? X : 254.
+ * reference: the host loop in kangaroo/_ext/dropoutord.py:55-68 */
+int dbk_dropoutord_mirror(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uint8_t* M,
+                          const uint32_t* regions, size_t nregion, size_t padding);
 
 /* ------------------------------------------------------------------ fused scan + bias + ReLU + pool */
 

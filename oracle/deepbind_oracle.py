@@ -281,11 +281,24 @@ def dropout_bp_te(dZ, rate):
     return dZ * (dZ.dtype.type(1) - p)[None, :]
 
 
-def dropoutord_fp_train(X, rate, U):
-    """kangaroo_smat/dropoutord.cu:41-52: keep iff U >= rate; dropped real bases become 254; 255 stays."""
+def dropoutord_fp_train(X, rate, U, regions=None, reverse_complement=False):
+    """kangaroo_smat/dropoutord.cu:41-52: M = (X == 255) or (U >= rate); Z = M ? X : 254.
+    With reverse complements (kangaroo/_ext/dropoutord.py:55-68) the reverse row's mask is the forward
+    row's flipped over the sequence part and Z is rebuilt as X with 254 wherever M is false."""
     X = np.asarray(X)
-    M = np.asarray(U).reshape(X.shape) >= rate
-    Z = np.where(M | (X == 255), X, np.uint8(254)).astype(np.uint8)
+    M = (X == 255) | (np.asarray(U).reshape(X.shape) >= rate)
+    Z = np.where(M, X, np.uint8(254)).astype(np.uint8)
+    if reverse_complement:
+        M = M.copy()
+        R = np.asarray(regions).astype(np.int64)
+        padsize = M.size - int(R[-1, -1])
+        Mf = M.reshape(-1)
+        for i in range(0, len(R), 2):
+            a, b = R[i]
+            c, d = R[i + 1]
+            Mf[c + padsize:d] = Mf[a + padsize:b][::-1]
+        Z = X.copy()
+        Z.reshape(-1)[~Mf] = 254
     return Z, M
 
 
@@ -461,13 +474,16 @@ def madd_bcast(A, b, k, dst):
 # whole-model forward / backward for a homogeneous batch of models on the model axis
 # layer order: kangaroo/kangaroo/model.py:45-132 ; deepity/_io_/load.py:51-72 ; cfg/*/M{1,2}.cfg
 # ----------------------------------------------------------------------------------------------
-def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None, train=False, matchrows=False):
-    """scan -> bias -> relu -> pool -> dropout -> dense(+bias[,relu,dense,bias]) -> (logistic)."""
+def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None, train=False, matchrows=False, input_keep=1.0):
+    """scan (-> * input_keep: the test-time side of input dropout, kangaroo/_ext/corr1ord.py:104-109) -> bias ->
+    relu -> pool -> dropout -> dense(+bias[,relu,dense,bias]) -> (logistic)."""
     m = params["Wc"].shape[0] // 4
     N = np.asarray(X).size
     st = {}
     Z0 = np.zeros((N, params["Wc"].shape[1]), params["Wc"].dtype)
     corr1ord(params["Wc"], X, Z0)
+    if input_keep != 1.0:
+        Z0 *= input_keep
     st["A0"] = relu_fprop(bias_fprop(Z0, params["bc"]))
     st["Pl"], st["I"] = poolrgn(st["A0"], R, pool, want_argmax=True)
     H = st["Pl"]
@@ -599,12 +615,12 @@ def maskout_revcomp(Z, reverse_complement):
     return Z[Zmask.ravel()], Zmask
 
 
-def eval_with_input_gradients(params, X, R, nmodel, pool, hidden, out, dropout_rate=None, reverse_complement=False):
+def eval_with_input_gradients(params, X, R, nmodel, pool, hidden, out, dropout_rate=None, reverse_complement=False, input_keep=1.0):
     """Test-mode forward pass, then back-propagation of dA = Z (targets 0, no batch mean, only
     output column 0, reverse-complement losers masked) down to the one-hot inputs: dX (N, 4).
     node.py:317-339, loss.py:98-109, elemwise.py:148-157 (test-mode dropout bprop), corr1ord.py:129-133."""
     dropout = None if dropout_rate is None else (np.asarray(dropout_rate, dtype=params["Wc"].dtype), None)
-    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=False)
+    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=False, input_keep=input_keep)
     Z = st["Zout"]
     dA = Z.copy()
     if reverse_complement:
@@ -626,7 +642,7 @@ def eval_with_input_gradients(params, X, R, nmodel, pool, hidden, out, dropout_r
     return Z, dX
 
 
-def gen_predictions(params, seqs, pool, hidden, out, dropout_rate=None, reverse_complement=False, want_gmaps=False):
+def gen_predictions(params, seqs, pool, hidden, out, dropout_rate=None, reverse_complement=False, want_gmaps=False, input_keep=1.0):
     """predict.py:168-260 for one model and one batch. Returns (predictions (nseq, 1), gmaps) where
     gmaps is None, or a list of (sequence string, (len, 4) map): the back-propagated input gradient
     (want_gmaps=True; with reverse complements only the winning strand's entry is kept), or the
@@ -640,12 +656,12 @@ def gen_predictions(params, seqs, pool, hidden, out, dropout_rate=None, reverse_
 
     def predict(Xb):
         dropout = None if dropout_rate is None else (np.asarray(dropout_rate, dtype=params["Wc"].dtype), None)
-        return model_forward(params, Xb, R, 1, pool, hidden, out=out, dropout=dropout, train=False)["Zout"]
+        return model_forward(params, Xb, R, 1, pool, hidden, out=out, dropout=dropout, train=False, input_keep=input_keep)["Zout"]
 
     if not want_gmaps:
         Z, _ = maskout_revcomp(predict(X), reverse_complement)
         return Z, None
-    Zall, dX = eval_with_input_gradients(params, X, R, 1, pool, hidden, out, dropout_rate, reverse_complement)
+    Zall, dX = eval_with_input_gradients(params, X, R, 1, pool, hidden, out, dropout_rate, reverse_complement, input_keep)
     Z, Zmask = maskout_revcomp(Zall, reverse_complement)
     if want_gmaps == "finite_diff":
         rcindex = [3, 2, 1, 0]
@@ -677,7 +693,7 @@ def gen_predictions(params, seqs, pool, hidden, out, dropout_rate=None, reverse_
 
 
 def gen_predictionmaps(params, seqs, pool, hidden, out, dropout_rate=None, reverse_complement=False, stride=1, windowsize=20,
-                       want_gmaps=False):
+                       want_gmaps=False, input_keep=1.0):
     """predict.py:263-345: every sequence is N-padded by windowsize-1 on both sides and cut into windows
     of `windowsize` every `stride` letters; each window is scored as a sequence of its own. Returns
     (list of per-sequence prediction maps, list of (len+windowsize-1, 4) averaged gradient maps | None)."""
@@ -685,7 +701,8 @@ def gen_predictionmaps(params, seqs, pool, hidden, out, dropout_rate=None, rever
     for raw in seqs:
         padseq = "N" * (windowsize - 1) + raw + "N" * (windowsize - 1)
         windows = [padseq[i:i + windowsize] for i in range(0, max(1, len(padseq) - windowsize + 1), stride)]
-        Z, wmaps = gen_predictions(params, windows, pool, hidden, out, dropout_rate, reverse_complement, want_gmaps=want_gmaps)
+        Z, wmaps = gen_predictions(params, windows, pool, hidden, out, dropout_rate, reverse_complement, want_gmaps=want_gmaps,
+                                   input_keep=input_keep)
         pmaps.append(Z.ravel().copy())
         if want_gmaps:
             gmap = np.zeros((len(raw) + windowsize - 1, 4), Z.dtype)

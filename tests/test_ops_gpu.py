@@ -343,6 +343,15 @@ def test_masks_dropout_and_loss_ops(ds, sm, ks):
     Zo, Mo = ks.dropoutord_fp_train(dev(Xo), 0.3, U=dev(Uo))
     Zor, Mor = orc.dropoutord_fp_train(Xo, np.float32(0.3), Uo)
     assert np.array_equal(host(Zo), Zor) and np.array_equal(host(Mo), Mor)
+    assert host(Mo)[Xo == 255].all()                                   # padding always reports "kept"
+    # reverse-complement rows: the reverse strand drops the mirrored letters
+    from deepbind_amd import data
+    seqs = ["".join("ACGTN"[v] for v in rng.integers(0, 5, int(rng.integers(1, 40)))) for _ in range(30)]
+    Xp, Rp = data.pack_sequences(seqs, 7, reverse_complement=True)
+    Up = rng.random(Xp.shape).astype(np.float32)
+    Zp, Mp = ks.dropoutord_fp_train(dev(Xp), 0.4, U=dev(Up), regions=dev(Rp), padding=7)
+    Zpr, Mpr = orc.dropoutord_fp_train(Xp, np.float32(0.4), Up, regions=Rp, reverse_complement=True)
+    assert np.array_equal(host(Zp), Zpr) and np.array_equal(host(Mp), Mpr)
     # maskout / zmask
     A = rng.standard_normal((n, nb)).astype(np.float32); A[3, 2] = np.nan
     Mk = rng.random((n, nb)) < 0.7; Mk[3, 2] = False

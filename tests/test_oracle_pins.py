@@ -337,6 +337,13 @@ def test_dropout_semantics():
     Xo = np.array([0, 1, 255, 3, 2], np.uint8)
     Zo, Mo = orc.dropoutord_fp_train(Xo, 0.5, np.array([0.9, 0.1, 0.1, 0.1, 0.7]))
     assert Zo.tolist() == [0, 254, 255, 254, 2]
+    assert Mo.tolist() == [True, False, True, False, True]            # padding reports "kept" (dropoutord.cu:47-49)
+    # reverse complements: "ACG" and its reverse complement "CGT", padding 2: the reverse row drops the mirrored letters
+    Xp, Rp = orc.pack(["ACG", "CGT"], 2)
+    Up = np.array([.9, .9, .1, .9, .9, .9, .9, .9, .9, .1, .9, .9])[:, None]      # drops fwd letter 0 (A); rev letter 1 drawn low too
+    Zp, Mp = orc.dropoutord_fp_train(Xp, 0.5, Up, regions=Rp, reverse_complement=True)
+    assert Zp.ravel().tolist() == [255, 255, 254, 1, 2, 255, 255, 1, 2, 254, 255, 255]   # rev "CGT" loses its T (pairs with A), keeps G
+    assert Mp.ravel().tolist() == [True, True, False, True, True, True, True, True, True, False, True, True]
 
 
 def test_whole_model_gradient_matches_finite_differences():

@@ -12,13 +12,15 @@ ACT, GRAD = 1e-5, 1e-4
 
 
 def _params(rng, m, F, pool, hidden, scale=0.5):
+    # dense weights small enough that the logistic output stays away from saturation: two strands that
+    # both round to 1.0f would be a tie in float32 but not in the float64 oracle
     k = F * (2 if pool == "all" else 1)
     f = lambda *s: (rng.standard_normal(s) * scale).astype(np.float32)
     p = {"Wc": f(4 * m, F), "bc": f(1, F) * 0.3}
     if hidden:
-        p.update(W1=f(k, hidden), b1=f(1, hidden) * 0.2, W2=f(hidden, 1), b2=f(1, 1) * 0.2 - 0.2)
+        p.update(W1=f(k, hidden) * 0.3, b1=f(1, hidden) * 0.2, W2=f(hidden, 1) * 0.3, b2=f(1, 1) * 0.2 - 0.2)
     else:
-        p.update(W1=f(k, 1), b1=f(1, 1) * 0.2 - 0.2)
+        p.update(W1=f(k, 1) * 0.2, b1=f(1, 1) * 0.2 - 0.2)
     return p
 
 
@@ -45,7 +47,7 @@ CASES = [("max", 8, "nll", False, 0.0, 24, 16), ("all", 0, "mse", False, 0.3, 16
 @pytest.mark.parametrize("mode", [False, True, "finite_diff"])
 def test_gen_predictions(pool, hidden, loss, rc, rate, m, F, mode):
     from deepbind_amd import predict
-    rng = np.random.default_rng(hash((pool, hidden, rc, m)) % 1000)
+    rng = np.random.default_rng(1000 * m + 10 * hidden + int(rc))
     p = _params(rng, m, F, pool, hidden)
     seqs = _seqs(rng, 7, 18, 30)                       # ragged: includes the pad-mutation quirk of short sequences
     out = "logistic" if loss == "nll" else "linear"

@@ -266,3 +266,71 @@ def test_graphed_group_step_matches_eager_group_step():
             pa, pb = a.get_params(), b.get_params()
             for k in pa:
                 assert np.array_equal(pa[k], pb[k]), "replay %d, %s/%d group, %s" % (i, a.pool, a.hidden, k)
+
+
+@pytest.mark.parametrize("mode", ["fused", "unfused"])
+@pytest.mark.parametrize("rc", [False, True])
+def test_input_dropout_train_steps_and_test_time_rescale(mode, rc):
+    """Input-base dropout: training scans the stream with dropped letters (mirrored on the reverse strand),
+    prediction scales the scan output by (1 - rate) instead."""
+    from deepbind_amd import data
+    from deepbind_amd.model import SequenceNet
+    rng = np.random.default_rng(31)
+    m, F, hid, rate_in = 8, 16, 8, 0.2
+    seqs = ["".join("ACGTN"[v] for v in rng.choice(5, int(rng.integers(12, 30)), p=[.24, .24, .24, .24, .04])) for _ in range(20)]
+    X, R = data.pack_sequences(seqs, m - 1, reverse_complement=rc)
+    n = len(R)
+    params = {"Wc": rng.standard_normal((4 * m, F)) * 0.3, "bc": rng.standard_normal((1, F)) * 0.1,
+              "W1": rng.standard_normal((F, hid)) * 0.3, "b1": rng.standard_normal((1, hid)) * 0.1,
+              "W2": rng.standard_normal((hid, 1)) * 0.3, "b2": rng.standard_normal((1, 1)) * 0.1}
+    params = {k: v.astype(np.float32) for k, v in params.items()}
+    Y = np.repeat((rng.random((len(seqs), 1)) < 0.5).astype(np.float32), 2 if rc else 1, axis=0)
+    net = SequenceNet(1, F, m, pool="max", hidden=hid, loss="nll", rate=0.05, momentum=0.9, mode=mode,
+                      reverse_complement=rc, input_dropout=rate_in)
+    net.set_params(params)
+    ref_p, ref_m = _f64(params), {k: np.zeros(v.shape) for k, v in params.items()}
+    Xd, Rd, Yd = dev(X), dev(R), dev(Y)
+    for step in range(2):
+        U = rng.random(X.shape).astype(np.float32)
+        net.train_step(Xd, Rd, Yd, U_input=dev(U))
+        Xdrop, _ = orc.dropoutord_fp_train(X, np.float32(rate_in), U, regions=R, reverse_complement=rc)
+        assert (Xdrop == 254).sum() > 10
+        _, g = orc.train_step(ref_p, ref_m, Xdrop, R, Y.astype(np.float64), 1, "max", hid, "nll", 0.05, 0.9, step=step,
+                              reverse_complement=rc)
+        got_g = net.get_grads()
+        for k in g:
+            assert_close(got_g[k], g[k], GRAD, "step %d grad %s" % (step, k))
+    # prediction: no letters dropped, scan output scaled
+    st = orc.model_forward(ref_p, X, R, 1, "max", hid, out="logistic", input_keep=1.0 - rate_in)
+    want = st["Zout"].reshape(-1, 2).max(axis=1, keepdims=True) if rc else st["Zout"]
+    assert_close(host(net.predict(Xd, Rd)), want, ACT, "test-time prediction")
+    assert_close(host(net.forward(Xd, Rd)["Z"]), st["Zout"], ACT, "test-time forward")
+
+
+def test_input_dropout_draws_from_the_library_generator_in_both_modes_and_under_a_graph():
+    from deepbind_amd import synth
+    from deepbind_amd.model import SequenceNet
+    cfg = synth.config3()
+    spec = cfg["spec"]
+    jit = np.random.default_rng(2)
+    params = {k: (v if not k.startswith("b") else (jit.standard_normal(v.shape) * 0.01).astype(np.float32)) for k, v in cfg["params"].items()}
+
+    def make(mode):
+        net = SequenceNet(1, spec.nfilter, spec.m, pool="max", hidden=32, loss="nll", rate=0.05, momentum=0.9, dropout=0.5,
+                          input_dropout=0.1, mode=mode)
+        net.rng_seed = 9
+        net.set_params(params)
+        return net
+
+    fused, layered, graphed = make("fused"), make("unfused"), make("fused")
+    X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
+    step = graphed.make_graphed_step(X, R, Y)
+    for i in range(3):
+        fused.train_step(X, R, Y)
+        layered.train_step(X, R, Y)
+        step()
+        a, b, c = fused.get_params(), layered.get_params(), graphed.get_params()
+        for k in a:
+            assert np.array_equal(a[k], c[k]), "graph replay %d differs in %s" % (i, k)
+            assert_close(b[k], a[k], GRAD, "layer-by-layer vs fused, step %d, %s" % (i, k))
+    assert fused._rng_offset == layered._rng_offset == graphed._rng_offset == int(graphed.rng_counter.item())
