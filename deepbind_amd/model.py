@@ -115,6 +115,46 @@ class SequenceNet(object):
         torch.cuda.synchronize()
         return {name: self.g[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
+    # ------------------------------------------------------------------ export
+    def _config(self):
+        return dict(nfilter=self.nfilter, m=self.m, pool=self.pool, hidden=self.hidden, loss=self.loss or "",
+                    reverse_complement=self.reverse_complement, input_dropout=self.input_dropout)
+
+    def slice_model(self, i):
+        """A single-model net holding model i's parameters and dropout rate, for export and prediction
+        (reference: slice_inst, deepity/deepity/node.py:148-163; hypertrain.py:136-162)."""
+        assert 0 <= i < self.ninst
+        one = SequenceNet(1, self.nfilter, self.m, pool=self.pool, hidden=self.hidden, loss=self.loss, dtype=self.dtype,
+                          dropout=float(self.dropout[i].item()), mode=self.mode, reverse_complement=self.reverse_complement,
+                          input_dropout=self.input_dropout, device=self.device)
+        src = self.get_params()
+        picked = {}
+        for name, shape, axis in self.layout:
+            blocks = np.split(src[name], self.ninst, axis=axis)
+            picked[name] = blocks[i]
+        one.set_params(picked)
+        return one
+
+    def save_npz(self, path):
+        """Writes the architecture and the parameters of a single-model net to one .npz file."""
+        assert self.ninst == 1, "slice one model out first"
+        cfg = self._config()
+        arrays = {"cfg_" + k: np.asarray(v) for k, v in cfg.items()}
+        arrays["cfg_dropout"] = np.asarray(float(self.dropout[0].item()))
+        arrays.update({"p_" + k: v for k, v in self.get_params().items()})
+        np.savez(path, **arrays)
+
+    @staticmethod
+    def load_npz(path, device="cuda", mode="fused"):
+        with np.load(path, allow_pickle=False) as f:
+            cfg = {k[4:]: f[k].item() for k in f.files if k.startswith("cfg_")}
+            params = {k[2:]: f[k] for k in f.files if k.startswith("p_")}
+        net = SequenceNet(1, int(cfg["nfilter"]), int(cfg["m"]), pool=str(cfg["pool"]), hidden=int(cfg["hidden"]),
+                          loss=(str(cfg["loss"]) or None), dropout=float(cfg["dropout"]), mode=mode,
+                          reverse_complement=bool(cfg["reverse_complement"]), input_dropout=float(cfg["input_dropout"]), device=device)
+        net.set_params(params)
+        return net
+
     # ------------------------------------------------------------------ forward
     def _drop_inputs(self, X, R, U_input=None):
         """Training-time input dropout; draws come from this net's generator position (device counter in
@@ -442,6 +482,13 @@ class ModelGroup(object):
             jobs.append((net, X, R, Y.index_select(1, ii).contiguous(),
                          Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
         return _graphed_step(jobs, self._streams())
+
+    def slice_model(self, j):
+        """Single-model net for model j of the original ordering."""
+        for idx, net in self.groups:
+            if j in idx:
+                return net.slice_model(idx.index(j))
+        raise IndexError(j)
 
     def predict(self, X, R):
         out = torch.empty((R.shape[0], self.nmodel), dtype=torch.float32, device=X.device)

@@ -334,3 +334,74 @@ def test_input_dropout_draws_from_the_library_generator_in_both_modes_and_under_
             assert np.array_equal(a[k], c[k]), "graph replay %d differs in %s" % (i, k)
             assert_close(b[k], a[k], GRAD, "layer-by-layer vs fused, step %d, %s" % (i, k))
     assert fused._rng_offset == layered._rng_offset == graphed._rng_offset == int(graphed.rng_counter.item())
+
+
+def test_slice_model_save_load_and_group_prediction(tmp_path):
+    """A model sliced out of a trained batch predicts exactly what its column of the batch predicts,
+    before and after a round trip through the .npz export."""
+    from deepbind_amd import synth
+    from deepbind_amd.model import ModelGroup, SequenceNet
+    cfg = synth.config4()
+    spec, hp = cfg["spec"], cfg["hp"]
+    grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
+                     decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"])
+    for idx, net in grp.groups:
+        net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
+    X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
+    for _ in range(2):
+        grp.train_step(X, R, Y, M)
+    scores = host(grp.predict(X, R))
+    for j in (0, 17, 44, 89):
+        one = grp.slice_model(j)
+        assert one.ninst == 1 and (one.pool, one.hidden) == (spec.pool[j], spec.hidden[j])
+        s1 = host(one.predict(X, R))
+        assert_close(s1[:, 0], scores[:, j], ACT, "model %d sliced" % j)
+        path = str(tmp_path / ("m%d.npz" % j))
+        one.save_npz(path)
+        back = SequenceNet.load_npz(path)
+        assert np.array_equal(host(back.predict(X, R)), s1)
+        for k, v in one.get_params().items():
+            assert np.array_equal(back.get_params()[k], v)
+
+
+def test_training_from_a_sequence_file_reduces_the_loss(tmp_path):
+    """Reader -> batcher -> reverse-complement training loop -> export -> prediction, on a planted motif."""
+    from deepbind_amd import datasource, predict
+    from deepbind_amd.model import SequenceNet
+    rng = np.random.default_rng(4)
+    lines = ["FoldID\tEventID\tseq\tBound"]
+    for i in range(256):
+        s = rng.integers(0, 4, 40)
+        bound = i % 2
+        if bound:
+            at = int(rng.integers(0, 32))
+            s[at:at + 8] = [2, 0, 3, 3, 0, 1, 0, 2]                      # GATTACAG
+            if rng.random() < 0.5:
+                s = 3 - s[::-1]                                           # planted on either strand
+        lines.append("%s\tseq%d\t%s\t%d" % ("ABC"[i % 3], i, "".join("ACGT"[v] for v in s), bound))
+    path = tmp_path / "train.seq"
+    path.write_text("\n".join(lines) + "\n")
+    d = datasource.SequenceData.fromtxt(str(path))
+    train, held = d.extract_fold("A")[:], d.extract_fold("C")
+    m = 10
+    net = SequenceNet(1, 8, m, pool="max", hidden=0, loss="nll", rate=0.05, momentum=0.9, reverse_complement=True, dropout=0.0)
+    init = np.random.default_rng(0)
+    net.set_params({"Wc": (init.standard_normal((4 * m, 8)) * 0.1).astype(np.float32), "bc": np.zeros((1, 8), np.float32),
+                    "W1": (init.standard_normal((8, 1)) * 0.1).astype(np.float32), "b1": np.zeros((1, 1), np.float32)})
+    batches = [{k: dev(v) for k, v in b.items() if k != "rowidx"} for b in d.asbatches(64, padding=m - 1, reverse_complement=True)]
+
+    def mean_loss():
+        return float(np.mean([net.loss_value(net.forward(b["X"], b["R"]), b["Y"], b["Ymask"])[0, 0] for b in batches]))
+
+    before = mean_loss()
+    for epoch in range(60):
+        for b in batches:
+            net.train_step(b["X"], b["R"], b["Y"], b["Ymask"])
+    after = mean_loss()
+    assert after < 0.5 * before, (before, after)
+    Z, _ = predict.gen_predictions(net, held.sequences)
+    auc_pairs = [(z, y) for z, y in zip(Z.ravel(), held.Y.ravel())]
+    pos = [z for z, y in auc_pairs if y == 1]
+    neg = [z for z, y in auc_pairs if y == 0]
+    auc = np.mean([p > q for p in pos for q in neg])
+    assert auc > 0.9, auc
