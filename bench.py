@@ -129,6 +129,7 @@ def main():
     ap.add_argument("--workload", default="config5", choices=["config5", "config5_small"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the secondary train-step throughput figures")
+    ap.add_argument("--train-only", action="store_true", help="only the train-step figures (for profiling the training kernels)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain copy kernel over 1 GiB (reference point for the HBM byte counters)")
     args = ap.parse_args()
@@ -141,6 +142,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
 
+    if args.train_only:
+        print(json.dumps({"train": train_throughput(steps=args.steps, warmup=args.warmup)}))
+        return
     nseq = 100000 if args.workload == "config5" else 5000
     cfg = synth.config5(seed=4, nseq=nseq)
     spec, p = cfg["spec"], cfg["params"]
@@ -209,7 +213,7 @@ def main():
     if not args.no_train:
         out["train"] = train_throughput()
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, nseq_c=min(nseq, 1000), nseq_np=min(nseq, 100))
+        out["cpu_baseline"] = cpu_baseline(cfg, nseq_c=min(nseq, 1000), nseq_np=min(nseq, 300))
     print(json.dumps(out))
 
 
