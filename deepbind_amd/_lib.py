@@ -60,6 +60,7 @@ _SIGNATURES = {
     "dbk_dropout_bp_tr": [_P, _I, _P, _P, _P, _Z],
     "dbk_dropout_bp_te": [_P, _I, _P, _P, _P, _Z, _Z, _Z],
     "dbk_uniform_fill": [_P, _P, _Z, _U64, _U64],
+    "dbk_normal_fill": [_P, _I, _P, _Z, _U64, _U64],
     "dbk_philox4x32_10": [_P, _P, _P],
     "dbk_add_rowvec": [_P, _I, _P, _P, _P, _Z, _Z],
     "dbk_colsum": [_P, _I, _P, _P, _Z, _Z],

@@ -178,6 +178,21 @@ __global__ void k_uniform_fill(float* U, size_t n, uint64_t seed, uint64_t offse
 {
     GRID_STRIDE(i, n) U[i] = uniform_at(seed, offset, i);
 }
+// Standard normals by Box-Muller from two independent Philox streams (third counter word 0 / 1), one value
+// per element so that element i depends only on (seed, offset, i).
+template <typename T> __global__ void k_normal_fill(T* Z, size_t n, uint64_t seed, uint64_t offset)
+{
+    GRID_STRIDE(i, n) {
+        const uint64_t ctr = offset + (uint64_t)(i >> 2);
+        uint32_t a[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u};
+        uint32_t b[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 1u, 0u};
+        philox4x32_10(a, (uint32_t)seed, (uint32_t)(seed >> 32));
+        philox4x32_10(b, (uint32_t)seed, (uint32_t)(seed >> 32));
+        const float u1 = ((float)(a[i & 3] >> 8) + 1.0f) * (1.0f / 16777216.0f);      // (0, 1]
+        const float u2 = (float)(b[i & 3] >> 8) * (1.0f / 16777216.0f);               // [0, 1)
+        Z[i] = (T)(sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2));
+    }
+}
 __global__ void k_counter_add(unsigned long long* ctr, unsigned long long delta) { if (threadIdx.x == 0 && blockIdx.x == 0) ctr[0] += delta; }
 template <typename T> __global__ void k_sub_scale(const T* Z, const T* Y, T scale, T* dZ, size_t n)
 {
@@ -346,6 +361,18 @@ int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uin
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(U != nullptr, "ValueError: U must not be null");
     hipLaunchKernelGGL(k_uniform_fill, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), U, n, seed, offset);
+    DBK_LAUNCH_OK();
+}
+
+int dbk_normal_fill(dbk_stream_t stream, int dtype, void* Z, size_t n, uint64_t seed, uint64_t offset)
+{
+    DBK_CHECK(dtype == DBK_F32 || dtype == DBK_F64, "TypeError: dtype must be float32 or float64");
+    if (n == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(Z != nullptr, "ValueError: Z must not be null");
+    if (dtype == DBK_F32)
+        hipLaunchKernelGGL(k_normal_fill<float>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), (float*)Z, n, seed, offset);
+    else
+        hipLaunchKernelGGL(k_normal_fill<double>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), (double*)Z, n, seed, offset);
     DBK_LAUNCH_OK();
 }
 

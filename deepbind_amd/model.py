@@ -34,7 +34,7 @@ class SequenceNet(object):
     def __init__(self, nmodel, nfilter, m, pool="max", hidden=32, loss="nll", dtype=torch.float32,
                  rate=0.01, momentum=0.9, decay_conv=0.0, decay_full=0.0, dropout=0.0,
                  weight_decay_start=100, nesterov=True, mode="fused", reverse_complement=False, input_dropout=0.0,
-                 device="cuda"):
+                 start_training=0, device="cuda"):
         assert pool in ("max", "avg", "all") and loss in ("nll", "mse", None)
         self.ninst, self.nfilter, self.m = int(nmodel), int(nfilter), int(m)
         self.pool, self.hidden, self.loss = pool, int(hidden), loss
@@ -48,6 +48,8 @@ class SequenceNet(object):
         # this probability; at test time the scan output is scaled by (1 - rate) instead
         # (reference: kangaroo/_ext/dropoutord.py:42-74, kangaroo/_ext/corr1ord.py:104-109)
         self.input_dropout = float(input_dropout)
+        # the scan filters' gradient is zeroed while step < start_training (reference: kangaroo/_ext/corr1ord.py:135-136)
+        self.start_training = int(start_training)
         self.step_count = 0
         ni, nf = self.ninst, self.nfilter
         self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
@@ -106,6 +108,45 @@ class SequenceNet(object):
             src = np.asarray(params[name])
             assert tuple(src.shape) == tuple(shape), "%s: expected %s, got %s" % (name, shape, src.shape)
             self.p[name].copy_(torch.as_tensor(src, dtype=self.dtype))
+
+    def init_params(self, init_conv=0.01, init_full=0.01, init_mu=0.0, seed=0):
+        """Random initial parameters the way the reference's trainer sets them up (deepity/deepity/sgd.py:333-352):
+        weights = randn * init (one scale per model, spread with madd_bcast), biases = init_mu.
+        init_conv / init_full / init_mu: scalar or one value per model. The normal deviates come from
+        the library's generator, so equal seeds give equal parameters."""
+        self.P.zero_()
+        offset = 0
+        for name, shape, axis in self.layout:
+            view = self.p[name]
+            flat = view.view(-1, 1)
+            per = view.numel() // self.ninst if axis == 0 else shape[1] // self.ninst      # block length of one model
+            if name.startswith("W"):
+                scale = self._vec(init_conv if name == "Wc" else init_full)
+                ds.madd_bcast(sm.randn(flat.shape[0], 1, dtype=self.dtype, seed=seed, offset=offset, device=self.device), scale, per, flat)
+                offset += (flat.shape[0] + 3) // 4
+            elif np.any(np.asarray(init_mu) != 0):
+                ds.madd_bcast(torch.ones_like(flat), self._vec(init_mu), per, flat)
+        self.mP.zero_()
+
+    def penalty_value(self):
+        """Per-model L1 weight cost (1 x ninst) that the reference adds to the reported loss once
+        step >= weight_decay_start: decay_conv * sum|Wc| + decay_full * (sum|W1| + sum|W2|).
+        (reference: kangaroo/_ext/corr1ord.py:111-115, deepity/std/full.py:92-109)"""
+        ni = self.ninst
+        if self.weight_decay_start > self.step_count:
+            return np.zeros((1, ni))
+        p = self.p
+        conv = sm.sum_axis0(sm.mul_sign(p["Wc"], p["Wc"]))                     # |W| summed over taps and channels
+        torch.cuda.synchronize()
+        cost = conv.cpu().numpy().astype(np.float64).reshape(ni, -1).sum(axis=1) * self.decay_conv.cpu().numpy().ravel()
+        for name in ("W1", "W2"):
+            if name in p:
+                absw = sm.mul_sign(p[name], p[name]).view(ni, -1)                # model-major rows: one row per model
+                ones = torch.ones((absw.shape[1], 1), dtype=self.dtype, device=self.device)
+                rows = sm.dot(absw.contiguous(), ones)
+                torch.cuda.synchronize()
+                cost = cost + rows.cpu().numpy().astype(np.float64).ravel() * self.decay_full.cpu().numpy().ravel()
+        return cost.reshape(1, ni)
 
     def get_params(self):
         torch.cuda.synchronize()
@@ -315,6 +356,8 @@ class SequenceNet(object):
             ks.corr1ord_bprop_W(g["Wc"], X, dZ0, 4)
         if self.weight_decay_start <= self.step_count:
             self._add_decay()
+        if self.step_count < self.start_training:
+            g["Wc"].zero_()
 
     def _add_decay(self):
         p, g, ni = self.p, self.g, self.ninst
@@ -344,6 +387,8 @@ class SequenceNet(object):
         ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, pooled, amax, dpooled, g["Wc"], g["bc"])
         if self.weight_decay_start <= self.step_count:
             self._add_decay()
+        if self.step_count < self.start_training:
+            g["Wc"].zero_()
         return Z
 
     # ------------------------------------------------------------------ one optimiser step
@@ -352,7 +397,8 @@ class SequenceNet(object):
         returns a function that replays it: for launch-bound batch sizes the step then costs one
         graph launch instead of ~10 kernel launches. Dropout masks stay fresh on every replay because
         the generator position lives in device memory. The graph bakes in whether L1 decay is
-        active, so it is re-captured when the step counter crosses weight_decay_start."""
+        active and whether the scan filters are still frozen, so it is re-captured when the step
+        counter crosses weight_decay_start or start_training."""
         return _graphed_step([(self, X, R, Y, Ymask)])
 
     def train_step(self, X, R, Y, Ymask=None, U=None, U_input=None):
@@ -392,7 +438,7 @@ def _graphed_step(jobs, streams=None):
     state = {"graph": None, "decay": None}
 
     def decay_flags():
-        return tuple(net.weight_decay_start <= net.step_count for net, *_ in jobs)
+        return tuple((net.weight_decay_start <= net.step_count, net.step_count < net.start_training) for net, *_ in jobs)
 
     def one(net, X, R, Y, Ymask):
         return lambda: ds.gradstep(net.P, net.dP, net.drate, net.mP, net.mrate,

@@ -29,6 +29,14 @@ def asarray(a, dtype=None, device="cuda"):
     return torch.as_tensor(a, dtype=dtype).to(device).contiguous()
 
 
+def randn(nrow, ncol, dtype=torch.float32, seed=0, offset=0, device="cuda"):
+    """(nrow x ncol) standard normal deviates from the library's counter-based generator at (seed, offset).
+    reference: smat.randn (cuRAND there; the streams differ, the distribution does not)"""
+    Z = torch.empty((nrow, ncol), dtype=dtype, device=device)
+    call("dbk_normal_fill", stream(), dtype_code(Z), ptr(Z), Z.numel(), int(seed), int(offset))
+    return Z
+
+
 def sync():
     call("dbk_sync", stream())
 

@@ -220,6 +220,10 @@ int dbk_dropout_bp_te(dbk_stream_t stream, int dtype, const void* dZ, const void
  * The reference draws from cuRAND's per-thread XORWOW states (smat_cuda/cuda_context.cpp:210-242),
  * which cannot be reproduced without the CUDA SDK; this generator is the library's own. */
 int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uint64_t offset);
+/* Standard normal deviates from the same generator (Box-Muller on two Philox streams, one value per
+ * element, element i depends only on (seed, offset, i)); used for the initial weights.
+ * reference: sm.randn in the parameter set-up, deepity/deepity/sgd.py:337-341 (cuRAND there) */
+int dbk_normal_fill(dbk_stream_t stream, int dtype, void* Z, size_t n, uint64_t seed, uint64_t offset);
 /* Host-side block function of that generator, for known-answer tests. */
 int dbk_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
 

@@ -551,7 +551,7 @@ PARAM_AXIS = {"Wc": 1, "bc": 1, "W1": 0, "b1": 1, "W2": 0, "b2": 1}
 
 
 def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum, Ymask=None, dropout=None,
-               decay_conv=0.0, decay_full=0.0, step=0, weight_decay_start=100, reverse_complement=False):
+               decay_conv=0.0, decay_full=0.0, step=0, weight_decay_start=100, reverse_complement=False, start_training=0):
     """Nesterov step in place on params / mom (dicts of arrays). dropout = (rates, U) or None."""
     names = [n for n in ("Wc", "bc", "W1", "b1", "W2", "b2") if n in params]
     eta = {n: _per_element(rate, params[n].shape, nmodel, PARAM_AXIS[n]).astype(params[n].dtype) for n in names}
@@ -573,9 +573,20 @@ def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum,
             if n in params:
                 Wn = params[n]
                 madd_bcast(sign(Wn), np.broadcast_to(np.asarray(decay_full, dtype=Wn.dtype), (nmodel,)), Wn.size // nmodel, g[n])
+    if start_training > step:
+        g["Wc"] = g["Wc"] * 0                                      # kangaroo/_ext/corr1ord.py:135-136
     for n in names:
         gradstep_nesterov2(params[n], g[n].astype(params[n].dtype), eta[n], mom[n], mu[n])
     return st, g
+
+
+def weight_cost(params, nmodel, decay_conv, decay_full):
+    """Per-model L1 cost added to the reported loss (kangaroo/_ext/corr1ord.py:111-115, deepity/std/full.py:92-109)."""
+    C = np.abs(params["Wc"]).sum(axis=0).reshape((nmodel, -1)).sum(axis=1) * np.broadcast_to(decay_conv, (nmodel,))
+    for n in ("W1", "W2"):
+        if n in params:
+            C = C + np.abs(params[n]).reshape((nmodel, -1)).sum(axis=1) * np.broadcast_to(decay_full, (nmodel,))
+    return C.reshape(1, nmodel)
 
 
 # ----------------------------------------------------------------------------------------------

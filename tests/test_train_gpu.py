@@ -405,3 +405,46 @@ def test_training_from_a_sequence_file_reduces_the_loss(tmp_path):
     neg = [z for z, y in auc_pairs if y == 0]
     auc = np.mean([p > q for p in pos for q in neg])
     assert auc > 0.9, auc
+
+
+def test_init_params_penalty_and_frozen_filters():
+    """Trainer set-up pieces: randn * per-model scale (+ bias shift), the L1 cost added to the reported loss,
+    and the scan filters staying frozen while step < start_training."""
+    from deepbind_amd import smat, synth
+    from deepbind_amd.model import SequenceNet
+    Zn = host(smat.randn(1 << 18, 1, seed=3))
+    assert abs(Zn.mean()) < 0.01 and abs(Zn.std() - 1.0) < 0.01 and abs((Zn ** 4).mean() - 3.0) < 0.1
+    assert np.array_equal(Zn, host(smat.randn(1 << 18, 1, seed=3))) and not np.array_equal(Zn, host(smat.randn(1 << 18, 1, seed=4)))
+    assert host(smat.randn(64, 2, dtype=torch.float64, seed=3)).dtype == np.float64
+
+    cfg = synth.config3()
+    spec = cfg["spec"]
+    ni = 6
+    scales = np.array([0.01, 0.02, 0.04, 0.08, 0.16, 0.32])
+    net = SequenceNet(ni, spec.nfilter, spec.m, pool="max", hidden=32, loss="nll", rate=0.05, momentum=0.9,
+                      decay_conv=np.linspace(1e-4, 6e-4, ni), decay_full=np.linspace(1e-3, 6e-3, ni), weight_decay_start=1,
+                      start_training=2)
+    net.init_params(init_conv=scales, init_full=2 * scales, init_mu=0.5, seed=11)
+    p = net.get_params()
+    for b in range(ni):
+        assert abs(p["Wc"][:, 16 * b:16 * (b + 1)].std() / scales[b] - 1) < 0.1
+        assert abs(p["W1"][16 * b:16 * (b + 1)].std() / (2 * scales[b]) - 1) < 0.15
+        assert abs(p["W2"][32 * b:32 * (b + 1)].std() / (2 * scales[b]) - 1) < 0.5
+    assert np.all(p["bc"] == 0.5) and np.all(p["b1"] == 0.5) and np.all(p["b2"] == 0.5)
+    # cost: zero before weight_decay_start, the per-model L1 sums after
+    assert np.all(net.penalty_value() == 0)
+    X, R = dev(cfg["X"]), dev(cfg["R"])
+    Y = dev(np.repeat(cfg["Y"], ni, axis=1))
+    ref_p, ref_m = _f64(p), {k: np.zeros(v.shape) for k, v in p.items()}
+    for step in range(3):
+        before = net.get_params()["Wc"]
+        net.train_step(X, R, Y)
+        orc.train_step(ref_p, ref_m, cfg["X"], cfg["R"], np.repeat(cfg["Y"], ni, axis=1).astype(np.float64), ni, "max", 32, "nll",
+                       0.05, 0.9, decay_conv=np.linspace(1e-4, 6e-4, ni), decay_full=np.linspace(1e-3, 6e-3, ni), step=step,
+                       weight_decay_start=1, start_training=2)
+        after = net.get_params()
+        assert np.array_equal(before, after["Wc"]) == (step < 2), "filters frozen exactly while step < start_training (step %d)" % step
+        for k in ref_p:
+            assert_close(after[k], ref_p[k], GRAD, "step %d %s" % (step, k))
+    want = orc.weight_cost(_f64(net.get_params()), ni, np.linspace(1e-4, 6e-4, ni), np.linspace(1e-3, 6e-3, ni))
+    assert_close(net.penalty_value(), want, ACT, "L1 cost")
