@@ -84,8 +84,10 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
                                               const float* __restrict__ b1, const float* __restrict__ W2,
                                               const float* __restrict__ b2, bool apply_logistic, float* __restrict__ scores)
 {
-    extern __shared__ float hsm[];
-    const unsigned b = blockIdx.y;
+    extern __shared__ __align__(16) float hsm[];
+    // models vary fastest over the grid: the workgroups that share a tile of rows run together, so each
+    // 4 KB row of the feature matrix is pulled from HBM once and served to its 64 models from L2
+    const unsigned b = blockIdx.x;
     const int h1 = hidden > 0 ? hidden : 1;
     float* w1s = hsm;                       // [k][h1]
     float* b1s = w1s + (size_t)k * h1;      // [h1]
@@ -96,7 +98,7 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
     __syncthreads();
     const float sc = in_scale ? in_scale[b] : 1.0f;
     const float bias2 = hidden > 0 ? b2[b] : 0.0f;
-    for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n; r += (size_t)gridDim.x * blockDim.x) {
+    for (size_t r = (size_t)blockIdx.y * blockDim.x + threadIdx.x; r < n; r += (size_t)gridDim.y * blockDim.x) {
         const float* x = pooled + r * (size_t)k * nblock + (size_t)b * k;
         float xr[KMAX];
 #pragma unroll
@@ -104,7 +106,32 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
         float out;
         if (hidden > 0) {
             out = 0.0f;
-            for (int h = 0; h < hidden; ++h) {
+            int h = 0;
+            // four hidden units at a time: one 16-byte broadcast read of LDS feeds four multiply-adds
+            // (hidden % 4 == 0 keeps the reads aligned; taps ascending per unit, units ascending in the output sum)
+            if ((hidden & 3) == 0) {
+                for (; h < hidden; h += 4) {
+                    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+#pragma unroll
+                    for (int kk = 0; kk < KMAX; ++kk)
+                        if (kk < k) {
+                            const float4 w = *reinterpret_cast<const float4*>(w1s + kk * hidden + h);
+                            // fused multiply-add, as the reference's GEMM library issues them
+                            a0 = __builtin_fmaf(xr[kk], w.x, a0);
+                            a1 = __builtin_fmaf(xr[kk], w.y, a1);
+                            a2 = __builtin_fmaf(xr[kk], w.z, a2);
+                            a3 = __builtin_fmaf(xr[kk], w.w, a3);
+                        }
+                    const float4 bb = *reinterpret_cast<const float4*>(b1s + h);
+                    const float4 ww = *reinterpret_cast<const float4*>(w2s + h);
+                    a0 += bb.x; a1 += bb.y; a2 += bb.z; a3 += bb.w;
+                    out += (a0 > 0.0f ? a0 : 0.0f) * ww.x;
+                    out += (a1 > 0.0f ? a1 : 0.0f) * ww.y;
+                    out += (a2 > 0.0f ? a2 : 0.0f) * ww.z;
+                    out += (a3 > 0.0f ? a3 : 0.0f) * ww.w;
+                }
+            }
+            for (; h < hidden; ++h) {
                 float a = 0.0f;
 #pragma unroll
                 for (int kk = 0; kk < KMAX; ++kk)
@@ -123,6 +150,83 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
         }
         if (apply_logistic) out = 1.0f / (1.0f + expf(-out));
         scores[r * (size_t)nblock + b] = out;
+    }
+}
+
+// Scoring head, coalesced variant for hidden % 4 == 0: a workgroup owns 16 consecutive models and a tile of
+// 16 rows per pass; lane = (row, model) with the model fastest, so a wave's reads of the feature matrix
+// cover four contiguous 16*k*4-byte row segments. The 16 models' first-layer weights sit in LDS as
+// [input][hidden/4][model][4]: the 16 lanes of a row read one aligned 256-byte line per ds_read_b128,
+// and the four rows of a wave read the same line.
+constexpr int HG = 16;
+template <int KMAX>
+__global__ __launch_bounds__(256) void k_head16(size_t n, int nblock, int k, int hidden, const float* __restrict__ pooled,
+                                                const float* __restrict__ in_scale, const float* __restrict__ W1,
+                                                const float* __restrict__ b1, const float* __restrict__ W2,
+                                                const float* __restrict__ b2, bool apply_logistic, float* __restrict__ scores)
+{
+    extern __shared__ __align__(16) float hsm[];
+    const int hq = hidden >> 2;
+    float* w1s = hsm;                                   // [k][hq][HG][4]
+    float* b1s = w1s + (size_t)k * hidden * HG;         // [hq][HG][4]
+    float* w2s = b1s + (size_t)hidden * HG;             // [hq][HG][4]
+    const unsigned g = threadIdx.x & (HG - 1), rl = threadIdx.x >> 4;
+    const unsigned m0 = blockIdx.x * HG;                // first model of this workgroup
+    for (int e = threadIdx.x; e < k * hidden * HG; e += blockDim.x) {
+        // destination order: e = ((kk*hq + h4)*HG + gg)*4 + c
+        const int c = e & 3, gg = (e >> 2) & (HG - 1), rest = e >> 6, h4 = rest % hq, kk = rest / hq;
+        const unsigned mdl = m0 + gg;
+        w1s[e] = mdl < (unsigned)nblock ? W1[((size_t)mdl * k + kk) * hidden + h4 * 4 + c] : 0.0f;
+    }
+    for (int e = threadIdx.x; e < hidden * HG; e += blockDim.x) {
+        const int c = e & 3, gg = (e >> 2) & (HG - 1), h4 = e >> 6;
+        const unsigned mdl = m0 + gg;
+        b1s[e] = mdl < (unsigned)nblock ? b1[(size_t)mdl * hidden + h4 * 4 + c] : 0.0f;
+        w2s[e] = mdl < (unsigned)nblock ? W2[(size_t)mdl * hidden + h4 * 4 + c] : 0.0f;
+    }
+    __syncthreads();
+    const unsigned mdl = m0 + g;
+    const bool live = mdl < (unsigned)nblock;
+    const float sc = (in_scale && live) ? in_scale[mdl] : 1.0f;
+    const float bias2 = live ? b2[mdl] : 0.0f;
+    const float4* w1v = reinterpret_cast<const float4*>(w1s) + g;
+    const float4* b1v = reinterpret_cast<const float4*>(b1s) + g;
+    const float4* w2v = reinterpret_cast<const float4*>(w2s) + g;
+    if (!live) return;                                   // (after the only barrier)
+    const size_t rstep = (size_t)gridDim.y * 16, rowlen = (size_t)k * nblock;
+    size_t r = (size_t)blockIdx.y * 16 + rl;
+    float xn[KMAX];                                      // next row's inputs, fetched while this row is computed
+#pragma unroll
+    for (int kk = 0; kk < KMAX; ++kk) xn[kk] = (kk < k && r < n) ? pooled[r * rowlen + (size_t)mdl * k + kk] : 0.0f;
+    for (; r < n; r += rstep) {
+        float xr[KMAX];
+#pragma unroll
+        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = xn[kk] * sc;
+        const size_t rn = r + rstep;
+#pragma unroll
+        for (int kk = 0; kk < KMAX; ++kk) xn[kk] = (kk < k && rn < n) ? pooled[rn * rowlen + (size_t)mdl * k + kk] : 0.0f;
+        float out = 0.0f;
+        for (int h4 = 0; h4 < hq; ++h4) {
+            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+#pragma unroll
+            for (int kk = 0; kk < KMAX; ++kk)
+                if (kk < k) {
+                    const float4 w = w1v[(kk * hq + h4) * HG];
+                    a0 = __builtin_fmaf(xr[kk], w.x, a0);
+                    a1 = __builtin_fmaf(xr[kk], w.y, a1);
+                    a2 = __builtin_fmaf(xr[kk], w.z, a2);
+                    a3 = __builtin_fmaf(xr[kk], w.w, a3);
+                }
+            const float4 bb = b1v[h4 * HG], ww = w2v[h4 * HG];
+            a0 += bb.x; a1 += bb.y; a2 += bb.z; a3 += bb.w;
+            out += (a0 > 0.0f ? a0 : 0.0f) * ww.x;
+            out += (a1 > 0.0f ? a1 : 0.0f) * ww.y;
+            out += (a2 > 0.0f ? a2 : 0.0f) * ww.z;
+            out += (a3 > 0.0f ? a3 : 0.0f) * ww.w;
+        }
+        out += bias2;
+        if (apply_logistic) out = 1.0f / (1.0f + expf(-out));
+        scores[r * (size_t)nblock + mdl] = out;
     }
 }
 
@@ -219,14 +323,24 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
     DBK_CHECK(pooled && W1 && b1 && scores, "ValueError: null pointer argument");
     DBK_CHECK(hidden == 0 || (W2 && b2), "ValueError: hidden layer requested but W2/b2 are null");
     DBK_CHECK(k <= HEAD_MAXK, "ValueError: the fused head takes at most %d inputs per model (got %d)", HEAD_MAXK, k);
-    DBK_CHECK(nblock <= 65535, "ValueError: too many models (%d) for one launch", nblock);
     const int h1 = hidden > 0 ? hidden : 1;
     size_t smem = ((size_t)k * h1 + h1 + hidden) * sizeof(float);
     DBK_CHECK(smem <= 65536, "ValueError: head weights (%zu bytes per model) do not fit in LDS", smem);
     unsigned gx = dbk::divup(n, 256);
     if (gx > 2048u) gx = 2048u;
+    const size_t smem16 = ((size_t)k * hidden + 2 * (size_t)hidden) * HG * sizeof(float);
+    if (hidden > 0 && (hidden & 3) == 0 && smem16 <= 65536 && n >= 4096) {
+        // bulk scoring: 16 models per workgroup, coalesced reads of the feature matrix
+        unsigned gy = dbk::divup(n, 16 * 32);                // each workgroup makes ~32 passes with its staged weights
+        if (gy > 65535u) gy = 65535u;
+        auto kern16 = k <= 16 ? k_head16<16> : (k <= 32 ? k_head16<32> : k_head16<64>);
+        DBK_HIP(hipFuncSetAttribute((const void*)kern16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem16));
+        hipLaunchKernelGGL(kern16, dim3(dbk::divup(nblock, HG), gy), dim3(256), smem16, dbk::as_stream(stream), n, nblock, k, hidden, pooled,
+                           in_scale, W1, b1, W2, b2, apply_logistic != 0, scores);
+        DBK_LAUNCH_OK();
+    }
     auto kern = k <= 16 ? k_head<16> : (k <= 32 ? k_head<32> : k_head<64>);
-    hipLaunchKernelGGL(kern, dim3(gx, nblock), dim3(256), smem, dbk::as_stream(stream), n, nblock, k, hidden, pooled, in_scale,
+    hipLaunchKernelGGL(kern, dim3(nblock, gx), dim3(256), smem, dbk::as_stream(stream), n, nblock, k, hidden, pooled, in_scale,
                        W1, b1, W2, b2, apply_logistic != 0, scores);
     DBK_LAUNCH_OK();
 }

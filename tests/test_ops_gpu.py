@@ -289,6 +289,21 @@ def test_head_fprop(ds):
     assert_close(host(got0), ref0, ACT, "scores (no hidden)")
 
 
+@pytest.mark.parametrize("k,h,nb", [(16, 32, 37), (32, 8, 16), (16, 64, 5)])
+def test_head_fprop_bulk_rows(ds, k, h, nb):
+    """Row counts that take the 16-models-per-workgroup kernel; model count not a multiple of 16; dropout rescale."""
+    rng = np.random.default_rng(40 + k + h)
+    n = 5001
+    Pl = np.abs(rng.standard_normal((n, k * nb))).astype(np.float32)
+    W1 = (rng.standard_normal((k * nb, h)) * 0.3).astype(np.float32); b1 = (rng.standard_normal((1, h * nb)) * 0.1).astype(np.float32)
+    W2 = (rng.standard_normal((h * nb, 1)) * 0.3).astype(np.float32); b2 = (rng.standard_normal((1, nb)) * 0.1).astype(np.float32)
+    rate = rng.choice([0.0, 0.25, 0.5], size=nb).astype(np.float32)
+    H = orc.relu_fprop(orc.bias_fprop(orc.blockwise_dot(orc.dropout_fp_test(Pl, rate), W1, nb), b1))
+    ref = orc.logistic(orc.bias_fprop(orc.blockwise_dot(H, W2, nb), b2))
+    got = ds.head_fprop(dev(Pl), dev(W1), dev(b1), dev(W2), dev(b2), nblock=nb, in_scale=1 - rate, apply_logistic=True)
+    assert_close(host(got), ref, ACT, "probabilities")
+
+
 # ------------------------------------------------------------------------------------------ elementwise / optimiser
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_gradstep_and_madd_bcast(ds, dtype):
