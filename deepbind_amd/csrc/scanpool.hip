@@ -283,31 +283,39 @@ __global__ __launch_bounds__(256) void scanpool_bprop_kernel(const float* __rest
     }
 }
 
-// Adds g at (tap j, letter of X[i+j]) for j < m into this lane's column of a [tap][channel][FT] table.
-// Taps are handled eight at a time with all LDS reads issued before the writes (distinct taps are
-// distinct cells), so a position costs two LDS round trips per eight taps instead of sixteen.
-__device__ __forceinline__ void add_position(float* mine, const uint8_t* __restrict__ xs, unsigned m, float g)
+// For up to four positions i_u with gradients g_u: adds g_u at (tap j, letter of X[i_u+j]) for j < m into
+// this lane's column of a [tap][channel][FT] table. Taps go eight at a time: the letters of all four
+// positions are loaded first (32 independent global loads in flight), then each position's eight cells
+// are read, updated and written (distinct taps are distinct cells), positions in ascending order.
+__device__ __forceinline__ void add_positions4(float* mine, const uint8_t* __restrict__ X, const size_t (&pos)[4],
+                                               const float (&g)[4], const bool (&on)[4], unsigned m)
 {
-    const float gq = g * 0.25f;
     for (unsigned j0 = 0; j0 < m; j0 += 8) {
-        unsigned l[8];
-        float v[8];
+        unsigned l[4][8];
 #pragma unroll
-        for (unsigned t = 0; t < 8; ++t) l[t] = j0 + t < m ? letter_of(xs[j0 + t]) : 5u;
+        for (int u = 0; u < 4; ++u) {
 #pragma unroll
-        for (unsigned t = 0; t < 8; ++t) v[t] = l[t] < 4u ? mine[((j0 + t) * 4 + l[t]) * FT] : 0.0f;
+            for (unsigned t = 0; t < 8; ++t) l[u][t] = (on[u] && j0 + t < m) ? letter_of(X[pos[u] + j0 + t]) : 5u;
+        }
 #pragma unroll
-        for (unsigned t = 0; t < 8; ++t)
-            if (l[t] < 4u) mine[((j0 + t) * 4 + l[t]) * FT] = v[t] + g;
+        for (int u = 0; u < 4; ++u) {
+            const float gu = g[u], gq = gu * 0.25f;
+            float v[8];
 #pragma unroll
-        for (unsigned t = 0; t < 8; ++t)
-            if (l[t] == 4u) {
-                float* cell = mine + (size_t)(j0 + t) * 4 * FT;
-                cell[0 * FT] += gq;
-                cell[1 * FT] += gq;
-                cell[2 * FT] += gq;
-                cell[3 * FT] += gq;
-            }
+            for (unsigned t = 0; t < 8; ++t) v[t] = l[u][t] < 4u ? mine[((j0 + t) * 4 + l[u][t]) * FT] : 0.0f;
+#pragma unroll
+            for (unsigned t = 0; t < 8; ++t)
+                if (l[u][t] < 4u) mine[((j0 + t) * 4 + l[u][t]) * FT] = v[t] + gu;
+#pragma unroll
+            for (unsigned t = 0; t < 8; ++t)
+                if (l[u][t] == 4u) {
+                    float* cell = mine + (size_t)(j0 + t) * 4 * FT;
+                    cell[0 * FT] += gq;
+                    cell[1 * FT] += gq;
+                    cell[2 * FT] += gq;
+                    cell[3 * FT] += gq;
+                }
+        }
     }
 }
 
@@ -348,13 +356,13 @@ __global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, u
                     g[u] = pv > 0.0f ? gd : 0.0f;
                 }
             }
+            bool on[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                if (g[u] != 0.0f) {
-                    db += g[u];
-                    if (pos[u] < n) add_position(mine, X + pos[u], m, g[u]);
-                }
+                if (g[u] != 0.0f) db += g[u];
+                on[u] = g[u] != 0.0f && pos[u] < n;
             }
+            add_positions4(mine, X, pos, g, on, m);
         }
         float* out = slabs + (size_t)blockIdx.x * stride;
         for (unsigned row = 0; row < 4 * m; ++row) out[(size_t)row * F + f] = mine[row * FT];
