@@ -661,15 +661,17 @@ int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, s
     using namespace dbk_scanpool_general;
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
-    DBK_CHECK(ptype == DBK_PT_AVG || argmax != nullptr, "ValueError: pooledmaps_argmax must be specified for max pooling.");
     if (nfilter == 0) { dbk::clear_error(); return 0; }
-    DBK_CHECK(W && bias && X && dW && dbias, "ValueError: null pointer argument");
+    DBK_CHECK(W && bias && dW && dbias, "ValueError: null pointer argument");
     if (nregion == 0) {
-        DBK_HIP(hipMemsetAsync(dbias, 0, nfilter * sizeof(float), dbk::as_stream(stream)));
-        dbk::clear_error();
-        return 0;
+        // no regions: the bias gradient is written as zero by the slab reduction over zero slabs
+        // (a kernel rather than a memset, so that the call can sit in a captured graph)
+        hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(nfilter)), dim3(256), 0, dbk::as_stream(stream), dW, dbias,
+                           (const float*)nullptr, (size_t)0, nfilter, 0u);
+        DBK_LAUNCH_OK();
     }
-    DBK_CHECK(regions && pooled && dpooled, "ValueError: null pointer argument");
+    DBK_CHECK(ptype == DBK_PT_AVG || argmax != nullptr, "ValueError: pooledmaps_argmax must be specified for max pooling.");
+    DBK_CHECK(X && regions && pooled && dpooled, "ValueError: null pointer argument");
     hipStream_t st = dbk::as_stream(stream);
     switch (ptype) {
     case DBK_PT_MAX: return launch_bprop_pt<DBK_PT_MAX>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias);

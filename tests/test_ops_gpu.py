@@ -450,3 +450,45 @@ def test_scanpool_kmer_regions_in_any_order(ks, B, lo, hi, m, F):
     perm = rng.permutation(B)
     P2, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R[perm]), "max", path="kmer")
     assert_close(host(P2), Pr[perm], ACT, "shuffled order")
+
+
+# ------------------------------------------------------------------------------------------ empty and degenerate inputs
+def test_empty_and_degenerate_inputs(ks, ds):
+    """Zero regions, streams shorter than the filter, zero rows: every entry point must
+    return the defined (empty or all-padding) result without touching memory it does not own."""
+    rng = np.random.default_rng(12)
+    m, F = 6, 20
+    W = (rng.standard_normal((4 * m, F)) * 0.3).astype(np.float32)
+    b = (rng.standard_normal((1, F)) * 0.3).astype(np.float32)
+    Wd, bd = dev(W), dev(b)
+    # no regions at all
+    X = random_codes(rng, 40, 0.1)
+    R0 = np.zeros((0, 2), np.uint32)
+    for ptype in ("max", "avg", "all"):
+        P, I = ks.scanpool_fprop(Wd, bd, dev(X), dev(R0), ptype, want_argmax=(ptype != "avg"))
+        assert P.shape == (0, F * (2 if ptype == "all" else 1))
+        dW, db = dev(np.ones_like(W)), dev(np.full_like(b, 5.0))
+        ks.scanpool_bprop(Wd, bd, dev(X), dev(R0), ptype, P, I, torch.zeros_like(P), dW, db)
+        assert np.array_equal(host(dW), np.ones_like(W)) and np.array_equal(host(db), np.zeros_like(b))
+    # a stream shorter than the filter: the scan defines no row, every row of the map is relu(bias)
+    Xs = random_codes(rng, m - 2, 0.0)
+    Rs = np.array([[0, m - 2]], np.uint32)
+    A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), Xs, Rs, "all")
+    P, I = ks.scanpool_fprop(Wd, bd, dev(Xs), dev(Rs), "all", want_argmax=True)
+    assert_close(host(P), Pr, ACT, "short stream")
+    assert np.array_equal(host(I), Ir)
+    Z = dev(np.full((m - 2, F), 3.0, np.float32))
+    ks.corr1ord(Wd, dev(Xs), Z, 4)
+    assert np.array_equal(host(Z), np.full((m - 2, F), 3.0, np.float32))        # rows >= n are left untouched
+    # (zero-length regions are outside the reference's domain: its kernels read the region's first row
+    # unconditionally, poolrgn.cuh:64-66, and the batcher never produces one; not tested)
+    # zero rows through the dense head and the elementwise ops
+    e = torch.zeros((0, 16 * 3), dtype=torch.float32, device="cuda")
+    W1 = dev(rng.standard_normal((48, 8)).astype(np.float32)); b1 = dev(np.zeros((1, 24), np.float32))
+    W2 = dev(rng.standard_normal((24, 1)).astype(np.float32)); b2 = dev(np.zeros((1, 3), np.float32))
+    assert ds.head_fprop(e, W1, b1, W2, b2, nblock=3).shape == (0, 3)
+    assert ds.blockwise_dot(e, W1, 3).shape == (0, 24)
+    Zd, Md = ds.dropout_fp_train(e, dev(np.full(3, 0.5, np.float32)), False)
+    assert Zd.shape == e.shape and Md.shape == e.shape
+    Ze, Me = ks.dropoutord_fp_train(torch.zeros((0, 1), dtype=torch.uint8, device="cuda"), 0.5)
+    assert Ze.numel() == 0 and Me.numel() == 0
