@@ -635,6 +635,9 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream, const float* W, const float*
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
+    // argmax entries are flat 32-bit indices row*nfilter + f into the (virtual) map, as in the reference (uindex_t)
+    DBK_CHECK(!argmax || (double)N * (double)nfilter <= 4294967296.0,
+              "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
     return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr);
@@ -647,6 +650,9 @@ int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, s
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
+    // argmax entries are flat 32-bit indices row*nfilter + f into the (virtual) map, as in the reference (uindex_t)
+    DBK_CHECK(!argmax || (double)N * (double)nfilter <= 4294967296.0,
+              "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
     int rc = dbk_scanpool_kmer::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax);

@@ -492,3 +492,40 @@ def test_empty_and_degenerate_inputs(ks, ds):
     assert Zd.shape == e.shape and Md.shape == e.shape
     Ze, Me = ks.dropoutord_fp_train(torch.zeros((0, 1), dtype=torch.uint8, device="cuda"), 0.5)
     assert Ze.numel() == 0 and Me.numel() == 0
+
+
+@pytest.mark.parametrize("ptype", ["max", "all"])
+def test_scanpool_extreme_shapes(ks, ptype):
+    """One very long region (a chromosome-scale scan: many staging chunks per region) and very many one-letter
+    regions in the same call, against the plain-C oracle; forward on every path and the fused backward."""
+    from oracle import oracle_c
+    rng = np.random.default_rng(77)
+    m, F = 24, 40
+    lens = [150001] + [1] * 20000 + [3000] + [2] * 5000
+    ords = [rng.integers(0, 4, L, dtype=np.uint8) for L in lens]
+    for o in ords[:3]:
+        o[rng.random(o.size) < 0.01] = 255
+    from deepbind_amd import data
+    X, R = data.pack_ordinals(ords, m - 1)
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
+    b = (rng.standard_normal((1, F)) * 0.1).astype(np.float32)
+    pt = {"max": 0, "all": 3}[ptype]
+    Pr, Ir = oracle_c.scanpool(W, b, X, R, pt, want_argmax=True)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True)
+    assert_close(host(P), Pr, ACT, "pooled (general, argmax)")
+    same = host(I) == Ir
+    assert same.mean() > 0.999                                       # the rest are float32 round-off ties between rows
+    if ptype == "max":
+        Pk, _ = ks.scanpool_fprop(Wd, bd, Xd, Rd, "max", path="kmer")
+        assert_close(host(Pk), Pr, ACT, "pooled (table kernel)")
+    # backward: linear in dpooled, so two calls with g and 2g must give dW2 = 2 dW1 (bit-exact) and run-to-run identical
+    dP = dev(rng.standard_normal(Pr.shape).astype(np.float32))
+    outs = []
+    for scale in (1.0, 2.0, 1.0):
+        dW, db = dev(np.zeros_like(W)), dev(np.zeros_like(b))
+        ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P, I, dP * scale, dW, db)
+        outs.append((host(dW), host(db)))
+    assert np.array_equal(outs[0][0], outs[2][0]) and np.array_equal(outs[0][1], outs[2][1])
+    assert np.array_equal(outs[1][0], 2 * outs[0][0]) and np.array_equal(outs[1][1], 2 * outs[0][1])
+    assert np.isfinite(outs[0][0]).all() and np.abs(outs[0][0]).max() > 0
