@@ -40,7 +40,7 @@ _SIGNATURES = {
     "dbk_scanpool_fprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
     "dbk_scanpool_fprop_general": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
     "dbk_scanpool_fprop_kmer": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
-    "dbk_scanpool_bprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P, _P, _P],
+    "dbk_scanpool_bprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P, _P, _P, _I],
     "dbk_blockwise_dot": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
     "dbk_blockwise_dot_nt": [_P, _I, _I, _I, _I, _I, _P, _P, _P],
     "dbk_blockwise_dot_tn": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
@@ -70,8 +70,9 @@ _SIGNATURES = {
     "dbk_logistic": [_P, _I, _P, _P, _Z],
     "dbk_loss_terms": [_P, _I, _I, _P, _P, _P, _Z],
     "dbk_sub_scale": [_P, _I, _P, _P, _D, _P, _Z],
-    "dbk_head_train": [_P, _Z, _I, _I, _I, _I, _I, _P, _P, _P, _U64, _U64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
+    "dbk_head_train": [_P, _Z, _I, _I, _I, _I, _I, _P, _P, _P, _U64, _U64, _P, _U64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "dbk_counter_add": [_P, _P, _U64],
+    "dbk_l1_decay": [_P, _I, _P, _P, _P, _Z],
     "dbk_head_fprop": [_P, _Z, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
 }
 

@@ -180,6 +180,14 @@ __global__ void k_uniform_fill(float* U, size_t n, uint64_t seed, uint64_t offse
 }
 // Standard normals by Box-Muller from two independent Philox streams (third counter word 0 / 1), one value
 // per element so that element i depends only on (seed, offset, i).
+template <typename T> __global__ void k_l1_decay(const T* P, const T* decay, T* dP, size_t n)
+{
+    GRID_STRIDE(i, n) {
+        const T w = P[i];
+        const T sg = (T)((w > (T)0) - (w < (T)0));
+        dP[i] += sg * decay[i];
+    }
+}
 template <typename T> __global__ void k_normal_fill(T* Z, size_t n, uint64_t seed, uint64_t offset)
 {
     GRID_STRIDE(i, n) {
@@ -361,6 +369,18 @@ int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uin
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(U != nullptr, "ValueError: U must not be null");
     hipLaunchKernelGGL(k_uniform_fill, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), U, n, seed, offset);
+    DBK_LAUNCH_OK();
+}
+
+int dbk_l1_decay(dbk_stream_t stream, int dtype, const void* P, const void* decay, void* dP, size_t n)
+{
+    DBK_CHECK(dtype == DBK_F32 || dtype == DBK_F64, "TypeError: dtype must be float32 or float64");
+    if (n == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(P && decay && dP, "ValueError: null pointer argument");
+    if (dtype == DBK_F32)
+        hipLaunchKernelGGL(k_l1_decay<float>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), (const float*)P, (const float*)decay, (float*)dP, n);
+    else
+        hipLaunchKernelGGL(k_l1_decay<double>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), (const double*)P, (const double*)decay, (double*)dP, n);
     DBK_LAUNCH_OK();
 }
 

@@ -27,7 +27,8 @@ struct head_args {
     int nblock, k, hidden, loss_kind, revcomp;
     const float *pooled, *rate, *U;
     unsigned long long seed, offset;
-    const unsigned long long* counter;
+    unsigned long long* counter;
+    unsigned long long counter_advance;
     const float *W1, *b1, *W2, *b2, *Y;
     const uint8_t* Ymask;
     float *Z, *dpooled, *dW1, *db1, *dW2, *db2, *loss;
@@ -204,13 +205,15 @@ __global__ void k_head_reduce(head_args a)
         else if (idx == nW1 + 2 * h1) { if (hidden > 0) a.db2[b] = s; }
         else if (a.loss) a.loss[b] = a.loss_kind == 0 ? -s / (float)a.n : 0.5f * s / (float)a.n;
     }
+    // every workgroup of the forward/backward kernel has read the generator position by now: move it on
+    if (a.counter && a.counter_advance && blockIdx.x == 0 && threadIdx.x == 0) a.counter[0] += a.counter_advance;
 }
 
 }  // namespace
 
 extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden, int loss_kind, int reverse_complement,
                               const float* pooled, const float* rate, const float* U, uint64_t seed, uint64_t offset,
-                              const uint64_t* counter,
+                              uint64_t* counter, uint64_t counter_advance,
                               const float* W1, const float* b1, const float* W2, const float* b2,
                               const float* Y, const uint8_t* Ymask,
                               float* Z, float* dpooled, float* dW1, float* db1, float* dW2, float* db2, float* loss)
@@ -228,7 +231,7 @@ extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, 
     DBK_CHECK(nchunk <= 65535, "ValueError: the fused head takes at most %d rows per call (got %zu)", 65535 * RB, n);
     head_args a;
     a.n = n; a.nblock = nblock; a.k = k; a.hidden = hidden; a.loss_kind = loss_kind; a.revcomp = reverse_complement;
-    a.pooled = pooled; a.rate = rate; a.U = U; a.seed = seed; a.offset = offset; a.counter = (const unsigned long long*)counter;
+    a.pooled = pooled; a.rate = rate; a.U = U; a.seed = seed; a.offset = offset; a.counter = (unsigned long long*)counter; a.counter_advance = counter_advance;
     a.W1 = W1; a.b1 = b1; a.W2 = W2; a.b2 = b2; a.Y = Y; a.Ymask = Ymask;
     a.Z = Z; a.dpooled = dpooled; a.dW1 = dW1; a.db1 = db1; a.dW2 = dW2; a.db2 = db2; a.loss = loss;
     a.nchunk = (unsigned)nchunk;

@@ -477,9 +477,10 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
     }
 }
 
-// Fixed-shape tree sum over slabs of nW + nB entries each: dW[e] += total for e < nW, dbias[e - nW] = total after that.
+// Fixed-shape tree sum over slabs of nW + nB entries each: dW[e] += total (or = total with overwrite) for e < nW,
+// dbias[e - nW] = total after that.
 __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ dbias, const float* __restrict__ slabs,
-                                    size_t nW, size_t nB, unsigned nslab)
+                                    size_t nW, size_t nB, unsigned nslab, bool overwrite)
 {
     const size_t nelem = nW + nB;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < nelem; e += (size_t)gridDim.x * blockDim.x) {
@@ -489,7 +490,7 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
             for (unsigned s = 0; s < 8; ++s) buf[s] = base + s < nslab ? slabs[(size_t)(base + s) * nelem + e] : 0.0f;
             total += ((buf[0] + buf[1]) + (buf[2] + buf[3])) + ((buf[4] + buf[5]) + (buf[6] + buf[7]));
         }
-        if (e < nW) dW[e] += total;
+        if (e < nW) dW[e] = overwrite ? total : dW[e] + total;
         else dbias[e - nW] = total;
     }
 }
@@ -548,7 +549,7 @@ void launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, con
 template <int PT>
 int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                     const uint32_t* R, size_t P, const float* pooled, const uint32_t* argmax, const float* dpooled,
-                    float* dW, float* dbias)
+                    float* dW, float* dbias, bool overwrite)
 {
     const unsigned ftiles = dbk::divup(F, FT);
     DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
@@ -571,7 +572,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P,
                            pooled, argmax, dpooled, slabs, stride);
-        hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gx);
+        hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gx, overwrite);
         DBK_LAUNCH_OK();
     }
     // sparse half: ~2048 single-wave workgroups, at least four regions each
@@ -604,7 +605,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         else if (mt == 16) launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
         else launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
     }
-    hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd);
+    hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd, overwrite);
     DBK_LAUNCH_OK();
 }
 
@@ -662,7 +663,7 @@ int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, s
 
 int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
                        const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
-                       const float* pooled, const uint32_t* argmax, const float* dpooled, float* dW, float* dbias)
+                       const float* pooled, const uint32_t* argmax, const float* dpooled, float* dW, float* dbias, int overwrite)
 {
     using namespace dbk_scanpool_general;
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
@@ -673,16 +674,16 @@ int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, s
         // no regions: the bias gradient is written as zero by the slab reduction over zero slabs
         // (a kernel rather than a memset, so that the call can sit in a captured graph)
         hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(nfilter)), dim3(256), 0, dbk::as_stream(stream), dW, dbias,
-                           (const float*)nullptr, (size_t)0, nfilter, 0u);
+                           (const float*)nullptr, (size_t)(overwrite ? 4 * m * nfilter : 0), nfilter, 0u, overwrite != 0);
         DBK_LAUNCH_OK();
     }
     DBK_CHECK(ptype == DBK_PT_AVG || argmax != nullptr, "ValueError: pooledmaps_argmax must be specified for max pooling.");
     DBK_CHECK(X && regions && pooled && dpooled, "ValueError: null pointer argument");
     hipStream_t st = dbk::as_stream(stream);
     switch (ptype) {
-    case DBK_PT_MAX: return launch_bprop_pt<DBK_PT_MAX>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias);
-    case DBK_PT_AVG: return launch_bprop_pt<DBK_PT_AVG>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias);
-    default:         return launch_bprop_pt<DBK_PT_ALL>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias);
+    case DBK_PT_MAX: return launch_bprop_pt<DBK_PT_MAX>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0);
+    case DBK_PT_AVG: return launch_bprop_pt<DBK_PT_AVG>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0);
+    default:         return launch_bprop_pt<DBK_PT_ALL>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0);
     }
 }
 

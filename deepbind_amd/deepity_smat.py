@@ -239,9 +239,10 @@ def head_fprop(pooled, W1, b1, W2=None, b2=None, nblock=1, in_scale=None, apply_
 
 
 def head_train(pooled, W1, b1, W2, b2, Y, nblock, loss, dW1, db1, dW2=None, db2=None, Ymask=None, rate=None, U=None,
-               seed=0, offset=0, counter=None, reverse_complement=False, want_loss=False):
-    """Forward and backward of nblock dense heads in one launch. Returns (Z, dpooled, loss|None);
-    the weight gradients are written into dW1, db1, dW2, db2. float32 only."""
+               seed=0, offset=0, counter=None, counter_advance=0, reverse_complement=False, want_loss=False):
+    """Forward and backward of nblock dense heads. Returns (Z, dpooled, loss|None); the weight gradients
+    are written into dW1, db1, dW2, db2. With `counter` (device int64) the dropout generator position is
+    read from it and moved on by `counter_advance` once the masks are drawn. float32 only."""
     require(pooled.dtype == torch.float32, "TypeError: the fused head is float32 only")
     n = pooled.shape[0]
     k = pooled.shape[1] // nblock
@@ -251,9 +252,15 @@ def head_train(pooled, W1, b1, W2, b2, Y, nblock, loss, dW1, db1, dW2=None, db2=
     L = torch.empty((1, nblock), dtype=torch.float32, device=pooled.device) if want_loss else None
     r = None if rate is None else _vec(rate, pooled)
     call("dbk_head_train", stream(), n, nblock, k, hidden, {"nll": 0, "mse": 1}[loss], int(bool(reverse_complement)),
-         ptr(pooled), ptr(r), ptr(U), int(seed), int(offset), ptr(counter), ptr(W1), ptr(b1), ptr(W2), ptr(b2), ptr(Y), ptr(Ymask),
+         ptr(pooled), ptr(r), ptr(U), int(seed), int(offset), ptr(counter), int(counter_advance), ptr(W1), ptr(b1), ptr(W2), ptr(b2), ptr(Y), ptr(Ymask),
          ptr(Z), ptr(dpooled), ptr(dW1), ptr(db1), ptr(dW2), ptr(db2), ptr(L))
     return Z, dpooled, L
+
+
+def l1_decay(P, decay, dP):
+    """dP += sign(P) * decay, elementwise over a whole flat parameter vector (decay: one coefficient per element)."""
+    require(P.shape == dP.shape == decay.shape and P.dtype == dP.dtype == decay.dtype, "ValueError: P, decay and dP must match")
+    call("dbk_l1_decay", stream(), dtype_code(P), ptr(P), ptr(decay), ptr(dP), P.numel())
 
 
 def counter_add(counter, delta):

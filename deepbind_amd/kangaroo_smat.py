@@ -152,8 +152,8 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto"):
     return pooled, argmax
 
 
-def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db):
-    """Backward of scanpool_fprop: dW += filter gradient, db[:] = bias gradient."""
+def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db, overwrite=False):
+    """Backward of scanpool_fprop: dW += filter gradient (dW[:] = with overwrite), db[:] = bias gradient."""
     _u8(X)
     _regions(regions)
     require(W.dtype == torch.float32 and dpooled.dtype == torch.float32, "TypeError: the fused path is float32 only")
@@ -161,4 +161,4 @@ def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db):
     require(dpooled.shape == pooled.shape, "ValueError: dpooled must have pooled's shape")
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
     call("dbk_scanpool_bprop", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype],
-         ptr(pooled), ptr(argmax), ptr(dpooled), ptr(dW), ptr(db))
+         ptr(pooled), ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)))

@@ -74,6 +74,7 @@ class SequenceNet(object):
         self.set_rates(rate, momentum)
         self.decay_conv = self._vec(decay_conv)
         self.decay_full = self._vec(decay_full)
+        self.decay_vec = self._build_decay_vec()
         self.dropout = self._vec(dropout)
         self.use_dropout = bool(np.any(np.asarray(dropout) > 0))
         # position of the dropout generator, kept on the device so that a captured graph advances it
@@ -345,10 +346,10 @@ class SequenceNet(object):
         dH0 = ds.blockwise_dot_nt(dA1, p["W1"], ni)
         if self.use_dropout:
             dH0 = ds.dropout_bp_tr(dH0, st["M"]) if "M" in st else ds.dropout_bp_te(dH0, self.dropout)
-        g["Wc"].zero_()
         if self.mode == "fused":
-            ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, st["pooled"], st["argmax"], dH0, g["Wc"], g["bc"])
+            ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, st["pooled"], st["argmax"], dH0, g["Wc"], g["bc"], overwrite=True)
         else:
+            g["Wc"].zero_()
             dA0 = sm.zeros_like(st["A0"])
             ks.poolrgn_bprop(dA0, R, dH0, st["argmax"], self.pool)
             dZ0 = sm.mul_sign(dA0, st["A0"])
@@ -359,15 +360,25 @@ class SequenceNet(object):
         if self.step_count < self.start_training:
             g["Wc"].zero_()
 
-    def _add_decay(self):
-        p, g, ni = self.p, self.g, self.ninst
+    def _build_decay_vec(self):
+        """One L1 coefficient per element of the flat parameter vector (zero for biases): what
+        madd_bcast(sign(W), decay, k, dW) multiplies each sign by (reference: deepity/std/full.py:111-119)."""
+        ni = self.ninst
+        vec = torch.zeros_like(self.P)
+        ones = torch.ones_like(self.P)
+        span = {name: (int(a), int(b)) for (name, _, _), a, b in zip(self.layout, self.offsets[:-1], self.offsets[1:])}
+        view = lambda name, t: t[span[name][0]:span[name][1]]
         # the reference passes rows/ninst as the block length for the scan filters although their
         # models lie along columns (kangaroo/_ext/corr1ord.py:126); kept as is for step parity
-        kq = max(1, p["Wc"].shape[0] // ni)
-        ds.madd_bcast(sm.sign(p["Wc"]), self.decay_conv, kq, g["Wc"])
-        ds.madd_bcast(sm.sign(p["W1"]), self.decay_full, p["W1"].numel() // ni, g["W1"])
-        if self.hidden > 0:
-            ds.madd_bcast(sm.sign(p["W2"]), self.decay_full, p["W2"].numel() // ni, g["W2"])
+        kq = max(1, self.p["Wc"].shape[0] // ni)
+        ds.madd_bcast(view("Wc", ones), self.decay_conv, kq, view("Wc", vec))
+        for name in ("W1", "W2"):
+            if name in self.p:
+                ds.madd_bcast(view(name, ones), self.decay_full, self.p[name].numel() // ni, view(name, vec))
+        return vec
+
+    def _add_decay(self):
+        ds.l1_decay(self.P, self.decay_vec, self.dP)
 
     def _grad_fused(self, X, R, Y, Ymask, U, U_input=None):
         """Gradient of one batch in a handful of launches: fused scan+pool forward, the whole dense head
@@ -376,15 +387,13 @@ class SequenceNet(object):
         X = self._drop_inputs(X, R, U_input)
         pooled, amax = ks.scanpool_fprop(p["Wc"], p["bc"], X, R, self.pool, want_argmax=True)
         rate = self.dropout if self.use_dropout else None
+        draws = (pooled.numel() + 3) // 4 if (rate is not None and U is None) else 0
         Z, dpooled, _ = ds.head_train(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), Y, self.ninst, self.loss,
                                       g["W1"], g["b1"], g.get("W2"), g.get("b2"), Ymask=Ymask, rate=rate, U=U,
-                                      seed=self.rng_seed, counter=self.rng_counter,
+                                      seed=self.rng_seed, counter=self.rng_counter, counter_advance=draws,
                                       reverse_complement=self.reverse_complement)
-        if rate is not None and U is None:
-            ds.counter_add(self.rng_counter, (pooled.numel() + 3) // 4)
-            self._rng_offset += (pooled.numel() + 3) // 4
-        g["Wc"].zero_()
-        ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, pooled, amax, dpooled, g["Wc"], g["bc"])
+        self._rng_offset += draws
+        ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, pooled, amax, dpooled, g["Wc"], g["bc"], overwrite=True)
         if self.weight_decay_start <= self.step_count:
             self._add_decay()
         if self.step_count < self.start_training:

@@ -140,7 +140,8 @@ int dbk_scanpool_fprop_kmer(dbk_stream_t stream,
                             float* pooled, uint32_t* argmax);
 
 /* Backward of the fused chain: given dpooled (same layout as pooled), the forward's pooled and
- * argmax, accumulates dW (C*m, F) += and writes dbias (1, F) =. Deterministic (no float atomics).
+ * argmax, accumulates dW (C*m, F) += (as corr1ord_bprop_W does; with overwrite != 0 it is written
+ * instead, which saves the caller a fill) and writes dbias (1, F) =. Deterministic (no float atomics).
  * reference chain: poolrgn_bprop -> relu bprop -> bias bprop -> corr1ord_bprop_W
  * (kangaroo/_ext/poolrgn.py:78-82, deepity/std/elemwise.py:78,172-180, kangaroo/_ext/corr1ord.py:120-138) */
 int dbk_scanpool_bprop(dbk_stream_t stream,
@@ -148,7 +149,7 @@ int dbk_scanpool_bprop(dbk_stream_t stream,
                        const uint8_t* X, size_t N,
                        const uint32_t* regions, size_t nregion, int ptype,
                        const float* pooled, const uint32_t* argmax, const float* dpooled,
-                       float* dW, float* dbias);
+                       float* dW, float* dbias, int overwrite);
 
 /* ------------------------------------------------------------------ dense head (deepity_smat) */
 
@@ -220,6 +221,11 @@ int dbk_dropout_bp_te(dbk_stream_t stream, int dtype, const void* dZ, const void
  * The reference draws from cuRAND's per-thread XORWOW states (smat_cuda/cuda_context.cpp:210-242),
  * which cannot be reproduced without the CUDA SDK; this generator is the library's own. */
 int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uint64_t offset);
+/* dP[i] += sign(P[i]) * decay[i]: the L1 weight-decay term of every parameter in one pass over the flat
+ * parameter vector (decay holds each element's coefficient, zero for biases).
+ * reference: madd_bcast(sign(W), decay, k, dW) per weight matrix, deepity/std/full.py:111-119,
+ * kangaroo/_ext/corr1ord.py:124-126 */
+int dbk_l1_decay(dbk_stream_t stream, int dtype, const void* P, const void* decay, void* dP, size_t n);
 /* Standard normal deviates from the same generator (Box-Muller on two Philox streams, one value per
  * element, element i depends only on (seed, offset, i)); used for the initial weights.
  * reference: sm.randn in the parameter set-up, deepity/deepity/sgd.py:337-341 (cuRAND there) */
@@ -261,19 +267,21 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
                    const float* W1, const float* b1, const float* W2, const float* b2,
                    int apply_logistic, float* scores);
 
-/* Forward AND backward of the dense head for nblock models in one launch (one workgroup per model):
+/* Forward AND backward of the dense head for nblock models in two launches (workgroups of one model x
+ * 32 rows, then an ordered sum over the row chunks):
  * dropout (rate per model, NULL = none; uniforms from U when given, else from the generator at
- * (seed, offset), or at (seed, *counter) when counter is a device pointer) -> dense (+bias, ReLU, dense
+ * (seed, offset), or at (seed, *counter) when counter is a device pointer; after the masks are drawn
+ * *counter is advanced by counter_advance) -> dense (+bias, ReLU, dense
  * when hidden > 0) -> bias -> logistic (loss_kind 0) or identity (loss_kind 1) -> dA = (Z-Y)/n masked by
  * Ymask (may be NULL) and, with reverse_complement, by the pair rule of dbk_calc_zmask -> all gradients.
  * Writes Z (n, nblock), dpooled (n, k*nblock), dW1, db1, dW2, db2 (overwritten, not accumulated) and,
  * if loss is not NULL, the per-model mean loss (nblock). Masks drawn here equal those of
- * dbk_dropout_fp_tr for the same (seed, offset). float32; k <= 64. Deterministic.
+ * dbk_dropout_fp_tr for the same (seed, offset). float32. Deterministic.
  * Replaces the reference's layer-by-layer head in a training step (deepity/std/elemwise.py:71-180,
  * full.py:78-119, softmax.py:58-77, loss.py:98-119). */
 int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden, int loss_kind, int reverse_complement,
                    const float* pooled, const float* rate, const float* U, uint64_t seed, uint64_t offset,
-                   const uint64_t* counter,
+                   uint64_t* counter, uint64_t counter_advance,
                    const float* W1, const float* b1, const float* W2, const float* b2,
                    const float* Y, const uint8_t* Ymask,
                    float* Z, float* dpooled, float* dW1, float* db1, float* dW2, float* db2, float* loss);
