@@ -121,6 +121,75 @@ def train_throughput(steps=30, warmup=5):
     return out
 
 
+def ops_throughput(reps=5):
+    """Per-operator figures for the drop-in operators and the general fused kernels on a mid-size batch
+    (8192 sequences x 101 nt, 16 models x 16 motifs x width 24: N = 1.02 M rows, F = 256, map = 1.04 GB).
+    bytes = algorithmic HBM bytes (operands read once, results written once); adds = N * F * m."""
+    import torch
+    from deepbind_amd import data, kangaroo_smat as ks, smat as sm
+    rng = np.random.default_rng(7)
+    B, L, m, F = 8192, 101, 24, 256
+    codes = rng.integers(0, 4, (B, L), dtype=np.uint8)
+    codes[rng.random((B, L)) < 0.01] = 255
+    Xh, Rh = data.pack_uniform_ordinals(codes, m - 1)
+    X, R = torch.from_numpy(Xh).cuda(), torch.from_numpy(Rh).cuda()
+    N = X.numel()
+    W = torch.randn(4 * m, F, device="cuda") * 0.1
+    b = torch.randn(1, F, device="cuda") * 0.1
+    Z = sm.zeros((N, F))
+    mapbytes, adds = N * F * 4, float(N) * F * m
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    out = {"workload": "%d sequences x %d nt, %d filters of width %d: N = %d rows, map %.2f GB" % (B, L, F, m, N, mapbytes / 1e9)}
+
+    def rec(name, ms, nbytes, nadds=None):
+        r = {"ms": ms, "GBs": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+        if nadds:
+            r["Tadds_s"] = nadds / ms / 1e9
+            r["fp32_frac"] = nadds / ms / 1e9 / FP32_VECTOR_PEAK_TFLOPS
+        out[name] = r
+
+    rec("corr1ord", timed(lambda: ks.corr1ord(W, X, Z, 4)), N + mapbytes, adds)
+    A = sm.relu(sm.add_rowvec(Z, b))
+    rec("bias+relu (2 launches)", timed(lambda: sm.relu(sm.add_rowvec(Z, b))), 4 * mapbytes)
+    for pt in ("max", "all"):
+        nout = B * F * 4 * (2 if pt == "all" else 1)
+        rec("poolrgn[%s]" % pt, timed(lambda: ks.poolrgn(A, R, pt, want_argmax=True)), mapbytes + nout + B * F * 4)
+        P, I = ks.poolrgn(A, R, pt, want_argmax=True)
+        dP = torch.randn_like(P)
+        dA = sm.zeros_like(A)
+        rec("poolrgn_bprop[%s]" % pt, timed(lambda: ks.poolrgn_bprop(dA, R, dP, I, pt)),
+            (2 * mapbytes if pt == "all" else 2 * B * F * 4) + nout)
+        del dA
+    dZ = torch.randn_like(Z)
+    dW = torch.zeros_like(W)
+    rec("corr1ord_bprop_W", timed(lambda: ks.corr1ord_bprop_W(dW, X, dZ, 4)), N + mapbytes, adds)
+    dX = sm.zeros((N, 4))
+    rec("corr1ord_bprop_X", timed(lambda: ks.corr1ord_bprop_X(dX, W, dZ, 4)), mapbytes + N * 16, adds)
+    del dZ, Z, A
+    db = torch.zeros_like(b)
+    for pt in ("max", "all"):
+        nout = B * F * 4 * (2 if pt == "all" else 1)
+        rec("scanpool_fprop general[%s, argmax]" % pt, timed(lambda: ks.scanpool_fprop(W, b, X, R, pt, want_argmax=True, path="general")),
+            N + nout + B * F * 4, adds)
+        P, I = ks.scanpool_fprop(W, b, X, R, pt, want_argmax=True, path="general")
+        dP = torch.randn_like(P)
+        rec("scanpool_bprop[%s]" % pt, timed(lambda: ks.scanpool_bprop(W, b, X, R, pt, P, I, dP, dW, db, overwrite=True)),
+            N + 2 * nout + B * F * 4, adds if pt == "all" else float(B) * F * m)
+    rec("scanpool_fprop table[max]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "max", path="kmer")), N + B * F * 4, adds)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,6 +198,7 @@ def main():
     ap.add_argument("--workload", default="config5", choices=["config5", "config5_small"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the secondary train-step throughput figures")
+    ap.add_argument("--ops", action="store_true", help="only the per-operator figures of the drop-in and general fused kernels")
     ap.add_argument("--train-only", action="store_true", help="only the train-step figures (for profiling the training kernels)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain copy kernel over 1 GiB (reference point for the HBM byte counters)")
@@ -144,6 +214,9 @@ def main():
 
     if args.train_only:
         print(json.dumps({"train": train_throughput(steps=args.steps, warmup=args.warmup)}))
+        return
+    if args.ops:
+        print(json.dumps({"ops": ops_throughput()}))
         return
     nseq = 100000 if args.workload == "config5" else 5000
     cfg = synth.config5(seed=4, nseq=nseq)

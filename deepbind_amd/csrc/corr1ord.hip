@@ -188,9 +188,233 @@ __global__ __launch_bounds__(256) void corr1ord_bprop_X_kernel(T* __restrict__ d
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Kernels for filters of at most MT taps (MT = 8, 16, 24, 32). All lanes of a wave look at the same
+// positions, so the letters of a 16-position window are read once into scalar registers.
+// ---------------------------------------------------------------------------------------------
+constexpr unsigned WSUBS = 4;             // windows of PSUB positions per wave and staging round
+
+// forward: every (position, tap) is one LDS read with an immediate offset; taps in ascending order,
+// so the sums are bit-identical to the any-length kernel's. A workgroup builds its filter tile's
+// table once and walks chunks of 256 positions.
+template <typename T, int MT>
+__global__ __launch_bounds__(256) void corr1ord_window_kernel(const T* __restrict__ W, unsigned m, unsigned F,
+                                                              const uint8_t* __restrict__ X, size_t n, T* __restrict__ Z)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    T* lut = reinterpret_cast<T*>(smem);                                   // [MT][NL][FT], zero rows past m
+    uint8_t* xl = smem + (size_t)MT * NL * FT * sizeof(T);                 // 4-byte aligned
+    const unsigned nw = blockDim.x >> 6, chunk = nw * WSUBS * PSUB;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
+    const size_t N = n + m - 1;
+    build_letter_table(lut, W, m, F, f0, MT);
+    for (size_t c0 = (size_t)blockIdx.x * chunk; c0 < n; c0 += (size_t)gridDim.x * chunk) {
+        const unsigned rows = (unsigned)((n - c0) < chunk ? (n - c0) : chunk);
+        __syncthreads();
+        stage(xl, X, N, c0, window_span<MT>(rows));
+        __syncthreads();
+#pragma unroll 1
+        for (unsigned s = 0; s < WSUBS; ++s) {
+            const unsigned p0 = (s * nw + wave) * PSUB;
+            if (p0 >= rows) break;
+            unsigned wq[window<MT>::words];
+            load_window<MT>(xl, p0, wq);
+            T acc[PSUB];
+            scan16_window<MT>(lut, wq, lane, acc);
+            if (f < F) {
+#pragma unroll
+                for (int p = 0; p < PSUB; ++p)
+                    if (p0 + p < rows) Z[(c0 + p0 + p) * F + f] = acc[p];
+            }
+        }
+    }
+}
+
+// filter gradient, pass 1: a lane keeps its filter's whole [tap][channel] column in registers; the
+// window's letters become four scalar weights (1 for the matching channel, 1/4 each for N, else 0)
+// applied as fused multiply-adds with exact products, i.e. one rounding per addition like a plain add.
+// Workgroup y walks chunks y, y+gridDim.y, ... in ascending order; its waves are folded in wave order.
+template <int MT>
+__global__ __launch_bounds__(256) void corr1ord_bprop_W_window_kernel(float* __restrict__ partial, unsigned m, unsigned F,
+                                                                      const uint8_t* __restrict__ X, size_t n,
+                                                                      const float* __restrict__ dZ)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* fold = reinterpret_cast<float*>(smem);                          // [MT*4][FT]
+    uint8_t* xl = smem + (size_t)MT * 4 * FT * sizeof(float);
+    const unsigned nw = blockDim.x >> 6, chunk = nw * WSUBS * PSUB;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned f0 = blockIdx.x * FT, f = f0 + lane;
+    const size_t N = n + m - 1;
+    float aw[MT][4];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) aw[j][0] = aw[j][1] = aw[j][2] = aw[j][3] = 0.0f;
+    for (size_t c0 = (size_t)blockIdx.y * chunk; c0 < n; c0 += (size_t)gridDim.y * chunk) {
+        const unsigned rows = (unsigned)((n - c0) < chunk ? (n - c0) : chunk);
+        __syncthreads();
+        stage(xl, X, N, c0, window_span<MT>(rows));
+        __syncthreads();
+#pragma unroll 1
+        for (unsigned s = 0; s < WSUBS; ++s) {
+            const unsigned p0 = (s * nw + wave) * PSUB;
+            if (p0 >= rows) break;
+            float g[PSUB];
+#pragma unroll
+            for (int p = 0; p < PSUB; ++p) g[p] = (f < F && p0 + p < rows) ? dZ[(c0 + p0 + p) * F + f] : 0.0f;
+            unsigned wq[window<MT>::words];
+            load_window<MT>(xl, p0, wq);
+#pragma unroll
+            for (int q = 0; q < PSUB + MT - 1; ++q) {
+                const unsigned l = window_letter(wq, q);
+                const float base = l == 4u ? 0.25f : 0.0f;
+                const float m0 = l == 0u ? 1.0f : base, m1 = l == 1u ? 1.0f : base;
+                const float m2 = l == 2u ? 1.0f : base, m3 = l == 3u ? 1.0f : base;
+#pragma unroll
+                for (int p = 0; p < PSUB; ++p) {
+                    const int j = q - p;
+                    if (j >= 0 && j < MT) {
+                        aw[j][0] = __builtin_fmaf(g[p], m0, aw[j][0]);
+                        aw[j][1] = __builtin_fmaf(g[p], m1, aw[j][1]);
+                        aw[j][2] = __builtin_fmaf(g[p], m2, aw[j][2]);
+                        aw[j][3] = __builtin_fmaf(g[p], m3, aw[j][3]);
+                    }
+                }
+            }
+        }
+    }
+    float* mine = fold + lane;
+    for (unsigned w = 0; w < nw; ++w) {
+        __syncthreads();
+        if (wave == w) {
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                if ((unsigned)j < m) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float* cell = mine + (j * 4 + c) * FT;
+                        *cell = w == 0 ? aw[j][c] : *cell + aw[j][c];
+                    }
+                }
+        }
+    }
+    __syncthreads();
+    float* out = partial + (size_t)blockIdx.y * (4 * m) * F;
+    for (unsigned e = threadIdx.x; e < m * 4 * FT; e += blockDim.x) {
+        const unsigned row = e / FT, fl = e % FT;
+        if (f0 + fl < F) out[(size_t)row * F + f0 + fl] = fold[e];
+    }
+}
+
+// input gradient: a wave owns RPW consecutive rows and walks the filter tiles; a lane holds its filter's
+// [tap][channel] weights in registers and a ring of the last MT gradient rows, so each row of dZ is read
+// once per tile and each (row, tap, channel) is one multiply-add. Row sums over the 64 filters of a tile
+// go through LDS eight rows at a time: every lane parks its 32 partial sums, then lane v < 32 adds up
+// value v over the 64 lanes in lane order (a fixed order); tiles are added in ascending order into the
+// wave's rows in LDS.
+constexpr int XR_STRIDE = 65;             // odd row stride: the 32 column sums read 32 different banks
+constexpr int XR_AHEAD = 4;               // rows of dZ in flight per lane
+
+template <int MT, int RPW>
+__global__ __launch_bounds__(256) void corr1ord_bprop_X_ring_kernel(float* __restrict__ dX, size_t n, const float* __restrict__ W,
+                                                                    unsigned m, unsigned F, const float* __restrict__ dZ)
+{
+    static_assert(RPW % MT == 0 && MT % 8 == 0 && MT % XR_AHEAD == 0, "a wave's rows are walked in blocks of MT, reduced eight at a time");
+    __shared__ float rows_acc[4][RPW * 4];
+    __shared__ float parts[4][32 * XR_STRIDE];
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t i0 = ((size_t)blockIdx.x * 4 + wave) * RPW;
+    if (i0 >= n) return;                                                   // (no barriers in this kernel)
+    float* acc = rows_acc[wave];
+    float* part = parts[wave];
+    for (unsigned e = lane; e < RPW * 4; e += 64) acc[e] = 0.0f;
+    const unsigned ftiles = (F + FT - 1) / FT;
+    for (unsigned t = 0; t < ftiles; ++t) {
+        const unsigned f = t * FT + lane;
+        const bool live = f < F;
+        float w[MT][4];
+#pragma unroll
+        for (int k = 0; k < MT; ++k) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) w[k][c] = (live && (unsigned)k < m) ? W[(size_t)(4 * k + c) * F + f] : 0.0f;
+        }
+        // ring slot r holds row i with i % MT == r (i0 is a multiple of MT); start with the MT-1 rows before i0
+        float ring[MT];
+        ring[0] = 0.0f;
+#pragma unroll
+        for (int r = 1; r < MT; ++r) {
+            const bool have = i0 + r >= (size_t)MT;                         // row i0 - MT + r exists
+            ring[r] = (live && have) ? dZ[(i0 - MT + r) * F + f] : 0.0f;
+        }
+        // rows are fetched XR_AHEAD positions before they are used (MT is a multiple of XR_AHEAD, so the
+        // slot of a row is a compile-time index)
+        float pre[XR_AHEAD];
+#pragma unroll
+        for (int d = 0; d < XR_AHEAD; ++d) pre[d] = (live && i0 + d < n) ? dZ[(i0 + d) * F + f] : 0.0f;
+#pragma unroll 1
+        for (unsigned b0 = 0; b0 < RPW; b0 += MT) {
+            if (i0 + b0 >= n) break;
+#pragma unroll
+            for (int u = 0; u < MT; ++u) {
+                ring[u] = pre[u % XR_AHEAD];
+                {
+                    const size_t i = i0 + b0 + u + XR_AHEAD;
+                    pre[u % XR_AHEAD] = (live && i < n) ? dZ[i * F + f] : 0.0f;
+                }
+                float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+#pragma unroll
+                for (int k = 0; k < MT; ++k) {
+                    const float dz = ring[(u - k + MT) % MT];              // row i - k
+                    s0 = __builtin_fmaf(dz, w[k][0], s0);
+                    s1 = __builtin_fmaf(dz, w[k][1], s1);
+                    s2 = __builtin_fmaf(dz, w[k][2], s2);
+                    s3 = __builtin_fmaf(dz, w[k][3], s3);
+                }
+                float* mine = part + ((u & 7) * 4) * XR_STRIDE + lane;
+                mine[0 * XR_STRIDE] = s0;
+                mine[1 * XR_STRIDE] = s1;
+                mine[2 * XR_STRIDE] = s2;
+                mine[3 * XR_STRIDE] = s3;
+                if ((u & 7) == 7) {
+                    // the wave's own LDS accesses execute in program order; no other wave touches `part`
+                    __builtin_amdgcn_wave_barrier();
+                    if (lane < 32) {
+                        const float* col = part + lane * XR_STRIDE;
+                        float tot = 0.0f;
+#pragma unroll 16
+                        for (int l = 0; l < 64; ++l) tot += col[l];
+                        acc[(b0 + u - 7) * 4 + lane] += tot;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        }
+    }
+    for (unsigned e = lane; e < RPW * 4; e += 64) {
+        const size_t i = i0 + e / 4;
+        if (i < n) dX[i * 4 + (e & 3)] += acc[e];
+    }
+}
+
 template <typename T>
 int launch_fprop(hipStream_t st, const T* W, size_t m, size_t F, const uint8_t* X, size_t n, T* Z)
 {
+    const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 24 ? 24 : (m <= 32 ? 32 : 0)));
+    if (mt) {
+        const unsigned ftiles = dbk::divup(F, FT), chunk = 4 * WSUBS * PSUB;
+        DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
+        const size_t smem_w = (size_t)mt * NL * FT * sizeof(T) + ((chunk + mt - 1 + 7) & ~(size_t)3);
+        if (smem_w <= lds_limit()) {
+            unsigned gx = 1024u / ftiles;                      // a few resident workgroups per CU, each building its table once
+            if (gx < 1) gx = 1;
+            if (gx > dbk::divup(n, chunk)) gx = dbk::divup(n, chunk);
+            auto kw = mt == 8 ? corr1ord_window_kernel<T, 8> : mt == 16 ? corr1ord_window_kernel<T, 16>
+                    : mt == 24 ? corr1ord_window_kernel<T, 24> : corr1ord_window_kernel<T, 32>;
+            DBK_HIP(hipFuncSetAttribute((const void*)kw, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_w));
+            hipLaunchKernelGGL(kw, dim3(gx, ftiles), dim3(256), smem_w, st, W, (unsigned)m, (unsigned)F, X, n, Z);
+            DBK_LAUNCH_OK();
+        }
+    }
     constexpr int NW = 4, PW = 64;
     size_t smem = m * NL * FT * sizeof(T) + (NW * PW + m - 1);
     DBK_CHECK(smem <= lds_limit(), "ValueError: filter length %zu needs %zu bytes of LDS (limit %zu)", m, smem, lds_limit());
@@ -199,6 +423,38 @@ int launch_fprop(hipStream_t st, const T* W, size_t m, size_t F, const uint8_t* 
     dim3 grid(dbk::divup(n, NW * PW), dbk::divup(F, FT));
     DBK_CHECK(grid.y <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
     hipLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, st, W, (unsigned)m, (unsigned)F, X, n, Z);
+    DBK_LAUNCH_OK();
+}
+
+// float32 filters of at most 24 taps: register-resident gradient columns
+inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, const uint8_t* X, size_t n, const float* dZ)
+{
+    const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : 24);
+    const unsigned ftiles = dbk::divup(F, FT), chunk = 4 * WSUBS * PSUB;
+    const unsigned nchunk = dbk::divup(n, chunk);
+    unsigned gy = 768u / ftiles;                               // three workgroups fit a CU
+    if (gy < 1) gy = 1;
+    if (gy > nchunk) gy = nchunk;
+    const size_t nelem = 4 * m * F;
+    float* partial = (float*)dbk::workspace(nelem * gy * sizeof(float), st);
+    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", nelem * gy * sizeof(float));
+    const size_t smem = (size_t)mt * 4 * FT * sizeof(float) + ((chunk + mt - 1 + 7) & ~(size_t)3);
+    auto kern = mt == 8 ? corr1ord_bprop_W_window_kernel<8> : mt == 16 ? corr1ord_bprop_W_window_kernel<16> : corr1ord_bprop_W_window_kernel<24>;
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3(ftiles, gy), dim3(256), smem, st, partial, (unsigned)m, (unsigned)F, X, n, dZ);
+    hipLaunchKernelGGL(reduce_partials_kernel<float>, dim3(dbk::ew_grid(nelem)), dim3(256), 0, st, dW, (const float*)partial, nelem, gy);
+    DBK_LAUNCH_OK();
+}
+
+inline int launch_bprop_X_ring(hipStream_t st, float* dX, size_t n, const float* W, size_t m, size_t F, const float* dZ)
+{
+    if (m <= 8) {
+        hipLaunchKernelGGL((corr1ord_bprop_X_ring_kernel<8, 96>), dim3(dbk::divup(n, 4 * 96)), dim3(256), 0, st, dX, n, W, (unsigned)m, (unsigned)F, dZ);
+    } else if (m <= 16) {
+        hipLaunchKernelGGL((corr1ord_bprop_X_ring_kernel<16, 96>), dim3(dbk::divup(n, 4 * 96)), dim3(256), 0, st, dX, n, W, (unsigned)m, (unsigned)F, dZ);
+    } else {
+        hipLaunchKernelGGL((corr1ord_bprop_X_ring_kernel<24, 96>), dim3(dbk::divup(n, 4 * 96)), dim3(256), 0, st, dX, n, W, (unsigned)m, (unsigned)F, dZ);
+    }
     DBK_LAUNCH_OK();
 }
 
@@ -259,6 +515,7 @@ int dbk_corr1ord_bprop_W(dbk_stream_t stream, int dtype, void* dW, size_t m, siz
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(dW && X && dZ, "ValueError: null pointer argument");
+    if (dtype == DBK_F32 && m <= 24) return launch_bprop_W_window(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     if (dtype == DBK_F32) return launch_bprop_W<float>(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     return launch_bprop_W<double>(dbk::as_stream(stream), (double*)dW, m, nfilter, X, n, (const double*)dZ);
 }
@@ -271,6 +528,7 @@ int dbk_corr1ord_bprop_X(dbk_stream_t stream, int dtype, void* dX, size_t n, siz
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(dX && W && dZ, "ValueError: null pointer argument");
+    if (dtype == DBK_F32 && m <= 24) return launch_bprop_X_ring(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     if (dtype == DBK_F32) return launch_bprop_X<float>(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     return launch_bprop_X<double>(dbk::as_stream(stream), (double*)dX, n, (const double*)W, m, nfilter, (const double*)dZ);
 }
