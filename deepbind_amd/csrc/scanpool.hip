@@ -230,15 +230,29 @@ __global__ __launch_bounds__(256) void scanpool_bprop_kernel(const float* __rest
 // this lane's column of a [tap][channel][FT] table. Taps go eight at a time: the letters of all four
 // positions are loaded first (32 independent global loads in flight), then each position's eight cells
 // are read, updated and written (distinct taps are distinct cells), positions in ascending order.
-__device__ __forceinline__ void add_positions4(float* mine, const uint8_t* __restrict__ X, const size_t (&pos)[4],
+__device__ __forceinline__ void add_positions4(float* mine, const uint8_t* __restrict__ X, size_t N, const size_t (&pos)[4],
                                                const float (&g)[4], const bool (&on)[4], unsigned m)
 {
     for (unsigned j0 = 0; j0 < m; j0 += 8) {
+        // eight letters = three aligned 32-bit loads shifted into place (a lane's window starts at any byte);
+        // a word is only fetched if it starts before the end of the stream
         unsigned l[4][8];
+        const uintptr_t xend = reinterpret_cast<uintptr_t>(X) + N;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
+            const uintptr_t addr = reinterpret_cast<uintptr_t>(X) + pos[u] + j0;
+            const uintptr_t base = addr & ~(uintptr_t)3;
+            const unsigned sh = (unsigned)(addr & 3);
+            unsigned w[3];
 #pragma unroll
-            for (unsigned t = 0; t < 8; ++t) l[u][t] = (on[u] && j0 + t < m) ? letter_of(X[pos[u] + j0 + t]) : 5u;
+            for (int t = 0; t < 3; ++t)
+                w[t] = (on[u] && base + 4 * t < xend) ? *reinterpret_cast<const unsigned*>(base + 4 * t) : 0xffffffffu;
+            const unsigned lo = __builtin_amdgcn_alignbyte(w[1], w[0], sh), hi = __builtin_amdgcn_alignbyte(w[2], w[1], sh);
+#pragma unroll
+            for (unsigned t = 0; t < 8; ++t) {
+                const unsigned code = ((t < 4 ? lo : hi) >> ((t & 3) * 8)) & 0xffu;
+                l[u][t] = (on[u] && j0 + t < m) ? letter_of(code) : 5u;
+            }
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -305,7 +319,7 @@ __global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, u
                 if (g[u] != 0.0f) db += g[u];
                 on[u] = g[u] != 0.0f && pos[u] < n;
             }
-            add_positions4(mine, X, pos, g, on, m);
+            add_positions4(mine, X, N, pos, g, on, m);
         }
         float* out = slabs + (size_t)blockIdx.x * stride;
         for (unsigned row = 0; row < 4 * m; ++row) out[(size_t)row * F + f] = mine[row * FT];
