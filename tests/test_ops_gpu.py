@@ -71,33 +71,45 @@ def test_corr1ord_rejects_bad_arguments(ks):
         ks.corr1ord(W, dev(np.zeros(20, np.float32)), dev(np.zeros((20, 4), np.float32)), 4)
 
 
-@pytest.mark.parametrize("N,m,F,dense", [(400, 24, 16, True), (3000, 16, 100, True), (2000, 24, 64, False), (50, 7, 5, True)])
-def test_corr1ord_bprop_W(ks, N, m, F, dense):
+@pytest.mark.parametrize("N,m,F,dense,dtype", [(400, 24, 16, True, np.float32), (3000, 16, 100, True, np.float32),
+                                               (2000, 24, 64, False, np.float32), (50, 7, 5, True, np.float32),
+                                               (70000, 24, 200, True, np.float32), (900, 30, 40, True, np.float32),
+                                               (600, 24, 33, True, np.float64), (20, 24, 8, True, np.float32)])
+def test_corr1ord_bprop_W(ks, N, m, F, dense, dtype):
+    """Several chunks per workgroup (N = 70000), the any-length kernel (m = 30), float64, and a stream shorter
+    than the filter (no row defined: the gradient is zero)."""
     rng = np.random.default_rng(N + F)
     X = random_codes(rng, N, 0.05, 0.02)
-    dZ = rng.standard_normal((N, F)).astype(np.float32)
+    dZ = rng.standard_normal((N, F)).astype(dtype)
     if not dense:
         dZ[rng.random((N, F)) < 0.98] = 0                              # 1-sparse-like, as after max pooling
     ref = np.zeros((4 * m, F), np.float64)
     orc.corr1ord_bprop_W(ref, X, dZ.astype(np.float64))
-    dW = dev(np.ones((4 * m, F), np.float32))                          # accumulates onto existing content
+    dW = dev(np.ones((4 * m, F), dtype))                               # accumulates onto existing content
     ks.corr1ord_bprop_W(dW, dev(X), dev(dZ), 4)
-    assert_close(host(dW), ref + 1.0, GRAD, "dW")
+    assert_close(host(dW), ref + 1.0, GRAD if dtype == np.float32 else 1e-12, "dW")
     # run-to-run bit stability (no float atomics)
-    dW2 = dev(np.ones((4 * m, F), np.float32))
+    dW2 = dev(np.ones((4 * m, F), dtype))
     ks.corr1ord_bprop_W(dW2, dev(X), dev(dZ), 4)
     assert np.array_equal(host(dW), host(dW2))
 
 
-def test_corr1ord_bprop_X(ks):
-    rng = np.random.default_rng(5)
-    n, m, F = 300, 24, 48
-    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
-    dZ = rng.standard_normal((n, F)).astype(np.float32)
+@pytest.mark.parametrize("n,m,F,dtype", [(300, 24, 48, np.float32), (1000, 11, 130, np.float32), (97, 5, 64, np.float32),
+                                         (5000, 24, 256, np.float32), (3, 16, 7, np.float32), (50, 30, 20, np.float32),
+                                         (400, 24, 70, np.float64)])
+def test_corr1ord_bprop_X(ks, n, m, F, dtype):
+    """Row counts around the per-wave block of 96 rows, several filter tiles, fewer rows than taps, the
+    any-length kernel (m = 30) and float64; accumulates into dX and is bit-stable."""
+    rng = np.random.default_rng(5 + n)
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(dtype)
+    dZ = rng.standard_normal((n, F)).astype(dtype)
     ref = np.ones((n, 4)); orc.corr1ord_bprop_X(ref, W.astype(np.float64), dZ.astype(np.float64))
-    dX = dev(np.ones((n, 4), np.float32))
+    dX = dev(np.ones((n, 4), dtype))
     ks.corr1ord_bprop_X(dX, dev(W), dev(dZ), 4)
-    assert_close(host(dX), ref, GRAD, "dX")
+    assert_close(host(dX), ref, GRAD if dtype == np.float32 else 1e-12, "dX")
+    dX2 = dev(np.ones((n, 4), dtype))
+    ks.corr1ord_bprop_X(dX2, dev(W), dev(dZ), 4)
+    assert np.array_equal(host(dX), host(dX2))
 
 
 # ------------------------------------------------------------------------------------------ pooling
