@@ -126,19 +126,42 @@ template <typename T> __global__ void k_add_rowvec(const T* X, const T* b, T* Z,
 {
     GRID_STRIDE(i, n * m) Z[i] = X[i] + b[i % m];
 }
-// 64 columns per workgroup; wave w sums rows w, w+4, ... in ascending order and the four partial
-// sums are combined in wave order: a fixed summation order, independent of the launch
-template <typename T> __global__ __launch_bounds__(256) void k_colsum(const T* X, T* out, size_t n, size_t m)
+// Column sums in a fixed order. Workgroup (x, y) takes 64 columns and row slice y; wave w sums rows
+// w, w+4, ... of the slice in ascending order (four rows in flight), the four waves are combined in
+// wave order, and k_colsum_fold adds the slices in ascending order: the summation order depends only
+// on the shape.
+template <typename T> __global__ __launch_bounds__(256) void k_colsum(const T* __restrict__ X, T* __restrict__ out, size_t n, size_t m,
+                                                                      size_t rows_per_slice)
 {
     __shared__ T part[4][64];
     const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const size_t c = (size_t)blockIdx.x * 64 + lane;
+    const size_t r0 = (size_t)blockIdx.y * rows_per_slice;
+    const size_t r1 = r0 + rows_per_slice < n ? r0 + rows_per_slice : n;
     T s = (T)0;
-    if (c < m)
-        for (size_t r = w; r < n; r += 4) s += X[r * m + c];
+    if (c < m) {
+        size_t r = r0 + w;
+        for (; r + 12 < r1; r += 16) {
+            const T a0 = X[r * m + c], a1 = X[(r + 4) * m + c], a2 = X[(r + 8) * m + c], a3 = X[(r + 12) * m + c];
+            s += a0;
+            s += a1;
+            s += a2;
+            s += a3;
+        }
+        for (; r < r1; r += 4) s += X[r * m + c];
+    }
     part[w][lane] = s;
     __syncthreads();
-    if (w == 0 && c < m) out[c] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+    if (w == 0 && c < m) out[(size_t)blockIdx.y * m + c] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+}
+template <typename T> __global__ void k_colsum_fold(const T* __restrict__ partial, T* __restrict__ out, size_t m, unsigned nslice)
+{
+    GRID_STRIDE(c, m) {
+        T s = partial[c];
+#pragma unroll 8
+        for (unsigned y = 1; y < nslice; ++y) s += partial[(size_t)y * m + c];
+        out[c] = s;
+    }
 }
 template <typename T> __global__ void k_relu(const T* X, T* Z, size_t n)
 {
@@ -224,6 +247,27 @@ template <typename T> __global__ void k_sub_scale(const T* Z, const T* Y, T scal
         DBK_LAUNCH_OK();                                                                                   \
     } while (0)
 #define A(...) __VA_ARGS__
+
+template <typename T>
+int launch_colsum(hipStream_t st, const T* X, T* out, size_t n, size_t m)
+{
+    const unsigned tiles = dbk::divup(m, 64);
+    // slices of at least 256 rows, about 2048 workgroups in all
+    size_t nslice = (n + 255) / 256;
+    const size_t cap = 2048u / tiles > 0 ? 2048u / tiles : 1;
+    if (nslice > cap) nslice = cap;
+    if (nslice < 1) nslice = 1;
+    const size_t rows_per = (n + nslice - 1) / nslice;
+    if (nslice == 1) {
+        hipLaunchKernelGGL(k_colsum<T>, dim3(tiles, 1), dim3(256), 0, st, X, out, n, m, rows_per);
+        return 0;
+    }
+    T* partial = (T*)dbk::workspace(nslice * m * sizeof(T), st);
+    if (!partial) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", nslice * m * sizeof(T)); return 1; }
+    hipLaunchKernelGGL(k_colsum<T>, dim3(tiles, (unsigned)nslice), dim3(256), 0, st, X, partial, n, m, rows_per);
+    hipLaunchKernelGGL(k_colsum_fold<T>, dim3(dbk::ew_grid(m)), dim3(256), 0, st, (const T*)partial, out, m, (unsigned)nslice);
+    return 0;
+}
 
 extern "C" {
 
@@ -333,9 +377,11 @@ int dbk_colsum(dbk_stream_t stream, int dtype, const void* X, void* out, size_t 
 {
     DBK_DTYPE_OK(dtype);
     if (m == 0) { dbk::clear_error(); return 0; }
-    DBK_CHECK(dbk::divup(m, 64) <= 0x7fffffffu, "ValueError: too many columns");
-    if (dtype == DBK_F32) hipLaunchKernelGGL(k_colsum<float>, dim3(dbk::divup(m, 64)), dim3(256), 0, dbk::as_stream(stream), CF32(X), F32(out), n, m);
-    else hipLaunchKernelGGL(k_colsum<double>, dim3(dbk::divup(m, 64)), dim3(256), 0, dbk::as_stream(stream), CF64(X), F64(out), n, m);
+    DBK_CHECK(dbk::divup(m, 64) <= 65535u, "ValueError: too many columns");
+    DBK_CHECK(out && (X || n == 0), "ValueError: null pointer argument");
+    int rc = dtype == DBK_F32 ? launch_colsum<float>(dbk::as_stream(stream), CF32(X), F32(out), n, m)
+                              : launch_colsum<double>(dbk::as_stream(stream), CF64(X), F64(out), n, m);
+    if (rc) return rc;
     DBK_LAUNCH_OK();
 }
 int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)

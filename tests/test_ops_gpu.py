@@ -464,6 +464,18 @@ def test_scanpool_kmer_regions_in_any_order(ks, B, lo, hi, m, F):
     assert_close(host(P2), Pr[perm], ACT, "shuffled order")
 
 
+@pytest.mark.parametrize("n,m,dtype", [(1, 5, np.float32), (255, 64, np.float32), (13591, 720, np.float32), (100000, 70, np.float32),
+                                       (4097, 1, np.float64), (0, 9, np.float32)])
+def test_column_sums(sm, n, m, dtype):
+    """One slice and many slices of rows, column counts off the 64-wide tile, bit-stability, zero rows."""
+    rng = np.random.default_rng(n + m)
+    X = rng.standard_normal((n, m)).astype(dtype)
+    got = host(sm.sum_axis0(dev(X)))
+    assert got.shape == (1, m)
+    assert_close(got, X.astype(np.float64).sum(axis=0, keepdims=True), ACT if dtype == np.float32 else 1e-12, "column sums")
+    assert np.array_equal(got, host(sm.sum_axis0(dev(X))))
+
+
 # ------------------------------------------------------------------------------------------ empty and degenerate inputs
 def test_empty_and_degenerate_inputs(ks, ds):
     """Zero regions, streams shorter than the filter, zero rows: every entry point must
