@@ -187,6 +187,18 @@ def ops_throughput(reps=5):
         rec("scanpool_bprop[%s]" % pt, timed(lambda: ks.scanpool_bprop(W, b, X, R, pt, P, I, dP, dW, db, overwrite=True)),
             N + 2 * nout + B * F * 4, adds if pt == "all" else float(B) * F * m)
     rec("scanpool_fprop table[max]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "max", path="kmer")), N + B * F * 4, adds)
+    del X, R, W, b, dW, db, dX, P, I, dP
+    # per-model dense layer at bulk-scoring size: 100 000 rows, 64 models, 16 -> 32
+    from deepbind_amd import deepity_smat as ds
+    n, nb, k, h = 100000, 64, 16, 32
+    Xp = torch.randn(n, k * nb, device="cuda")
+    W1 = torch.randn(k * nb, h, device="cuda") * 0.1
+    dH = torch.randn(n, h * nb, device="cuda")
+    io = (n * k * nb + n * h * nb + k * nb * h) * 4
+    rec("blockwise_dot 100000x(64x16)->(64x32)", timed(lambda: ds.blockwise_dot(Xp, W1, nb)), io)
+    rec("blockwise_dot_nt", timed(lambda: ds.blockwise_dot_nt(dH, W1, nb)), io)
+    rec("blockwise_dot_tn", timed(lambda: ds.blockwise_dot_tn(Xp, dH, nb, W1)), io)
+    rec("sum_axis0 100000x2048", timed(lambda: sm.sum_axis0(dH)), n * h * nb * 4)
     return out
 
 

@@ -74,6 +74,188 @@ __global__ __launch_bounds__(256) void k_bdot_tn(int nblock, size_t n, int m, in
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Bulk variants (many rows). A workgroup takes TG = 16 consecutive models; lane = (row, model) with the
+// model fastest, so a wave reads and writes contiguous row segments spanning 16 models, and the 16
+// models' weights sit in LDS as [input][output/4][model][4]: one aligned 256-byte line per 16 lanes and
+// ds_read_b128. Multiply-adds are fused (as in the reference's GEMM library); inputs ascending.
+// ---------------------------------------------------------------------------------------------
+constexpr int TG = 16;
+
+template <typename T> struct alignas(4 * sizeof(T)) vec4 { T x, y, z, w; };
+
+template <typename T>
+__device__ void stage_weights16(T* ws, const T* __restrict__ W, int nblock, unsigned m0, int k, int m, int p, int off)
+{
+    const int mq = m >> 2;
+    for (int e = threadIdx.x; e < k * m * TG; e += blockDim.x) {
+        // destination order: e = ((kk*mq + c4)*TG + g)*4 + c
+        const int c = e & 3, g = (e >> 2) & (TG - 1), rest = e >> 6, c4 = rest % mq, kk = rest / mq;
+        const unsigned mdl = m0 + g;
+        ws[e] = mdl < (unsigned)nblock ? W[((size_t)mdl * p + off + kk) * m + c4 * 4 + c] : (T)0;
+    }
+}
+
+// Z[r, b*m + c] (accumulate ? += : =) sum_kk X[r, xb + kk] * W[(b*p + off + kk)*m + c]
+template <typename T, int KMAX, int MMAX>
+__global__ __launch_bounds__(256) void k_bdot_tile(int nblock, size_t n, int m, int k, int p, int off, bool bcast, bool accumulate,
+                                                   const T* __restrict__ X, const T* __restrict__ W, T* __restrict__ Z)
+{
+    extern __shared__ __align__(16) unsigned char tsm[];
+    T* ws = reinterpret_cast<T*>(tsm);
+    const unsigned g = threadIdx.x & (TG - 1), rl = threadIdx.x >> 4, m0 = blockIdx.x * TG, mdl = m0 + g;
+    stage_weights16(ws, W, nblock, m0, k, m, p, off);
+    __syncthreads();
+    if (mdl >= (unsigned)nblock) return;
+    const int mq = m >> 2;
+    const size_t ldx = (size_t)k * (bcast ? 1 : nblock), ldz = (size_t)m * nblock;
+    const vec4<T>* wv = reinterpret_cast<const vec4<T>*>(ws) + g;
+    const size_t rstep = (size_t)gridDim.y * 16, xoff = bcast ? 0 : (size_t)mdl * k;
+    size_t r = (size_t)blockIdx.y * 16 + rl;
+    T xn[KMAX];                                          // next row's inputs, fetched while this row is computed
+#pragma unroll
+    for (int kk = 0; kk < KMAX; ++kk) xn[kk] = (kk < k && r < n) ? X[r * ldx + xoff + kk] : (T)0;
+    for (; r < n; r += rstep) {
+        T xr[KMAX];
+#pragma unroll
+        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = xn[kk];
+        const size_t rn = r + rstep;
+#pragma unroll
+        for (int kk = 0; kk < KMAX; ++kk) xn[kk] = (kk < k && rn < n) ? X[rn * ldx + xoff + kk] : (T)0;
+        T* z = Z + r * ldz + (size_t)mdl * m;
+#pragma unroll
+        for (int c4 = 0; c4 < MMAX / 4; ++c4) {
+            if (c4 < mq) {
+                T a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+#pragma unroll
+                for (int kk = 0; kk < KMAX; ++kk)
+                    if (kk < k) {
+                        const vec4<T> w = wv[(kk * mq + c4) * TG];
+                        a0 = __builtin_fma(xr[kk], w.x, a0);
+                        a1 = __builtin_fma(xr[kk], w.y, a1);
+                        a2 = __builtin_fma(xr[kk], w.z, a2);
+                        a3 = __builtin_fma(xr[kk], w.w, a3);
+                    }
+                vec4<T>* zo = reinterpret_cast<vec4<T>*>(z) + c4;
+                if (accumulate) { const vec4<T> o = *zo; a0 += o.x; a1 += o.y; a2 += o.z; a3 += o.w; }
+                *zo = vec4<T>{a0, a1, a2, a3};
+            }
+        }
+    }
+}
+
+// dX[r, b*k + kk] = sum_c dZ[r, b*m + c] * W[(b*p + off + kk)*m + c]
+template <typename T, int KMAX, int MMAX>
+__global__ __launch_bounds__(256) void k_bdot_nt_tile(int nblock, size_t n, int m, int k, int p, int off,
+                                                      const T* __restrict__ dZ, const T* __restrict__ W, T* __restrict__ dX)
+{
+    extern __shared__ __align__(16) unsigned char tsm[];
+    T* ws = reinterpret_cast<T*>(tsm);
+    const unsigned g = threadIdx.x & (TG - 1), rl = threadIdx.x >> 4, m0 = blockIdx.x * TG, mdl = m0 + g;
+    stage_weights16(ws, W, nblock, m0, k, m, p, off);
+    __syncthreads();
+    if (mdl >= (unsigned)nblock) return;
+    const int mq = m >> 2;
+    const size_t ldx = (size_t)k * nblock, ldz = (size_t)m * nblock;
+    const vec4<T>* wv = reinterpret_cast<const vec4<T>*>(ws) + g;
+    const size_t rstep = (size_t)gridDim.y * 16;
+    size_t r = (size_t)blockIdx.y * 16 + rl;
+    vec4<T> dn[MMAX / 4];                                // next row's gradient, fetched while this row is computed
+#pragma unroll
+    for (int c4 = 0; c4 < MMAX / 4; ++c4)
+        dn[c4] = (c4 < mq && r < n) ? reinterpret_cast<const vec4<T>*>(dZ + r * ldz + (size_t)mdl * m)[c4] : vec4<T>{0, 0, 0, 0};
+    for (; r < n; r += rstep) {
+        vec4<T> d[MMAX / 4];
+#pragma unroll
+        for (int c4 = 0; c4 < MMAX / 4; ++c4) d[c4] = dn[c4];
+        const size_t rn = r + rstep;
+#pragma unroll
+        for (int c4 = 0; c4 < MMAX / 4; ++c4)
+            dn[c4] = (c4 < mq && rn < n) ? reinterpret_cast<const vec4<T>*>(dZ + rn * ldz + (size_t)mdl * m)[c4] : vec4<T>{0, 0, 0, 0};
+        T* dx = dX + r * ldx + (size_t)mdl * k;
+#pragma unroll
+        for (int kk = 0; kk < KMAX; ++kk) {
+            if (kk < k) {
+                T s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+#pragma unroll
+                for (int c4 = 0; c4 < MMAX / 4; ++c4)
+                    if (c4 < mq) {
+                        const vec4<T> w = wv[(kk * mq + c4) * TG];
+                        s0 = __builtin_fma(d[c4].x, w.x, s0);
+                        s1 = __builtin_fma(d[c4].y, w.y, s1);
+                        s2 = __builtin_fma(d[c4].z, w.z, s2);
+                        s3 = __builtin_fma(d[c4].w, w.w, s3);
+                    }
+                dx[kk] = (s0 + s1) + (s2 + s3);
+            }
+        }
+    }
+}
+
+// dW partial sums: workgroup (b, y) takes model b and row chunk y, stages 64 rows of the model's
+// X (64 x k) and dZ (64 x m) columns in LDS at a time, and thread e owns output elements e, e+256, ...
+// (rows ascending). k_bdot_tn_fold adds the chunks in ascending order.
+constexpr int TN_ROWS = 64, TN_CHUNK = 1024, TN_OWN = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void k_bdot_tn_tile(int nblock, size_t n, int m, int k, bool bcast,
+                                                      const T* __restrict__ X, const T* __restrict__ dZ, T* __restrict__ partial)
+{
+    extern __shared__ __align__(16) unsigned char tsm[];
+    const int ks = k | 1, ms = m | 1;                        // odd strides: no bank conflicts while staging
+    T* xs = reinterpret_cast<T*>(tsm);                       // [TN_ROWS][ks]
+    T* ds_ = xs + TN_ROWS * ks;                              // [TN_ROWS][ms]
+    const unsigned b = blockIdx.x;
+    const size_t ldx = (size_t)k * (bcast ? 1 : nblock), ldz = (size_t)m * nblock;
+    const size_t r0 = (size_t)blockIdx.y * TN_CHUNK;
+    const size_t r1 = r0 + TN_CHUNK < n ? r0 + TN_CHUNK : n;
+    const int nout = k * m;
+    T acc[TN_OWN];
+#pragma unroll
+    for (int i = 0; i < TN_OWN; ++i) acc[i] = (T)0;
+    for (size_t t0 = r0; t0 < r1; t0 += TN_ROWS) {
+        const int rows = (int)(r1 - t0 < (size_t)TN_ROWS ? r1 - t0 : (size_t)TN_ROWS);
+        __syncthreads();
+        for (int e = threadIdx.x; e < TN_ROWS * k; e += blockDim.x) {
+            const int rr = e / k, kk = e % k;
+            xs[rr * ks + kk] = rr < rows ? X[(t0 + rr) * ldx + (bcast ? 0 : (size_t)b * k) + kk] : (T)0;
+        }
+        for (int e = threadIdx.x; e < TN_ROWS * m; e += blockDim.x) {
+            const int rr = e / m, c = e % m;
+            ds_[rr * ms + c] = rr < rows ? dZ[(t0 + rr) * ldz + (size_t)b * m + c] : (T)0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TN_OWN; ++i) {
+            const int e = threadIdx.x + i * 256;
+            if (e < nout) {
+                const int kk = e / m, c = e % m;
+                T s = acc[i];
+#pragma unroll 8
+                for (int rr = 0; rr < TN_ROWS; ++rr) s = __builtin_fma(xs[rr * ks + kk], ds_[rr * ms + c], s);
+                acc[i] = s;
+            }
+        }
+    }
+    T* out = partial + ((size_t)blockIdx.y * nblock + b) * nout;
+#pragma unroll
+    for (int i = 0; i < TN_OWN; ++i) {
+        const int e = threadIdx.x + i * 256;
+        if (e < nout) out[e] = acc[i];
+    }
+}
+template <typename T>
+__global__ void k_bdot_tn_fold(int nblock, int m, int k, int p, int off, unsigned nchunk, const T* __restrict__ partial, T* __restrict__ dW)
+{
+    const size_t nout = (size_t)k * m, total = nout * nblock;
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+        const unsigned b = (unsigned)(e / nout), idx = (unsigned)(e % nout), kk = idx / m, c = idx % m;
+        T s = partial[e];
+#pragma unroll 8
+        for (unsigned y = 1; y < nchunk; ++y) s += partial[(size_t)y * total + e];
+        dW[((size_t)b * p + off + kk) * m + c] = s;
+    }
+}
+
 // Scoring head: a workgroup owns one model and a tile of 256 rows. The model's weights (a few KB)
 // are staged in LDS once and read back as wave-wide broadcasts; each thread keeps its row's k inputs
 // in registers (one contiguous k*4-byte read of HBM per thread) and writes one score.
@@ -230,6 +412,65 @@ __global__ __launch_bounds__(256) void k_head16(size_t n, int nblock, int k, int
     }
 }
 
+inline bool bulk_ok(int n, int m, int k) { return n >= 2048 && (m & 3) == 0 && m <= 64 && k <= 64; }
+
+// returns -1 when the shape does not fit the bulk kernel (the caller falls back), else the launch status
+template <typename T>
+int launch_bdot_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int off, bool bcast, bool accumulate,
+                     const T* X, const T* W, T* Z)
+{
+    const size_t smem = (size_t)k * m * TG * sizeof(T);
+    if (smem > 65536) return -1;
+    unsigned gy = dbk::divup((size_t)n, 16 * 32);
+    if (gy > 65535u) gy = 65535u;
+    const dim3 grid(dbk::divup(nblock, TG), gy);
+#define DBK_BDOT_CASE(KM, MM)                                                                                         \
+    if (k <= KM && m <= MM) {                                                                                         \
+        auto kern = k_bdot_tile<T, KM, MM>;                                                                           \
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -1; \
+        hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, nblock, (size_t)n, m, k, p, off, bcast, accumulate, X, W, Z); \
+        return 0;                                                                                                     \
+    }
+    DBK_BDOT_CASE(16, 32) DBK_BDOT_CASE(32, 32) DBK_BDOT_CASE(64, 32) DBK_BDOT_CASE(16, 64) DBK_BDOT_CASE(32, 64) DBK_BDOT_CASE(64, 64)
+#undef DBK_BDOT_CASE
+    return -1;
+}
+
+template <typename T>
+int launch_bdot_nt_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int off, const T* dZ, const T* W, T* dX)
+{
+    const size_t smem = (size_t)k * m * TG * sizeof(T);
+    if (smem > 65536) return -1;
+    unsigned gy = dbk::divup((size_t)n, 16 * 32);
+    if (gy > 65535u) gy = 65535u;
+    const dim3 grid(dbk::divup(nblock, TG), gy);
+#define DBK_BDOT_CASE(KM, MM)                                                                                         \
+    if (k <= KM && m <= MM) {                                                                                         \
+        auto kern = k_bdot_nt_tile<T, KM, MM>;                                                                        \
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -1; \
+        hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, nblock, (size_t)n, m, k, p, off, dZ, W, dX);             \
+        return 0;                                                                                                     \
+    }
+    DBK_BDOT_CASE(16, 32) DBK_BDOT_CASE(32, 32) DBK_BDOT_CASE(64, 32) DBK_BDOT_CASE(16, 64) DBK_BDOT_CASE(32, 64) DBK_BDOT_CASE(64, 64)
+#undef DBK_BDOT_CASE
+    return -1;
+}
+
+template <typename T>
+int launch_bdot_tn_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int off, bool bcast, const T* X, const T* dZ, T* dW)
+{
+    const unsigned nchunk = dbk::divup((size_t)n, TN_CHUNK);
+    const size_t nout = (size_t)k * m * nblock;
+    T* partial = (T*)dbk::workspace(nout * nchunk * sizeof(T), st);
+    if (!partial) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", nout * nchunk * sizeof(T)); return 1; }
+    const size_t smem = (size_t)TN_ROWS * ((k | 1) + (m | 1)) * sizeof(T);
+    auto kern = k_bdot_tn_tile<T>;
+    hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(kern, dim3(nblock, nchunk), dim3(256), smem, st, nblock, (size_t)n, m, k, bcast, X, dZ, partial);
+    hipLaunchKernelGGL(k_bdot_tn_fold<T>, dim3(dbk::ew_grid(nout)), dim3(256), 0, st, nblock, m, k, p, off, nchunk, (const T*)partial, dW);
+    return 0;
+}
+
 int check_dims(int nblock, int n, int m, int k, int p, int off)
 {
     DBK_CHECK(nblock >= 1, "ValueError: nblock must be >= 1, got %d", nblock);
@@ -249,6 +490,12 @@ int dbk_blockwise_dot_combined(dbk_stream_t stream, int dtype, int nblock, int X
     if (check_dims(nblock, n, m, k, p, Xoffset)) return 1;
     if (n == 0 || m == 0 || k == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(X && W && Z, "ValueError: null pointer argument");
+    if (bulk_ok(n, m, k)) {
+        const int rc = dtype == DBK_F32
+            ? launch_bdot_tile<float>(dbk::as_stream(stream), nblock, n, m, k, p, Xoffset, Xbroadcast != 0, Xoffset != 0, (const float*)X, (const float*)W, (float*)Z)
+            : launch_bdot_tile<double>(dbk::as_stream(stream), nblock, n, m, k, p, Xoffset, Xbroadcast != 0, Xoffset != 0, (const double*)X, (const double*)W, (double*)Z);
+        if (rc >= 0) { if (rc) return rc; DBK_LAUNCH_OK(); }
+    }
     size_t total = (size_t)n * m * nblock;
     if (dtype == DBK_F32)
         hipLaunchKernelGGL(k_bdot<float>, dim3(dbk::ew_grid(total)), dim3(256), 0, dbk::as_stream(stream), nblock, (size_t)n, m, k, p,
@@ -272,6 +519,12 @@ int dbk_blockwise_dot_nt_combined(dbk_stream_t stream, int dtype, int nblock, in
     if (check_dims(nblock, n, m, k, p, Xoffset)) return 1;
     if (n == 0 || m == 0 || k == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(dX && W && dZ, "ValueError: null pointer argument");
+    if (bulk_ok(n, m, k)) {
+        const int rc = dtype == DBK_F32
+            ? launch_bdot_nt_tile<float>(dbk::as_stream(stream), nblock, n, m, k, p, Xoffset, (const float*)dZ, (const float*)W, (float*)dX)
+            : launch_bdot_nt_tile<double>(dbk::as_stream(stream), nblock, n, m, k, p, Xoffset, (const double*)dZ, (const double*)W, (double*)dX);
+        if (rc >= 0) { if (rc) return rc; DBK_LAUNCH_OK(); }
+    }
     size_t total = (size_t)n * k * nblock;
     if (dtype == DBK_F32)
         hipLaunchKernelGGL(k_bdot_nt<float>, dim3(dbk::ew_grid(total)), dim3(256), 0, dbk::as_stream(stream), nblock, (size_t)n, m, k, p,
@@ -295,6 +548,13 @@ int dbk_blockwise_dot_tn_combined(dbk_stream_t stream, int dtype, int nblock, in
     if (check_dims(nblock, n, m, k, p, Xoffset)) return 1;
     if (n == 0 || m == 0 || k == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(X && dW && dZ, "ValueError: null pointer argument");
+    if (n >= 2048 && k * m <= 256 * TN_OWN) {
+        const int rc = dtype == DBK_F32
+            ? launch_bdot_tn_tile<float>(dbk::as_stream(stream), nblock, n, m, k, p, Xoffset, Xbroadcast != 0, (const float*)X, (const float*)dZ, (float*)dW)
+            : launch_bdot_tn_tile<double>(dbk::as_stream(stream), nblock, n, m, k, p, Xoffset, Xbroadcast != 0, (const double*)X, (const double*)dZ, (double*)dW);
+        if (rc) return rc;
+        DBK_LAUNCH_OK();
+    }
     size_t total = (size_t)nblock * k * m;                 // one wave per element
     unsigned grid = dbk::divup(total, 4);
     if (grid > 256u * 16u) grid = 256u * 16u;

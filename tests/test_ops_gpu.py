@@ -316,6 +316,36 @@ def test_head_fprop_bulk_rows(ds, k, h, nb):
     assert_close(host(got), ref, ACT, "probabilities")
 
 
+@pytest.mark.parametrize("n,k,m,nb,dtype", [(2048, 16, 32, 7, np.float32), (5003, 32, 4, 33, np.float32), (3000, 16, 1, 5, np.float32),
+                                            (2500, 64, 64, 3, np.float32), (2100, 16, 32, 18, np.float64), (2049, 5, 12, 16, np.float32)])
+def test_blockwise_dot_family_bulk_rows(ds, n, k, m, nb, dtype):
+    """Row counts that take the bulk kernels (16 models per workgroup; chunked weight gradient), model counts
+    off the group size, output widths that are / are not multiples of four (the latter fall back), float64."""
+    rng = np.random.default_rng(n + k + m)
+    tol = ACT if dtype == np.float32 else 1e-12
+    X = rng.standard_normal((n, k * nb)).astype(dtype)
+    W = rng.standard_normal((k * nb, m)).astype(dtype)
+    dZ = rng.standard_normal((n, m * nb)).astype(dtype)
+    X64, W64, dZ64 = X.astype(np.float64), W.astype(np.float64), dZ.astype(np.float64)
+    assert_close(host(ds.blockwise_dot(dev(X), dev(W), nb)), orc.blockwise_dot(X64, W64, nb), tol, "Z")
+    assert_close(host(ds.blockwise_dot_nt(dev(dZ), dev(W), nb)), orc.blockwise_dot_nt(dZ64, W64, nb), tol * 10, "dX")
+    got = host(ds.blockwise_dot_tn(dev(X), dev(dZ), nb, dev(W)))
+    assert_close(got, orc.blockwise_dot_tn(X64, dZ64, nb, W64), tol * 10, "dW")
+    assert np.array_equal(got, host(ds.blockwise_dot_tn(dev(X), dev(dZ), nb, dev(W))))
+    # combined: conv features + a shared feature block
+    k2 = 8
+    X2 = rng.standard_normal((n, k2)).astype(dtype)
+    Wc = rng.standard_normal(((k + k2) * nb, m)).astype(dtype)
+    Xl, bc = [X, X2], [False, True]
+    assert_close(host(ds.blockwise_dot_combined([dev(X), dev(X2)], dev(Wc), nb, bc)),
+                 orc.blockwise_dot_combined([X64, X2.astype(np.float64)], Wc.astype(np.float64), nb, bc), tol * 3, "Zc")
+    dXs = ds.blockwise_dot_nt_combined([dev(X), dev(X2)], dev(dZ), dev(Wc), nb, bc)
+    dXr = orc.blockwise_dot_nt_combined([X64, X2.astype(np.float64)], dZ64, Wc.astype(np.float64), nb, bc)
+    assert_close(host(dXs[0]), dXr[0], tol * 10, "dX combined")
+    dWc = host(ds.blockwise_dot_tn_combined([dev(X), dev(X2)], dev(dZ), dev(Wc), nb, bc))
+    assert_close(dWc, orc.blockwise_dot_tn_combined([X64, X2.astype(np.float64)], dZ64, Wc.astype(np.float64), nb, bc), tol * 10, "dW combined")
+
+
 # ------------------------------------------------------------------------------------------ elementwise / optimiser
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_gradstep_and_madd_bcast(ds, dtype):
