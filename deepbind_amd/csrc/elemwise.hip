@@ -55,26 +55,88 @@ template <typename T> __global__ void k_calc_zmask(const T* Z, uint8_t* M, size_
 template <typename T> __global__ void k_dropout_fp_tr(const T* X, const T* rate, T* Z, uint8_t* M, size_t n, size_t m, size_t k,
                                                       const float* U, uint64_t seed, uint64_t offset)
 {
-    GRID_STRIDE(i, n) {
-        T p = rate[(i / k) % m];
-        float u = U ? U[i] : uniform_at(seed, offset, i);
-        bool keep = (T)u >= p;
-        M[i] = keep;
-        Z[i] = X[i] * (T)keep;
+    // a thread takes four consecutive elements: they share one call of the generator, and (when the arrays
+    // allow it) one 16-byte load, one 16-byte store and one 4-byte mask store
+    const bool vec = sizeof(T) == 4 && (n & 3) == 0 && ((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Z)) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(M) & 3) == 0 && (!U || (reinterpret_cast<uintptr_t>(U) & 15) == 0);
+    GRID_STRIDE(q, (n + 3) / 4) {
+        float u4[4];
+        if (!U) dbk_rng::uniform4_at(seed, offset, q, u4);
+        if (vec) {
+            if (U) { const float4 uu = reinterpret_cast<const float4*>(U)[q]; u4[0] = uu.x; u4[1] = uu.y; u4[2] = uu.z; u4[3] = uu.w; }
+            const float4 x = reinterpret_cast<const float4*>(X)[q];
+            const float xs[4] = {x.x, x.y, x.z, x.w};
+            float zs[4];
+            unsigned mk = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const size_t i = 4 * q + j;
+                const bool keep = (T)u4[j] >= rate[(i / k) % m];
+                mk |= (unsigned)keep << (8 * j);
+                zs[j] = xs[j] * (float)keep;
+            }
+            reinterpret_cast<float4*>(Z)[q] = make_float4(zs[0], zs[1], zs[2], zs[3]);
+            reinterpret_cast<unsigned*>(M)[q] = mk;
+            continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const size_t i = 4 * q + j;
+            if (i < n) {
+                T p = rate[(i / k) % m];
+                float u = U ? U[i] : u4[j];
+                bool keep = (T)u >= p;
+                M[i] = keep;
+                Z[i] = X[i] * (T)keep;
+            }
+        }
     }
 }
 template <typename T> __global__ void k_dropout_fp_tr_match(const T* X, const T* rate, T* Z, uint8_t* M, size_t nrow, size_t ncol,
                                                             size_t k, const float* U, uint64_t seed, uint64_t offset)
 {
-    GRID_STRIDE(i, nrow * ncol / 2) {
-        size_t row = (i / ncol) * 2, col = i % ncol;
-        T p = rate[col / k];
-        size_t i0 = row * ncol + col, i1 = i0 + ncol;
-        float u = U ? U[i0] : uniform_at(seed, offset, i);
-        bool keep = (T)u >= p;
-        M[i0] = keep; M[i1] = keep;
-        Z[i0] = X[i0] * (T)keep;
-        Z[i1] = X[i1] * (T)keep;
+    const size_t npair = nrow * ncol / 2;
+    const bool vec = sizeof(T) == 4 && (ncol & 3) == 0 && ((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Z)) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(M) & 3) == 0;
+    GRID_STRIDE(q, (npair + 3) / 4) {
+        float u4[4];
+        if (!U) dbk_rng::uniform4_at(seed, offset, q, u4);
+        if (vec) {
+            // four consecutive pair indices are four consecutive columns of one row pair
+            const size_t i = 4 * q, row = (i / ncol) * 2, col = i % ncol, i0 = row * ncol + col, i1 = i0 + ncol;
+            if (U) { u4[0] = U[i0]; u4[1] = U[i0 + 1]; u4[2] = U[i0 + 2]; u4[3] = U[i0 + 3]; }
+            const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(X) + i0);
+            const float4 b = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(X) + i1);
+            const float as[4] = {a.x, a.y, a.z, a.w}, bs[4] = {b.x, b.y, b.z, b.w};
+            float za[4], zb[4];
+            unsigned mk = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool keep = (T)u4[j] >= rate[(col + j) / k];
+                mk |= (unsigned)keep << (8 * j);
+                za[j] = as[j] * (float)keep;
+                zb[j] = bs[j] * (float)keep;
+            }
+            *reinterpret_cast<float4*>(reinterpret_cast<float*>(Z) + i0) = make_float4(za[0], za[1], za[2], za[3]);
+            *reinterpret_cast<float4*>(reinterpret_cast<float*>(Z) + i1) = make_float4(zb[0], zb[1], zb[2], zb[3]);
+            *reinterpret_cast<unsigned*>(M + i0) = mk;
+            *reinterpret_cast<unsigned*>(M + i1) = mk;
+            continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const size_t i = 4 * q + j;                    // pair index: the draw both rows of a pair share
+            if (i < npair) {
+                size_t row = (i / ncol) * 2, col = i % ncol;
+                T p = rate[col / k];
+                size_t i0 = row * ncol + col, i1 = i0 + ncol;
+                float u = U ? U[i0] : u4[j];
+                bool keep = (T)u >= p;
+                M[i0] = keep; M[i1] = keep;
+                Z[i0] = X[i0] * (T)keep;
+                Z[i1] = X[i1] * (T)keep;
+            }
+        }
     }
 }
 template <typename T> __global__ void k_dropout_scale(const T* X, const T* rate, T* Z, size_t n, size_t m, size_t k)
@@ -89,12 +151,36 @@ __global__ void k_dropoutord(const uint8_t* X, uint8_t* Z, uint8_t* M, size_t n,
                              const unsigned long long* counter)
 {
     if (counter) offset = counter[0];
-    GRID_STRIDE(i, n) {
-        float u = U ? U[i] : uniform_at(seed, offset, i);
-        uint8_t x = X[i];
-        bool mask = x == 255 || u >= rate;                  // padding always passes (and reports "kept")
-        M[i] = mask;
-        Z[i] = mask ? x : (uint8_t)254;
+    GRID_STRIDE(q, (n + 3) / 4) {
+        float u4[4];
+        if (!U) dbk_rng::uniform4_at(seed, offset, q, u4);
+        if (4 * q + 3 < n && ((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Z) | reinterpret_cast<uintptr_t>(M)) & 3) == 0) {
+            // four letters per 32-bit word
+            const unsigned xw = reinterpret_cast<const unsigned*>(X)[q];
+            unsigned zw = 0, mw = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const unsigned x = (xw >> (8 * j)) & 0xffu;
+                const float u = U ? U[4 * q + j] : u4[j];
+                const bool mask = x == 255u || u >= rate;
+                mw |= (unsigned)mask << (8 * j);
+                zw |= (mask ? x : 254u) << (8 * j);
+            }
+            reinterpret_cast<unsigned*>(Z)[q] = zw;
+            reinterpret_cast<unsigned*>(M)[q] = mw;
+            continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const size_t i = 4 * q + j;
+            if (i < n) {
+                float u = U ? U[i] : u4[j];
+                uint8_t x = X[i];
+                bool mask = x == 255 || u >= rate;          // padding always passes (and reports "kept")
+                M[i] = mask;
+                Z[i] = mask ? x : (uint8_t)254;
+            }
+        }
     }
 }
 // One workgroup per (fwd, rev) pair of regions: the reverse strand drops the mirrored letters of the
@@ -199,7 +285,17 @@ template <typename T> __global__ void k_loss_terms(int kind, const T* Z, const T
 }
 __global__ void k_uniform_fill(float* U, size_t n, uint64_t seed, uint64_t offset)
 {
-    GRID_STRIDE(i, n) U[i] = uniform_at(seed, offset, i);
+    GRID_STRIDE(q, (n + 3) / 4) {
+        float u4[4];
+        dbk_rng::uniform4_at(seed, offset, q, u4);
+        if (4 * q + 3 < n && (reinterpret_cast<uintptr_t>(U) & 15) == 0) {
+            reinterpret_cast<float4*>(U)[q] = make_float4(u4[0], u4[1], u4[2], u4[3]);
+            continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (4 * q + j < n) U[4 * q + j] = u4[j];
+    }
 }
 // Standard normals by Box-Muller from two independent Philox streams (third counter word 0 / 1), one value
 // per element so that element i depends only on (seed, offset, i).
@@ -213,15 +309,19 @@ template <typename T> __global__ void k_l1_decay(const T* P, const T* decay, T* 
 }
 template <typename T> __global__ void k_normal_fill(T* Z, size_t n, uint64_t seed, uint64_t offset)
 {
-    GRID_STRIDE(i, n) {
-        const uint64_t ctr = offset + (uint64_t)(i >> 2);
+    GRID_STRIDE(q, (n + 3) / 4) {
+        const uint64_t ctr = offset + (uint64_t)q;
         uint32_t a[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u};
         uint32_t b[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 1u, 0u};
         philox4x32_10(a, (uint32_t)seed, (uint32_t)(seed >> 32));
         philox4x32_10(b, (uint32_t)seed, (uint32_t)(seed >> 32));
-        const float u1 = ((float)(a[i & 3] >> 8) + 1.0f) * (1.0f / 16777216.0f);      // (0, 1]
-        const float u2 = (float)(b[i & 3] >> 8) * (1.0f / 16777216.0f);               // [0, 1)
-        Z[i] = (T)(sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const size_t i = 4 * q + j;
+            const float u1 = ((float)(a[j] >> 8) + 1.0f) * (1.0f / 16777216.0f);      // (0, 1]
+            const float u2 = (float)(b[j] >> 8) * (1.0f / 16777216.0f);               // [0, 1)
+            if (i < n) Z[i] = (T)(sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2));
+        }
     }
 }
 __global__ void k_counter_add(unsigned long long* ctr, unsigned long long delta) { if (threadIdx.x == 0 && blockIdx.x == 0) ctr[0] += delta; }

@@ -31,4 +31,14 @@ __device__ inline float uniform_at(uint64_t seed, uint64_t offset, size_t i)
     return (float)(c[i & 3] >> 8) * (1.0f / 16777216.0f);
 }
 
+// The four uniforms of flat elements 4q .. 4q+3 (one generator call).
+__device__ inline void uniform4_at(uint64_t seed, uint64_t offset, size_t q, float u[4])
+{
+    uint64_t ctr = offset + (uint64_t)q;
+    uint32_t c[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u};
+    philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) u[j] = (float)(c[j] >> 8) * (1.0f / 16777216.0f);
+}
+
 }  // namespace dbk_rng
