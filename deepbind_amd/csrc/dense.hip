@@ -84,6 +84,9 @@ constexpr int TG = 16;
 
 template <typename T> struct alignas(4 * sizeof(T)) vec4 { T x, y, z, w; };
 
+__device__ __forceinline__ float fma_t(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_t(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
 template <typename T>
 __device__ void stage_weights16(T* ws, const T* __restrict__ W, int nblock, unsigned m0, int k, int m, int p, int off)
 {
@@ -131,10 +134,10 @@ __global__ __launch_bounds__(256) void k_bdot_tile(int nblock, size_t n, int m, 
                 for (int kk = 0; kk < KMAX; ++kk)
                     if (kk < k) {
                         const vec4<T> w = wv[(kk * mq + c4) * TG];
-                        a0 = __builtin_fma(xr[kk], w.x, a0);
-                        a1 = __builtin_fma(xr[kk], w.y, a1);
-                        a2 = __builtin_fma(xr[kk], w.z, a2);
-                        a3 = __builtin_fma(xr[kk], w.w, a3);
+                        a0 = fma_t(xr[kk], w.x, a0);
+                        a1 = fma_t(xr[kk], w.y, a1);
+                        a2 = fma_t(xr[kk], w.z, a2);
+                        a3 = fma_t(xr[kk], w.w, a3);
                     }
                 vec4<T>* zo = reinterpret_cast<vec4<T>*>(z) + c4;
                 if (accumulate) { const vec4<T> o = *zo; a0 += o.x; a1 += o.y; a2 += o.z; a3 += o.w; }
@@ -181,14 +184,65 @@ __global__ __launch_bounds__(256) void k_bdot_nt_tile(int nblock, size_t n, int 
                 for (int c4 = 0; c4 < MMAX / 4; ++c4)
                     if (c4 < mq) {
                         const vec4<T> w = wv[(kk * mq + c4) * TG];
-                        s0 = __builtin_fma(d[c4].x, w.x, s0);
-                        s1 = __builtin_fma(d[c4].y, w.y, s1);
-                        s2 = __builtin_fma(d[c4].z, w.z, s2);
-                        s3 = __builtin_fma(d[c4].w, w.w, s3);
+                        s0 = fma_t(d[c4].x, w.x, s0);
+                        s1 = fma_t(d[c4].y, w.y, s1);
+                        s2 = fma_t(d[c4].z, w.z, s2);
+                        s3 = fma_t(d[c4].w, w.w, s3);
                     }
                 dx[kk] = (s0 + s1) + (s2 + s3);
             }
         }
+    }
+}
+
+// Row-tile kernel shared by dot and dot_nt when the output width per model `no` is 4, 8, 16, 32 or 64:
+// out[r, b*no + o] (+)= sum_i in[r, inbase(b) + i] * w_b[i][o]. no/4 adjacent lanes share one (row, model)
+// and own four outputs each, so a wave stores whole contiguous row segments (16 bytes per lane, lanes
+// adjacent) and the 16 lanes of a quarter-wave read one aligned 256-byte line of the weights, which sit
+// in LDS as [input][model][output]. `transpose` stages w_b[i][o] = W_b[o][i] (the dot_nt case).
+template <typename T, int IMAX>
+__global__ __launch_bounds__(256) void k_bdot_rowtile(int nblock, size_t n, int ni, int no, bool bcast, bool accumulate, bool transpose,
+                                                      int m, int p, int off,
+                                                      const T* __restrict__ in, const T* __restrict__ W, T* __restrict__ out)
+{
+    extern __shared__ __align__(16) unsigned char tsm[];
+    T* ws = reinterpret_cast<T*>(tsm);                                     // [ni][TG][no]
+    const unsigned m0 = blockIdx.x * TG;
+    for (int e = threadIdx.x; e < ni * TG * no; e += blockDim.x) {
+        const int o = e % no, g = (e / no) % TG, i = e / (no * TG);
+        const unsigned mdl = m0 + g;
+        // W_b is (k rows = inputs of dot, m columns); dot: (i, o) = (row, col); dot_nt: (i, o) = (col, row)
+        const size_t src = transpose ? ((size_t)mdl * p + off + o) * m + i : ((size_t)mdl * p + off + i) * m + o;
+        ws[e] = mdl < (unsigned)nblock ? W[src] : (T)0;
+    }
+    __syncthreads();
+    const int lpm = no >> 2;                                               // lanes per (row, model)
+    const unsigned j = threadIdx.x % lpm, pm = threadIdx.x / lpm, g = pm % TG, rl = pm / TG;
+    const unsigned rpp = 256 / (lpm * TG);                                 // rows per pass
+    const unsigned mdl = m0 + g;
+    if (mdl >= (unsigned)nblock) return;
+    const size_t ldin = (size_t)ni * (bcast ? 1 : nblock), ldout = (size_t)no * nblock;
+    const size_t inoff = bcast ? 0 : (size_t)mdl * ni;
+    const vec4<T>* wv = reinterpret_cast<const vec4<T>*>(ws + (size_t)g * no) + j;
+    const int wstep = TG * no / 4;                                         // vec4 stride between inputs
+    for (size_t r = (size_t)blockIdx.y * rpp + rl; r < n; r += (size_t)gridDim.y * rpp) {
+        const T* x = in + r * ldin + inoff;
+        T xr[IMAX];
+#pragma unroll
+        for (int i = 0; i < IMAX; ++i) xr[i] = i < ni ? x[i] : (T)0;
+        T a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+#pragma unroll
+        for (int i = 0; i < IMAX; ++i)
+            if (i < ni) {
+                const vec4<T> w = wv[i * wstep];
+                a0 = fma_t(xr[i], w.x, a0);
+                a1 = fma_t(xr[i], w.y, a1);
+                a2 = fma_t(xr[i], w.z, a2);
+                a3 = fma_t(xr[i], w.w, a3);
+            }
+        vec4<T>* zo = reinterpret_cast<vec4<T>*>(out + r * ldout + (size_t)mdl * no) + j;
+        if (accumulate) { const vec4<T> o = *zo; a0 += o.x; a1 += o.y; a2 += o.z; a3 += o.w; }
+        *zo = vec4<T>{a0, a1, a2, a3};
     }
 }
 
@@ -231,7 +285,7 @@ __global__ __launch_bounds__(256) void k_bdot_tn_tile(int nblock, size_t n, int 
                 const int kk = e / m, c = e % m;
                 T s = acc[i];
 #pragma unroll 8
-                for (int rr = 0; rr < TN_ROWS; ++rr) s = __builtin_fma(xs[rr * ks + kk], ds_[rr * ms + c], s);
+                for (int rr = 0; rr < TN_ROWS; ++rr) s = fma_t(xs[rr * ks + kk], ds_[rr * ms + c], s);
                 acc[i] = s;
             }
         }
@@ -412,17 +466,45 @@ __global__ __launch_bounds__(256) void k_head16(size_t n, int nblock, int k, int
     }
 }
 
+// Row-slice count for the kernels that stage 16 models' weights per workgroup: about 1024 workgroups in all
+// (a few per CU), so that staging is paid once per many rows.
+inline unsigned row_slices(size_t n, unsigned rows_per_pass, unsigned ngroups)
+{
+    unsigned cap = 1024u / (ngroups ? ngroups : 1u);
+    if (cap < 1) cap = 1;
+    unsigned gy = dbk::divup(n, rows_per_pass);
+    if (gy > cap) gy = cap;
+    if (gy > 65535u) gy = 65535u;
+    return gy < 1 ? 1 : gy;
+}
+
 inline bool bulk_ok(int n, int m, int k) { return n >= 2048 && (m & 3) == 0 && m <= 64 && k <= 64; }
 
 // returns -1 when the shape does not fit the bulk kernel (the caller falls back), else the launch status
 template <typename T>
+int launch_rowtile(hipStream_t st, int nblock, int n, int ni, int no, bool bcast, bool accumulate, bool transpose, int m, int p, int off,
+                   const T* in, const T* W, T* out)
+{
+    if (!(no == 4 || no == 8 || no == 16 || no == 32 || no == 64) || ni > 64) return -1;
+    const size_t smem = (size_t)ni * no * TG * sizeof(T);
+    if (smem > 65536) return -1;
+    const unsigned rpp = 256 / ((no / 4) * TG);
+    const unsigned gy = row_slices((size_t)n, rpp, dbk::divup(nblock, TG));
+    const dim3 grid(dbk::divup(nblock, TG), gy);
+    auto kern = ni <= 16 ? k_bdot_rowtile<T, 16> : (ni <= 32 ? k_bdot_rowtile<T, 32> : k_bdot_rowtile<T, 64>);
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -1;
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, nblock, (size_t)n, ni, no, bcast, accumulate, transpose, m, p, off, in, W, out);
+    return 0;
+}
+
+template <typename T>
 int launch_bdot_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int off, bool bcast, bool accumulate,
                      const T* X, const T* W, T* Z)
 {
+    if (launch_rowtile<T>(st, nblock, n, k, m, bcast, accumulate, false, m, p, off, X, W, Z) == 0) return 0;
     const size_t smem = (size_t)k * m * TG * sizeof(T);
     if (smem > 65536) return -1;
-    unsigned gy = dbk::divup((size_t)n, 16 * 32);
-    if (gy > 65535u) gy = 65535u;
+    const unsigned gy = row_slices((size_t)n, 16, dbk::divup(nblock, TG));
     const dim3 grid(dbk::divup(nblock, TG), gy);
 #define DBK_BDOT_CASE(KM, MM)                                                                                         \
     if (k <= KM && m <= MM) {                                                                                         \
@@ -439,10 +521,10 @@ int launch_bdot_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int
 template <typename T>
 int launch_bdot_nt_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int off, const T* dZ, const T* W, T* dX)
 {
+    if (launch_rowtile<T>(st, nblock, n, m, k, false, false, true, m, p, off, dZ, W, dX) == 0) return 0;
     const size_t smem = (size_t)k * m * TG * sizeof(T);
     if (smem > 65536) return -1;
-    unsigned gy = dbk::divup((size_t)n, 16 * 32);
-    if (gy > 65535u) gy = 65535u;
+    const unsigned gy = row_slices((size_t)n, 16, dbk::divup(nblock, TG));
     const dim3 grid(dbk::divup(nblock, TG), gy);
 #define DBK_BDOT_CASE(KM, MM)                                                                                         \
     if (k <= KM && m <= MM) {                                                                                         \
@@ -591,8 +673,7 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
     const size_t smem16 = ((size_t)k * hidden + 2 * (size_t)hidden) * HG * sizeof(float);
     if (hidden > 0 && (hidden & 3) == 0 && smem16 <= 65536 && n >= 4096) {
         // bulk scoring: 16 models per workgroup, coalesced reads of the feature matrix
-        unsigned gy = dbk::divup(n, 16 * 32);                // each workgroup makes ~32 passes with its staged weights
-        if (gy > 65535u) gy = 65535u;
+        const unsigned gy = row_slices(n, 16, dbk::divup(nblock, HG));
         auto kern16 = k <= 16 ? k_head16<16> : (k <= 32 ? k_head16<32> : k_head16<64>);
         DBK_HIP(hipFuncSetAttribute((const void*)kern16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem16));
         hipLaunchKernelGGL(kern16, dim3(dbk::divup(nblock, HG), gy), dim3(256), smem16, dbk::as_stream(stream), n, nblock, k, hidden, pooled,
