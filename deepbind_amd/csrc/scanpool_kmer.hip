@@ -55,33 +55,48 @@ constexpr int KPAD = 128;            // index bytes readable past the end of the
 
 __device__ __forceinline__ unsigned letter5(unsigned code) { return code < 4u ? code : 4u; }
 
-// flag[0] = 1 if a region is reversed or reaches past row ndef, the last row the scan defines
-// (the fast kernel then stands down)
-__global__ void check_regions_kernel(const uint32_t* __restrict__ R, size_t P, size_t ndef, unsigned* flag)
-{
-    __shared__ unsigned bad;
-    if (threadIdx.x == 0) bad = 0;
-    __syncthreads();
-    unsigned mine = 0;
-    for (size_t r = threadIdx.x; r < P; r += blockDim.x)
-        if (R[2 * r + 1] < R[2 * r] || R[2 * r + 1] > ndef) mine = 1;
-    if (mine) atomicOr(&bad, 1u);
-    __syncthreads();
-    if (threadIdx.x == 0) flag[0] = bad;
-}
+__global__ void clear_flag_kernel(unsigned* flag) { flag[0] = 0; }
 
 // K[t] = 25*l(X[t]) + 5*l(X[t+1]) + l(X[t+2]) for t < N + KPAD, reading past the end as N (letter 4).
-// Sets flag[0] when a code 254 ("contributes nothing") is present: the table has no letter for it.
-__global__ __launch_bounds__(256) void kmer_index_kernel(const uint8_t* __restrict__ X, size_t N, uint8_t* __restrict__ K, unsigned* flag)
+// Sets flag[0] (cleared beforehand) when the table kernel must stand down: a code 254 ("contributes
+// nothing") is present, for which the table has no letter, or a region is reversed or reaches past
+// row ndef, the last row the scan defines. A thread makes four indices from two aligned 32-bit loads.
+__global__ __launch_bounds__(256) void kmer_index_kernel(const uint8_t* __restrict__ X, size_t N, uint8_t* __restrict__ K, unsigned* flag,
+                                                         const uint32_t* __restrict__ R, size_t P, size_t ndef)
 {
-    const size_t total = N + KPAD;
-    unsigned saw = 0;
-    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (size_t)gridDim.x * blockDim.x) {
+    const size_t total = N + KPAD;                       // a multiple of 4 is not required: the tail is done bytewise
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nthread = (size_t)gridDim.x * blockDim.x;
+    unsigned bad = 0;
+    for (size_t r = tid; r < P; r += nthread) {
+        const uint2 ab = reinterpret_cast<const uint2*>(R)[r];
+        bad |= (ab.y < ab.x || ab.y > ndef);
+    }
+    const bool aligned = (reinterpret_cast<uintptr_t>(X) & 3) == 0 && (reinterpret_cast<uintptr_t>(K) & 3) == 0;
+    const size_t nquad = aligned ? total / 4 : 0;
+    const size_t nword = (N + 3) / 4;                    // 32-bit words of X that may be read
+    for (size_t q = tid; q < nquad; q += nthread) {
+        unsigned w0 = q < nword ? reinterpret_cast<const unsigned*>(X)[q] : 0xffffffffu;
+        unsigned w1 = q + 1 < nword ? reinterpret_cast<const unsigned*>(X)[q + 1] : 0xffffffffu;
+        unsigned l[6];
+#pragma unroll
+        for (int j = 0; j < 6; ++j) {
+            const size_t t = 4 * q + j;
+            unsigned c = ((j < 4 ? w0 : w1) >> (8 * (j & 3))) & 0xffu;
+            if (t >= N) c = 255u;                        // bytes of the last word past the end of the stream
+            bad |= (j < 4 && c == 254u);
+            l[j] = letter5(c);
+        }
+        unsigned out = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) out |= (25u * l[j] + 5u * l[j + 1] + l[j + 2]) << (8 * j);
+        reinterpret_cast<unsigned*>(K)[q] = out;
+    }
+    for (size_t t = 4 * nquad + tid; t < total; t += nthread) {
         unsigned c0 = t < N ? X[t] : 255u, c1 = t + 1 < N ? X[t + 1] : 255u, c2 = t + 2 < N ? X[t + 2] : 255u;
-        saw |= (c0 == 254u);
+        bad |= (c0 == 254u);
         K[t] = (uint8_t)(25u * letter5(c0) + 5u * letter5(c1) + letter5(c2));
     }
-    if (saw) atomicOr(flag, 1u);
+    if (bad) atomicOr(flag, 1u);
 }
 
 // Value of `v` held by lane `src` of the caller's row of 16 lanes (DPP row_share, folded by the
@@ -290,8 +305,8 @@ int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size
     unsigned* flag = (unsigned*)ws;
     uint8_t* K = ws + 256;
     const size_t ndef = N + 1 >= m + 1 ? N - m + 1 : 0;          // rows the scan defines
-    hipLaunchKernelGGL(check_regions_kernel, dim3(1), dim3(1024), 0, st, R, P, ndef, flag);
-    hipLaunchKernelGGL(kmer_index_kernel, dim3(dbk::ew_grid(N + KPAD)), dim3(256), 0, st, X, N, K, flag);
+    hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, st, flag);
+    hipLaunchKernelGGL(kmer_index_kernel, dim3(dbk::ew_grid((N + KPAD) / 4 + 1)), dim3(256), 0, st, X, N, K, flag, R, P, ndef);
     int G = (int)((m + 2) / 3);
     G += G & 1;
     int rc;
