@@ -187,6 +187,10 @@ def ops_throughput(reps=5):
         rec("scanpool_bprop[%s]" % pt, timed(lambda: ks.scanpool_bprop(W, b, X, R, pt, P, I, dP, dW, db, overwrite=True)),
             N + 2 * nout + B * F * 4, adds if pt == "all" else float(B) * F * m)
     rec("scanpool_fprop table[max]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "max", path="kmer")), N + B * F * 4, adds)
+    rec("scanpool_fprop table[max, argmax]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "max", want_argmax=True, path="kmer")),
+        N + 2 * B * F * 4, adds)
+    rec("scanpool_fprop table[all, argmax]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "all", want_argmax=True, path="kmer")),
+        N + 3 * B * F * 4, adds)
     del X, R, W, b, dW, db, dX, P, I, dP
     # per-model dense layer at bulk-scoring size: 100 000 rows, 64 models, 16 -> 32
     from deepbind_amd import deepity_smat as ds

@@ -1,4 +1,4 @@
-// Fast path of the fused scan + bias + ReLU + max-pool forward: a 3-mer lookup table in LDS.
+// Fast path of the fused scan + bias + ReLU + region pooling forward: a 3-mer lookup table in LDS.
 //
 // The scan is a gather-add: Z[p,f] = sum_j w(j, X[p+j], f). Grouping taps three at a time turns
 // it into G = ceil(m/3) adds per (position, filter): Z[p,f] = sum_g L_g[kmer(p+3g)][f], where
@@ -30,8 +30,13 @@
 //    position read a 126th table entry that is all poison, which sinks exactly the positions that
 //    lie beyond the region. The running max ignores both, and ReLU follows the max.
 //
-// Shapes this path declines (filter length > 24, average pooling, argmax, code 254 present, regions
-// reaching past the last row the scan defines) go through the general kernel in scanpool.hip.
+// Pooling variants share the loop: the running max (plain, or with the index of the winning triple of
+// positions, whose exact position is settled at the region's end by re-adding those three positions'
+// entries in the same order), and / or the running sum of rectified values for average pooling
+// (positions outside the region carry a poison term, so their rectified value is exactly zero).
+//
+// Shapes this path declines (filter length > 24, code 254 present, regions reaching past the last row
+// the scan defines) go through the general kernel in scanpool.hip.
 //
 // Reference chain being fused: kangaroo/_ext/corr1ord.py:97-117 -> deepity/std/elemwise.py:162-180,71-82
 // -> kangaroo/_ext/poolrgn.py:56-76 (kernels corr1ord.cuh:139-157, poolrgn.cuh:44-79).
@@ -111,9 +116,12 @@ __device__ __forceinline__ unsigned row_share(unsigned v)
 //   k0, k1    table byte offsets (triple index * bytes per triple) of this block's positions, spread
 //             over the stream's 16 lanes: lane i holds position i in k0 and position 16+i in k1
 //   acc       ring of partial sums (2 filters per lane), mx the running max
-template <int G>
+// MODE bits: what a finished position is folded into
+constexpr int M_MAX = 1, M_ARG = 2, M_SUM = 4;
+
+template <int G, int MODE>
 __device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigned k0, unsigned k1,
-                                           float2 (&acc)[3][G], float2& mx, unsigned lanebase)
+                                           float2 (&acc)[3][G], float2& mx, uint2& best, float2& sum, unsigned lanebase, unsigned triple0)
 {
     constexpr int H = G / 2;
 #pragma unroll
@@ -141,18 +149,57 @@ __device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigne
                 acc[c][s1].x += v.z; acc[c][s1].y += v.w;
             }
         }
-        // group G-1 just landed in slot (q+1) mod G of each class: three finished positions
+        // group G-1 just landed in slot (q+1) mod G of each class: three finished positions, in text order
         const int cs = (q + 1) % G;
-        mx.x = fmaxf(fmaxf(mx.x, acc[0][cs].x), acc[1][cs].x); mx.y = fmaxf(fmaxf(mx.y, acc[0][cs].y), acc[1][cs].y);
-        mx.x = fmaxf(mx.x, acc[2][cs].x); mx.y = fmaxf(mx.y, acc[2][cs].y);
+        if (MODE & M_ARG) {
+            // remember which triple of positions holds the running maximum (strictly greater: the earliest
+            // triple wins ties); the position inside the triple is settled when the region ends
+            const float m3x = fmaxf(fmaxf(acc[0][cs].x, acc[1][cs].x), acc[2][cs].x);
+            const float m3y = fmaxf(fmaxf(acc[0][cs].y, acc[1][cs].y), acc[2][cs].y);
+            const bool ux = m3x > mx.x, uy = m3y > mx.y;
+            mx.x = ux ? m3x : mx.x;
+            mx.y = uy ? m3y : mx.y;
+            best.x = ux ? triple0 + q : best.x;
+            best.y = uy ? triple0 + q : best.y;
+        } else if (MODE & M_MAX) {
+            mx.x = fmaxf(fmaxf(mx.x, acc[0][cs].x), acc[1][cs].x); mx.y = fmaxf(fmaxf(mx.y, acc[0][cs].y), acc[1][cs].y);
+            mx.x = fmaxf(mx.x, acc[2][cs].x); mx.y = fmaxf(mx.y, acc[2][cs].y);
+        }
+        if (MODE & M_SUM) {
+            // positions outside the region carry a poison term: their rectified value is exactly 0
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                sum.x += fmaxf(acc[c][cs].x, 0.f);
+                sum.y += fmaxf(acc[c][cs].y, 0.f);
+            }
+        }
     }
 }
 
-template <int G, int MAXT>
+// The sum of one position's G table entries for this lane's two filters, groups in ascending order:
+// the same additions, in the same order, as the ring performs.
+template <int G>
+__device__ __forceinline__ float2 rescan_position(const char* __restrict__ lds, const uint8_t* __restrict__ K, size_t t0, unsigned lanebase)
+{
+    constexpr unsigned KSTRIDE = G * ROWB;
+    float2 z = make_float2(0.f, 0.f);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const unsigned km = K[t0 + 3 * g];
+        const float4 v = *reinterpret_cast<const float4*>(lds + km * KSTRIDE + lanebase + (g >> 1) * 256);
+        const float vx = (g & 1) ? v.z : v.x, vy = (g & 1) ? v.w : v.y;
+        if (g == 0) { z.x = vx; z.y = vy; }
+        else { z.x += vx; z.y += vy; }
+    }
+    return z;
+}
+
+template <int G, int MAXT, int MODE>
 __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __restrict__ W, const float* __restrict__ bias,
                                                             unsigned m, unsigned F, const uint8_t* __restrict__ K, size_t N,
                                                             const uint32_t* __restrict__ R, unsigned P, unsigned nsplit,
-                                                            const unsigned* __restrict__ flag, float* __restrict__ pooled)
+                                                            const unsigned* __restrict__ flag, float* __restrict__ pooled,
+                                                            uint32_t* __restrict__ argmax)
 {
     constexpr int STEPS = 3 * G;
     constexpr unsigned KSTRIDE = G * ROWB;                     // bytes per triple: G/2 lines of 256 B
@@ -230,6 +277,8 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
 #pragma unroll
         for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
     float2 mx = make_float2(POISON, POISON);
+    uint2 best = make_uint2(0u, 0u);
+    float2 sum = make_float2(0.f, 0.f);
     unsigned blk = 0;
     const char* lds = reinterpret_cast<const char*>(smem);
 
@@ -241,19 +290,54 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
         unsigned n0, n1;
         if (last) fetch(a_next, (r < P && r + nstream < P) ? rows_next + TAIL : 0u, 0u, n0, n1);
         else fetch(a + (blk + 1) * STEPS, rows + TAIL, (blk + 1) * STEPS, n0, n1);
-        scan_block<G>(lds, k0, k1, acc, mx, lanebase);
+        scan_block<G, MODE>(lds, k0, k1, acc, mx, best, sum, lanebase, blk * (unsigned)G);
         k0 = n0;
         k1 = n1;
         if (last) {
             // ReLU and store this lane's two of the region's 32 pooled features
             if (active) {
                 const unsigned f = f0 + (lane & 15u) * 2;
-                float* out = pooled + (size_t)r * F + f;
-                if (f + 0 < F) out[0] = fmaxf(mx.x, 0.f);
-                if (f + 1 < F) out[1] = fmaxf(mx.y, 0.f);
+                const float inv = 1.0f / (float)rows;
+                if (MODE == M_SUM) {
+                    float* out = pooled + (size_t)r * F + f;
+                    if (f + 0 < F) out[0] = sum.x * inv;
+                    if (f + 1 < F) out[1] = sum.y * inv;
+                } else if (MODE & M_SUM) {
+                    float* out = pooled + ((size_t)r * F + f) * 2;           // (max, avg) interleaved per filter
+                    if (f + 0 < F) { out[0] = fmaxf(mx.x, 0.f); out[1] = sum.x * inv; }
+                    if (f + 1 < F) { out[2] = fmaxf(mx.y, 0.f); out[3] = sum.y * inv; }
+                } else {
+                    float* out = pooled + (size_t)r * F + f;
+                    if (f + 0 < F) out[0] = fmaxf(mx.x, 0.f);
+                    if (f + 1 < F) out[1] = fmaxf(mx.y, 0.f);
+                }
+                if (MODE & M_ARG) {
+                    // first row of the region whose rectified value equals the maximum: the region's first row when
+                    // nothing is positive, else the first position of the winning triple that reproduces the maximum
+                    unsigned px = 0, py = 0;
+                    if (mx.x > 0.f) {
+#pragma unroll
+                        for (int c = 2; c >= 0; --c) {
+                            const int p = (int)(3u * best.x) + c - (int)TAIL;
+                            if (p >= 0 && (unsigned)p < rows && rescan_position<G>(lds, K, (size_t)a + p, lanebase).x == mx.x) px = (unsigned)p;
+                        }
+                    }
+                    if (mx.y > 0.f) {
+#pragma unroll
+                        for (int c = 2; c >= 0; --c) {
+                            const int p = (int)(3u * best.y) + c - (int)TAIL;
+                            if (p >= 0 && (unsigned)p < rows && rescan_position<G>(lds, K, (size_t)a + p, lanebase).y == mx.y) py = (unsigned)p;
+                        }
+                    }
+                    uint32_t* am = argmax + (size_t)r * F + f;
+                    if (f + 0 < F) am[0] = (uint32_t)(((size_t)a + px) * F + f);
+                    if (f + 1 < F) am[1] = (uint32_t)(((size_t)a + py) * F + f + 1);
+                }
             }
             // new region: everything still in the ring belongs to the old one
             mx = make_float2(POISON, POISON);
+            best = make_uint2(0u, 0u);
+            sum = make_float2(0.f, 0.f);
 #pragma unroll
             for (int c = 0; c < 3; ++c)
 #pragma unroll
@@ -270,9 +354,25 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
     }
 }
 
+template <int G, int MODE>
+int launch_mode(hipStream_t st, unsigned nwave, unsigned grid, size_t smem, const float* W, const float* bias, size_t m, size_t F,
+                const uint8_t* K, size_t N, const uint32_t* R, size_t P, unsigned nsplit, const unsigned* flag, float* pooled,
+                uint32_t* argmax)
+{
+    // the plain max kernel exists for 8, 12 and 16 waves (tuning knob); the other modes for 12
+    auto kern = scanpool_kmer_kernel<G, 768, MODE>;
+    if (MODE == M_MAX && nwave == 8) kern = scanpool_kmer_kernel<G, 512, M_MAX>;
+    if (MODE == M_MAX && nwave == 16) kern = scanpool_kmer_kernel<G, 1024, M_MAX>;
+    if (MODE != M_MAX) nwave = 12;
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(nwave * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, K, N, R,
+                       (unsigned)P, nsplit, flag, pooled, argmax);
+    return 0;
+}
+
 template <int G>
 int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* K, size_t N,
-           const uint32_t* R, size_t P, const unsigned* flag, float* pooled)
+           const uint32_t* R, size_t P, const unsigned* flag, int ptype, float* pooled, uint32_t* argmax)
 {
     size_t smem = ((size_t)(NKMER + 1) * G * FTILE + (size_t)3 * G * 5 * FTILE) * sizeof(float);
     if (smem > dbk_scan::lds_limit()) return -1;
@@ -283,19 +383,22 @@ int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F
     unsigned nwave = 12;
     if (const char* e = getenv("DBK_KMER_WAVES")) nwave = (unsigned)atoi(e);     // tuning knob
     if (nwave != 8 && nwave != 12 && nwave != 16) nwave = 12;
+    if (ptype != DBK_PT_MAX || argmax) nwave = 12;
     while (nsplit > 1 && (size_t)(nsplit - 1) * nwave * 4 >= P) --nsplit;       // no more streams than regions
-    auto kern = nwave == 8 ? scanpool_kmer_kernel<G, 512> : (nwave == 12 ? scanpool_kmer_kernel<G, 768> : scanpool_kmer_kernel<G, 1024>);
-    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL(kern, dim3(ntile * nsplit), dim3(nwave * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, K, N, R,
-                       (unsigned)P, nsplit, flag, pooled);
-    return 0;
+    const unsigned grid = ntile * nsplit;
+#define DBK_GO(MODE) return launch_mode<G, MODE>(st, nwave, grid, smem, W, bias, m, F, K, N, R, P, nsplit, flag, pooled, argmax)
+    if (ptype == DBK_PT_MAX) { if (argmax) DBK_GO(M_MAX | M_ARG); DBK_GO(M_MAX); }
+    if (ptype == DBK_PT_ALL) { if (argmax) DBK_GO(M_MAX | M_SUM | M_ARG); DBK_GO(M_MAX | M_SUM); }
+    DBK_GO(M_SUM);
+#undef DBK_GO
 }
 
 // force: take the fast path whenever the shape allows, regardless of problem size
 int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, bool force)
 {
-    if (ptype != DBK_PT_MAX || argmax != nullptr) return -1;
+    if (ptype != DBK_PT_MAX && ptype != DBK_PT_AVG && ptype != DBK_PT_ALL) return -1;
+    if (ptype == DBK_PT_AVG && argmax != nullptr) return -1;
     if (m > 24 || N == 0 || N > 0x7fffff00u || P > 0x7fff0000u) return -1;
     // a filter tile's table costs ~0.1 M position-equivalents to build: only worth it for bulk work
     if (!force && (double)N * dbk::divup(F, FTILE) < 2.0e6) return -1;
@@ -311,10 +414,10 @@ int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size
     G += G & 1;
     int rc;
     switch (G) {
-    case 2: rc = launch<2>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
-    case 4: rc = launch<4>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
-    case 6: rc = launch<6>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
-    default: rc = launch<8>(st, W, bias, m, F, K, N, R, P, flag, pooled); break;
+    case 2: rc = launch<2>(st, W, bias, m, F, K, N, R, P, flag, ptype, pooled, argmax); break;
+    case 4: rc = launch<4>(st, W, bias, m, F, K, N, R, P, flag, ptype, pooled, argmax); break;
+    case 6: rc = launch<6>(st, W, bias, m, F, K, N, R, P, flag, ptype, pooled, argmax); break;
+    default: rc = launch<8>(st, W, bias, m, F, K, N, R, P, flag, ptype, pooled, argmax); break;
     }
     if (rc != 0) return rc;
     // inputs the table cannot express (code 254, regions outside the sequence): the general kernel
@@ -338,7 +441,10 @@ extern "C" int dbk_scanpool_fprop_kmer(dbk_stream_t stream, const float* W, cons
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
+    DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
+    DBK_CHECK(!argmax || (double)N * (double)nfilter <= 4294967296.0,
+              "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
     int rc = dbk_scanpool_kmer::fprop_impl(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, true);
-    DBK_CHECK(rc >= 0, "NotImplementedError: the k-mer table path takes max pooling without argmax and filter length <= 24");
+    DBK_CHECK(rc >= 0, "NotImplementedError: the k-mer table path takes max / avg / all pooling and filter length <= 24");
     return rc;
 }

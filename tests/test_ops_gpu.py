@@ -467,7 +467,59 @@ def test_scanpool_kmer_path_device_side_fallbacks(ks):
     assert_close(host(P), Pr, ACT, "pooled with a region past the last scan row")
     from deepbind_amd._lib import DeepbindError
     with pytest.raises(DeepbindError):
-        ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "all", path="kmer")
+        ks.scanpool_fprop(dev(W[:, :8].repeat(2, axis=0)[:4 * 30].copy()), dev(b[:, :8].copy()), dev(X), dev(R), "max", path="kmer")   # 30 taps
+
+
+@pytest.mark.parametrize("ptype", ["max", "avg", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(200, 101, 101, 24, 64), (150, 30, 60, 16, 40), (60, 1, 30, 24, 33), (90, 40, 90, 7, 32)])
+def test_scanpool_kmer_path_pooling_variants_and_argmax(ks, ptype, B, lo, hi, m, F):
+    """The table kernel's average / max+average pooling and its argmax (winning triple of positions, settled
+    exactly at the region's end) against the oracle, with the general kernel as a second opinion."""
+    rng, W, b, X, R = _fused_case(7000 + B + m + F, B, lo, hi, m, F, pn=0.04)
+    b = b - 0.05                                                    # some filters never fire in some regions: argmax = first row
+    A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
+    want = ptype != "avg"
+    P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=want, path="kmer")
+    assert_close(host(P), Pr, ACT, "pooled (%s, table kernel)" % ptype)
+    Pg, Ig = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=want, path="general")
+    assert_close(host(P), host(Pg), ACT, "table vs general")
+    if want:
+        got = host(I)
+        agree = got == Ir
+        assert agree.mean() > 0.995                                 # float32 round-off can move a near-tie
+        # wherever the index differs from the float64 oracle the two rows must be a float32 tie
+        rows, cols = np.nonzero(~agree)
+        Af = A.astype(np.float32)
+        for r_, c_ in zip(rows[:50], cols[:50]):
+            i_got, i_ref = got[r_, c_] // F, Ir[r_, c_] // F
+            assert got[r_, c_] % F == c_ and R[r_, 0] <= i_got < R[r_, 1]
+            assert abs(Af[i_got, c_] - Af[i_ref, c_]) <= 1e-5 * max(1.0, abs(Af[i_ref, c_]))
+        zero = Pr[:, ::2] == 0 if ptype == "all" else Pr == 0
+        assert zero.any() and np.array_equal(got[zero] // F, np.broadcast_to(R[:, :1], got.shape)[zero])
+    else:
+        assert I is None
+
+
+def test_scanpool_kmer_argmax_takes_the_first_of_exactly_equal_rows(ks):
+    """A sequence made of one 40-letter unit repeated: every window value recurs bit-for-bit 40 rows later,
+    so the maximum is attained several times and the index must be the first occurrence."""
+    rng = np.random.default_rng(3)
+    m, F = 24, 32
+    unit = rng.integers(0, 4, 40, dtype=np.uint8)
+    ords = [np.tile(unit, 5), np.tile(unit[::-1].copy(), 3)]
+    from deepbind_amd import data
+    X, R = data.pack_ordinals(ords, m - 1)
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
+    b = np.zeros((1, F), np.float32)
+    A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, "max")
+    rows_ref = Ir // F
+    # the oracle's maxima really are attained more than once
+    repeats = sum(int((A[R[r_, 0]:R[r_, 1], c_] == Pr[r_, c_]).sum() > 1) for r_ in range(2) for c_ in range(F))
+    assert repeats > F
+    for path in ("kmer", "general"):
+        P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max", want_argmax=True, path=path)
+        assert np.array_equal(host(I) // F, rows_ref), path
+        assert np.array_equal(host(I) % F, np.broadcast_to(np.arange(F), (2, F)))
 
 
 def test_scanpool_auto_path_bulk(ks):
