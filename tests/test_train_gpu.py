@@ -478,3 +478,28 @@ def test_gradcheck_float64_layer_by_layer(pool, hidden, loss):
     net.backward = bad
     with pytest.raises(AssertionError, match="W1 FAILED"):
         gradcheck(net, dev(X), dev(R), Y, Ymask, ncheck=30, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("pool", ["max", "all"])
+def test_bulk_batch_training_step_uses_the_table_kernel_and_matches_layer_by_layer(pool):
+    """A batch large enough for the fused forward to pick the table kernel (with argmax for the backward pass):
+    one training step must agree with the layer-by-layer drop-in operators, and be bit-stable."""
+    from deepbind_amd import data
+    from deepbind_amd.model import SequenceNet
+    rng = np.random.default_rng(13)
+    B, L, m, ni = 12000, 101, 24, 4
+    codes = rng.integers(0, 4, (B, L), dtype=np.uint8)
+    codes[rng.random((B, L)) < 0.01] = 255
+    X, R = data.pack_uniform_ordinals(codes, m - 1)
+    Y = (rng.random((B, ni)) < 0.5).astype(np.float32)
+    nets = []
+    for mode in ("fused", "unfused", "fused"):
+        net = SequenceNet(ni, 16, m, pool=pool, hidden=32, loss="nll", rate=0.05, momentum=0.9, mode=mode, dropout=0.0)
+        net.init_params(init_conv=0.05, init_full=0.1, init_mu=0.01, seed=3)
+        net.train_step(dev(X), dev(R), dev(Y))
+        nets.append(net)
+    a, b, c = (n.get_grads() for n in nets)
+    for k in a:
+        assert_close(a[k], b[k], GRAD, "fused vs layer-by-layer gradient %s" % k)
+        assert np.array_equal(a[k], c[k]), "run-to-run difference in %s" % k
+    assert np.abs(a["Wc"]).max() > 0
