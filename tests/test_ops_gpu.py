@@ -635,3 +635,28 @@ def test_scanpool_extreme_shapes(ks, ptype):
     assert np.array_equal(outs[0][0], outs[2][0]) and np.array_equal(outs[0][1], outs[2][1])
     assert np.array_equal(outs[1][0], 2 * outs[0][0]) and np.array_equal(outs[1][1], 2 * outs[0][1])
     assert np.isfinite(outs[0][0]).all() and np.abs(outs[0][0]).max() > 0
+
+
+def test_config5_full_size_against_subsampled_checkers(ks):
+    """The full bulk-scoring workload (100 000 x 500 nt, 1024 filters): rows of the table kernel's result are
+    checked against the general kernel and the plain-C oracle run on random subsets of the regions (same
+    packed stream, region table subsampled), and a permuted region table must permute the rows and nothing else."""
+    from deepbind_amd import synth
+    from oracle import oracle_c
+    cfg = synth.config5(seed=4, nseq=100000)
+    p = cfg["params"]
+    W, b, X, R = dev(p["Wc"]), dev(p["bc"]), dev(cfg["X"]), dev(cfg["R"])
+    P, _ = ks.scanpool_fprop(W, b, X, R, "max")
+    assert tuple(P.shape) == (100000, 1024) and bool(torch.isfinite(P).all()) and float(P.min()) >= 0.0
+    rng = np.random.default_rng(0)
+    pick = np.sort(rng.choice(100000, 1500, replace=False))
+    Rs = np.ascontiguousarray(cfg["R"][pick])
+    Pg, _ = ks.scanpool_fprop(W, b, X, dev(Rs), "max", path="general")
+    sub = host(P[torch.as_tensor(pick, device="cuda")])
+    assert_close(sub, host(Pg), ACT, "table kernel vs general kernel on 1500 regions")
+    few = pick[:120]
+    Pc, _ = oracle_c.scanpool(p["Wc"], p["bc"], cfg["X"], np.ascontiguousarray(cfg["R"][few]), 0)
+    assert_close(sub[:120], Pc, ACT, "table kernel vs C oracle on 120 regions")
+    perm = rng.permutation(100000)
+    Pp, _ = ks.scanpool_fprop(W, b, X, dev(np.ascontiguousarray(cfg["R"][perm])), "max")
+    assert torch.equal(Pp, P[torch.as_tensor(perm, device="cuda")])
