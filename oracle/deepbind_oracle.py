@@ -19,6 +19,7 @@ checks live in tests/test_oracle_pins.py):
                         unit tests compare against (smat/tests/unittest.py:425-471,531-623)
   blockwise_dot*      - np.dot per block; no reference test exists at that boundary
                         (closed form only): PARITY UNPINNED beyond the per-block np.dot identity
+  weight_cost         - scalar loops over each model's own weights
   gradstep*           - three-line closed form (gradstep.cu:41-72) vs. an unrolled scalar loop
   dropout masks       - the reference draws them from cuRAND (not reproducible without the
                         CUDA SDK): masks are INPUTS here (uniforms U supplied by the caller);

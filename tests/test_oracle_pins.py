@@ -377,3 +377,17 @@ def test_whole_model_gradient_matches_finite_differences():
                 flat[idx] = old
                 np.testing.assert_allclose(g[name].reshape(-1)[idx], (cp - cm) / 2e-6, rtol=2e-5, atol=1e-8,
                                            err_msg="%s[%d] pool=%s" % (name, idx, pool))
+
+
+def test_weight_cost_is_the_per_model_l1_norm_times_decay():
+    """Scalar loops over each model's own weights (scan filters lie along columns, dense weights in row blocks)."""
+    rng = np.random.default_rng(4)
+    nm, nf, m, hid = 3, 2, 4, 5
+    p = {"Wc": rng.standard_normal((4 * m, nf * nm)), "W1": rng.standard_normal((nf * nm, hid)), "W2": rng.standard_normal((hid * nm, 1))}
+    dc, df = np.array([0.1, 0.2, 0.3]), np.array([1.0, 2.0, 3.0])
+    want = np.zeros(nm)
+    for b in range(nm):
+        conv = sum(abs(p["Wc"][r, c]) for r in range(4 * m) for c in range(nf * b, nf * (b + 1)))
+        full = sum(abs(v) for v in p["W1"][nf * b:nf * (b + 1)].ravel()) + sum(abs(v) for v in p["W2"][hid * b:hid * (b + 1)].ravel())
+        want[b] = dc[b] * conv + df[b] * full
+    np.testing.assert_allclose(orc.weight_cost(p, nm, dc, df).ravel(), want, rtol=1e-12)
