@@ -74,7 +74,24 @@ _SIGNATURES = {
     "dbk_counter_add": [_P, _P, _U64],
     "dbk_l1_decay": [_P, _I, _P, _P, _P, _Z],
     "dbk_head_fprop": [_P, _Z, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
+    "dbk_train_step": [_P, _P],
 }
+
+
+class TrainStepArgs(ctypes.Structure):
+    """dbk_train_step_args of the public header, field for field."""
+    _fields_ = [
+        ("nmodel", _Z), ("nfilter", _Z), ("m", _Z), ("hidden", _Z),
+        ("ptype", _I), ("loss_kind", _I), ("reverse_complement", _I), ("nesterov", _I),
+        ("nparam", _Z),
+        ("P", _P), ("dP", _P), ("mP", _P), ("drate", _P), ("mrate", _P),
+        ("off_Wc", _Z), ("off_bc", _Z), ("off_W1", _Z), ("off_b1", _Z), ("off_W2", _Z), ("off_b2", _Z),
+        ("X", _P), ("N", _Z), ("regions", _P), ("nregion", _Z), ("Y", _P), ("Ymask", _P),
+        ("input_rate", _F), ("Xdrop", _P), ("Mdrop", _P),
+        ("rate", _P), ("seed", _U64), ("counter", _P),
+        ("decay", _P), ("freeze_scan", _I),
+        ("pooled", _P), ("argmax", _P), ("Z", _P), ("dpooled", _P), ("loss", _P),
+    ]
 
 _dll = None
 

@@ -1,0 +1,92 @@
+// One whole optimiser step of a model group, issued from native code.
+//
+// A step on a small minibatch is eight to ten launches of 2-50 us each, so its cost is what the host
+// spends per launch. Issued from here that is ~2.6 us per launch (measured on MI355X); from a scripting
+// host, or as nodes of a multi-branch HIP graph, it is 6-8 us. The step is the body of the reference
+// trainer's loop (deepity/deepity/sgd.py:98-135: gradstep with the batch gradient as its callback,
+// deepity_smat.py:77-117), with the gradient computed by the fused kernels:
+//
+//   [P += mrate*mP]                                   Nesterov look-ahead       (gradstep.cu:41-51)
+//   [Xd = input dropout(X)]                           dropoutord.py:50-70
+//   pooled, argmax = scanpool_fprop(Wc, bc, Xd)       corr1ord -> bias -> relu -> poolrgn
+//   Z, dpooled, dW1.. = head_train(pooled, Y)         dropout -> full (-> relu -> full) -> bias -> loss
+//   dWc, dbc = scanpool_bprop(dpooled)
+//   [dP += decay * sign(P)]                           L1 decay once it is switched on (full.py:111-119)
+//   [dWc = 0]                                         scan filters still frozen
+//   mP = mrate*mP - drate*dP ; P += ...               momentum / Nesterov update  (gradstep.cu:53-72)
+//
+// The same entry points a caller would use one by one are called in the same order, so the result is
+// bit-identical to issuing them separately.
+#include "dbk_common.h"
+
+namespace {
+
+__global__ void k_zero_f32(float* p, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.0f;
+}
+
+}  // namespace
+
+extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
+{
+    DBK_CHECK(a != nullptr, "ValueError: null argument block");
+    DBK_CHECK(a->nmodel >= 1 && a->nfilter >= 1 && a->m >= 1, "ValueError: nmodel, nfilter and m must be >= 1");
+    DBK_CHECK(a->ptype == DBK_PT_MAX || a->ptype == DBK_PT_AVG || a->ptype == DBK_PT_ALL,
+              "ValueError: the fused step takes max, avg or all pooling");
+    DBK_CHECK(a->P && a->dP && a->mP && a->drate && a->mrate, "ValueError: null parameter vector");
+    DBK_CHECK(a->X && a->regions && a->Y && a->pooled && a->Z && a->dpooled, "ValueError: null batch or work buffer");
+    DBK_CHECK(a->ptype == DBK_PT_AVG || a->argmax, "ValueError: max / all pooling needs the argmax work buffer");
+    DBK_CHECK(a->input_rate <= 0.0f || (a->Xdrop && a->Mdrop), "ValueError: input dropout needs the Xdrop and Mdrop work buffers");
+    DBK_CHECK(!(a->rate || a->input_rate > 0.0f) || a->counter, "ValueError: dropout needs the device generator position");
+    const size_t F = a->nmodel * a->nfilter;                       // filters of all models, side by side
+    const size_t k = a->nfilter * (a->ptype == DBK_PT_ALL ? 2 : 1); // pooled features per model
+    const size_t nWc = 4 * a->m * F;
+    const size_t nW1 = k * a->nmodel * (a->hidden ? a->hidden : 1), nb1 = a->nmodel * (a->hidden ? a->hidden : 1);
+    const size_t nW2 = a->hidden ? a->hidden * a->nmodel : 0, nb2 = a->hidden ? a->nmodel : 0;
+    const size_t need[6] = { a->off_Wc + nWc, a->off_bc + F, a->off_W1 + nW1, a->off_b1 + nb1,
+                             a->off_W2 + nW2, a->off_b2 + nb2 };
+    for (size_t v : need) DBK_CHECK(v <= a->nparam, "ValueError: a parameter block reaches past the flat vector (%zu > %zu)", v, a->nparam);
+
+    float* const P = a->P;
+    float* const dP = a->dP;
+    int rc;
+    if (a->nesterov) {
+        rc = dbk_gradstep_nesterov1(stream, DBK_F32, a->nparam, P, a->mP, a->mrate);
+        if (rc) return rc;
+    }
+    const uint8_t* X = a->X;
+    if (a->input_rate > 0.0f) {
+        rc = dbk_dropoutord_fp_tr(stream, a->X, a->Xdrop, a->Mdrop, a->N, a->input_rate, a->seed, 0, a->counter);
+        if (rc) return rc;
+        if (a->reverse_complement) {
+            rc = dbk_dropoutord_mirror(stream, a->X, a->Xdrop, a->Mdrop, a->regions, a->nregion, a->m - 1);
+            if (rc) return rc;
+        }
+        rc = dbk_counter_add(stream, a->counter, (a->N + 3) / 4);
+        if (rc) return rc;
+        X = a->Xdrop;
+    }
+    rc = dbk_scanpool_fprop(stream, P + a->off_Wc, P + a->off_bc, a->m, F, X, a->N, a->regions, a->nregion, a->ptype,
+                            a->pooled, a->argmax);
+    if (rc) return rc;
+    const uint64_t draws = a->rate ? (a->nregion * k * a->nmodel + 3) / 4 : 0;
+    rc = dbk_head_train(stream, a->nregion, (int)a->nmodel, (int)k, (int)a->hidden, a->loss_kind, a->reverse_complement,
+                        a->pooled, a->rate, nullptr, a->seed, 0, a->counter, draws,
+                        P + a->off_W1, P + a->off_b1, a->hidden ? P + a->off_W2 : nullptr, a->hidden ? P + a->off_b2 : nullptr,
+                        a->Y, a->Ymask, a->Z, a->dpooled,
+                        dP + a->off_W1, dP + a->off_b1, a->hidden ? dP + a->off_W2 : nullptr, a->hidden ? dP + a->off_b2 : nullptr,
+                        a->loss);
+    if (rc) return rc;
+    rc = dbk_scanpool_bprop(stream, P + a->off_Wc, P + a->off_bc, a->m, F, X, a->N, a->regions, a->nregion, a->ptype,
+                            a->pooled, a->argmax, a->dpooled, dP + a->off_Wc, dP + a->off_bc, 1);
+    if (rc) return rc;
+    if (a->decay) {
+        rc = dbk_l1_decay(stream, DBK_F32, P, a->decay, dP, a->nparam);
+        if (rc) return rc;
+    }
+    if (a->freeze_scan) hipLaunchKernelGGL(k_zero_f32, dim3(dbk::ew_grid(nWc)), dim3(256), 0, dbk::as_stream(stream), dP + a->off_Wc, nWc);
+    if (a->nesterov) rc = dbk_gradstep_nesterov2(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
+    else rc = dbk_gradstep(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
+    return rc;
+}

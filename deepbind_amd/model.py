@@ -22,9 +22,12 @@ forward and one backward; "unfused" calls the drop-in operators one by one, as t
 All models of one SequenceNet share pool type and hidden size; a calibration batch that mixes
 architectures is run as one SequenceNet per architecture (see ModelGroup).
 """
+import ctypes
+
 import numpy as np
 import torch
 
+from . import _lib
 from . import deepity_smat as ds
 from . import kangaroo_smat as ks
 from . import smat as sm
@@ -51,6 +54,9 @@ class SequenceNet(object):
         # the scan filters' gradient is zeroed while step < start_training (reference: kangaroo/_ext/corr1ord.py:135-136)
         self.start_training = int(start_training)
         self.step_count = 0
+        self._step_args = None               # argument block and work buffers of the natively issued step
+        self._step_bufs = {}
+        self._busy_stream = None             # side stream a ModelGroup left this net's last step on
         ni, nf = self.ninst, self.nfilter
         self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
         h = self.hidden
@@ -96,6 +102,7 @@ class SequenceNet(object):
 
     def set_rates(self, rate, momentum):
         """Per-model learning and momentum rates spread over the flat vectors."""
+        self.join()
         self.drate.zero_()
         self.mrate.zero_()
         ones = torch.ones_like(self.P)
@@ -105,6 +112,7 @@ class SequenceNet(object):
 
     def set_params(self, params):
         """Copies a dict of NumPy arrays shaped like the layout into the flat parameter vector."""
+        self.join()
         for name, shape, _ in self.layout:
             src = np.asarray(params[name])
             assert tuple(src.shape) == tuple(shape), "%s: expected %s, got %s" % (name, shape, src.shape)
@@ -115,6 +123,7 @@ class SequenceNet(object):
         weights = randn * init (one scale per model, spread with madd_bcast), biases = init_mu.
         init_conv / init_full / init_mu: scalar or one value per model. The normal deviates come from
         the library's generator, so equal seeds give equal parameters."""
+        self.join()
         self.P.zero_()
         offset = 0
         for name, shape, axis in self.layout:
@@ -136,6 +145,7 @@ class SequenceNet(object):
         ni = self.ninst
         if self.weight_decay_start > self.step_count:
             return np.zeros((1, ni))
+        self.join()
         p = self.p
         conv = sm.sum_axis0(sm.mul_sign(p["Wc"], p["Wc"]))                     # |W| summed over taps and channels
         torch.cuda.synchronize()
@@ -150,10 +160,12 @@ class SequenceNet(object):
         return cost.reshape(1, ni)
 
     def get_params(self):
+        self.join()
         torch.cuda.synchronize()
         return {name: self.p[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
     def get_grads(self):
+        self.join()
         torch.cuda.synchronize()
         return {name: self.g[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
@@ -234,6 +246,7 @@ class SequenceNet(object):
     def forward(self, X, R, train=False, U=None, want_argmax=False):
         """Returns the state dict of one forward pass; st["Z"] are the predictions (n x ninst)."""
         p, ni = self.p, self.ninst
+        self.join()
         st = {}
         st["pooled"], st["argmax"], st["A0"] = self._conv_forward(X, R, want_argmax, train=train)
         H0 = st["pooled"]
@@ -264,6 +277,7 @@ class SequenceNet(object):
     def predict(self, X, R):
         """Test-mode predictions through the fused scoring head (dropout rescale folded in)."""
         p = self.p
+        self.join()
         pooled, _, _ = self._conv_forward(X, R, False)
         if self.dtype != torch.float32:
             Z = self.forward(X, R)["Z"]
@@ -282,6 +296,7 @@ class SequenceNet(object):
         (reference: deepity/deepity/node.py:298-341, kangaroo/kangaroo/predict.py:168-193,
         kangaroo/_ext/corr1ord.py:129-133, deepity/std/elemwise.py:148-157)"""
         p, ni = self.p, self.ninst
+        self.join()
         Z0 = sm.zeros((X.numel(), p["Wc"].shape[1]), dtype=self.dtype, device=self.device)
         ks.corr1ord(p["Wc"], X, Z0, 4)
         if self.input_dropout > 0:
@@ -330,6 +345,7 @@ class SequenceNet(object):
     def backward(self, X, R, st, Y, Ymask=None):
         """Fills dP with the gradient of the summed per-model losses (plus L1 decay when active)."""
         p, g, ni = self.p, self.g, self.ninst
+        self.join()
         dA = sm.sub_scale(st["Z"], Y, 1.0 / st["Z"].shape[0])
         if Ymask is not None:
             ds.maskout(Ymask, dA)
@@ -401,6 +417,70 @@ class SequenceNet(object):
         return Z
 
     # ------------------------------------------------------------------ one optimiser step
+    def join(self):
+        """Orders the current stream after this net's last step when a ModelGroup issued it on a side stream."""
+        if self._busy_stream is not None:
+            torch.cuda.current_stream().wait_stream(self._busy_stream)
+            self._busy_stream = None
+
+    def _native_step(self, X, R, Y, Ymask=None, stream=None):
+        """One fused step through dbk_train_step: one library call issues every launch of the step (the
+        scripting host otherwise pays several microseconds per launch, which is what bounds a step on a
+        small minibatch). Same kernels in the same order as gradstep(..., _grad_fused), so the same bits.
+        stream: torch stream to issue on (default: the current one)."""
+        ks._u8(X)
+        ks._regions(R)
+        ni, P = self.ninst, R.shape[0]
+        _lib.require(R.shape[1] == 2, "ValueError: the fused path takes 2-column regions")
+        _lib.require(Y.dtype == torch.float32 and tuple(Y.shape) == (P, ni), "ValueError: Y must be float32 (rows x models)")
+        _lib.require(Ymask is None or (Ymask.dtype == torch.bool and tuple(Ymask.shape) == (P, ni)), "ValueError: Ymask must be bool (rows x models)")
+        a = self._step_args
+        if a is None:
+            a = self._step_args = _lib.TrainStepArgs()
+            off = {name: int(o) for (name, _, _), o in zip(self.layout, self.offsets[:-1])}
+            a.nmodel, a.nfilter, a.m, a.hidden = ni, self.nfilter, self.m, self.hidden
+            a.ptype, a.loss_kind = _lib.str2pooltype[self.pool], {"nll": 0, "mse": 1}[self.loss]
+            a.reverse_complement = int(self.reverse_complement)
+            a.nparam = self.P.numel()
+            a.P, a.dP, a.mP = self.P.data_ptr(), self.dP.data_ptr(), self.mP.data_ptr()
+            a.drate, a.mrate = self.drate.data_ptr(), self.mrate.data_ptr()
+            a.off_Wc, a.off_bc, a.off_W1, a.off_b1 = off["Wc"], off["bc"], off["W1"], off["b1"]
+            a.off_W2, a.off_b2 = off.get("W2", 0), off.get("b2", 0)
+            a.rate = self.dropout.data_ptr() if self.use_dropout else None
+            a.counter = self.rng_counter.data_ptr()
+        key = (X.numel(), P)
+        buf = self._step_bufs.get(key)
+        if buf is None:
+            if len(self._step_bufs) >= 4:
+                self._step_bufs.clear()
+            dev = self.P.device
+            with torch.cuda.stream(stream if stream is not None else torch.cuda.current_stream()):   # owned by the issuing stream
+                buf = self._step_bufs[key] = dict(
+                    pooled=torch.empty((P, self.k * ni), dtype=torch.float32, device=dev),
+                    dpooled=torch.empty((P, self.k * ni), dtype=torch.float32, device=dev),
+                    argmax=torch.empty((P, self.nfilter * ni), dtype=ks.uindex, device=dev) if self.pool != "avg" else None,
+                    Z=torch.empty((P, ni), dtype=torch.float32, device=dev),
+                    Xdrop=torch.empty(X.numel(), dtype=torch.uint8, device=dev) if self.input_dropout > 0 else None,
+                    Mdrop=torch.empty(X.numel(), dtype=torch.bool, device=dev) if self.input_dropout > 0 else None)
+        a.nesterov, a.seed = int(bool(self.nesterov)), int(self.rng_seed)
+        pv = lambda t: None if t is None else _lib.ptr(t).value          # checks device + contiguity
+        a.X, a.N, a.regions, a.nregion = pv(X), X.numel(), pv(R), P
+        a.Y, a.Ymask = pv(Y), pv(Ymask)
+        a.input_rate = self.input_dropout
+        for name, t in buf.items():
+            setattr(a, name, None if t is None else t.data_ptr())
+        a.decay = self.decay_vec.data_ptr() if self.weight_decay_start <= self.step_count else None
+        a.freeze_scan = int(self.step_count < self.start_training)
+        a.loss = None
+        handle = _lib.stream() if stream is None else ctypes.c_void_p(stream.cuda_stream)
+        _lib.call("dbk_train_step", handle, ctypes.addressof(a))
+        if self.input_dropout > 0:
+            self._rng_offset += (X.numel() + 3) // 4
+        if self.use_dropout:
+            self._rng_offset += (P * self.k * ni + 3) // 4
+        self.step_count += 1
+        return buf["Z"]
+
     def make_graphed_step(self, X, R, Y, Ymask=None):
         """Captures one fused training step on the given (static) batch tensors into a HIP graph and
         returns a function that replays it: for launch-bound batch sizes the step then costs one
@@ -414,6 +494,10 @@ class SequenceNet(object):
         """One optimiser step. U / U_input optionally supply the uniforms of the pooled-feature and the
         input dropout (otherwise the library's generator draws them)."""
         fused = self.mode == "fused" and self.dtype == torch.float32 and self.loss is not None
+        self.join()
+        if fused and U is None and U_input is None:
+            self._native_step(X, R, Y, Ymask)
+            return
 
         def grad():
             if fused:
@@ -485,6 +569,8 @@ def _graphed_step(jobs, streams=None):
         state["graph"], state["decay"] = g, decay_flags()
 
     def step():
+        for net, *_ in jobs:
+            net.join()
         if state["graph"] is None or state["decay"] != decay_flags():
             capture()
         state["graph"].replay()
@@ -512,26 +598,73 @@ class ModelGroup(object):
             kw = {k: (np.asarray(v)[idx] if np.ndim(v) else v) for k, v in per_model.items()}
             self.groups.append((idx, SequenceNet(len(idx), nfilter, m, pool=key[0], hidden=key[1], loss=loss, **kw)))
         self.streams = None
+        self._batch_key, self._batch, self._targets = None, None, None
 
     def _streams(self):
         if self.streams is None:
             self.streams = [torch.cuda.Stream() for _ in self.groups]
         return self.streams
 
-    def train_step(self, X, R, Y, Ymask=None, U=None):
-        """U, when given, is a list with one uniforms tensor per architecture group (see self.groups)."""
-        def one(gi, idx, net):
-            def run():
-                ii = torch.as_tensor(idx, device=Y.device)
-                Yg = Y.index_select(1, ii).contiguous()
-                Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
-                net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
-            return run
-        _side_by_side(self._streams(), [one(gi, idx, net) for gi, (idx, net) in enumerate(self.groups)])
+    def train_step(self, X, R, Y, Ymask=None, U=None, join=True):
+        """One step of every architecture group on the shared batch. Each group's step is one native
+        call on the group's own stream (all of default priority), so the host spends a few microseconds
+        per launch and the groups' small kernels overlap on the GPU.
+        join=False leaves the step in flight on the group streams: the next train_step carries on there,
+        and join() - which predict / slice_model / make_graphed_step and every accessor of the nets call -
+        orders the current stream after it. A loop that only steps thereby saves the stream events of a
+        fork and a join per step (about 10 us of host time each).
+        U, when given, is a list with one uniforms tensor per architecture group (see self.groups); that
+        path goes through the layer wrappers."""
+        streams = self._streams()
+        native = U is None and all(net.mode == "fused" and net.dtype == torch.float32 and net.loss is not None
+                                   for _, net in self.groups)
+        if not native:
+            def one(gi, idx, net):
+                def run():
+                    ii = torch.as_tensor(idx, device=Y.device)
+                    Yg = Y.index_select(1, ii).contiguous()
+                    Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
+                    net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
+                return run
+            self.join()
+            _side_by_side(streams, [one(gi, idx, net) for gi, (idx, net) in enumerate(self.groups)])
+            return
+        key = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in (X, R, Y, Ymask) if t is not None)
+        in_flight = all(net._busy_stream is s for (_, net), s in zip(self.groups, streams))
+        if key != self._batch_key or not in_flight:
+            # fork: the group streams wait for whatever produced the batch (and for anything the current
+            # stream did to the nets since they were joined)
+            self.join()
+            if key != self._batch_key:
+                self._targets = []
+                for idx, _ in self.groups:
+                    ii = torch.as_tensor(idx, device=Y.device)
+                    self._targets.append((Y.index_select(1, ii).contiguous(),
+                                          Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
+                for t in [X, R, Y, Ymask] + [t for pair in self._targets for t in pair]:
+                    if t is not None:
+                        for s in streams:
+                            t.record_stream(s)
+                self._batch_key, self._batch = key, (X, R, Y, Ymask)
+            ev = torch.cuda.Event()
+            ev.record()
+            for s in streams:
+                s.wait_event(ev)
+        for (idx, net), s, (Yg, Mg) in zip(self.groups, streams, self._targets):
+            net._native_step(X, R, Yg, Mg, stream=s)
+            net._busy_stream = s
+        if join:
+            self.join()
+
+    def join(self):
+        """Orders the current stream after the steps left in flight on the group streams."""
+        for _, net in self.groups:
+            net.join()
 
     def make_graphed_step(self, X, R, Y, Ymask=None):
         """One HIP graph holding the fused training step of every architecture group on a static batch."""
         jobs = []
+        self.join()
         for idx, net in self.groups:
             ii = torch.as_tensor(idx, device=Y.device)
             jobs.append((net, X, R, Y.index_select(1, ii).contiguous(),
@@ -540,6 +673,7 @@ class ModelGroup(object):
 
     def slice_model(self, j):
         """Single-model net for model j of the original ordering."""
+        self.join()
         for idx, net in self.groups:
             if j in idx:
                 return net.slice_model(idx.index(j))
@@ -547,6 +681,7 @@ class ModelGroup(object):
 
     def predict(self, X, R):
         out = torch.empty((R.shape[0], self.nmodel), dtype=torch.float32, device=X.device)
+        self.join()
         for idx, net in self.groups:
             out[:, torch.as_tensor(idx, device=X.device)] = net.predict(X, R)
         return out

@@ -289,6 +289,44 @@ int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
  * captured HIP graph draws fresh masks on every replay). */
 int dbk_counter_add(dbk_stream_t stream, uint64_t* counter, uint64_t delta);
 
+/* ------------------------------------------------------------------ one whole optimiser step */
+
+/* Everything one step of a group of `nmodel` same-architecture models touches. The parameters, their
+ * gradients and the momentum live in flat float32 vectors of nparam elements, as the reference trainer
+ * keeps them (deepity/deepity/sgd.py:287-331); off_* are the element offsets of the blocks inside them:
+ * Wc (4m, nmodel*nfilter), bc (nmodel*nfilter), W1 (k*nmodel, hidden|1), b1 (hidden*nmodel | nmodel),
+ * W2 (hidden*nmodel, 1), b2 (nmodel) with k = nfilter (x2 for all-pooling); W2 / b2 only when hidden > 0.
+ * Work buffers are the caller's: pooled and dpooled (nregion, k*nmodel), argmax (nregion,
+ * nmodel*nfilter; unused for avg pooling), Z (nregion, nmodel), and with input dropout Xdrop, Mdrop (N). */
+typedef struct dbk_train_step_args {
+    size_t nmodel, nfilter, m, hidden;      /* architecture: filters per model, filter length, hidden units (0 = none) */
+    int ptype, loss_kind;                   /* DBK_PT_MAX / AVG / ALL; 0 = logistic + nll, 1 = identity + mse */
+    int reverse_complement, nesterov;
+    size_t nparam;
+    float *P, *dP, *mP;
+    const float *drate, *mrate;             /* per-element learning and momentum rates */
+    size_t off_Wc, off_bc, off_W1, off_b1, off_W2, off_b2;
+    const uint8_t* X; size_t N;             /* packed batch (see dbk_corr1ord) */
+    const uint32_t* regions; size_t nregion; /* (nregion, 2) row ranges */
+    const float* Y; const uint8_t* Ymask;   /* targets (nregion, nmodel); mask may be NULL */
+    float input_rate;                       /* input-base dropout rate, 0 = off */
+    uint8_t *Xdrop, *Mdrop;
+    const float* rate;                      /* pooled-feature dropout rate per model, NULL = off */
+    uint64_t seed; uint64_t* counter;       /* generator seed and its position in device memory */
+    const float* decay;                     /* L1 coefficient per element of P, NULL while decay is off */
+    int freeze_scan;                        /* zero the scan filters' gradient (filters not yet training) */
+    float* pooled; uint32_t* argmax; float* Z; float* dpooled;
+    float* loss;                            /* per-model mean loss (nmodel), may be NULL */
+} dbk_train_step_args;
+
+/* One optimiser step, all launches issued from native code on `stream`:
+ * [Nesterov look-ahead] -> [input dropout] -> dbk_scanpool_fprop -> dbk_head_train -> dbk_scanpool_bprop
+ * -> [dbk_l1_decay] -> [zero dWc] -> momentum / Nesterov update. Bit-identical to calling those entry
+ * points one by one; exists because a step on a small minibatch is bound by the host's cost per launch.
+ * reference: the body of the trainer's loop, deepity/deepity/sgd.py:98-135 (gradstep with the batch
+ * gradient as callback, deepity_smat.py:77-117, gradstep.cu:41-72). */
+int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* args);
+
 #ifdef __cplusplus
 }
 #endif

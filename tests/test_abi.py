@@ -53,6 +53,39 @@ def test_argument_errors_surface_through_last_error():
         raise AssertionError("expected DeepbindError")
 
 
+def test_train_step_argument_block_layout_matches_the_header():
+    """The ctypes mirror of dbk_train_step_args is read field for field by the library's own checks,
+    which run on the host before anything touches a device."""
+    from deepbind_amd import _lib
+    lib = _lib.dll()
+    assert lib.dbk_train_step(None, None) != 0 and b"null argument block" in lib.dbk_last_error()
+    a = _lib.TrainStepArgs()
+    a.nmodel, a.nfilter, a.m, a.hidden = 3, 5, 7, 2
+    a.ptype, a.loss_kind, a.reverse_complement, a.nesterov = _lib.PT_ALL, 0, 0, 1
+    for f in ("P", "dP", "mP", "drate", "mrate", "X", "regions", "Y", "pooled", "Z", "dpooled", "argmax"):
+        setattr(a, f, 1)
+    a.nparam = 1000
+    # blocks: Wc 4*7*15 = 420, bc 15, W1 (10*3)*2 = 60, b1 6, W2 6, b2 3
+    a.off_Wc, a.off_bc, a.off_W1, a.off_b1, a.off_W2, a.off_b2 = 0, 420, 435, 495, 501, 998
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0
+    assert b"reaches past the flat vector (1001 > 1000)" in lib.dbk_last_error()        # off_b2 + nmodel
+    a.off_b2, a.off_W1 = 507, 941
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0
+    assert b"(1001 > 1000)" in lib.dbk_last_error()                                     # off_W1 + k*nmodel*hidden
+    a.off_W1, a.ptype = 435, 2
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"max, avg or all pooling" in lib.dbk_last_error()
+    a.ptype, a.argmax = _lib.PT_MAX, None
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"argmax work buffer" in lib.dbk_last_error()
+    a.argmax, a.input_rate = 1, 0.25
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"Xdrop and Mdrop" in lib.dbk_last_error()
+    a.Xdrop, a.Mdrop = 1, 1
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"generator position" in lib.dbk_last_error()
+    a.input_rate, a.rate = 0.0, 1
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"generator position" in lib.dbk_last_error()
+    a.rate, a.dpooled = None, None
+    assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"null batch or work buffer" in lib.dbk_last_error()
+
+
 def test_philox_known_answers():
     """Published Philox4x32-10 vectors (Random123 kat_vectors)."""
     from deepbind_amd import _lib

@@ -503,3 +503,84 @@ def test_bulk_batch_training_step_uses_the_table_kernel_and_matches_layer_by_lay
         assert_close(a[k], b[k], GRAD, "fused vs layer-by-layer gradient %s" % k)
         assert np.array_equal(a[k], c[k]), "run-to-run difference in %s" % k
     assert np.abs(a["Wc"]).max() > 0
+
+
+@pytest.mark.parametrize("pool,hidden,loss,nesterov,rc", [("max", 0, "nll", True, False), ("all", 8, "mse", False, False),
+                                                           ("avg", 4, "nll", True, True), ("all", 0, "nll", True, True)])
+def test_natively_issued_step_equals_the_step_issued_call_by_call(pool, hidden, loss, nesterov, rc):
+    """dbk_train_step against the same entry points called one by one from the host: every variant of the
+    step (pooling, hidden layer, loss, plain momentum, reverse complements with mirrored input dropout,
+    frozen filters, the L1-decay switch-on) must leave bit-identical parameters, momenta, gradients and
+    generator position."""
+    from deepbind_amd import data, deepity_smat as ds
+    from deepbind_amd.model import SequenceNet
+    rng = np.random.default_rng(17)
+    ni, nf, m = 3, 5, 9
+    seqs = ["".join(rng.choice(list("ACGTN"), p=[.24, .24, .24, .24, .04], size=rng.integers(12, 40))) for _ in range(24)]
+    if rc:
+        seqs = orc.insert_reverse_complements(seqs)
+    Xh, Rh = data.pack_sequences(seqs, m - 1)
+    X, R = dev(Xh), dev(Rh)
+    Y = dev(rng.random((len(seqs), ni)).astype(np.float32))
+    M = dev(rng.random((len(seqs), ni)) < 0.8)
+
+    def make():
+        net = SequenceNet(ni, nf, m, pool=pool, hidden=hidden, loss=loss, rate=[0.05, 0.02, 0.1], momentum=0.8,
+                          dropout=[0.0, 0.3, 0.5], decay_conv=1e-3, decay_full=[1e-3, 0.0, 1e-2], weight_decay_start=2,
+                          nesterov=nesterov, reverse_complement=rc, input_dropout=0.2 if rc else 0.0, start_training=1)
+        net.rng_seed = 11
+        net.init_params(0.3, 0.3, 0.05, seed=4)
+        return net
+
+    native, stepwise = make(), make()
+    for i in range(4):
+        native.train_step(X, R, Y, M)
+        ds.gradstep(stepwise.P, stepwise.dP, stepwise.drate, stepwise.mP, stepwise.mrate,
+                    lambda: stepwise._grad_fused(X, R, Y, M, None), nesterov=nesterov)
+        stepwise.step_count += 1
+        torch.cuda.synchronize()
+        for name in ("P", "dP", "mP"):
+            a, b = getattr(native, name).cpu().numpy(), getattr(stepwise, name).cpu().numpy()
+            assert np.array_equal(a, b), "step %d: %s differs" % (i, name)
+        assert int(native.rng_counter.item()) == int(stepwise.rng_counter.item()) == native._rng_offset == stepwise._rng_offset
+    assert np.abs(native.mP.cpu().numpy()).max() > 0 and native.step_count == 4
+
+
+def test_group_steps_left_in_flight_match_joined_steps_across_changing_batches():
+    """ModelGroup.train_step(join=False) keeps the architecture groups running on their own streams from
+    step to step; joined steps, un-joined steps, a change of batch in between and accessors that join
+    implicitly must all give the same bits."""
+    from deepbind_amd import synth
+    from deepbind_amd.model import ModelGroup
+    cfg = synth.config4()
+    spec, hp = cfg["spec"], cfg["hp"]
+
+    def make():
+        grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
+                         decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"], weight_decay_start=3)
+        for gi, (idx, net) in enumerate(grp.groups):
+            net.rng_seed = 100 + gi
+            net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
+        return grp
+
+    joined, flying = make(), make()
+    X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
+    rng = np.random.default_rng(3)
+    Y2 = dev(rng.random(cfg["Y"].shape).astype(np.float32))
+    half = cfg["R"].shape[0] // 2                                    # a second, smaller batch: the first half of the regions
+    R3, Y3, M3 = dev(cfg["R"][:half]), dev(cfg["Y"][:half]), dev(cfg["Ymask"][:half])
+    batches = [(X, R, Y, M)] * 3 + [(X, R, Y2, M)] * 2 + [(X, R3, Y3, M3)] * 2 + [(X, R, Y, M)]
+    for i, (bx, br, by, bm) in enumerate(batches):
+        joined.train_step(bx, br, by, bm)
+        flying.train_step(bx, br, by, bm, join=False)
+        if i == 4:
+            # an accessor in the middle joins by itself and the next step forks again
+            pa = flying.predict(X, R)
+            assert np.array_equal(host(pa), host(joined.predict(X, R)))
+    pred_a, pred_b = host(flying.predict(X, R)), host(joined.predict(X, R))      # predict() joins first
+    assert np.array_equal(pred_a, pred_b)
+    for (_, a), (_, b) in zip(joined.groups, flying.groups):
+        pa, pb = a.get_params(), b.get_params()
+        for k in pa:
+            assert np.array_equal(pa[k], pb[k]), "%s/%d group, %s" % (a.pool, a.hidden, k)
+        assert a.step_count == b.step_count == len(batches) and a._rng_offset == b._rng_offset
