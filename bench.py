@@ -189,6 +189,14 @@ def ops_throughput(reps=5):
         dP = torch.randn_like(P)
         rec("scanpool_bprop[%s]" % pt, timed(lambda: ks.scanpool_bprop(W, b, X, R, pt, P, I, dP, dW, db, overwrite=True)),
             N + 2 * nout + B * F * 4, adds if pt == "all" else float(B) * F * m)
+        if pt == "all":
+            # with the forward pass leaving 1 bit per (row, filter) for the backward pass (N * F / 8 bytes each way)
+            act = ks.activity_words(X, W)
+            rec("scanpool_fprop general[all, argmax, masks]", timed(lambda: ks.scanpool_fprop(W, b, X, R, pt, want_argmax=True, act=act)),
+                N + nout + B * F * 4 + N * F // 8, adds)
+            rec("scanpool_bprop[all, masks]", timed(lambda: ks.scanpool_bprop(W, b, X, R, pt, P, I, dP, dW, db, overwrite=True, act=act)),
+                N + 2 * nout + B * F * 4 + N * F // 8, adds)
+            del act
     rec("scanpool_fprop table[max]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "max", path="kmer")), N + B * F * 4, adds)
     rec("scanpool_fprop table[max, argmax]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "max", want_argmax=True, path="kmer")),
         N + 2 * B * F * 4, adds)

@@ -37,10 +37,10 @@ _SIGNATURES = {
     "dbk_dropoutord_fp_tr": [_P, _P, _P, _P, _Z, _F, _U64, _U64, _P],
     "dbk_dropoutord_mirror": [_P, _P, _P, _P, _P, _Z, _Z],
     "dbk_dropoutord_fp_tr_u": [_P, _P, _P, _P, _Z, _F, _P],
-    "dbk_scanpool_fprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
-    "dbk_scanpool_fprop_general": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
+    "dbk_scanpool_fprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
+    "dbk_scanpool_fprop_general": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
     "dbk_scanpool_fprop_kmer": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
-    "dbk_scanpool_bprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P, _P, _P, _I],
+    "dbk_scanpool_bprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P, _P, _P, _I, _P],
     "dbk_blockwise_dot": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
     "dbk_blockwise_dot_nt": [_P, _I, _I, _I, _I, _I, _P, _P, _P],
     "dbk_blockwise_dot_tn": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
@@ -90,7 +90,7 @@ class TrainStepArgs(ctypes.Structure):
         ("input_rate", _F), ("Xdrop", _P), ("Mdrop", _P),
         ("rate", _P), ("seed", _U64), ("counter", _P),
         ("decay", _P), ("freeze_scan", _I),
-        ("pooled", _P), ("argmax", _P), ("Z", _P), ("dpooled", _P), ("loss", _P),
+        ("pooled", _P), ("argmax", _P), ("Z", _P), ("dpooled", _P), ("loss", _P), ("act", _P),
     ]
 
 _dll = None

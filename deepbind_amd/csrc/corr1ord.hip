@@ -193,6 +193,7 @@ __global__ __launch_bounds__(256) void corr1ord_bprop_X_kernel(T* __restrict__ d
 // positions, so the letters of a 16-position window are read once into scalar registers.
 // ---------------------------------------------------------------------------------------------
 constexpr unsigned WSUBS = 4;             // windows of PSUB positions per wave and staging round
+constexpr unsigned WSUBS_W = 8;           // the same for the filter-gradient kernel
 
 // forward: every (position, tap) is one LDS read with an immediate offset; taps in ascending order,
 // so the sums are bit-identical to the any-length kernel's. A workgroup builds its filter tile's
@@ -231,9 +232,10 @@ __global__ __launch_bounds__(256) void corr1ord_window_kernel(const T* __restric
     }
 }
 
-// filter gradient, pass 1: a lane keeps its filter's whole [tap][channel] column in registers; the
-// window's letters become four scalar weights (1 for the matching channel, 1/4 each for N, else 0)
-// applied as fused multiply-adds with exact products, i.e. one rounding per addition like a plain add.
+// filter gradient, pass 1: a lane keeps its filter's whole [letter][tap] column in registers; the window's
+// letters (scalars) pick the register plane each gradient value is added into through the register index
+// mode: one addition per (position, tap). "Mean of the four" letters collect in a plane of their own that
+// is spread over the four channels (x 1/4) at the end.
 // Workgroup y walks chunks y, y+gridDim.y, ... in ascending order; its waves are folded in wave order.
 template <int MT>
 __global__ __launch_bounds__(256) void corr1ord_bprop_W_window_kernel(float* __restrict__ partial, unsigned m, unsigned F,
@@ -243,46 +245,38 @@ __global__ __launch_bounds__(256) void corr1ord_bprop_W_window_kernel(float* __r
     extern __shared__ __align__(16) unsigned char smem[];
     float* fold = reinterpret_cast<float*>(smem);                          // [MT*4][FT]
     uint8_t* xl = smem + (size_t)MT * 4 * FT * sizeof(float);
-    const unsigned nw = blockDim.x >> 6, chunk = nw * WSUBS * PSUB;
+    const unsigned nw = blockDim.x >> 6, chunk = nw * WSUBS_W * PSUB;
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const unsigned f0 = blockIdx.x * FT, f = f0 + lane;
     const size_t N = n + m - 1;
-    float aw[MT][4];
-#pragma unroll
-    for (int j = 0; j < MT; ++j) aw[j][0] = aw[j][1] = aw[j][2] = aw[j][3] = 0.0f;
+    grad_planes<MT> planes;                                                // [letter][tap] accumulators in fixed registers
+    planes.clear();
     for (size_t c0 = (size_t)blockIdx.y * chunk; c0 < n; c0 += (size_t)gridDim.y * chunk) {
         const unsigned rows = (unsigned)((n - c0) < chunk ? (n - c0) : chunk);
         __syncthreads();
         stage(xl, X, N, c0, window_span<MT>(rows));
         __syncthreads();
+        // the next window's gradient rows are requested before this window's additions start
+        float g[PSUB], gn[PSUB];
+        auto fetch = [&](unsigned p0, float (&dst)[PSUB]) {
+#pragma unroll
+            for (int p = 0; p < PSUB; ++p) dst[p] = (f < F && p0 + p < rows) ? dZ[(c0 + p0 + p) * F + f] : 0.0f;
+        };
+        fetch(wave * PSUB, g);
 #pragma unroll 1
-        for (unsigned s = 0; s < WSUBS; ++s) {
+        for (unsigned s = 0; s < WSUBS_W; ++s) {
             const unsigned p0 = (s * nw + wave) * PSUB;
             if (p0 >= rows) break;
-            float g[PSUB];
-#pragma unroll
-            for (int p = 0; p < PSUB; ++p) g[p] = (f < F && p0 + p < rows) ? dZ[(c0 + p0 + p) * F + f] : 0.0f;
+            fetch(p0 + nw * PSUB, gn);                                     // all zero past the chunk's rows
             unsigned wq[window<MT>::words];
             load_window<MT>(xl, p0, wq);
+            grad_planes_window<MT>(planes, wq, g);                         // one add per (position, tap)
 #pragma unroll
-            for (int q = 0; q < PSUB + MT - 1; ++q) {
-                const unsigned l = window_letter(wq, q);
-                const float base = l == 4u ? 0.25f : 0.0f;
-                const float m0 = l == 0u ? 1.0f : base, m1 = l == 1u ? 1.0f : base;
-                const float m2 = l == 2u ? 1.0f : base, m3 = l == 3u ? 1.0f : base;
-#pragma unroll
-                for (int p = 0; p < PSUB; ++p) {
-                    const int j = q - p;
-                    if (j >= 0 && j < MT) {
-                        aw[j][0] = __builtin_fmaf(g[p], m0, aw[j][0]);
-                        aw[j][1] = __builtin_fmaf(g[p], m1, aw[j][1]);
-                        aw[j][2] = __builtin_fmaf(g[p], m2, aw[j][2]);
-                        aw[j][3] = __builtin_fmaf(g[p], m3, aw[j][3]);
-                    }
-                }
-            }
+            for (int p = 0; p < PSUB; ++p) g[p] = gn[p];
         }
     }
+    float aw[MT][4];
+    grad_planes_read<MT>(planes, aw);
     float* mine = fold + lane;
     for (unsigned w = 0; w < nw; ++w) {
         __syncthreads();
@@ -430,9 +424,9 @@ int launch_fprop(hipStream_t st, const T* W, size_t m, size_t F, const uint8_t* 
 inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, const uint8_t* X, size_t n, const float* dZ)
 {
     const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : 24);
-    const unsigned ftiles = dbk::divup(F, FT), chunk = 4 * WSUBS * PSUB;
+    const unsigned ftiles = dbk::divup(F, FT), chunk = 4 * WSUBS_W * PSUB;
     const unsigned nchunk = dbk::divup(n, chunk);
-    unsigned gy = 768u / ftiles;                               // three workgroups fit a CU
+    unsigned gy = (mt == 8 ? 768u : 512u) / ftiles;           // three workgroups fit a CU with 8 taps' register planes, else two
     if (gy < 1) gy = 1;
     if (gy > nchunk) gy = nchunk;
     const size_t nelem = 4 * m * F;

@@ -55,7 +55,7 @@ extern "C" {
 
 const char* dbk_last_error(void) { return dbk::g_err; }
 
-int dbk_version(void) { return 1; }
+int dbk_version(void) { return 2; }
 
 int dbk_device_count(void)
 {

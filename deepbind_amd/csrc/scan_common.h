@@ -1,6 +1,7 @@
 // Pieces shared by the scan kernels: the 6-letter alphabet and the [tap][letter][filter] LDS table.
 #pragma once
 #include "dbk_common.h"
+#include <utility>
 
 namespace dbk_scan {
 
@@ -89,6 +90,100 @@ __device__ __forceinline__ void scan16_window(const T* __restrict__ lut, const u
                          "+v"(acc[14]), "+v"(acc[15]));
         }
     }
+}
+
+// ---- filter-gradient accumulation through the VGPR index mode -------------------------------------
+// dW[tap j][letter c][filter] += g[position p] for every (p, j) of a window whose letter at p + j is c.
+// The letter is the same for all lanes (a scalar), the filter is the lane. Spelled with ordinary
+// arithmetic this takes four multiply-adds per (p, j) (letter weights 1 / 0 / 1/4 per channel); with
+// the accumulators laid out as six planes of MT consecutive registers - plane = letter: A, C, G, T,
+// "mean of the four", "nothing" - and the hardware's register index mode (s_set_gpr_idx_on: M0[7:0]
+// is added to the register number of src0 and dst), it is ONE v_add_f32 per (p, j) plus one scalar
+// instruction per letter. The planes live in fixed registers v96.. so that the instruction text can
+// name them; the compiler keeps everything else below. Plane 4 is spread over the four channels
+// (x 1/4) and plane 5 is dropped when the planes are read out.
+typedef float v32f __attribute__((ext_vector_type(32)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+constexpr int GRAD_PLANES = 6;
+
+template <int MT> struct grad_planes {
+    static_assert(MT == 8 || MT == 16 || MT == 24, "plane sets exist for 8, 16 and 24 taps");
+    v32f t0, t1, t2, t3;            // v[96:127], v[128:159], v[160:191], v[192:223]   (as many as 6*MT needs)
+    v16f u0;                        // MT = 8: v[128:143], MT = 24: v[224:239]
+    __device__ __forceinline__ void clear()
+    {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) t0[i] = t1[i] = t2[i] = t3[i] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) u0[i] = 0.0f;
+    }
+    // register e of the plane set (plane * MT + tap)
+    template <int E> __device__ __forceinline__ float reg() const
+    {
+        static_assert(E >= 0 && E < GRAD_PLANES * MT, "register outside the plane set");
+        if constexpr (MT == 8) return E < 32 ? t0[E % 32] : u0[(E - 32) % 16];
+        else if constexpr (E < 32) return t0[E % 32];
+        else if constexpr (E < 64) return t1[E % 32];
+        else if constexpr (E < 96) return t2[E % 32];
+        else if constexpr (E < 128) return t3[E % 32];
+        else return u0[(E - 128) % 16];
+    }
+    // gradient of tap J, channel C: the letter's own plane plus a quarter of the "mean" plane
+    template <int J, int C> __device__ __forceinline__ float grad() const { return reg<C * MT + J>() + 0.25f * reg<4 * MT + J>(); }
+};
+
+#define DBK_GP_LIST(...) __VA_ARGS__
+#define DBK_GP_SLOT(P) ".if ((%c[q] - " #P ") >= 0) && ((%c[q] - " #P ") < %c[mt])\n\t" \
+                       "v_add_f32 v[96 + %c[q] - " #P "], v[96 + %c[q] - " #P "], %[g" #P "]\n\t.endif\n\t"
+#define DBK_GP_ASM(PLANES)                                                                                          \
+    asm volatile("s_set_gpr_idx_on %[idx], 0x9\n\t"                                                                  \
+                 DBK_GP_SLOT(0) DBK_GP_SLOT(1) DBK_GP_SLOT(2) DBK_GP_SLOT(3) DBK_GP_SLOT(4) DBK_GP_SLOT(5) DBK_GP_SLOT(6)   \
+                 DBK_GP_SLOT(7) DBK_GP_SLOT(8) DBK_GP_SLOT(9) DBK_GP_SLOT(10) DBK_GP_SLOT(11) DBK_GP_SLOT(12)            \
+                 DBK_GP_SLOT(13) DBK_GP_SLOT(14) DBK_GP_SLOT(15)                                                     \
+                 "s_set_gpr_idx_off"                                                                                \
+                 : PLANES                                                                                           \
+                 : [idx] "s"(idx), [q] "n"(Q), [mt] "n"(MT), [g0] "v"(g[0]), [g1] "v"(g[1]), [g2] "v"(g[2]),        \
+                   [g3] "v"(g[3]), [g4] "v"(g[4]), [g5] "v"(g[5]), [g6] "v"(g[6]), [g7] "v"(g[7]), [g8] "v"(g[8]),  \
+                   [g9] "v"(g[9]), [g10] "v"(g[10]), [g11] "v"(g[11]), [g12] "v"(g[12]), [g13] "v"(g[13]),          \
+                   [g14] "v"(g[14]), [g15] "v"(g[15]))
+
+// All (p, j) pairs of the window that meet letter position Q: tap j = Q - p of position p.
+template <int Q, int MT>
+__device__ __forceinline__ void grad_planes_add(grad_planes<MT>& A, unsigned letter, const float (&g)[PSUB])
+{
+    static_assert(PSUB == 16, "the instruction text lists 16 positions");
+    // M0 (which the index lives in while the mode is on) is left changed: the compiler never carries a value
+    // in M0 across other code - it writes M0 immediately before each instruction that reads it - and saving
+    // and restoring it here costs more than the sixteen additions (measured: +48 %).
+    const unsigned idx = letter * (unsigned)MT;          // first register of the letter's plane, relative to v96
+    if constexpr (MT == 8) DBK_GP_ASM(DBK_GP_LIST("+{v[96:127]}"(A.t0), "+{v[128:143]}"(A.u0)));
+    else if constexpr (MT == 16) DBK_GP_ASM(DBK_GP_LIST("+{v[96:127]}"(A.t0), "+{v[128:159]}"(A.t1), "+{v[160:191]}"(A.t2)));
+    else DBK_GP_ASM(DBK_GP_LIST("+{v[96:127]}"(A.t0), "+{v[128:159]}"(A.t1), "+{v[160:191]}"(A.t2), "+{v[192:223]}"(A.t3), "+{v[224:239]}"(A.u0)));
+}
+
+template <int MT, int... Q>
+__device__ __forceinline__ void grad_planes_window(grad_planes<MT>& A, const unsigned (&wq)[window<MT>::words], const float (&g)[PSUB],
+                                                   std::integer_sequence<int, Q...>)
+{
+    (grad_planes_add<Q, MT>(A, window_letter(wq, Q), g), ...);
+}
+// Adds one sub-chunk (PSUB positions with gradients g, window letters wq) into the planes.
+template <int MT>
+__device__ __forceinline__ void grad_planes_window(grad_planes<MT>& A, const unsigned (&wq)[window<MT>::words], const float (&g)[PSUB])
+{
+    grad_planes_window<MT>(A, wq, g, std::make_integer_sequence<int, PSUB + MT - 1>{});
+}
+
+template <int MT, int... E>
+__device__ __forceinline__ void grad_planes_read(const grad_planes<MT>& A, float (&aw)[MT][4], std::integer_sequence<int, E...>)
+{
+    ((aw[E / 4][E % 4] = A.template grad<E / 4, E % 4>()), ...);
+}
+// The finished [tap][channel] gradient column of this lane's filter.
+template <int MT>
+__device__ __forceinline__ void grad_planes_read(const grad_planes<MT>& A, float (&aw)[MT][4])
+{
+    grad_planes_read<MT>(A, aw, std::make_integer_sequence<int, 4 * MT>{});
 }
 
 // Stages letters for absolute positions [c0, c0+cnt) into xl; past the end of X -> "nothing".

@@ -44,7 +44,8 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
                                                              unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
                                                              const uint32_t* __restrict__ R, size_t P,
                                                              float* __restrict__ pooled, uint32_t* __restrict__ argmax,
-                                                             const unsigned* __restrict__ run_if_flag)
+                                                             const unsigned* __restrict__ run_if_flag,
+                                                             unsigned long long* __restrict__ act)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     // when given, the launch only does work if the device flag is set (fallback behind the k-mer kernel)
@@ -81,6 +82,18 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
                     scan16_window<MT ? MT : 1>(lut, wq, lane, acc);
                 } else {
                     scan16(lut, xl, m, p0, lane, acc);
+                }
+                if (act) {
+                    // which rectifiers are open, for the backward pass: one 64-bit lane mask per (row, filter tile);
+                    // lane p of the wave stores row p's
+                    unsigned long long mine = 0;
+#pragma unroll
+                    for (int p = 0; p < PSUB; ++p) {
+                        const size_t i = c0 + p0 + p;
+                        const unsigned long long open = __ballot(((i < n ? acc[p] : 0.0f) + bf) > 0.0f);
+                        if (lane == (unsigned)p) mine = open;
+                    }
+                    if (lane < (unsigned)PSUB && p0 + lane < rows) act[(c0 + p0 + lane) * gridDim.y + blockIdx.y] = mine;
                 }
 #pragma unroll
                 for (int p = 0; p < PSUB; ++p) {
@@ -353,9 +366,8 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
     build_letter_table(lut, W, m, F, f0, MT);
     const float bf = f < F ? bias[f] : 0.0f;
     float db = 0.0f;
-    float aw[MT][4];
-#pragma unroll
-    for (int j = 0; j < MT; ++j) aw[j][0] = aw[j][1] = aw[j][2] = aw[j][3] = 0.0f;
+    grad_planes<MT> planes;                                        // [letter][tap] accumulators in fixed registers
+    planes.clear();
 
     for (size_t r = blockIdx.x; r < P; r += gridDim.x) {
         const size_t a = R[2 * r], b = R[2 * r + 1];
@@ -384,26 +396,12 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
                     db += gg;
                     g[p] = i < n ? gg : 0.0f;                   // rows past the scan's end carry bias only
                 }
-#pragma unroll
-                for (int q = 0; q < PSUB + MT - 1; ++q) {
-                    const unsigned l = window_letter(wq, q);
-                    const float base = l == 4u ? 0.25f : 0.0f;
-                    const float m0 = l == 0u ? 1.0f : base, m1 = l == 1u ? 1.0f : base;
-                    const float m2 = l == 2u ? 1.0f : base, m3 = l == 3u ? 1.0f : base;
-#pragma unroll
-                    for (int p = 0; p < PSUB; ++p) {
-                        const int j = q - p;
-                        if (j >= 0 && j < MT) {
-                            aw[j][0] = __builtin_fmaf(g[p], m0, aw[j][0]);
-                            aw[j][1] = __builtin_fmaf(g[p], m1, aw[j][1]);
-                            aw[j][2] = __builtin_fmaf(g[p], m2, aw[j][2]);
-                            aw[j][3] = __builtin_fmaf(g[p], m3, aw[j][3]);
-                        }
-                    }
-                }
+                grad_planes_window<MT>(planes, wq, g);         // one add per (position, tap), the letter picks the plane
             }
         }
     }
+    float aw[MT][4];
+    grad_planes_read<MT>(planes, aw);
     // fold the waves in wave order through the (now unused) letter table's memory
     dbacc[wave * FT + lane] = db;
     float* fold = lut + lane;
@@ -452,25 +450,117 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
     }
 }
 
+// Dense half of the backward pass when the forward pass left its activity masks (one 64-bit lane mask per
+// row and filter tile: bit l set = the rectifier of filter tile*64 + l is open at that row): nothing is
+// recomputed and no table is needed. Per window of 16 positions a wave reads 16 masks (lane p reads row p's,
+// one window ahead), turns each into this lane's gradient value (davg/count or 0) and adds the window
+// into the register planes, one addition per (position, tap).
+template <int PT, int MT>
+__global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                       const uint32_t* __restrict__ R, size_t P,
+                                                                       const float* __restrict__ dpooled,
+                                                                       const unsigned long long* __restrict__ act,
+                                                                       float* __restrict__ slabs, size_t stride)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const unsigned nw = blockDim.x >> 6;
+    const unsigned chunk = nw * XCH_SUBS * PSUB;
+    float* lut = reinterpret_cast<float*>(smem);                   // [MT*4][FT]: only the cross-wave fold at the end uses it
+    float* dbacc = lut + (size_t)MT * 4 * FT;                      // [nw][FT]
+    uint8_t* xl = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT);
+
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
+    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
+    float db = 0.0f;
+    grad_planes<MT> planes;
+    planes.clear();
+
+    for (size_t r = blockIdx.x; r < P; r += gridDim.x) {
+        const size_t a = R[2 * r], b = R[2 * r + 1];
+        const size_t j0 = r * F + f;
+        const float gavg = f < F ? (PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1]) / (float)(b - a) : 0.0f;
+        for (size_t c0 = a; c0 < b; c0 += chunk) {
+            const unsigned rows = (unsigned)((b - c0) < chunk ? (b - c0) : chunk);
+            __syncthreads();
+            stage(xl, X, N, c0, window_span<MT>(rows));
+            __syncthreads();
+            auto fetch = [&](unsigned p0) -> unsigned long long {      // rows past the chunk read as "closed"
+                return (lane < (unsigned)PSUB && p0 + lane < rows) ? act[(c0 + p0 + lane) * gridDim.y + blockIdx.y] : 0ull;
+            };
+            unsigned long long mk = fetch(wave * PSUB);
+#pragma unroll 1
+            for (unsigned s = 0; s < XCH_SUBS; ++s) {
+                const unsigned p0 = (s * nw + wave) * PSUB;
+                if (p0 >= rows) break;
+                const unsigned long long mkn = fetch(p0 + nw * PSUB);
+                unsigned wq[window<MT>::words];
+                load_window<MT>(xl, p0, wq);
+                float g[PSUB];
+#pragma unroll
+                for (int p = 0; p < PSUB; ++p) {
+                    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)mk, p);
+                    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(mk >> 32), p);
+                    const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
+                    const float gg = open ? gavg : 0.0f;
+                    db += gg;
+                    g[p] = c0 + p0 + p < n ? gg : 0.0f;            // rows past the scan's end carry bias only
+                }
+                grad_planes_window<MT>(planes, wq, g);
+                mk = mkn;
+            }
+        }
+    }
+    float aw[MT][4];
+    grad_planes_read<MT>(planes, aw);
+    dbacc[wave * FT + lane] = db;
+    float* fold = lut + lane;
+    for (unsigned w = 0; w < nw; ++w) {
+        __syncthreads();
+        if (wave == w) {
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                if ((unsigned)j < m) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float* cell = fold + (j * 4 + c) * FT;
+                        *cell = w == 0 ? aw[j][c] : *cell + aw[j][c];
+                    }
+                }
+        }
+    }
+    __syncthreads();
+    float* out = slabs + (size_t)blockIdx.x * stride;
+    for (unsigned e = threadIdx.x; e < m * 4 * FT; e += blockDim.x) {
+        const unsigned row = e / FT, fl = e % FT;
+        if (f0 + fl < F) out[(size_t)row * F + f0 + fl] = lut[e];
+    }
+    if (wave == 0 && f < F) {
+        float t = dbacc[lane];
+        for (unsigned w = 1; w < nw; ++w) t += dbacc[w * FT + lane];
+        out[(size_t)4 * m * F + f] = t;
+    }
+}
+
 template <int PT, int MT>
 void launch_fprop_mt(hipStream_t st, unsigned gx, unsigned ftiles, unsigned nw, size_t smem, const float* W, const float* bias, size_t m,
                      size_t F, const uint8_t* X, size_t N, const uint32_t* R, size_t P, float* pooled, uint32_t* argmax,
-                     const unsigned* run_if_flag)
+                     const unsigned* run_if_flag, unsigned long long* act)
 {
     if (argmax) {
         auto kern = scanpool_fprop_kernel<PT, true, MT>;
         hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag, act);
     } else {
         auto kern = scanpool_fprop_kernel<PT, false, MT>;
         hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag, act);
     }
 }
 
 template <int PT>
 int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
-                    const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, const unsigned* run_if_flag)
+                    const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, const unsigned* run_if_flag, unsigned long long* act)
 {
     const unsigned nw = 4;
     const unsigned chunk = nw * XCH_SUBS * PSUB;
@@ -485,19 +575,26 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     if (gx < 1) gx = 1;
     if (gx > P) gx = (unsigned)P;
     switch (mt) {
-    case 8:  launch_fprop_mt<PT, 8>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
-    case 16: launch_fprop_mt<PT, 16>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
-    case 24: launch_fprop_mt<PT, 24>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
-    case 32: launch_fprop_mt<PT, 32>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
-    default: launch_fprop_mt<PT, 0>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag); break;
+    case 8:  launch_fprop_mt<PT, 8>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    case 16: launch_fprop_mt<PT, 16>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    case 24: launch_fprop_mt<PT, 24>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    case 32: launch_fprop_mt<PT, 32>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    default: launch_fprop_mt<PT, 0>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
     }
     DBK_LAUNCH_OK();
 }
 
 template <int PT, int MT>
 void launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, const float* W, const float* bias, size_t m, size_t F,
-                  const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* dpooled, float* slabs, size_t stride)
+                  const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* dpooled, const unsigned long long* act,
+                  float* slabs, size_t stride)
 {
+    if (act) {
+        auto kern = scanpool_bprop_dense_act_kernel<PT, MT>;
+        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, (unsigned)m, (unsigned)F, X, N, R, P, dpooled, act, slabs, stride);
+        return;
+    }
     auto kern = scanpool_bprop_dense_kernel<PT, MT>;
     hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, dpooled, slabs, stride);
@@ -506,7 +603,7 @@ void launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, con
 template <int PT>
 int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                     const uint32_t* R, size_t P, const float* pooled, const uint32_t* argmax, const float* dpooled,
-                    float* dW, float* dbias, bool overwrite)
+                    float* dW, float* dbias, bool overwrite, const unsigned long long* act)
 {
     const unsigned ftiles = dbk::divup(F, FT);
     DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
@@ -539,9 +636,10 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);
         if (gxs < 1) gxs = 1;
     }
-    // dense half: ~768 four-wave workgroups (three resident per CU)
+    // dense half: four-wave workgroups, as many as are resident at once (its register planes leave room for
+    // two per CU, three with 8 taps)
     if (PT != DBK_PT_MAX) {
-        gxd = 768u / ftiles;
+        gxd = (mt == 8 ? 768u : 512u) / ftiles;
         if (gxd < 1) gxd = 1;
         if (gxd > P) gxd = (unsigned)P;
     }
@@ -558,21 +656,22 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     if (gxd) {
         constexpr int PD = PT == DBK_PT_MAX ? DBK_PT_AVG : PT;
         float* sd = slabs + stride * gxs;
-        if (mt == 8) launch_dense<PD, 8>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
-        else if (mt == 16) launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
-        else launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, sd, stride);
+        if (mt == 8) launch_dense<PD, 8>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, act, sd, stride);
+        else if (mt == 16) launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, act, sd, stride);
+        else launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, act, sd, stride);
     }
     hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd, overwrite);
     DBK_LAUNCH_OK();
 }
 
 int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
-          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, const unsigned* run_if_flag)
+          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, const unsigned* run_if_flag,
+          unsigned long long* act)
 {
     switch (ptype) {
-    case DBK_PT_MAX: return launch_fprop_pt<DBK_PT_MAX>(st, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag);
-    case DBK_PT_AVG: return launch_fprop_pt<DBK_PT_AVG>(st, W, bias, m, F, X, N, R, P, pooled, nullptr, run_if_flag);
-    default:         return launch_fprop_pt<DBK_PT_ALL>(st, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag);
+    case DBK_PT_MAX: return launch_fprop_pt<DBK_PT_MAX>(st, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act);
+    case DBK_PT_AVG: return launch_fprop_pt<DBK_PT_AVG>(st, W, bias, m, F, X, N, R, P, pooled, nullptr, run_if_flag, act);
+    default:         return launch_fprop_pt<DBK_PT_ALL>(st, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act);
     }
 }
 
@@ -588,7 +687,7 @@ extern "C" {
 
 int dbk_scanpool_fprop_general(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
                                const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
-                               float* pooled, uint32_t* argmax)
+                               float* pooled, uint32_t* argmax, uint64_t* act)
 {
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
@@ -598,12 +697,13 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream, const float* W, const float*
               "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
-    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr);
+    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr,
+                                       reinterpret_cast<unsigned long long*>(act));
 }
 
 int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
                        const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
-                       float* pooled, uint32_t* argmax)
+                       float* pooled, uint32_t* argmax, uint64_t* act)
 {
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
@@ -613,14 +713,20 @@ int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, s
               "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
-    int rc = dbk_scanpool_kmer::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax);
-    if (rc >= 0) return rc;
-    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr);
+    // the activity masks are written by the general kernel only (the k-mer table is worth its set-up for bulk scoring,
+    // where no backward pass follows)
+    if (!act) {
+        int rc = dbk_scanpool_kmer::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax);
+        if (rc >= 0) return rc;
+    }
+    return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr,
+                                       reinterpret_cast<unsigned long long*>(act));
 }
 
 int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
                        const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
-                       const float* pooled, const uint32_t* argmax, const float* dpooled, float* dW, float* dbias, int overwrite)
+                       const float* pooled, const uint32_t* argmax, const float* dpooled, float* dW, float* dbias, int overwrite,
+                       const uint64_t* act)
 {
     using namespace dbk_scanpool_general;
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
@@ -637,10 +743,11 @@ int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, s
     DBK_CHECK(ptype == DBK_PT_AVG || argmax != nullptr, "ValueError: pooledmaps_argmax must be specified for max pooling.");
     DBK_CHECK(X && regions && pooled && dpooled, "ValueError: null pointer argument");
     hipStream_t st = dbk::as_stream(stream);
+    const unsigned long long* am = reinterpret_cast<const unsigned long long*>(act);
     switch (ptype) {
-    case DBK_PT_MAX: return launch_bprop_pt<DBK_PT_MAX>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0);
-    case DBK_PT_AVG: return launch_bprop_pt<DBK_PT_AVG>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0);
-    default:         return launch_bprop_pt<DBK_PT_ALL>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0);
+    case DBK_PT_MAX: return launch_bprop_pt<DBK_PT_MAX>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0, am);
+    case DBK_PT_AVG: return launch_bprop_pt<DBK_PT_AVG>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0, am);
+    default:         return launch_bprop_pt<DBK_PT_ALL>(st, W, bias, m, nfilter, X, N, regions, nregion, pooled, argmax, dpooled, dW, dbias, overwrite != 0, am);
     }
 }
 

@@ -47,7 +47,8 @@
 
 namespace dbk_scanpool_general {
 int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
-          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, const unsigned* run_if_flag);
+          const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, const unsigned* run_if_flag,
+          unsigned long long* act);
 }
 
 namespace dbk_scanpool_kmer {
@@ -422,7 +423,7 @@ int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size
     if (rc != 0) return rc;
     // inputs the table cannot express (code 254, regions outside the sequence): the general kernel
     // runs instead, gated on the same device flag so that no host synchronisation is needed
-    rc = dbk_scanpool_general::fprop(st, W, bias, m, F, X, N, R, P, ptype, pooled, argmax, flag);
+    rc = dbk_scanpool_general::fprop(st, W, bias, m, F, X, N, R, P, ptype, pooled, argmax, flag, nullptr);
     return rc;
 }
 

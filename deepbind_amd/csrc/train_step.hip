@@ -67,8 +67,9 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
         if (rc) return rc;
         X = a->Xdrop;
     }
+    uint64_t* act = a->ptype == DBK_PT_MAX ? nullptr : a->act;      // only the average part of the backward pass reads the masks
     rc = dbk_scanpool_fprop(stream, P + a->off_Wc, P + a->off_bc, a->m, F, X, a->N, a->regions, a->nregion, a->ptype,
-                            a->pooled, a->argmax);
+                            a->pooled, a->argmax, act);
     if (rc) return rc;
     const uint64_t draws = a->rate ? (a->nregion * k * a->nmodel + 3) / 4 : 0;
     rc = dbk_head_train(stream, a->nregion, (int)a->nmodel, (int)k, (int)a->hidden, a->loss_kind, a->reverse_complement,
@@ -79,7 +80,7 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
                         a->loss);
     if (rc) return rc;
     rc = dbk_scanpool_bprop(stream, P + a->off_Wc, P + a->off_bc, a->m, F, X, a->N, a->regions, a->nregion, a->ptype,
-                            a->pooled, a->argmax, a->dpooled, dP + a->off_Wc, dP + a->off_bc, 1);
+                            a->pooled, a->argmax, a->dpooled, dP + a->off_Wc, dP + a->off_bc, 1, act);
     if (rc) return rc;
     if (a->decay) {
         rc = dbk_l1_decay(stream, DBK_F32, P, a->decay, dP, a->nparam);

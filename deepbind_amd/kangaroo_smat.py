@@ -134,10 +134,17 @@ def dropoutord_fp_train(X, rate, U=None, regions=None, padding=None, seed=None, 
 # ------------------------------------------------------------------------------------------------
 # fused scan + bias + ReLU + pool
 # ------------------------------------------------------------------------------------------------
-def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto"):
+def activity_words(X, W):
+    """Empty buffer for the activity masks of scanpool_fprop: one 64-bit word per row of X and tile of 64 filters."""
+    return torch.empty((X.numel(), (W.shape[1] + 63) // 64), dtype=torch.int64, device=W.device)
+
+
+def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=None):
     """pool(relu(corr1ord(W, X) + b)) per region without storing the (N x P) map.
     Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only.
-    path: "auto" lets the library choose, "general" / "kmer" force one kernel."""
+    path: "auto" lets the library choose, "general" / "kmer" force one kernel.
+    act (optional, from activity_words): receives 1 bit per row and filter - rectifier open or not - which
+    scanpool_bprop takes in place of recomputing the map (general kernel only)."""
     _u8(X)
     _regions(regions)
     require(regions.shape[1] == 2, "ValueError: the fused path takes 2-column regions")
@@ -147,13 +154,26 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto"):
     pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
     argmax = torch.empty((P, F), dtype=uindex, device=W.device) if (want_argmax and ptype in ("max", "all")) else None
     entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "kmer": "dbk_scanpool_fprop_kmer"}[path]
-    call(entry, stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(),
-         ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax))
+    args = [stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax)]
+    if path != "kmer":
+        args.append(_act(act, X, F))
+    else:
+        require(act is None, "ValueError: the table kernel does not write activity masks")
+    call(entry, *args)
     return pooled, argmax
 
 
-def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db, overwrite=False):
-    """Backward of scanpool_fprop: dW += filter gradient (dW[:] = with overwrite), db[:] = bias gradient."""
+def _act(act, X, F):
+    if act is None:
+        return None
+    require(act.dtype == torch.int64 and act.numel() == X.numel() * ((F + 63) // 64),
+            "ValueError: act must hold one 64-bit word per row of X and tile of 64 filters")
+    return ptr(act)
+
+
+def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db, overwrite=False, act=None):
+    """Backward of scanpool_fprop: dW += filter gradient (dW[:] = with overwrite), db[:] = bias gradient.
+    act: the activity masks the forward call filled (same W, b, X, regions), if it was given any."""
     _u8(X)
     _regions(regions)
     require(W.dtype == torch.float32 and dpooled.dtype == torch.float32, "TypeError: the fused path is float32 only")
@@ -161,4 +181,4 @@ def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db, ove
     require(dpooled.shape == pooled.shape, "ValueError: dpooled must have pooled's shape")
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
     call("dbk_scanpool_bprop", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype],
-         ptr(pooled), ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)))
+         ptr(pooled), ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)), _act(act, X, F))

@@ -401,7 +401,9 @@ class SequenceNet(object):
         forward+backward (+ chunk reduction), fused scan+pool backward (+ slab reduction)."""
         p, g = self.p, self.g
         X = self._drop_inputs(X, R, U_input)
-        pooled, amax = ks.scanpool_fprop(p["Wc"], p["bc"], X, R, self.pool, want_argmax=True)
+        # average pooling: the forward pass leaves 1 bit per (row, filter), rectifier open or not, for the backward pass
+        act = ks.activity_words(X, p["Wc"]) if self.pool != "max" else None
+        pooled, amax = ks.scanpool_fprop(p["Wc"], p["bc"], X, R, self.pool, want_argmax=True, act=act)
         rate = self.dropout if self.use_dropout else None
         draws = (pooled.numel() + 3) // 4 if (rate is not None and U is None) else 0
         Z, dpooled, _ = ds.head_train(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), Y, self.ninst, self.loss,
@@ -409,7 +411,7 @@ class SequenceNet(object):
                                       seed=self.rng_seed, counter=self.rng_counter, counter_advance=draws,
                                       reverse_complement=self.reverse_complement)
         self._rng_offset += draws
-        ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, pooled, amax, dpooled, g["Wc"], g["bc"], overwrite=True)
+        ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, pooled, amax, dpooled, g["Wc"], g["bc"], overwrite=True, act=act)
         if self.weight_decay_start <= self.step_count:
             self._add_decay()
         if self.step_count < self.start_training:
@@ -460,6 +462,7 @@ class SequenceNet(object):
                     dpooled=torch.empty((P, self.k * ni), dtype=torch.float32, device=dev),
                     argmax=torch.empty((P, self.nfilter * ni), dtype=ks.uindex, device=dev) if self.pool != "avg" else None,
                     Z=torch.empty((P, ni), dtype=torch.float32, device=dev),
+                    act=ks.activity_words(X, self.p["Wc"]) if self.pool != "max" else None,
                     Xdrop=torch.empty(X.numel(), dtype=torch.uint8, device=dev) if self.input_dropout > 0 else None,
                     Mdrop=torch.empty(X.numel(), dtype=torch.bool, device=dev) if self.input_dropout > 0 else None)
         a.nesterov, a.seed = int(bool(self.nesterov)), int(self.rng_seed)

@@ -114,12 +114,17 @@ int dbk_dropoutord_mirror(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uin
  * reaching past N contribute nothing (the unfused chain leaves those rows at relu(bias)).
  * float32 only. Replaces the chain corr1ord -> bias -> relu -> poolrgn
  * (reference: kangaroo/_ext/corr1ord.py:97-117, deepity/std/elemwise.py:71-82,162-180,
- *  kangaroo/_ext/poolrgn.py:56-76,153-174). */
+ *  kangaroo/_ext/poolrgn.py:56-76,153-174).
+ * act (may be NULL): N * ceil(nfilter/64) 64-bit words that receive, for every row inside a region and
+ * every tile of 64 filters, the mask of filters whose rectifier is open there (bit l = filter tile*64 + l):
+ * what the reference's relu node keeps as its output for the backward pass (elemwise.py:78), 1 bit per
+ * value. Hand it to dbk_scanpool_bprop and the average-pooling gradient needs no recomputation. With act
+ * the general kernel runs (the table kernel does not write it). */
 int dbk_scanpool_fprop(dbk_stream_t stream,
                        const float* W, const float* bias, size_t m, size_t nfilter,
                        const uint8_t* X, size_t N,
                        const uint32_t* regions, size_t nregion, int ptype,
-                       float* pooled, uint32_t* argmax);
+                       float* pooled, uint32_t* argmax, uint64_t* act);
 
 /* Same contract, always through the general kernel (any filter length that fits in LDS, any letter
  * code); dbk_scanpool_fprop picks a faster kernel when the shape allows and otherwise calls this. */
@@ -127,7 +132,7 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream,
                                const float* W, const float* bias, size_t m, size_t nfilter,
                                const uint8_t* X, size_t N,
                                const uint32_t* regions, size_t nregion, int ptype,
-                               float* pooled, uint32_t* argmax);
+                               float* pooled, uint32_t* argmax, uint64_t* act);
 
 /* Same contract through the 3-mer lookup-table kernel regardless of problem size; fails with
  * NotImplementedError for shapes that kernel does not take (filter length > 24, avg/all pooling,
@@ -142,6 +147,8 @@ int dbk_scanpool_fprop_kmer(dbk_stream_t stream,
 /* Backward of the fused chain: given dpooled (same layout as pooled), the forward's pooled and
  * argmax, accumulates dW (C*m, F) += (as corr1ord_bprop_W does; with overwrite != 0 it is written
  * instead, which saves the caller a fill) and writes dbias (1, F) =. Deterministic (no float atomics).
+ * act (may be NULL): the activity masks dbk_scanpool_fprop wrote for the same W, bias, X and regions;
+ * without them the avg / all gradient recomputes the map through the letter table.
  * reference chain: poolrgn_bprop -> relu bprop -> bias bprop -> corr1ord_bprop_W
  * (kangaroo/_ext/poolrgn.py:78-82, deepity/std/elemwise.py:78,172-180, kangaroo/_ext/corr1ord.py:120-138) */
 int dbk_scanpool_bprop(dbk_stream_t stream,
@@ -149,7 +156,7 @@ int dbk_scanpool_bprop(dbk_stream_t stream,
                        const uint8_t* X, size_t N,
                        const uint32_t* regions, size_t nregion, int ptype,
                        const float* pooled, const uint32_t* argmax, const float* dpooled,
-                       float* dW, float* dbias, int overwrite);
+                       float* dW, float* dbias, int overwrite, const uint64_t* act);
 
 /* ------------------------------------------------------------------ dense head (deepity_smat) */
 
@@ -317,6 +324,7 @@ typedef struct dbk_train_step_args {
     int freeze_scan;                        /* zero the scan filters' gradient (filters not yet training) */
     float* pooled; uint32_t* argmax; float* Z; float* dpooled;
     float* loss;                            /* per-model mean loss (nmodel), may be NULL */
+    uint64_t* act;                          /* activity masks (see dbk_scanpool_fprop), N * ceil(nmodel*nfilter/64) words; may be NULL */
 } dbk_train_step_args;
 
 /* One optimiser step, all launches issued from native code on `stream`:

@@ -23,7 +23,7 @@ def test_header_symbols_are_exported_and_bound():
         assert hasattr(lib, name), "header declares %s but the library does not export it" % name
     # the Python binding covers the header and nothing else
     assert sorted(_lib.exported_names()) == names
-    assert lib.dbk_version() == 1
+    assert lib.dbk_version() == 2
     assert lib.dbk_last_error() == b""
 
 
@@ -40,7 +40,7 @@ def test_argument_errors_surface_through_last_error():
     assert rc != 0 and b"pooledmaps_argmax must be specified" in lib.dbk_last_error()
     # the 32-bit argmax index cannot address 2^26 rows x 1024 filters: refused before any launch
     one = ctypes.c_void_p(1)
-    rc = lib.dbk_scanpool_fprop(None, one, one, 24, 1024, one, 1 << 26, one, 10, 0, one, one)
+    rc = lib.dbk_scanpool_fprop(None, one, one, 24, 1024, one, 1 << 26, one, 10, 0, one, one, None)
     assert rc != 0 and b"overflow the 32-bit argmax index" in lib.dbk_last_error()
     # empty work succeeds and clears the error text
     assert lib.dbk_corr1ord(None, 0, None, 5, 16, None, 0, 4, None) == 0

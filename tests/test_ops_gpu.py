@@ -245,6 +245,49 @@ def test_scanpool_bprop(ks, ptype, B, lo, hi, m, F):
     assert np.array_equal(host(dW), host(dW2)) and np.array_equal(host(db), host(db2))
 
 
+@pytest.mark.parametrize("ptype", ["avg", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (33, 1, 300, 11, 70), (17, 0, 9, 5, 33),
+                                          (25, 200, 300, 7, 64), (40, 20, 40, 24, 144), (12, 480, 520, 30, 40)])
+def test_scanpool_bprop_with_activity_masks_equals_recomputation(ks, ptype, B, lo, hi, m, F):
+    """The forward pass can leave one bit per (row, filter) - rectifier open or not - and the backward pass
+    then skips recomputing the map: same gradient values added in the same order, so the same bits. Also
+    checks the masks themselves against the oracle's activation map, with letters that contribute nothing
+    (code 254) and regions that end where the stream ends."""
+    rng, W, b, X, R = _fused_case(3 * B + F, B, lo, hi, m, F, p254=0.02)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    act = ks.activity_words(Xd, Wd)
+    act.fill_(-1)                                                      # rows outside every region keep this
+    P0, I0 = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="general")
+    P1, I1 = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, act=act)
+    assert np.array_equal(host(P0), host(P1))
+    if I0 is not None:
+        assert np.array_equal(host(I0), host(I1))
+    # bit l of word [row, tile] <=> activation of filter 64*tile + l is positive (to round-off: skip values near 0)
+    A, _, _ = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
+    words = host(act).view(np.uint64)
+    inside = np.zeros(len(X), bool)
+    for a_, b_ in R[:, :2]:
+        inside[a_:b_] = True
+    assert (words[~inside] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()
+    rows = np.nonzero(inside)[0]
+    bits = ((words[rows][:, np.arange(F) // 64] >> (np.arange(F) % 64).astype(np.uint64)) & np.uint64(1)).astype(bool)
+    Zpre = np.zeros((len(X), F))
+    orc.corr1ord(W.astype(np.float64), X, Zpre)
+    Zpre += b.astype(np.float64)
+    sure = np.abs(Zpre[rows]) > 1e-5
+    assert np.array_equal(bits[sure], (Zpre[rows] > 0)[sure])
+    if F % 64:
+        assert (words[rows][:, -1] >> np.uint64(F % 64) == 0).all()    # lanes past the last filter never report open
+    dP = dev(rng.standard_normal(tuple(P0.shape)).astype(np.float32))
+    dW0 = dev(np.zeros(W.shape, np.float32)); db0 = dev(np.zeros((1, F), np.float32))
+    dW1 = dev(np.ones(W.shape, np.float32)); db1 = dev(np.ones((1, F), np.float32))
+    ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P0, I0, dP, dW0, db0, overwrite=True)
+    ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P0, I0, dP, dW1, db1, overwrite=True, act=act)
+    assert np.array_equal(host(dW0), host(dW1)) and np.array_equal(host(db0), host(db1))
+    with pytest.raises(Exception):
+        ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, path="kmer", act=act)
+
+
 # ------------------------------------------------------------------------------------------ dense head
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_blockwise_dot_family(ds, dtype):
