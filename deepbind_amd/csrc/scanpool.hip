@@ -350,6 +350,7 @@ template <int PT, int MT>
 __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* __restrict__ W, const float* __restrict__ bias,
                                                                    unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
                                                                    const uint32_t* __restrict__ R, size_t P,
+                                                                   const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
                                                                    const float* __restrict__ dpooled,
                                                                    float* __restrict__ slabs, size_t stride)
 {
@@ -373,6 +374,11 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
         const size_t a = R[2 * r], b = R[2 * r + 1];
         const size_t j0 = r * F + f;
         const float gavg = f < F ? (PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1]) / (float)(b - a) : 0.0f;
+        // max+avg pooling: the maximum's gradient joins the average's at the winning row before the
+        // rectifier, as it does in the unpooled gradient map of the layer-by-layer chain
+        float gmax = 0.0f;
+        size_t imax = ~(size_t)0;
+        if (PT == DBK_PT_ALL && f < F && pooled[2 * j0] > 0.0f) { gmax = dpooled[2 * j0]; imax = argmax[j0] / F; }
         for (size_t c0 = a; c0 < b; c0 += chunk) {
             const unsigned rows = (unsigned)((b - c0) < chunk ? (b - c0) : chunk);
             __syncthreads();
@@ -392,7 +398,8 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_kernel(const float* 
                 for (int p = 0; p < PSUB; ++p) {
                     const size_t i = c0 + p0 + p;
                     const float z = (i < n ? g[p] : 0.0f) + bf;
-                    const float gg = (p0 + p < rows && z > 0.0f) ? gavg : 0.0f;
+                    float gg = (p0 + p < rows && z > 0.0f) ? gavg : 0.0f;
+                    if (PT == DBK_PT_ALL) gg += (p0 + p < rows && i == imax) ? gmax : 0.0f;
                     db += gg;
                     g[p] = i < n ? gg : 0.0f;                   // rows past the scan's end carry bias only
                 }
@@ -458,6 +465,7 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
 template <int PT, int MT>
 __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
                                                                        const uint32_t* __restrict__ R, size_t P,
+                                                                       const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
                                                                        const float* __restrict__ dpooled,
                                                                        const unsigned long long* __restrict__ act,
                                                                        float* __restrict__ slabs, size_t stride)
@@ -480,6 +488,9 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
         const size_t a = R[2 * r], b = R[2 * r + 1];
         const size_t j0 = r * F + f;
         const float gavg = f < F ? (PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1]) / (float)(b - a) : 0.0f;
+        float gmax = 0.0f;                                         // max+avg pooling: see the recomputing kernel
+        size_t imax = ~(size_t)0;
+        if (PT == DBK_PT_ALL && f < F && pooled[2 * j0] > 0.0f) { gmax = dpooled[2 * j0]; imax = argmax[j0] / F; }
         for (size_t c0 = a; c0 < b; c0 += chunk) {
             const unsigned rows = (unsigned)((b - c0) < chunk ? (b - c0) : chunk);
             __syncthreads();
@@ -502,7 +513,8 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
                     const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)mk, p);
                     const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(mk >> 32), p);
                     const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
-                    const float gg = open ? gavg : 0.0f;
+                    float gg = open ? gavg : 0.0f;
+                    if (PT == DBK_PT_ALL) gg += (p0 + p < rows && c0 + p0 + p == imax) ? gmax : 0.0f;
                     db += gg;
                     g[p] = c0 + p0 + p < n ? gg : 0.0f;            // rows past the scan's end carry bias only
                 }
@@ -586,18 +598,18 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
 
 template <int PT, int MT>
 void launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, const float* W, const float* bias, size_t m, size_t F,
-                  const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* dpooled, const unsigned long long* act,
-                  float* slabs, size_t stride)
+                  const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* pooled, const uint32_t* argmax,
+                  const float* dpooled, const unsigned long long* act, float* slabs, size_t stride)
 {
     if (act) {
         auto kern = scanpool_bprop_dense_act_kernel<PT, MT>;
         hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, (unsigned)m, (unsigned)F, X, N, R, P, dpooled, act, slabs, stride);
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
         return;
     }
     auto kern = scanpool_bprop_dense_kernel<PT, MT>;
     hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, dpooled, slabs, stride);
+    hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled, slabs, stride);
 }
 
 template <int PT>
@@ -631,7 +643,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     }
     // sparse half: ~2048 single-wave workgroups, at least four regions each
     unsigned gxs = 0, gxd = 0;
-    if (PT != DBK_PT_AVG) {
+    if (PT == DBK_PT_MAX) {                                       // with max+avg pooling the dense half carries the maxima along
         gxs = 2048u / ftiles;
         if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);
         if (gxs < 1) gxs = 1;
@@ -656,9 +668,9 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     if (gxd) {
         constexpr int PD = PT == DBK_PT_MAX ? DBK_PT_AVG : PT;
         float* sd = slabs + stride * gxs;
-        if (mt == 8) launch_dense<PD, 8>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, act, sd, stride);
-        else if (mt == 16) launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, act, sd, stride);
-        else launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, dpooled, act, sd, stride);
+        if (mt == 8) launch_dense<PD, 8>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
+        else if (mt == 16) launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
+        else launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
     }
     hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd, overwrite);
     DBK_LAUNCH_OK();
