@@ -243,58 +243,54 @@ __global__ __launch_bounds__(256) void scanpool_bprop_kernel(const float* __rest
 // this lane's column of a [tap][channel][FT] table. Taps go eight at a time: the letters of all four
 // positions are loaded first (32 independent global loads in flight), then each position's eight cells
 // are read, updated and written (distinct taps are distinct cells), positions in ascending order.
+// Adds g[u] at the MT-letter windows starting at pos[u], u = 0..3, into this lane's private column of the
+// LDS slab, laid out [tap][A, C, G, T, mean-of-four][filter]: every letter, "mean of the four" included,
+// touches exactly one cell, so a batch of eight taps is one LDS round trip (the mean row is spread over
+// the four channels when the slab is written out).
+constexpr int SPARSE_ROWS = 5;
+template <int MT>
 __device__ __forceinline__ void add_positions4(float* mine, const uint8_t* __restrict__ X, size_t N, const size_t (&pos)[4],
                                                const float (&g)[4], const bool (&on)[4], unsigned m)
 {
-    for (unsigned j0 = 0; j0 < m; j0 += 8) {
-        // eight letters = three aligned 32-bit loads shifted into place (a lane's window starts at any byte);
-        // a word is only fetched if it starts before the end of the stream
-        unsigned l[4][8];
-        const uintptr_t xend = reinterpret_cast<uintptr_t>(X) + N;
+    // The letters of all four windows first, so that their loads are in flight together: a window of MT
+    // letters starting at any byte is MT/4 + 1 aligned 32-bit words shifted into place; a word is only
+    // fetched if it starts before the end of the stream.
+    static_assert(MT % 8 == 0, "windows are taken eight letters at a time");
+    constexpr int NW = MT / 4 + 1;
+    unsigned w[4][NW], sh[4];
+    const uintptr_t xend = reinterpret_cast<uintptr_t>(X) + N;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(X) + pos[u];
+        const uintptr_t base = addr & ~(uintptr_t)3;
+        sh[u] = (unsigned)(addr & 3);
+#pragma unroll
+        for (int t = 0; t < NW; ++t)
+            w[u][t] = (on[u] && base + 4 * t < xend) ? *reinterpret_cast<const unsigned*>(base + 4 * t) : 0xffffffffu;
+    }
+#pragma unroll
+    for (unsigned j0 = 0; j0 < (unsigned)MT; j0 += 8) {
+        if (j0 >= m) break;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const uintptr_t addr = reinterpret_cast<uintptr_t>(X) + pos[u] + j0;
-            const uintptr_t base = addr & ~(uintptr_t)3;
-            const unsigned sh = (unsigned)(addr & 3);
-            unsigned w[3];
-#pragma unroll
-            for (int t = 0; t < 3; ++t)
-                w[t] = (on[u] && base + 4 * t < xend) ? *reinterpret_cast<const unsigned*>(base + 4 * t) : 0xffffffffu;
-            const unsigned lo = __builtin_amdgcn_alignbyte(w[1], w[0], sh), hi = __builtin_amdgcn_alignbyte(w[2], w[1], sh);
+            const unsigned lo = __builtin_amdgcn_alignbyte(w[u][j0 / 4 + 1], w[u][j0 / 4], sh[u]);
+            const unsigned hi = __builtin_amdgcn_alignbyte(w[u][j0 / 4 + 2], w[u][j0 / 4 + 1], sh[u]);     // j0/4 + 2 <= MT/4
+            unsigned l[8];
 #pragma unroll
             for (unsigned t = 0; t < 8; ++t) {
                 const unsigned code = ((t < 4 ? lo : hi) >> ((t & 3) * 8)) & 0xffu;
-                l[u][t] = (on[u] && j0 + t < m) ? letter_of(code) : 5u;
+                l[t] = (on[u] && j0 + t < m) ? letter_of(code) : 5u;
             }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const float gu = g[u], gq = gu * 0.25f;
             float v[8];
 #pragma unroll
-            for (unsigned t = 0; t < 8; ++t) v[t] = l[u][t] < 4u ? mine[((j0 + t) * 4 + l[u][t]) * FT] : 0.0f;
+            for (unsigned t = 0; t < 8; ++t) v[t] = l[t] < 5u ? mine[((j0 + t) * SPARSE_ROWS + l[t]) * FT] : 0.0f;
 #pragma unroll
             for (unsigned t = 0; t < 8; ++t)
-                if (l[u][t] < 4u) mine[((j0 + t) * 4 + l[u][t]) * FT] = v[t] + gu;
-#pragma unroll
-            for (unsigned t = 0; t < 8; ++t)
-                if (l[u][t] == 4u) {
-                    float* cell = mine + (size_t)(j0 + t) * 4 * FT;
-                    cell[0 * FT] += gq;
-                    cell[1 * FT] += gq;
-                    cell[2 * FT] += gq;
-                    cell[3 * FT] += gq;
-                }
+                if (l[t] < 5u) mine[((j0 + t) * SPARSE_ROWS + l[t]) * FT] = v[t] + g[u];
         }
     }
 }
-
-// Sparse half of the backward pass (max and max+avg pooling): one position per (region, filter)
-// receives the pooled gradient. One wave per workgroup, one lane per filter, a private
-// [tap][channel][FT] table in LDS that the wave writes out as its slab; regions are taken four at a
-// time so that their pooled / gradient / argmax loads are in flight together. Slab s of the launch
-// lives at slabs + s*stride: 4m*F gradient entries followed by F bias-gradient entries.
-template <int PT>
+template <int PT, int MT>
 __global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
                                                                    size_t P, const float* __restrict__ pooled,
                                                                    const uint32_t* __restrict__ argmax, const float* __restrict__ dpooled,
@@ -306,7 +302,7 @@ __global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, u
     const unsigned f = blockIdx.y * FT + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
     float* mine = table + lane;                                   // a lane only ever touches its own column: no barriers needed
-    for (unsigned row = 0; row < 4 * m; ++row) mine[row * FT] = 0.0f;
+    for (unsigned row = 0; row < SPARSE_ROWS * m; ++row) mine[row * FT] = 0.0f;
     float db = 0.0f;
     if (f < F) {
         const size_t gx = gridDim.x;
@@ -332,10 +328,18 @@ __global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, u
                 if (g[u] != 0.0f) db += g[u];
                 on[u] = g[u] != 0.0f && pos[u] < n;
             }
-            add_positions4(mine, X, N, pos, g, on, m);
+            add_positions4<MT>(mine, X, N, pos, g, on, m);
         }
         float* out = slabs + (size_t)blockIdx.x * stride;
-        for (unsigned row = 0; row < 4 * m; ++row) out[(size_t)row * F + f] = mine[row * FT];
+        for (unsigned j = 0; j < m; ++j) {
+            const float* tap = mine + (size_t)j * SPARSE_ROWS * FT;
+            const float q = 0.25f * tap[4 * FT];
+            float* o = out + (size_t)(4 * j) * F + f;
+            o[0] = tap[0] + q;
+            o[F] = tap[FT] + q;
+            o[2 * (size_t)F] = tap[2 * FT] + q;
+            o[3 * (size_t)F] = tap[3 * FT] + q;
+        }
         out[(size_t)4 * m * F + f] = db;
     }
 }
@@ -645,7 +649,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     unsigned gxs = 0, gxd = 0;
     if (PT == DBK_PT_MAX) {                                       // with max+avg pooling the dense half carries the maxima along
         gxs = 2048u / ftiles;
-        if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);
+        if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);   // more regions per workgroup only lengthens its chain of dependent loads
         if (gxs < 1) gxs = 1;
     }
     // dense half: four-wave workgroups, as many as are resident at once (its register planes leave room for
@@ -655,13 +659,14 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         if (gxd < 1) gxd = 1;
         if (gxd > P) gxd = (unsigned)P;
     }
-    const size_t smem_s = m * 4 * FT * sizeof(float);
+    const size_t smem_s = m * SPARSE_ROWS * FT * sizeof(float);
     const size_t smem_d = ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3);
     DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
     float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float), st);
     DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * (gxs + gxd) * sizeof(float));
     if (gxs) {
-        auto kern = scanpool_bprop_sparse_kernel<PT == DBK_PT_AVG ? DBK_PT_MAX : PT>;
+        constexpr int PS = PT == DBK_PT_AVG ? DBK_PT_MAX : PT;
+        auto kern = mt == 8 ? scanpool_bprop_sparse_kernel<PS, 8> : mt == 16 ? scanpool_bprop_sparse_kernel<PS, 16> : scanpool_bprop_sparse_kernel<PS, 24>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_s));
         hipLaunchKernelGGL(kern, dim3(gxs, ftiles), dim3(64), smem_s, st, (unsigned)m, (unsigned)F, X, N, P, pooled, argmax, dpooled, slabs, stride);
     }
