@@ -232,6 +232,42 @@ __global__ __launch_bounds__(256) void corr1ord_window_kernel(const T* __restric
     }
 }
 
+// forward, float32 and at most 24 taps: the lane's filter weights sit in register planes and the scan needs
+// no table in LDS (one index-mode v_add_f32 per position and tap). Same additions in the same order as above.
+template <int MT>
+__global__ __launch_bounds__(256) void corr1ord_planes_kernel(const float* __restrict__ W, unsigned m, unsigned F,
+                                                              const uint8_t* __restrict__ X, size_t n, float* __restrict__ Z)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    uint8_t* xl = smem;
+    const unsigned nw = blockDim.x >> 6, chunk = nw * WSUBS_W * PSUB;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
+    const size_t N = n + m - 1;
+    grad_planes<MT> planes;
+    weight_planes_load<MT>(planes, W, m, F, f);
+    for (size_t c0 = (size_t)blockIdx.x * chunk; c0 < n; c0 += (size_t)gridDim.x * chunk) {
+        const unsigned rows = (unsigned)((n - c0) < chunk ? (n - c0) : chunk);
+        __syncthreads();
+        stage(xl, X, N, c0, window_span<MT>(rows));
+        __syncthreads();
+#pragma unroll 1
+        for (unsigned s = 0; s < WSUBS_W; ++s) {
+            const unsigned p0 = (s * nw + wave) * PSUB;
+            if (p0 >= rows) break;
+            unsigned wq[window<MT>::words];
+            load_window<MT>(xl, p0, wq);
+            float acc[PSUB];
+            scan16_planes<MT>(planes, wq, acc);
+            if (f < F) {
+#pragma unroll
+                for (int p = 0; p < PSUB; ++p)
+                    if (p0 + p < rows) Z[(c0 + p0 + p) * F + f] = acc[p];
+            }
+        }
+    }
+}
+
 // filter gradient, pass 1: a lane keeps its filter's whole [letter][tap] column in registers; the window's
 // letters (scalars) pick the register plane each gradient value is added into through the register index
 // mode: one addition per (position, tap). "Mean of the four" letters collect in a plane of their own that
@@ -394,6 +430,19 @@ template <typename T>
 int launch_fprop(hipStream_t st, const T* W, size_t m, size_t F, const uint8_t* X, size_t n, T* Z)
 {
     const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 24 ? 24 : (m <= 32 ? 32 : 0)));
+    if constexpr (sizeof(T) == 4) {
+        if (mt && mt <= 24) {
+            const unsigned ftiles = dbk::divup(F, FT), chunk = 4 * WSUBS_W * PSUB;
+            DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
+            const size_t smem_p = (chunk + mt - 1 + 7) & ~(size_t)3;
+            unsigned gx = (mt == 8 ? 768u : 512u) / ftiles;         // the register planes leave room for two workgroups per CU (three with 8 taps)
+            if (gx < 1) gx = 1;
+            if (gx > dbk::divup(n, chunk)) gx = dbk::divup(n, chunk);
+            auto kp = mt == 8 ? corr1ord_planes_kernel<8> : mt == 16 ? corr1ord_planes_kernel<16> : corr1ord_planes_kernel<24>;
+            hipLaunchKernelGGL(kp, dim3(gx, ftiles), dim3(256), smem_p, st, (const float*)W, (unsigned)m, (unsigned)F, X, n, (float*)Z);
+            DBK_LAUNCH_OK();
+        }
+    }
     if (mt) {
         const unsigned ftiles = dbk::divup(F, FT), chunk = 4 * WSUBS * PSUB;
         DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);

@@ -128,6 +128,16 @@ template <int MT> struct grad_planes {
         else if constexpr (E < 128) return t3[E % 32];
         else return u0[(E - 128) % 16];
     }
+    template <int E> __device__ __forceinline__ void set(float v)
+    {
+        static_assert(E >= 0 && E < GRAD_PLANES * MT, "register outside the plane set");
+        if constexpr (MT == 8) { if constexpr (E < 32) t0[E % 32] = v; else u0[(E - 32) % 16] = v; }
+        else if constexpr (E < 32) t0[E % 32] = v;
+        else if constexpr (E < 64) t1[E % 32] = v;
+        else if constexpr (E < 96) t2[E % 32] = v;
+        else if constexpr (E < 128) t3[E % 32] = v;
+        else u0[(E - 128) % 16] = v;
+    }
     // gradient of tap J, channel C: the letter's own plane plus a quarter of the "mean" plane
     template <int J, int C> __device__ __forceinline__ float grad() const { return reg<C * MT + J>() + 0.25f * reg<4 * MT + J>(); }
 };
@@ -184,6 +194,84 @@ template <int MT>
 __device__ __forceinline__ void grad_planes_read(const grad_planes<MT>& A, float (&aw)[MT][4])
 {
     grad_planes_read<MT>(A, aw, std::make_integer_sequence<int, 4 * MT>{});
+}
+
+// ---- the forward scan through the same register planes ---------------------------------------------
+// With the lane's filter weights in the planes ([letter][tap]: A, C, G, T, mean of the four, zero) the
+// scan needs no table in LDS: Z[p] += plane[letter(p + j)][j] is one v_add_f32 whose first source is
+// picked by the register index mode. Taps are added in ascending order per position and the mean row is
+// formed as in the LDS table, so the sums are bit-identical to the table kernels'.
+template <int MT, int J>
+__device__ __forceinline__ void weight_planes_tap(grad_planes<MT>& A, const float* __restrict__ W, unsigned m, unsigned F, unsigned f)
+{
+    float w0 = 0.0f, w1 = 0.0f, w2 = 0.0f, w3 = 0.0f;
+    if (f < F && (unsigned)J < m) {
+        w0 = W[(4 * J + 0) * (size_t)F + f];
+        w1 = W[(4 * J + 1) * (size_t)F + f];
+        w2 = W[(4 * J + 2) * (size_t)F + f];
+        w3 = W[(4 * J + 3) * (size_t)F + f];
+    }
+    float z = w0;
+    z += w1;
+    z += w2;
+    z += w3;
+    A.template set<0 * MT + J>(w0);
+    A.template set<1 * MT + J>(w1);
+    A.template set<2 * MT + J>(w2);
+    A.template set<3 * MT + J>(w3);
+    A.template set<4 * MT + J>(z * 0.25f);
+    A.template set<5 * MT + J>(0.0f);
+}
+template <int MT, int... J>
+__device__ __forceinline__ void weight_planes_load(grad_planes<MT>& A, const float* __restrict__ W, unsigned m, unsigned F, unsigned f,
+                                                   std::integer_sequence<int, J...>)
+{
+    (weight_planes_tap<MT, J>(A, W, m, F, f), ...);
+}
+// Fills the planes with filter f's weights from W (4m, F); taps >= m and filters >= F read as zero.
+template <int MT>
+__device__ __forceinline__ void weight_planes_load(grad_planes<MT>& A, const float* __restrict__ W, unsigned m, unsigned F, unsigned f)
+{
+    A.clear();
+    weight_planes_load<MT>(A, W, m, F, f, std::make_integer_sequence<int, MT>{});
+}
+
+#define DBK_WP_SLOT(P) ".if ((%c[q] - " #P ") >= 0) && ((%c[q] - " #P ") < %c[mt])\n\t" \
+                       "v_add_f32 %[a" #P "], v[96 + %c[q] - " #P "], %[a" #P "]\n\t.endif\n\t"
+#define DBK_WP_ASM(PLANES)                                                                                          \
+    asm volatile("s_set_gpr_idx_on %[idx], 0x1\n\t"                                                                  \
+                 DBK_WP_SLOT(0) DBK_WP_SLOT(1) DBK_WP_SLOT(2) DBK_WP_SLOT(3) DBK_WP_SLOT(4) DBK_WP_SLOT(5) DBK_WP_SLOT(6)   \
+                 DBK_WP_SLOT(7) DBK_WP_SLOT(8) DBK_WP_SLOT(9) DBK_WP_SLOT(10) DBK_WP_SLOT(11) DBK_WP_SLOT(12)            \
+                 DBK_WP_SLOT(13) DBK_WP_SLOT(14) DBK_WP_SLOT(15)                                                     \
+                 "s_set_gpr_idx_off"                                                                                \
+                 : [a0] "+v"(acc[0]), [a1] "+v"(acc[1]), [a2] "+v"(acc[2]), [a3] "+v"(acc[3]), [a4] "+v"(acc[4]),   \
+                   [a5] "+v"(acc[5]), [a6] "+v"(acc[6]), [a7] "+v"(acc[7]), [a8] "+v"(acc[8]), [a9] "+v"(acc[9]),   \
+                   [a10] "+v"(acc[10]), [a11] "+v"(acc[11]), [a12] "+v"(acc[12]), [a13] "+v"(acc[13]),              \
+                   [a14] "+v"(acc[14]), [a15] "+v"(acc[15])                                                         \
+                 : PLANES, [idx] "s"(idx), [q] "n"(Q), [mt] "n"(MT))
+
+template <int Q, int MT>
+__device__ __forceinline__ void weight_planes_add(const grad_planes<MT>& A, unsigned letter, float (&acc)[PSUB])
+{
+    static_assert(PSUB == 16, "the instruction text lists 16 positions");
+    const unsigned idx = letter * (unsigned)MT;          // (M0 is left changed: see grad_planes_add)
+    if constexpr (MT == 8) DBK_WP_ASM(DBK_GP_LIST("{v[96:127]}"(A.t0), "{v[128:143]}"(A.u0)));
+    else if constexpr (MT == 16) DBK_WP_ASM(DBK_GP_LIST("{v[96:127]}"(A.t0), "{v[128:159]}"(A.t1), "{v[160:191]}"(A.t2)));
+    else DBK_WP_ASM(DBK_GP_LIST("{v[96:127]}"(A.t0), "{v[128:159]}"(A.t1), "{v[160:191]}"(A.t2), "{v[192:223]}"(A.t3), "{v[224:239]}"(A.u0)));
+}
+template <int MT, int... Q>
+__device__ __forceinline__ void scan16_planes(const grad_planes<MT>& A, const unsigned (&wq)[window<MT>::words], float (&acc)[PSUB],
+                                              std::integer_sequence<int, Q...>)
+{
+    (weight_planes_add<Q, MT>(A, window_letter(wq, Q), acc), ...);
+}
+// acc[p] = sum over taps of the window's weights for positions p = 0..15 (the counterpart of scan16_window).
+template <int MT>
+__device__ __forceinline__ void scan16_planes(const grad_planes<MT>& A, const unsigned (&wq)[window<MT>::words], float (&acc)[PSUB])
+{
+#pragma unroll
+    for (int p = 0; p < PSUB; ++p) acc[p] = 0.0f;
+    scan16_planes<MT>(A, wq, acc, std::make_integer_sequence<int, PSUB + MT - 1>{});
 }
 
 // Stages letters for absolute positions [c0, c0+cnt) into xl; past the end of X -> "nothing".
