@@ -488,55 +488,115 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
     extern __shared__ __align__(16) unsigned char smem[];
     const unsigned nw = blockDim.x >> 6;
     const unsigned chunk = nw * XCH_SUBS * PSUB;
+    constexpr unsigned XBUF = (4 * XCH_SUBS * PSUB + MT - 1 + 7) & ~3u;   // bytes of one letter buffer (>= window_span of a full chunk)
+    static_assert(XBUF <= 512, "a thread stages at most two letters per chunk");
     float* lut = reinterpret_cast<float*>(smem);                   // [MT*4][FT]: only the cross-wave fold at the end uses it
     float* dbacc = lut + (size_t)MT * 4 * FT;                      // [nw][FT]
-    uint8_t* xl = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT);
+    uint8_t* xbuf = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT);   // two letter buffers, used in turn
 
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
     const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
     float db = 0.0f;
     grad_planes<MT> planes;
     planes.clear();
 
-    for (size_t r = blockIdx.x; r < P; r += gridDim.x) {
-        const size_t a = R[2 * r], b = R[2 * r + 1];
-        const size_t j0 = r * F + f;
-        const float gavg = f < F ? (PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1]) / (float)(b - a) : 0.0f;
-        float gmax = 0.0f;                                         // max+avg pooling: see the recomputing kernel
-        size_t imax = ~(size_t)0;
-        if (PT == DBK_PT_ALL && f < F && pooled[2 * j0] > 0.0f) { gmax = dpooled[2 * j0]; imax = argmax[j0] / F; }
-        for (size_t c0 = a; c0 < b; c0 += chunk) {
-            const unsigned rows = (unsigned)((b - c0) < chunk ? (b - c0) : chunk);
-            __syncthreads();
-            stage(xl, X, N, c0, window_span<MT>(rows));
-            __syncthreads();
-            auto fetch = [&](unsigned p0) -> unsigned long long {      // rows past the chunk read as "closed"
-                return (lane < (unsigned)PSUB && p0 + lane < rows) ? act[(c0 + p0 + lane) * gridDim.y + blockIdx.y] : 0ull;
-            };
-            unsigned long long mk = fetch(wave * PSUB);
-#pragma unroll 1
-            for (unsigned s = 0; s < XCH_SUBS; ++s) {
-                const unsigned p0 = (s * nw + wave) * PSUB;
-                if (p0 >= rows) break;
-                const unsigned long long mkn = fetch(p0 + nw * PSUB);
-                unsigned wq[window<MT>::words];
-                load_window<MT>(xl, p0, wq);
-                float g[PSUB];
-#pragma unroll
-                for (int p = 0; p < PSUB; ++p) {
-                    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)mk, p);
-                    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(mk >> 32), p);
-                    const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
-                    float gg = open ? gavg : 0.0f;
-                    if (PT == DBK_PT_ALL) gg += (p0 + p < rows && c0 + p0 + p == imax) ? gmax : 0.0f;
-                    db += gg;
-                    g[p] = c0 + p0 + p < n ? gg : 0.0f;            // rows past the scan's end carry bias only
-                }
-                grad_planes_window<MT>(planes, wq, g);
-                mk = mkn;
+    // The work is a sequence of items (region, chunk of up to 256 rows). While an item is being added into the
+    // planes, everything the next item needs is already on its way: its letters (two per thread, parked in
+    // registers and put into the other LDS buffer afterwards), the next region's pooled gradients and the
+    // bounds of the region after that. One barrier per item.
+    auto rows_of = [&](size_t b_, size_t c_) -> unsigned { return c_ < b_ ? (unsigned)((b_ - c_) < chunk ? (b_ - c_) : chunk) : 0u; };
+    auto load_letters = [&](size_t c_, unsigned rows_, unsigned& v0, unsigned& v1) {
+        const unsigned cnt = window_span<MT>(rows_);
+        const size_t g0 = c_ + tid, g1 = g0 + 256;
+        v0 = (tid < cnt && g0 < N) ? letter_of(X[g0]) : 5u;
+        v1 = (tid + 256 < cnt && g1 < N) ? letter_of(X[g1]) : 5u;
+    };
+    auto store_letters = [&](uint8_t* buf, unsigned v0, unsigned v1) {
+        buf[tid] = (uint8_t)v0;
+        if (tid + 256 < XBUF) buf[tid + 256] = (uint8_t)v1;
+    };
+    struct pooled_in { float davg, pmax, dmax; unsigned arg; };
+    auto load_pooled = [&](size_t r_) -> pooled_in {
+        pooled_in q = { 0.0f, 0.0f, 0.0f, 0u };
+        if (f < F) {
+            const size_t j0 = r_ * F + f;
+            q.davg = PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1];
+            if (PT == DBK_PT_ALL) { q.pmax = pooled[2 * j0]; q.dmax = dpooled[2 * j0]; q.arg = argmax[j0]; }
+        }
+        return q;
+    };
+    float gavg = 0.0f, gmax = 0.0f;                                // max+avg pooling: see the recomputing kernel
+    size_t imax = ~(size_t)0;
+    auto enter_region = [&](const pooled_in& q, size_t a_, size_t b_) {
+        gavg = q.davg / (float)(b_ - a_);
+        gmax = 0.0f;
+        imax = ~(size_t)0;
+        if (PT == DBK_PT_ALL && q.pmax > 0.0f) { gmax = q.dmax; imax = q.arg / F; }
+    };
+
+    size_t r = blockIdx.x;
+    bool valid = r < P;
+    size_t a = 0, b = 0, c0 = 0, pa = 0, pb = 0;                   // (pa, pb): bounds of the region after this one
+    if (valid) {
+        a = R[2 * r]; b = R[2 * r + 1]; c0 = a;
+        if (r + gridDim.x < P) { pa = R[2 * (r + gridDim.x)]; pb = R[2 * (r + gridDim.x) + 1]; }
+        enter_region(load_pooled(r), a, b);
+        unsigned v0, v1;
+        load_letters(c0, rows_of(b, c0), v0, v1);
+        store_letters(xbuf, v0, v1);
+    }
+    __syncthreads();
+    unsigned cur = 0;
+    while (valid) {                                                // uniform over the workgroup
+        const unsigned rows = rows_of(b, c0);
+        // ---- the next item, and its loads
+        size_t nr = r, na = a, nb = b, nc0 = c0 + chunk;
+        const bool newregion = nc0 >= b;
+        if (newregion) { nr = r + gridDim.x; na = pa; nb = pb; nc0 = na; }
+        const bool nvalid = nr < P;
+        unsigned nv0 = 5u, nv1 = 5u;
+        pooled_in nq = { 0.0f, 0.0f, 0.0f, 0u };
+        size_t qa = 0, qb = 0;
+        if (nvalid) {
+            load_letters(nc0, rows_of(nb, nc0), nv0, nv1);
+            if (newregion) {
+                nq = load_pooled(nr);
+                if (nr + gridDim.x < P) { qa = R[2 * (nr + gridDim.x)]; qb = R[2 * (nr + gridDim.x) + 1]; }
             }
         }
+        // ---- this item
+        const uint8_t* xl = xbuf + cur * XBUF;
+        auto fetch = [&](unsigned p0) -> unsigned long long {          // rows past the chunk read as "closed"
+            return (lane < (unsigned)PSUB && p0 + lane < rows) ? act[(c0 + p0 + lane) * gridDim.y + blockIdx.y] : 0ull;
+        };
+        unsigned long long mk = fetch(wave * PSUB);
+#pragma unroll 1
+        for (unsigned s = 0; s < XCH_SUBS; ++s) {
+            const unsigned p0 = (s * nw + wave) * PSUB;
+            if (p0 >= rows) break;
+            const unsigned long long mkn = fetch(p0 + nw * PSUB);
+            unsigned wq[window<MT>::words];
+            load_window<MT>(xl, p0, wq);
+            float g[PSUB];
+#pragma unroll
+            for (int p = 0; p < PSUB; ++p) {
+                const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)mk, p);
+                const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(mk >> 32), p);
+                const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
+                float gg = open ? gavg : 0.0f;
+                if (PT == DBK_PT_ALL) gg += (p0 + p < rows && c0 + p0 + p == imax) ? gmax : 0.0f;
+                db += gg;
+                g[p] = c0 + p0 + p < n ? gg : 0.0f;                // rows past the scan's end carry bias only
+            }
+            grad_planes_window<MT>(planes, wq, g);
+            mk = mkn;
+        }
+        // ---- hand over
+        if (nvalid) store_letters(xbuf + (cur ^ 1u) * XBUF, nv0, nv1);
+        __syncthreads();
+        if (newregion && nvalid) { enter_region(nq, na, nb); pa = qa; pb = qb; }
+        r = nr; a = na; b = nb; c0 = nc0; valid = nvalid; cur ^= 1u;
     }
     float aw[MT][4];
     grad_planes_read<MT>(planes, aw);
