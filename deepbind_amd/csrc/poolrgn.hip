@@ -36,13 +36,22 @@ __global__ __launch_bounds__(256) void poolrgn_kernel(const T* __restrict__ U, s
     size_t xi = g.a * F + f;
     T x = U[xi];
     T y = x;
-    for (size_t i = g.a + g.step; i < g.b; i += g.step) {
-        const T v = U[i * F + f];
+    auto take = [&](size_t i, T v) {
         if (PT == DBK_PT_MAX || PT == DBK_PT_ALL) {
             if (v > x) { x = v; xi = i * F + f; }
         }
         if (PT != DBK_PT_MAX) y += v;
+    };
+    // eight rows per round: the loads of a round are in flight together, the rows are still taken in ascending order
+    size_t i = g.a + g.step;
+    for (; i + 7 * g.step < g.b; i += 8 * g.step) {
+        T v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v[t] = U[(i + t * g.step) * F + f];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) take(i + t * g.step, v[t]);
     }
+    for (; i < g.b; i += g.step) take(i, U[i * F + f]);
     const size_t j = r * F + f;
     if (PT == DBK_PT_MAX) {
         pooled[j] = x;
@@ -107,7 +116,18 @@ __global__ __launch_bounds__(256) void poolrgn_bprop_kernel(T* __restrict__ dU, 
     if (PT == DBK_PT_ALL) dy = dP[2 * j + 1] / (T)g.count;
     else if (PT == DBK_PT_AVG) dy = dP[j] / (T)g.count;
     else dy = dP[j];
-    for (size_t i = g.a; i < g.b; i += g.step) accumulate<ATOMIC>(&dU[i * F + f], dy);
+    size_t i = g.a;
+    if (!ATOMIC) {
+        // eight rows per round: read, add, write, with the eight reads in flight together
+        for (; i + 7 * g.step < g.b; i += 8 * g.step) {
+            T v[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) v[t] = dU[(i + t * g.step) * F + f];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) dU[(i + t * g.step) * F + f] = v[t] + dy;
+        }
+    }
+    for (; i < g.b; i += g.step) accumulate<ATOMIC>(&dU[i * F + f], dy);
     if (PT == DBK_PT_ALL) atomicAdd(&dU[argmax[j]], dP[2 * j]);
 }
 
