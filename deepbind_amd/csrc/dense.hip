@@ -547,7 +547,7 @@ int launch_bdot_tn_tile(hipStream_t st, int nblock, int n, int m, int k, int p, 
     if (!partial) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", nout * nchunk * sizeof(T)); return 1; }
     const size_t smem = (size_t)TN_ROWS * ((k | 1) + (m | 1)) * sizeof(T);
     auto kern = k_bdot_tn_tile<T>;
-    hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3(nblock, nchunk), dim3(256), smem, st, nblock, (size_t)n, m, k, bcast, X, dZ, partial);
     hipLaunchKernelGGL(k_bdot_tn_fold<T>, dim3(dbk::ew_grid(nout)), dim3(256), 0, st, nblock, m, k, p, off, nchunk, (const T*)partial, dW);
     return 0;

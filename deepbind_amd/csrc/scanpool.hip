@@ -630,19 +630,20 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
 }
 
 template <int PT, int MT>
-void launch_fprop_mt(hipStream_t st, unsigned gx, unsigned ftiles, unsigned nw, size_t smem, const float* W, const float* bias, size_t m,
+int launch_fprop_mt(hipStream_t st, unsigned gx, unsigned ftiles, unsigned nw, size_t smem, const float* W, const float* bias, size_t m,
                      size_t F, const uint8_t* X, size_t N, const uint32_t* R, size_t P, float* pooled, uint32_t* argmax,
                      const unsigned* run_if_flag, unsigned long long* act)
 {
     if (argmax) {
         auto kern = scanpool_fprop_kernel<PT, true, MT>;
-        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag, act);
     } else {
         auto kern = scanpool_fprop_kernel<PT, false, MT>;
-        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, run_if_flag, act);
     }
+    return 0;
 }
 
 template <int PT>
@@ -663,30 +664,33 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     unsigned gx = (mt == 16 ? 512u : 768u) / ftiles;
     if (gx < 1) gx = 1;
     if (gx > P) gx = (unsigned)P;
+    int rc = 0;
     switch (mt) {
-    case 8:  launch_fprop_mt<PT, 8>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
-    case 16: launch_fprop_mt<PT, 16>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
-    case 24: launch_fprop_mt<PT, 24>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
-    case 32: launch_fprop_mt<PT, 32>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
-    default: launch_fprop_mt<PT, 0>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    case 8:  rc = launch_fprop_mt<PT, 8>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    case 16: rc = launch_fprop_mt<PT, 16>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    case 24: rc = launch_fprop_mt<PT, 24>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    case 32: rc = launch_fprop_mt<PT, 32>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
+    default: rc = launch_fprop_mt<PT, 0>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
     }
+    if (rc) return rc;
     DBK_LAUNCH_OK();
 }
 
 template <int PT, int MT>
-void launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, const float* W, const float* bias, size_t m, size_t F,
+int launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, const float* W, const float* bias, size_t m, size_t F,
                   const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* pooled, const uint32_t* argmax,
                   const float* dpooled, const unsigned long long* act, float* slabs, size_t stride)
 {
     if (act) {
         auto kern = scanpool_bprop_dense_act_kernel<PT, MT>;
-        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
-        return;
+        return 0;
     }
     auto kern = scanpool_bprop_dense_kernel<PT, MT>;
-    hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled, slabs, stride);
+    return 0;
 }
 
 template <int PT>
@@ -746,9 +750,11 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     if (gxd) {
         constexpr int PD = PT == DBK_PT_MAX ? DBK_PT_AVG : PT;
         float* sd = slabs + stride * gxs;
-        if (mt == 8) launch_dense<PD, 8>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
-        else if (mt == 16) launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
-        else launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
+        int rc;
+        if (mt == 8) rc = launch_dense<PD, 8>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
+        else if (mt == 16) rc = launch_dense<PD, 16>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
+        else rc = launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
+        if (rc) return rc;
     }
     hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd, overwrite);
     DBK_LAUNCH_OK();
