@@ -53,11 +53,20 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
     float* w2s = b1s + h1;                  // [h1] (unused when hidden == 0)
     float* H0s = w2s + h1;                  // [RB][ks]  inputs after dropout
     float* H1s = H0s + RB * ks;             // [RB][hst] hidden activations (hidden > 0)
-    float* dAs = H1s + RB * hst;            // [RB]      gradient at the output pre-activation
+    float* D1s = H1s + RB * hst;            // [RB][hst] gradient at the hidden pre-activations
+    float* dAs = D1s + RB * hst;            // [RB]      gradient at the output pre-activation
     float* lss = dAs + RB;                  // [RB]      loss terms
     unsigned char* kept = reinterpret_cast<unsigned char*>(lss + RB);   // [RB][k] dropout keep flags
 
-    for (int e = tid; e < k * h1; e += NT) w1s[e] = a.W1[(size_t)b * k * h1 + e];
+    // four loads in flight per thread and round (a plain strided loop waits for each load before the next)
+    for (int e0 = tid; e0 < k * h1; e0 += 4 * NT) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = e0 + j * NT < k * h1 ? a.W1[(size_t)b * k * h1 + e0 + j * NT] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (e0 + j * NT < k * h1) w1s[e0 + j * NT] = v[j];
+    }
     for (int e = tid; e < h1; e += NT) b1s[e] = a.b1[(size_t)b * h1 + e];
     for (int e = tid; e < hidden; e += NT) w2s[e] = a.W2[(size_t)b * hidden + e];
     const float bias2 = hidden > 0 ? a.b2[b] : 0.0f;
@@ -66,23 +75,29 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
     const float inv_n = 1.0f / (float)a.n;
 
     // ---------------- inputs of the chunk, dropout applied (same element numbering as the stand-alone dropout kernels)
-    for (int e = tid; e < RB * k; e += NT) {
-        const int er = e / k, kk = e % k;
-        const size_t rr = r0 + er;
-        float x = 0.0f;
-        bool kp = true;
-        if (rr < a.n) {
-            const size_t col = (size_t)b * k + kk;
-            if (a.rate) {
-                float u;
-                if (a.U) u = a.U[(a.revcomp ? (rr & ~(size_t)1) : rr) * ncol + col];
-                else u = dbk_rng::uniform_at(a.seed, off, a.revcomp ? (rr >> 1) * ncol + col : rr * ncol + col);
+    for (int e0 = tid; e0 < RB * k; e0 += 4 * NT) {
+        float xv[4], uv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {                              // the loads of a round first
+            const int e = e0 + j * NT, er = e / k, kk = e % k;
+            const size_t rr = r0 + er, col = (size_t)b * k + kk;
+            const bool in = e < RB * k && rr < a.n;
+            xv[j] = in ? a.pooled[rr * ncol + col] : 0.0f;
+            uv[j] = (in && a.rate && a.U) ? a.U[(a.revcomp ? (rr & ~(size_t)1) : rr) * ncol + col] : 1.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e = e0 + j * NT, er = e / k, kk = e % k;
+            if (e >= RB * k) break;
+            const size_t rr = r0 + er, col = (size_t)b * k + kk;
+            bool kp = true;
+            if (rr < a.n && a.rate) {
+                const float u = a.U ? uv[j] : dbk_rng::uniform_at(a.seed, off, a.revcomp ? (rr >> 1) * ncol + col : rr * ncol + col);
                 kp = u >= p_drop;
             }
-            x = kp ? a.pooled[rr * ncol + col] : 0.0f;
+            H0s[er * ks + kk] = kp ? xv[j] : 0.0f;
+            kept[e] = kp;
         }
-        H0s[er * ks + kk] = x;
-        kept[e] = kp;
     }
     __syncthreads();
 
@@ -125,6 +140,10 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
         dAs[row] = dA;
         lss[row] = lterm;
     }
+    // gradient at the hidden pre-activations, once: the loops below then run without branches, so that their
+    // LDS reads can be issued back to back
+    if (hidden > 0)
+        for (int h = part; h < hidden; h += NP) D1s[row * hst + h] = H1s[row * hst + h] > 0.0f ? dA * w2s[h] : 0.0f;
     __syncthreads();
 
     // ---------------- gradient back to the pooled features: the row's lanes split the inputs
@@ -134,10 +153,8 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
             float g;
             if (hidden > 0) {
                 g = 0.0f;
-                for (int h = 0; h < hidden; ++h) {
-                    const float d1 = H1s[row * hst + h] > 0.0f ? dA * w2s[h] : 0.0f;
-                    g += d1 * w1s[kk * hidden + h];
-                }
+#pragma unroll 8
+                for (int h = 0; h < hidden; ++h) g += D1s[row * hst + h] * w1s[kk * hidden + h];
             } else {
                 g = dA * w1s[kk];
             }
@@ -151,14 +168,10 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
         const int kk = pidx / h1, h = pidx % h1;
         float s = 0.0f;
         if (hidden > 0) {
-            const float w2 = w2s[h];
-#pragma unroll 4
-            for (int rr = 0; rr < RB; ++rr) {
-                const float d1 = H1s[rr * hst + h] > 0.0f ? dAs[rr] * w2 : 0.0f;
-                s += H0s[rr * ks + kk] * d1;
-            }
+#pragma unroll 8
+            for (int rr = 0; rr < RB; ++rr) s += H0s[rr * ks + kk] * D1s[rr * hst + h];
         } else {
-#pragma unroll 4
+#pragma unroll 8
             for (int rr = 0; rr < RB; ++rr) s += H0s[rr * ks + kk] * dAs[rr];
         }
         part_out[pidx] = s;
@@ -166,11 +179,10 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
     for (int h = tid; h < h1; h += NT) {
         float gb1 = 0.0f, gW2 = 0.0f;
         if (hidden > 0) {
-            const float w2 = w2s[h];
+#pragma unroll 8
             for (int rr = 0; rr < RB; ++rr) {
-                const float hv = H1s[rr * hst + h], d = dAs[rr];
-                gb1 += hv > 0.0f ? d * w2 : 0.0f;
-                gW2 += hv * d;
+                gb1 += D1s[rr * hst + h];
+                gW2 += H1s[rr * hst + h] * dAs[rr];
             }
         } else {
             for (int rr = 0; rr < RB; ++rr) gb1 += dAs[rr];
@@ -225,7 +237,7 @@ extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, 
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(pooled && W1 && b1 && Y && Z && dpooled && dW1 && db1, "ValueError: null pointer argument");
     DBK_CHECK(hidden == 0 || (W2 && b2 && dW2 && db2), "ValueError: hidden layer requested but W2/b2/dW2/db2 are null");
-    const size_t smem = ((size_t)k * h1 + 2 * h1 + (size_t)RB * (k | 1) + (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
+    const size_t smem = ((size_t)k * h1 + 2 * h1 + (size_t)RB * (k | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
     DBK_CHECK(smem <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", k, hidden, smem);
     const size_t nchunk = (n + RB - 1) / RB;
     DBK_CHECK(nchunk <= 65535, "ValueError: the fused head takes at most %d rows per call (got %zu)", 65535 * RB, n);
