@@ -20,27 +20,33 @@ template <typename T>
 __device__ void build_letter_table(T* lut, const T* __restrict__ W, unsigned m, unsigned F, unsigned f0, unsigned mpad = 0)
 {
     if (mpad < m) mpad = m;
-    for (unsigned e = threadIdx.x; e < mpad * FT; e += blockDim.x) {
-        unsigned j = e / FT, fl = e % FT;
-        unsigned f = f0 + fl;
-        T w0 = 0, w1 = 0, w2 = 0, w3 = 0;
-        if (f < F && j < m) {
-            w0 = W[(4 * j + 0) * (size_t)F + f];
-            w1 = W[(4 * j + 1) * (size_t)F + f];
-            w2 = W[(4 * j + 2) * (size_t)F + f];
-            w3 = W[(4 * j + 3) * (size_t)F + f];
+    // two taps per thread and round, so that eight loads are in flight together (a plain strided loop waits
+    // for each round's loads before it issues the next)
+    for (unsigned e0 = threadIdx.x; e0 < mpad * FT; e0 += 2 * blockDim.x) {
+        T w[2][4];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const unsigned e = e0 + u * blockDim.x, j = e / FT, f = f0 + e % FT;
+            const bool in = e < mpad * FT && f < F && j < m;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) w[u][c] = in ? W[(4 * j + c) * (size_t)F + f] : (T)0;
         }
-        T z = w0;
-        z += w1;
-        z += w2;
-        z += w3;
-        T* row = lut + (size_t)j * NL * FT + fl;
-        row[0 * FT] = w0;
-        row[1 * FT] = w1;
-        row[2 * FT] = w2;
-        row[3 * FT] = w3;
-        row[4 * FT] = z * (T)0.25;
-        row[5 * FT] = (T)0;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const unsigned e = e0 + u * blockDim.x, j = e / FT, fl = e % FT;
+            if (e >= mpad * FT) break;
+            T z = w[u][0];
+            z += w[u][1];
+            z += w[u][2];
+            z += w[u][3];
+            T* row = lut + (size_t)j * NL * FT + fl;
+            row[0 * FT] = w[u][0];
+            row[1 * FT] = w[u][1];
+            row[2 * FT] = w[u][2];
+            row[3 * FT] = w[u][3];
+            row[4 * FT] = z * (T)0.25;
+            row[5 * FT] = (T)0;
+        }
     }
 }
 
