@@ -210,7 +210,15 @@ __global__ void k_head_reduce(head_args a)
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
         const unsigned b = (unsigned)(e / a.pstride), idx = (unsigned)(e % a.pstride);
         float s = 0.0f;
-        for (unsigned c = 0; c < a.nchunk; ++c) s += a.partial[((size_t)c * a.nblock + b) * a.pstride + idx];
+        // eight chunks in flight per round, added in ascending order
+        for (unsigned c0 = 0; c0 < a.nchunk; c0 += 8) {
+            float v[8];
+#pragma unroll
+            for (unsigned t = 0; t < 8; ++t) v[t] = c0 + t < a.nchunk ? a.partial[((size_t)(c0 + t) * a.nblock + b) * a.pstride + idx] : 0.0f;
+#pragma unroll
+            for (unsigned t = 0; t < 8; ++t)
+                if (c0 + t < a.nchunk) s += v[t];
+        }
         if (idx < nW1) a.dW1[(size_t)b * nW1 + idx] = s;
         else if (idx < nW1 + h1) a.db1[(size_t)b * h1 + (idx - nW1)] = s;
         else if (idx < nW1 + 2 * h1) { if (hidden > 0) a.dW2[(size_t)b * hidden + (idx - nW1 - h1)] = s; }

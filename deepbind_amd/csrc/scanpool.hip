@@ -462,10 +462,15 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
     const size_t nelem = nW + nB;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < nelem; e += (size_t)gridDim.x * blockDim.x) {
         float total = 0.0f;
-        for (unsigned base = 0; base < nslab; base += 8) {
-            float buf[8];
-            for (unsigned s = 0; s < 8; ++s) buf[s] = base + s < nslab ? slabs[(size_t)(base + s) * nelem + e] : 0.0f;
-            total += ((buf[0] + buf[1]) + (buf[2] + buf[3])) + ((buf[4] + buf[5]) + (buf[6] + buf[7]));
+        // 32 slabs in flight per round; they are added as four 8-wide trees in ascending order, whatever the round size
+        for (unsigned base = 0; base < nslab; base += 32) {
+            float buf[32];
+#pragma unroll
+            for (unsigned s = 0; s < 32; ++s) buf[s] = base + s < nslab ? slabs[(size_t)(base + s) * nelem + e] : 0.0f;
+#pragma unroll
+            for (unsigned q = 0; q < 32; q += 8)
+                if (base + q < nslab)
+                    total += ((buf[q] + buf[q + 1]) + (buf[q + 2] + buf[q + 3])) + ((buf[q + 4] + buf[q + 5]) + (buf[q + 6] + buf[q + 7]));
         }
         if (e < nW) dW[e] = overwrite ? total : dW[e] + total;
         else dbias[e - nW] = total;
