@@ -288,6 +288,41 @@ def test_scanpool_bprop_with_activity_masks_equals_recomputation(ks, ptype, B, l
         ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, path="kmer", act=act)
 
 
+@pytest.mark.parametrize("ptype", ["max", "all"])
+def test_scanpool_bprop_bulk_is_linear_and_independent_of_region_order(ks, ptype):
+    """Size-independent properties of the fused backward at a bulk size (4096 sequences x 101 nt, 128 filters of
+    width 24, through the activity masks for max+avg pooling): the gradient is linear in the pooled gradient,
+    and listing the regions in another order changes nothing but the order of the additions."""
+    from deepbind_amd import data
+    rng = np.random.default_rng(11)
+    B, L, m, F = 4096, 101, 24, 128
+    codes = rng.integers(0, 4, (B, L), dtype=np.uint8)
+    codes[rng.random((B, L)) < 0.01] = 255
+    Xh, Rh = data.pack_uniform_ordinals(codes, m - 1)
+    X, R = dev(Xh), dev(Rh)
+    W = dev((rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32))
+    b = dev((rng.standard_normal((1, F)) * 0.05).astype(np.float32))
+    act = ks.activity_words(X, W) if ptype == "all" else None
+    P, I = ks.scanpool_fprop(W, b, X, R, ptype, want_argmax=True, act=act)
+
+    def grad(dP, regions=R, pooled=P, amax=I):
+        dW = torch.empty_like(W); db = torch.empty_like(b)
+        ks.scanpool_bprop(W, b, X, regions, ptype, pooled, amax, dP, dW, db, overwrite=True, act=act)
+        return host(dW).astype(np.float64), host(db).astype(np.float64)
+
+    d1 = torch.randn_like(P); d2 = torch.randn_like(P)
+    (w1, b1), (w2, b2), (w12, b12) = grad(d1), grad(d2), grad(2.0 * d1 + d2)
+    assert_close(w12, 2.0 * w1 + w2, GRAD, "dW linear")
+    assert_close(b12, 2.0 * b1 + b2, GRAD, "db linear")
+    perm = rng.permutation(B)                                          # (on the host: unsigned index tensors cannot be gathered on the device)
+    wp, bp = grad(dev(host(d1)[perm]), dev(Rh[perm]), dev(host(P)[perm]), dev(host(I)[perm]))
+    assert_close(wp, w1, GRAD, "dW under a permutation of the regions")
+    assert_close(bp, b1, GRAD, "db under a permutation of the regions")
+    # the bias gradient is the plain sum of the gradients that pass the rectifier: for max pooling, of dP where pooled > 0
+    if ptype == "max":
+        assert_close(b1, (host(d1).astype(np.float64) * (host(P) > 0)).sum(axis=0, keepdims=True), GRAD, "db closed form")
+
+
 # ------------------------------------------------------------------------------------------ dense head
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_blockwise_dot_family(ds, dtype):
