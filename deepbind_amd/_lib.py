@@ -50,6 +50,8 @@ _SIGNATURES = {
     "dbk_gradstep": [_P, _I, _Z, _P, _P, _P, _P, _P],
     "dbk_gradstep_nesterov1": [_P, _I, _Z, _P, _P, _P],
     "dbk_gradstep_nesterov2": [_P, _I, _Z, _P, _P, _P, _P, _P],
+    "dbk_gradstep_lookahead": [_P, _I, _Z, _P, _P, _P, _P],
+    "dbk_gradstep_nesterov2_lookahead": [_P, _I, _Z, _P, _P, _P, _P, _P, _P],
     "dbk_madd_bcast": [_P, _I, _P, _P, _P, _Z, _Z, _Z],
     "dbk_maskout": [_P, _I, _P, _P, _Z],
     "dbk_calc_zmask": [_P, _I, _P, _P, _Z, _Z],
@@ -91,6 +93,7 @@ class TrainStepArgs(ctypes.Structure):
         ("rate", _P), ("seed", _U64), ("counter", _P),
         ("decay", _P), ("freeze_scan", _I),
         ("pooled", _P), ("argmax", _P), ("Z", _P), ("dpooled", _P), ("loss", _P), ("act", _P),
+        ("L", _P), ("L_ready", _I),
     ]
 
 _dll = None

@@ -35,6 +35,24 @@ template <typename T> __global__ void k_nesterov2(T* P, const T* dP, const T* dr
         P[i] -= delta;
     }
 }
+// Look-ahead kept beside the parameters: L = P + mrate*mP (the value nesterov1 leaves in P).
+template <typename T> __global__ void k_lookahead(T* L, const T* P, const T* mP, const T* mrate, size_t n)
+{
+    GRID_STRIDE(i, n) L[i] = P[i] + mrate[i] * mP[i];
+}
+// nesterov2 on the look-ahead L, leaving the new parameters in P and the NEXT step's look-ahead in L:
+// the same operations, in the same order, as nesterov2 followed by the next step's nesterov1.
+template <typename T> __global__ void k_nesterov2_lookahead(T* P, T* L, const T* dP, const T* drate, T* mP, const T* mrate, size_t n)
+{
+    GRID_STRIDE(i, n) {
+        const T delta = dP[i] * drate[i];
+        const T mom = mP[i] * mrate[i] - delta;
+        const T pn = L[i] - delta;
+        mP[i] = mom;
+        P[i] = pn;
+        L[i] = pn + mrate[i] * mom;
+    }
+}
 template <typename T> __global__ void k_madd_bcast(const T* A, const T* b, T* dst, size_t n, size_t m, size_t k)
 {
     GRID_STRIDE(i, n) dst[i] += A[i] * b[(i / k) % m];
@@ -382,6 +400,16 @@ int dbk_gradstep_nesterov1(dbk_stream_t stream, int dtype, size_t n, void* P, co
 int dbk_gradstep_nesterov2(dbk_stream_t stream, int dtype, size_t n, void* P, const void* dP, const void* drate, void* mP, const void* mrate)
 {
     EW2(k_nesterov2, n, A(F32(P), CF32(dP), CF32(drate), F32(mP), CF32(mrate), n), A(F64(P), CF64(dP), CF64(drate), F64(mP), CF64(mrate), n));
+}
+int dbk_gradstep_lookahead(dbk_stream_t stream, int dtype, size_t n, void* L, const void* P, const void* mP, const void* mrate)
+{
+    EW2(k_lookahead, n, A(F32(L), CF32(P), CF32(mP), CF32(mrate), n), A(F64(L), CF64(P), CF64(mP), CF64(mrate), n));
+}
+int dbk_gradstep_nesterov2_lookahead(dbk_stream_t stream, int dtype, size_t n, void* P, void* L, const void* dP, const void* drate,
+                                     void* mP, const void* mrate)
+{
+    EW2(k_nesterov2_lookahead, n, A(F32(P), F32(L), CF32(dP), CF32(drate), F32(mP), CF32(mrate), n),
+        A(F64(P), F64(L), CF64(dP), CF64(drate), F64(mP), CF64(mrate), n));
 }
 int dbk_madd_bcast(dbk_stream_t stream, int dtype, const void* A_, const void* b, void* dst, size_t n, size_t m, size_t k)
 {

@@ -6,7 +6,9 @@
 // trainer's loop (deepity/deepity/sgd.py:98-135: gradstep with the batch gradient as its callback,
 // deepity_smat.py:77-117), with the gradient computed by the fused kernels:
 //
-//   [P += mrate*mP]                                   Nesterov look-ahead       (gradstep.cu:41-51)
+//   [P += mrate*mP]                                   Nesterov look-ahead       (gradstep.cu:41-51); kept in a vector
+//                                                     of its own when the caller provides one, and then formed by
+//                                                     the previous step's update kernel instead of a launch here
 //   [Xd = input dropout(X)]                           dropoutord.py:50-70
 //   pooled, argmax = scanpool_fprop(Wc, bc, Xd)       corr1ord -> bias -> relu -> poolrgn
 //   Z, dpooled, dW1.. = head_train(pooled, Y)         dropout -> full (-> relu -> full) -> bias -> loss
@@ -48,10 +50,18 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
                              a->off_W2 + nW2, a->off_b2 + nb2 };
     for (size_t v : need) DBK_CHECK(v <= a->nparam, "ValueError: a parameter block reaches past the flat vector (%zu > %zu)", v, a->nparam);
 
-    float* const P = a->P;
+    // Nesterov with a look-ahead vector: the step's weights are read from L = P + mrate*mP, which the previous
+    // step left there (L_ready) or which is formed now; otherwise the look-ahead is applied to P in place.
+    const bool beside = a->nesterov && a->L != nullptr;
+    float* const P = beside ? a->L : a->P;                         // where this step's weights are read
     float* const dP = a->dP;
     int rc;
-    if (a->nesterov) {
+    if (beside) {
+        if (!a->L_ready) {
+            rc = dbk_gradstep_lookahead(stream, DBK_F32, a->nparam, a->L, a->P, a->mP, a->mrate);
+            if (rc) return rc;
+        }
+    } else if (a->nesterov) {
         rc = dbk_gradstep_nesterov1(stream, DBK_F32, a->nparam, P, a->mP, a->mrate);
         if (rc) return rc;
     }
@@ -87,7 +97,8 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
         if (rc) return rc;
     }
     if (a->freeze_scan) hipLaunchKernelGGL(k_zero_f32, dim3(dbk::ew_grid(nWc)), dim3(256), 0, dbk::as_stream(stream), dP + a->off_Wc, nWc);
-    if (a->nesterov) rc = dbk_gradstep_nesterov2(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
+    if (beside) rc = dbk_gradstep_nesterov2_lookahead(stream, DBK_F32, a->nparam, a->P, a->L, dP, a->drate, a->mP, a->mrate);
+    else if (a->nesterov) rc = dbk_gradstep_nesterov2(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
     else rc = dbk_gradstep(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
     return rc;
 }

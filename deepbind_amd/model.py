@@ -56,6 +56,9 @@ class SequenceNet(object):
         self.step_count = 0
         self._step_args = None               # argument block and work buffers of the natively issued step
         self._step_bufs = {}
+        # Nesterov look-ahead kept beside the parameters by the natively issued step (each step's update kernel
+        # leaves the next step's look-ahead there); valid while nothing else has touched P, mP or mrate
+        self._L, self._L_versions = None, None
         self._busy_stream = None             # side stream a ModelGroup left this net's last step on
         ni, nf = self.ninst, self.nfilter
         self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
@@ -466,6 +469,17 @@ class SequenceNet(object):
                     Xdrop=torch.empty(X.numel(), dtype=torch.uint8, device=dev) if self.input_dropout > 0 else None,
                     Mdrop=torch.empty(X.numel(), dtype=torch.bool, device=dev) if self.input_dropout > 0 else None)
         a.nesterov, a.seed = int(bool(self.nesterov)), int(self.rng_seed)
+        if self.nesterov:
+            if self._L is None:
+                self._L = torch.empty_like(self.P)
+            a.L = self._L.data_ptr()
+            # in-place changes made through torch (set_params, set_rates, a view written by the caller) move these counters;
+            # the wrappers that write through raw pointers (the layer-by-layer and the graphed step) reset _L_versions
+            versions = (self.P._version, self.mP._version, self.mrate._version)
+            a.L_ready = int(self._L_versions == versions)
+            self._L_versions = versions
+        else:
+            a.L, a.L_ready = None, 0
         pv = lambda t: None if t is None else _lib.ptr(t).value          # checks device + contiguity
         a.X, a.N, a.regions, a.nregion = pv(X), X.numel(), pv(R), P
         a.Y, a.Ymask = pv(Y), pv(Ymask)
@@ -501,6 +515,8 @@ class SequenceNet(object):
         if fused and U is None and U_input is None:
             self._native_step(X, R, Y, Ymask)
             return
+
+        self._L_versions = None                 # the step below updates P and mP in place
 
         def grad():
             if fused:
@@ -574,6 +590,7 @@ def _graphed_step(jobs, streams=None):
     def step():
         for net, *_ in jobs:
             net.join()
+            net._L_versions = None              # the graph updates P and mP in place
         if state["graph"] is None or state["decay"] != decay_flags():
             capture()
         state["graph"].replay()

@@ -193,6 +193,16 @@ int dbk_gradstep_nesterov1(dbk_stream_t stream, int dtype, size_t n,
 int dbk_gradstep_nesterov2(dbk_stream_t stream, int dtype, size_t n,
                            void* P, const void* dP, const void* drate, void* mP, const void* mrate);
 
+/* The Nesterov step with the look-ahead kept in a vector L beside the parameters, which saves a launch
+ * per step: dbk_gradstep_lookahead sets L = P + mrate*mP (what nesterov1 leaves in P); the gradient is
+ * taken at L; dbk_gradstep_nesterov2_lookahead then does mP = mrate*mP - drate*dP, P = L - drate*dP and
+ * L = P + mrate*mP for the next step. Same operations in the same order as nesterov1 / nesterov2: the
+ * parameters come out bit-identical. (reference: gradstep.cu:41-72) */
+int dbk_gradstep_lookahead(dbk_stream_t stream, int dtype, size_t n,
+                           void* L, const void* P, const void* mP, const void* mrate);
+int dbk_gradstep_nesterov2_lookahead(dbk_stream_t stream, int dtype, size_t n,
+                                     void* P, void* L, const void* dP, const void* drate, void* mP, const void* mrate);
+
 /* dst[i] += A[i] * b[(i/k) % m] for i < n.
  * reference: launch_madd_bcast, deepity_smat.cpp:54-56, madd_bcast.cu:41-58 */
 int dbk_madd_bcast(dbk_stream_t stream, int dtype, const void* A, const void* b, void* dst,
@@ -325,12 +335,16 @@ typedef struct dbk_train_step_args {
     float* pooled; uint32_t* argmax; float* Z; float* dpooled;
     float* loss;                            /* per-model mean loss (nmodel), may be NULL */
     uint64_t* act;                          /* activity masks (see dbk_scanpool_fprop), N * ceil(nmodel*nfilter/64) words; may be NULL */
+    float* L;                               /* look-ahead vector (nparam), may be NULL: see dbk_gradstep_lookahead */
+    int L_ready;                            /* L already holds P + mrate*mP (left there by the previous step) */
 } dbk_train_step_args;
 
 /* One optimiser step, all launches issued from native code on `stream`:
  * [Nesterov look-ahead] -> [input dropout] -> dbk_scanpool_fprop -> dbk_head_train -> dbk_scanpool_bprop
  * -> [dbk_l1_decay] -> [zero dWc] -> momentum / Nesterov update. Bit-identical to calling those entry
  * points one by one; exists because a step on a small minibatch is bound by the host's cost per launch.
+ * With a look-ahead vector L (Nesterov only) the step reads its weights from L and ends by writing the
+ * next step's look-ahead there, so consecutive steps need no launch for it (L_ready).
  * reference: the body of the trainer's loop, deepity/deepity/sgd.py:98-135 (gradstep with the batch
  * gradient as callback, deepity_smat.py:77-117, gradstep.cu:41-72). */
 int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* args);

@@ -544,6 +544,30 @@ def test_natively_issued_step_equals_the_step_issued_call_by_call(pool, hidden, 
             assert np.array_equal(a, b), "step %d: %s differs" % (i, name)
         assert int(native.rng_counter.item()) == int(stepwise.rng_counter.item()) == native._rng_offset == stepwise._rng_offset
     assert np.abs(native.mP.cpu().numpy()).max() > 0 and native.step_count == 4
+    # the natively issued step keeps the Nesterov look-ahead beside the parameters from one step to the next; whatever
+    # changes the parameters, the momentum or the momentum rates in between must make it form the look-ahead afresh
+    if nesterov:
+        for change in ("params", "rates", "view", "layerwise"):
+            for net in (native, stepwise):
+                if change == "params":
+                    net.set_params({k: v * 0.5 for k, v in net.get_params().items()})
+                elif change == "rates":
+                    net.set_rates([0.03, 0.01, 0.2], 0.6)
+                elif change == "view":
+                    net.p["bc"].add_(0.25)
+            if change == "layerwise":
+                Ux = dev(rng.random((len(seqs), native.k * ni)).astype(np.float32))
+                Ui = dev(rng.random(Xh.shape).astype(np.float32)) if native.input_dropout > 0 else None
+                native.train_step(X, R, Y, M, U=Ux, U_input=Ui)           # goes through the wrappers, in place
+                stepwise.train_step(X, R, Y, M, U=Ux, U_input=Ui)
+            for _ in range(2):
+                native.train_step(X, R, Y, M)
+                ds.gradstep(stepwise.P, stepwise.dP, stepwise.drate, stepwise.mP, stepwise.mrate,
+                            lambda: stepwise._grad_fused(X, R, Y, M, None), nesterov=True)
+                stepwise.step_count += 1
+            torch.cuda.synchronize()
+            for name in ("P", "mP"):
+                assert np.array_equal(getattr(native, name).cpu().numpy(), getattr(stepwise, name).cpu().numpy()), (change, name)
 
 
 def test_group_steps_left_in_flight_match_joined_steps_across_changing_batches():
