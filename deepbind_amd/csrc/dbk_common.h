@@ -18,7 +18,21 @@ void clear_error();
 // launches are ordered within a stream, so consecutive calls on it can share the buffer, and calls on
 // different streams never do. At most 64 distinct streams per device; null when that is exceeded or
 // when memory runs out. Growing a buffer synchronises the device (and so cannot happen under capture).
-void* workspace(size_t bytes, hipStream_t stream);
+// `which` selects one of two independent buffers of the stream (a call that must keep one kernel's partial
+// results while another kernel fills its own uses the second).
+void* workspace(size_t bytes, hipStream_t stream, int which = 0);
+
+// While dbk_train_step runs, dbk_head_train and dbk_scanpool_bprop leave their partial results unreduced and
+// describe them here instead: the step's last kernel adds them up (in the order the stand-alone reduction
+// kernels use) and applies the parameter update in the same pass. Thread-local; null outside such a step.
+struct deferred_sums {
+    const float* head_partial = nullptr;    // [chunk][model][pstride] (see head_train.hip)
+    unsigned head_nchunk = 0, head_pstride = 0;
+    const float* slabs = nullptr;           // [slab][stride]: 4m*F filter gradients then F bias gradients
+    size_t slab_stride = 0;
+    unsigned nslab = 0;
+};
+deferred_sums*& deferred();
 
 inline hipStream_t as_stream(dbk_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -257,10 +257,17 @@ extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, 
     a.nchunk = (unsigned)nchunk;
     a.pstride = (unsigned)(k * h1 + 2 * h1 + 2);
     const size_t pbytes = nchunk * (size_t)nblock * a.pstride * sizeof(float);
-    a.partial = (float*)dbk::workspace(pbytes, dbk::as_stream(stream));
+    dbk::deferred_sums* later = dbk::deferred();                   // inside dbk_train_step: the chunk sums are taken by its last kernel
+    a.partial = (float*)dbk::workspace(pbytes, dbk::as_stream(stream), later ? 1 : 0);
     DBK_CHECK(a.partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", pbytes);
     DBK_HIP(hipFuncSetAttribute((const void*)k_head_train, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(k_head_train, dim3(nblock, (unsigned)nchunk), dim3(NT), smem, dbk::as_stream(stream), a);
-    hipLaunchKernelGGL(k_head_reduce, dim3(dbk::ew_grid((size_t)nblock * a.pstride)), dim3(256), 0, dbk::as_stream(stream), a);
+    if (later) {
+        later->head_partial = a.partial;
+        later->head_nchunk = a.nchunk;
+        later->head_pstride = a.pstride;
+    } else {
+        hipLaunchKernelGGL(k_head_reduce, dim3(dbk::ew_grid((size_t)nblock * a.pstride)), dim3(256), 0, dbk::as_stream(stream), a);
+    }
     DBK_LAUNCH_OK();
 }

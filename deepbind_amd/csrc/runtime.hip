@@ -17,14 +17,15 @@ void set_error(const char* fmt, ...)
 
 void clear_error() { g_err[0] = 0; }
 
-struct ws_t { hipStream_t stream = nullptr; void* ptr = nullptr; size_t bytes = 0; bool used = false; };
+struct ws_t { hipStream_t stream = nullptr; void* ptr[2] = {nullptr, nullptr}; size_t bytes[2] = {0, 0}; bool used = false; };
 constexpr int WS_DEVICES = 64, WS_STREAMS = 64;
 static ws_t g_ws[WS_DEVICES][WS_STREAMS];
 static std::mutex g_ws_mutex;
 
-void* workspace(size_t bytes, hipStream_t stream)
+void* workspace(size_t bytes, hipStream_t stream, int which)
 {
     int dev = 0;
+    if (which < 0 || which > 1) return nullptr;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= WS_DEVICES) return nullptr;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     ws_t* w = nullptr;
@@ -35,19 +36,22 @@ void* workspace(size_t bytes, hipStream_t stream)
     if (!w) return nullptr;
     w->used = true;
     w->stream = stream;
-    if (w->bytes >= bytes && w->ptr) return w->ptr;
-    if (w->ptr) {
+    if (w->bytes[which] >= bytes && w->ptr[which]) return w->ptr[which];
+    if (w->ptr[which]) {
         // earlier launches may still be reading the old buffer
         if (hipDeviceSynchronize() != hipSuccess) return nullptr;
-        (void)hipFree(w->ptr);
-        w->ptr = nullptr;
-        w->bytes = 0;
+        (void)hipFree(w->ptr[which]);
+        w->ptr[which] = nullptr;
+        w->bytes[which] = 0;
     }
     size_t want = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes + bytes / 4;
-    if (hipMalloc(&w->ptr, want) != hipSuccess) { w->ptr = nullptr; return nullptr; }
-    w->bytes = want;
-    return w->ptr;
+    if (hipMalloc(&w->ptr[which], want) != hipSuccess) { w->ptr[which] = nullptr; return nullptr; }
+    w->bytes[which] = want;
+    return w->ptr[which];
 }
+
+static thread_local deferred_sums* g_deferred = nullptr;
+deferred_sums*& deferred() { return g_deferred; }
 
 }  // namespace dbk
 

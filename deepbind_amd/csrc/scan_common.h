@@ -290,6 +290,23 @@ __device__ __forceinline__ void stage(uint8_t* xl, const uint8_t* __restrict__ X
 }
 
 
+// Element e summed over nslab slabs of nelem entries: 32 slabs in flight per round, added as four 8-wide trees in
+// ascending order, whatever the round size (the one summation order every reduction of slabs uses).
+__device__ __forceinline__ float slab_sum(const float* __restrict__ slabs, size_t nelem, size_t e, unsigned nslab)
+{
+    float total = 0.0f;
+    for (unsigned base = 0; base < nslab; base += 32) {
+        float buf[32];
+#pragma unroll
+        for (unsigned s = 0; s < 32; ++s) buf[s] = base + s < nslab ? slabs[(size_t)(base + s) * nelem + e] : 0.0f;
+#pragma unroll
+        for (unsigned q = 0; q < 32; q += 8)
+            if (base + q < nslab)
+                total += ((buf[q] + buf[q + 1]) + (buf[q + 2] + buf[q + 3])) + ((buf[q + 4] + buf[q + 5]) + (buf[q + 6] + buf[q + 7]));
+    }
+    return total;
+}
+
 inline size_t lds_limit()
 {
     static size_t cached = 0;

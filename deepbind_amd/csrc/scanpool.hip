@@ -461,17 +461,7 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
 {
     const size_t nelem = nW + nB;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < nelem; e += (size_t)gridDim.x * blockDim.x) {
-        float total = 0.0f;
-        // 32 slabs in flight per round; they are added as four 8-wide trees in ascending order, whatever the round size
-        for (unsigned base = 0; base < nslab; base += 32) {
-            float buf[32];
-#pragma unroll
-            for (unsigned s = 0; s < 32; ++s) buf[s] = base + s < nslab ? slabs[(size_t)(base + s) * nelem + e] : 0.0f;
-#pragma unroll
-            for (unsigned q = 0; q < 32; q += 8)
-                if (base + q < nslab)
-                    total += ((buf[q] + buf[q + 1]) + (buf[q + 2] + buf[q + 3])) + ((buf[q + 4] + buf[q + 5]) + (buf[q + 6] + buf[q + 7]));
-        }
+        const float total = slab_sum(slabs, nelem, e, nslab);
         if (e < nW) dW[e] = overwrite ? total : dW[e] + total;
         else dbias[e - nW] = total;
     }
@@ -724,7 +714,8 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P,
                            pooled, argmax, dpooled, slabs, stride);
-        hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gx, overwrite);
+        if (dbk::deferred_sums* later = dbk::deferred()) { later->slabs = slabs; later->slab_stride = stride; later->nslab = gx; }
+        else hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gx, overwrite);
         DBK_LAUNCH_OK();
     }
     // sparse half: ~2048 single-wave workgroups, at least four regions each
@@ -761,7 +752,8 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         else rc = launch_dense<PD, 24>(st, gxd, ftiles, smem_d, W, bias, m, F, X, N, R, P, pooled, argmax, dpooled, act, sd, stride);
         if (rc) return rc;
     }
-    hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd, overwrite);
+    if (dbk::deferred_sums* later = dbk::deferred()) { later->slabs = slabs; later->slab_stride = stride; later->nslab = gxs + gxd; }
+    else hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gxs + gxd, overwrite);
     DBK_LAUNCH_OK();
 }
 
@@ -834,6 +826,13 @@ int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, s
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && dW && dbias, "ValueError: null pointer argument");
+    if (nregion == 0 && dbk::deferred()) {
+        dbk::deferred()->slabs = nullptr;                          // zero slabs: the gradient is zero
+        dbk::deferred()->slab_stride = 4 * m * nfilter + nfilter;
+        dbk::deferred()->nslab = 0;
+        dbk::clear_error();
+        return 0;
+    }
     if (nregion == 0) {
         // no regions: the bias gradient is written as zero by the slab reduction over zero slabs
         // (a kernel rather than a memset, so that the call can sit in a captured graph)

@@ -20,8 +20,81 @@
 // The same entry points a caller would use one by one are called in the same order, so the result is
 // bit-identical to issuing them separately.
 #include "dbk_common.h"
+#include "scan_common.h"
 
 namespace {
+
+// The step's last kernel when the look-ahead lives beside the parameters: one pass over the flat vectors that
+//   * adds up the partial results the backward kernels left (slabs of the scan filters' gradient as
+//     reduce_slabs_kernel does, row chunks of the dense head's gradients as k_head_reduce does: same order),
+//   * adds the L1 term, zeroes the scan filters' gradient while they are frozen, stores the gradient,
+//   * applies the Nesterov update and forms the next step's look-ahead,
+//   * writes the per-model loss when asked and moves the dropout generator on.
+struct reduce_update_args {
+    size_t nparam;
+    float *P, *L, *dP, *mP;
+    const float *drate, *mrate, *decay;
+    size_t off_Wc, off_bc, off_W1, off_b1, off_W2, off_b2;
+    size_t nWc, nbc, nW1, nb1, nW2, nb2;
+    const float* slabs; size_t slab_stride; unsigned nslab;
+    const float* head_partial; unsigned nchunk, pstride;
+    unsigned nblock, k, h1, hidden;
+    int freeze_scan, loss_kind;
+    float* loss; size_t nrow;
+    unsigned long long* counter; unsigned long long counter_advance;
+};
+
+__device__ __forceinline__ float chunk_sum(const reduce_update_args& a, unsigned b, unsigned idx)
+{
+    float s = 0.0f;
+    for (unsigned c0 = 0; c0 < a.nchunk; c0 += 8) {                // eight chunks in flight per round, added in ascending order
+        float v[8];
+#pragma unroll
+        for (unsigned t = 0; t < 8; ++t) v[t] = c0 + t < a.nchunk ? a.head_partial[((size_t)(c0 + t) * a.nblock + b) * a.pstride + idx] : 0.0f;
+#pragma unroll
+        for (unsigned t = 0; t < 8; ++t)
+            if (c0 + t < a.nchunk) s += v[t];
+    }
+    return s;
+}
+
+__global__ __launch_bounds__(256) void k_reduce_update(reduce_update_args a)
+{
+    const unsigned nW1m = a.k * a.h1;                              // dense weights per model
+    const size_t total = a.nparam + (a.loss ? a.nblock : 0);
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+        if (e >= a.nparam) {                                       // per-model loss
+            const unsigned b = (unsigned)(e - a.nparam);
+            const float s = chunk_sum(a, b, nW1m + 2 * a.h1 + 1);
+            a.loss[b] = a.loss_kind == 0 ? -s / (float)a.nrow : 0.5f * s / (float)a.nrow;
+            continue;
+        }
+        float g;
+        bool scan_weight = false;
+        if (e - a.off_Wc < a.nWc) { g = dbk_scan::slab_sum(a.slabs, a.slab_stride, e - a.off_Wc, a.nslab); scan_weight = true; }
+        else if (e - a.off_bc < a.nbc) g = dbk_scan::slab_sum(a.slabs, a.slab_stride, a.nWc + (e - a.off_bc), a.nslab);
+        else if (e - a.off_W1 < a.nW1) { const size_t q = e - a.off_W1; g = chunk_sum(a, (unsigned)(q / nW1m), (unsigned)(q % nW1m)); }
+        else if (e - a.off_b1 < a.nb1) { const size_t q = e - a.off_b1; g = chunk_sum(a, (unsigned)(q / a.h1), nW1m + (unsigned)(q % a.h1)); }
+        else if (e - a.off_W2 < a.nW2) { const size_t q = e - a.off_W2; g = chunk_sum(a, (unsigned)(q / a.hidden), nW1m + a.h1 + (unsigned)(q % a.hidden)); }
+        else { const size_t q = e - a.off_b2; g = chunk_sum(a, (unsigned)q, nW1m + 2 * a.h1); }
+        const float look = a.L[e];
+        if (a.decay) {
+            const float sg = (float)((look > 0.0f) - (look < 0.0f));
+            g += sg * a.decay[e];
+        }
+        if (scan_weight && a.freeze_scan) g = 0.0f;
+        a.dP[e] = g;
+        const float rm = a.mrate[e];
+        const float delta = g * a.drate[e];
+        const float mom = a.mP[e] * rm - delta;
+        const float pn = look - delta;
+        a.mP[e] = mom;
+        a.P[e] = pn;
+        a.L[e] = pn + rm * mom;
+    }
+    // every workgroup of the head kernel has read the generator position long ago: move it on
+    if (a.counter && a.counter_advance && blockIdx.x == 0 && threadIdx.x == 0) a.counter[0] += a.counter_advance;
+}
 
 __global__ void k_zero_f32(float* p, size_t n)
 {
@@ -77,6 +150,10 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
         if (rc) return rc;
         X = a->Xdrop;
     }
+    // with the look-ahead beside the parameters the backward kernels leave their partial sums for the step's last kernel
+    dbk::deferred_sums later;
+    struct scope { dbk::deferred_sums*& slot; ~scope() { slot = nullptr; } } guard{dbk::deferred()};
+    if (beside) dbk::deferred() = &later;
     uint64_t* act = a->ptype == DBK_PT_MAX ? nullptr : a->act;      // only the average part of the backward pass reads the masks
     rc = dbk_scanpool_fprop(stream, P + a->off_Wc, P + a->off_bc, a->m, F, X, a->N, a->regions, a->nregion, a->ptype,
                             a->pooled, a->argmax, act);
@@ -92,13 +169,32 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
     rc = dbk_scanpool_bprop(stream, P + a->off_Wc, P + a->off_bc, a->m, F, X, a->N, a->regions, a->nregion, a->ptype,
                             a->pooled, a->argmax, a->dpooled, dP + a->off_Wc, dP + a->off_bc, 1, act);
     if (rc) return rc;
+    if (beside) {
+        dbk::deferred() = nullptr;
+        reduce_update_args u;
+        u.nparam = a->nparam;
+        u.P = a->P; u.L = a->L; u.dP = dP; u.mP = a->mP; u.drate = a->drate; u.mrate = a->mrate; u.decay = a->decay;
+        u.off_Wc = a->off_Wc; u.off_bc = a->off_bc; u.off_W1 = a->off_W1; u.off_b1 = a->off_b1;
+        u.off_W2 = a->hidden ? a->off_W2 : a->nparam; u.off_b2 = a->hidden ? a->off_b2 : a->nparam;
+        u.nWc = nWc; u.nbc = F; u.nW1 = nW1; u.nb1 = nb1; u.nW2 = nW2; u.nb2 = nb2;
+        u.slabs = later.slabs; u.slab_stride = later.slab_stride; u.nslab = later.nslab;
+        u.head_partial = later.head_partial; u.nchunk = later.head_nchunk; u.pstride = later.head_pstride;
+        u.nblock = (unsigned)a->nmodel; u.k = (unsigned)k; u.h1 = (unsigned)(a->hidden ? a->hidden : 1); u.hidden = (unsigned)a->hidden;
+        u.freeze_scan = a->freeze_scan; u.loss_kind = a->loss_kind; u.loss = a->loss; u.nrow = a->nregion;
+        u.counter = (unsigned long long*)a->counter; u.counter_advance = draws;
+        DBK_CHECK(nWc + F + nW1 + nb1 + nW2 + nb2 == a->nparam, "ValueError: the parameter blocks do not tile the flat vector (%zu of %zu elements)",
+                  nWc + F + nW1 + nb1 + nW2 + nb2, a->nparam);
+        DBK_CHECK((later.head_partial != nullptr || a->nregion == 0) && later.slab_stride == nWc + F,
+                  "RuntimeError: the backward kernels left no partial sums");
+        hipLaunchKernelGGL(k_reduce_update, dim3(dbk::ew_grid(a->nparam + a->nmodel)), dim3(256), 0, dbk::as_stream(stream), u);
+        DBK_LAUNCH_OK();
+    }
     if (a->decay) {
         rc = dbk_l1_decay(stream, DBK_F32, P, a->decay, dP, a->nparam);
         if (rc) return rc;
     }
     if (a->freeze_scan) hipLaunchKernelGGL(k_zero_f32, dim3(dbk::ew_grid(nWc)), dim3(256), 0, dbk::as_stream(stream), dP + a->off_Wc, nWc);
-    if (beside) rc = dbk_gradstep_nesterov2_lookahead(stream, DBK_F32, a->nparam, a->P, a->L, dP, a->drate, a->mP, a->mrate);
-    else if (a->nesterov) rc = dbk_gradstep_nesterov2(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
+    if (a->nesterov) rc = dbk_gradstep_nesterov2(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
     else rc = dbk_gradstep(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
     return rc;
 }
