@@ -442,6 +442,20 @@ def test_gradstep_and_madd_bcast(ds, dtype):
                     grad=lambda: called.append(1), nesterov=nesterov)
         assert called == [1]
         assert np.array_equal(host(P).ravel(), Pr) and np.array_equal(host(mP).ravel(), mPr)
+    # the look-ahead kept in a vector of its own: two steps give the bits of nesterov1 / nesterov2 applied in place
+    from deepbind_amd import _lib
+    Pr, mPr = P0.copy(), mP0.copy()
+    col = lambda a: dev(a.reshape(-1, 1))
+    P, mP, L, g1, g2, dr, mr = col(P0), col(mP0), col(np.zeros(n, dtype)), col(dP), col(dP * dtype(0.5)), col(drate), col(mrate)
+    dt = _lib.dtype_code(P)
+    _lib.call("dbk_gradstep_lookahead", _lib.stream(), dt, n, _lib.ptr(L), _lib.ptr(P), _lib.ptr(mP), _lib.ptr(mr))
+    for g, gh in ((g1, dP), (g2, dP * dtype(0.5))):
+        orc.gradstep_nesterov1(Pr, mPr, mrate)
+        assert np.array_equal(host(L).ravel(), Pr)                     # the gradient is taken at these look-ahead parameters
+        orc.gradstep_nesterov2(Pr, gh, drate, mPr, mrate)
+        _lib.call("dbk_gradstep_nesterov2_lookahead", _lib.stream(), dt, n, _lib.ptr(P), _lib.ptr(L), _lib.ptr(g), _lib.ptr(dr),
+                  _lib.ptr(mP), _lib.ptr(mr))
+        assert np.array_equal(host(P).ravel(), Pr) and np.array_equal(host(mP).ravel(), mPr)
     A = rng.standard_normal((24, 10)).astype(dtype); b = rng.standard_normal(3).astype(dtype)
     dst = rng.standard_normal((24, 10)).astype(dtype)
     ref = dst.copy(); orc.madd_bcast(A, b, 16, ref)
