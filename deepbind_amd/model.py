@@ -553,8 +553,11 @@ def _graphed_step(jobs, streams=None):
         return tuple((net.weight_decay_start <= net.step_count, net.step_count < net.start_training) for net, *_ in jobs)
 
     def one(net, X, R, Y, Ymask):
-        return lambda: ds.gradstep(net.P, net.dP, net.drate, net.mP, net.mrate,
-                                   lambda: net._grad_fused(X, R, Y, Ymask, None), nesterov=net.nesterov)
+        def run():
+            # the natively issued step on the capturing stream; the graph always forms its look-ahead itself
+            net._L_versions = None
+            net._native_step(X, R, Y, Ymask)
+        return run
 
     def body():
         if streams is None:
@@ -571,30 +574,32 @@ def _graphed_step(jobs, streams=None):
         cap = state["stream"]
         live = [t for net, *_ in jobs for t in (net.P, net.mP, net.dP, net.rng_counter)]
         saved = [t.clone() for t in live]
-        host_off = [net._rng_offset for net, *_ in jobs]
+        host_off = [(net._rng_offset, net.step_count) for net, *_ in jobs]
         cap.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(cap):
             body()
         torch.cuda.synchronize()
         for t, s_ in zip(live, saved):
             t.copy_(s_)
+        for (net, *_), (off, count) in zip(jobs, host_off):
+            net._rng_offset, net.step_count = off, count        # the warm-up step must not count (decay / freeze switches are baked in)
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g, stream=cap):
             body()
-        # capturing executes nothing on the device; only the host mirrors of the generator position moved
-        for (net, *_), off in zip(jobs, host_off):
-            net._rng_offset = off
+        # capturing executes nothing on the device; only the host mirrors of the step moved
+        for (net, *_), (off, count) in zip(jobs, host_off):
+            net._rng_offset, net.step_count = off, count
         state["graph"], state["decay"] = g, decay_flags()
 
     def step():
         for net, *_ in jobs:
             net.join()
-            net._L_versions = None              # the graph updates P and mP in place
         if state["graph"] is None or state["decay"] != decay_flags():
             capture()
         state["graph"].replay()
         for net, X, R, Y, Ymask in jobs:
+            net._L_versions = None              # (a step issued natively after this one forms its look-ahead afresh)
             if net.input_dropout > 0:
                 net._rng_offset += (X.numel() + 3) // 4
             if net.use_dropout:
