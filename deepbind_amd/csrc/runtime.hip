@@ -59,7 +59,7 @@ extern "C" {
 
 const char* dbk_last_error(void) { return dbk::g_err; }
 
-int dbk_version(void) { return 2; }
+int dbk_version(void) { return 3; }
 
 int dbk_device_count(void)
 {

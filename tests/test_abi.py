@@ -23,7 +23,7 @@ def test_header_symbols_are_exported_and_bound():
         assert hasattr(lib, name), "header declares %s but the library does not export it" % name
     # the Python binding covers the header and nothing else
     assert sorted(_lib.exported_names()) == names
-    assert lib.dbk_version() == 2
+    assert lib.dbk_version() == 3
     assert lib.dbk_last_error() == b""
 
 
