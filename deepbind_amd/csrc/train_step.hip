@@ -198,3 +198,5 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
     else rc = dbk_gradstep(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
     return rc;
 }
+
+extern "C" int dbk_train_step_args_size(void) { return (int)sizeof(dbk_train_step_args); }

@@ -348,6 +348,8 @@ typedef struct dbk_train_step_args {
  * reference: the body of the trainer's loop, deepity/deepity/sgd.py:98-135 (gradstep with the batch
  * gradient as callback, deepity_smat.py:77-117, gradstep.cu:41-72). */
 int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* args);
+/* sizeof(dbk_train_step_args) as the library was built, for bindings that mirror the block field by field. */
+int dbk_train_step_args_size(void);
 
 #ifdef __cplusplus
 }

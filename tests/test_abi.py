@@ -59,6 +59,7 @@ def test_train_step_argument_block_layout_matches_the_header():
     from deepbind_amd import _lib
     lib = _lib.dll()
     assert lib.dbk_train_step(None, None) != 0 and b"null argument block" in lib.dbk_last_error()
+    assert lib.dbk_train_step_args_size() == ctypes.sizeof(_lib.TrainStepArgs)
     a = _lib.TrainStepArgs()
     a.nmodel, a.nfilter, a.m, a.hidden = 3, 5, 7, 2
     a.ptype, a.loss_kind, a.reverse_complement, a.nesterov = _lib.PT_ALL, 0, 0, 1
