@@ -574,15 +574,20 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
             unsigned wq[window<MT>::words];
             load_window<MT>(xl, p0, wq);
             float g[PSUB];
+            // window-relative 32-bit positions of the winning row (this lane's; -1 when it lies elsewhere: it is always
+            // inside the region) and of the scan's end, so that the per-position tests are one 32-bit compare each
+            const size_t w0 = c0 + p0;
+            const int relmax = (PT == DBK_PT_ALL && imax >= w0 && imax - w0 < (size_t)PSUB) ? (int)(imax - w0) : -1;
+            const int nrel = n > w0 ? (n - w0 < (size_t)PSUB ? (int)(n - w0) : PSUB) : 0;
 #pragma unroll
             for (int p = 0; p < PSUB; ++p) {
                 const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)mk, p);
                 const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(mk >> 32), p);
                 const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
                 float gg = open ? gavg : 0.0f;
-                if (PT == DBK_PT_ALL) gg += (p0 + p < rows && c0 + p0 + p == imax) ? gmax : 0.0f;
+                if (PT == DBK_PT_ALL) gg += p == relmax ? gmax : 0.0f;
                 db += gg;
-                g[p] = c0 + p0 + p < n ? gg : 0.0f;                // rows past the scan's end carry bias only
+                g[p] = p < nrel ? gg : 0.0f;                       // rows past the scan's end carry bias only
             }
             grad_planes_window<MT>(planes, wq, g);
             mk = mkn;
