@@ -113,7 +113,8 @@ def train_throughput(steps=30, warmup=5):
     cfg = synth.config4()
     spec, hp = cfg["spec"], cfg["hp"]
     grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
-                     decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"])
+                     decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"],
+                     weight_decay_start=0)       # the L1 term is on in every timed step (steady state; a captured graph is re-captured when it switches on)
     for idx, net in grp.groups:
         net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
     X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
