@@ -67,9 +67,17 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
         for (int j = 0; j < 4; ++j)
             if (e0 + j * NT < k * h1) w1s[e0 + j * NT] = v[j];
     }
-    for (int e = tid; e < h1; e += NT) b1s[e] = a.b1[(size_t)b * h1 + e];
-    for (int e = tid; e < hidden; e += NT) w2s[e] = a.W2[(size_t)b * hidden + e];
+    for (int e = tid; e < h1; e += NT) {                          // both vectors' loads are issued before either is stored
+        const float vb = a.b1[(size_t)b * h1 + e];
+        const float vw = e < hidden ? a.W2[(size_t)b * hidden + e] : 0.0f;
+        b1s[e] = vb;
+        if (e < hidden) w2s[e] = vw;
+    }
     const float bias2 = hidden > 0 ? a.b2[b] : 0.0f;
+    // this row's target and mask are needed only after the forward pass: requested now, they arrive meanwhile
+    const size_t zi = live ? r * a.nblock + b : 0;
+    const float y_row = live ? a.Y[zi] : 0.0f;
+    const bool use_row = (live && a.Ymask) ? a.Ymask[zi] != 0 : true;
     const float p_drop = a.rate ? a.rate[b] : 0.0f;
     const unsigned long long off = a.counter ? a.counter[0] : a.offset;
     const float inv_n = 1.0f / (float)a.n;
@@ -107,6 +115,7 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
     if (hidden > 0) {
         for (int h = part; h < hidden; h += NP) {
             float s = 0.0f;
+#pragma unroll 8
             for (int kk = 0; kk < k; ++kk) s += x[kk] * w1s[kk * hidden + h];
             s += b1s[h];
             s = s > 0.0f ? s : 0.0f;
@@ -114,6 +123,7 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
             outp += s * w2s[h];
         }
     } else {
+#pragma unroll 4
         for (int kk = part; kk < k; kk += NP) outp += x[kk] * w1s[kk];
     }
     // butterfly over the row's lanes: every lane ends with the same bits
@@ -126,9 +136,8 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
     const float zo = __shfl_xor(z, NP, 64);
     float dA = 0.0f, lterm = 0.0f;
     if (live) {
-        const size_t zi = r * a.nblock + b;
-        const float y = a.Y[zi];
-        bool use = a.Ymask ? a.Ymask[zi] != 0 : true;
+        const float y = y_row;
+        bool use = use_row;
         if (a.revcomp) use = use && ((r & 1) ? !(zo >= z) : (z >= zo));
         if (use) {
             dA = (z - y) * inv_n;
