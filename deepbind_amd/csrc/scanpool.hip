@@ -530,12 +530,18 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
         if (PT == DBK_PT_ALL && q.pmax > 0.0f) { gmax = q.dmax; imax = q.arg / F; }
     };
 
+    // activity masks of the 16 rows from p0 of a chunk (lane p takes row p's); rows past the chunk read as "closed"
+    auto fetch = [&](size_t c_, unsigned rows_, unsigned p0) -> unsigned long long {
+        return (lane < (unsigned)PSUB && p0 + lane < rows_) ? act[(c_ + p0 + lane) * gridDim.y + blockIdx.y] : 0ull;
+    };
     size_t r = blockIdx.x;
     bool valid = r < P;
     size_t a = 0, b = 0, c0 = 0, pa = 0, pb = 0;                   // (pa, pb): bounds of the region after this one
+    unsigned long long mk_first = 0ull;                            // this wave's first masks of the current item
     if (valid) {
         a = R[2 * r]; b = R[2 * r + 1]; c0 = a;
         if (r + gridDim.x < P) { pa = R[2 * (r + gridDim.x)]; pb = R[2 * (r + gridDim.x) + 1]; }
+        mk_first = fetch(c0, rows_of(b, c0), wave * PSUB);
         enter_region(load_pooled(r), a, b);
         unsigned v0, v1;
         load_letters(c0, rows_of(b, c0), v0, v1);
@@ -560,17 +566,15 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
                 if (nr + gridDim.x < P) { qa = R[2 * (nr + gridDim.x)]; qb = R[2 * (nr + gridDim.x) + 1]; }
             }
         }
+        const unsigned long long mk_next = nvalid ? fetch(nc0, rows_of(nb, nc0), wave * PSUB) : 0ull;   // the next item's first masks
         // ---- this item
         const uint8_t* xl = xbuf + cur * XBUF;
-        auto fetch = [&](unsigned p0) -> unsigned long long {          // rows past the chunk read as "closed"
-            return (lane < (unsigned)PSUB && p0 + lane < rows) ? act[(c0 + p0 + lane) * gridDim.y + blockIdx.y] : 0ull;
-        };
-        unsigned long long mk = fetch(wave * PSUB);
+        unsigned long long mk = mk_first;
 #pragma unroll 1
         for (unsigned s = 0; s < XCH_SUBS; ++s) {
             const unsigned p0 = (s * nw + wave) * PSUB;
             if (p0 >= rows) break;
-            const unsigned long long mkn = fetch(p0 + nw * PSUB);
+            const unsigned long long mkn = fetch(c0, rows, p0 + nw * PSUB);
             unsigned wq[window<MT>::words];
             load_window<MT>(xl, p0, wq);
             float g[PSUB];
@@ -597,6 +601,7 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
         __syncthreads();
         if (newregion && nvalid) { enter_region(nq, na, nb); pa = qa; pb = qb; }
         r = nr; a = na; b = nb; c0 = nc0; valid = nvalid; cur ^= 1u;
+        mk_first = mk_next;
     }
     float aw[MT][4];
     grad_planes_read<MT>(planes, aw);
