@@ -125,6 +125,22 @@ def train_throughput(steps=30, warmup=5):
     return out
 
 
+def issue_rates(iters=4000):
+    """Sustained issue rate of one SIMD (1e9 wave-instructions/s) for the instructions the scan kernels are made of,
+    at 1-8 resident waves per SIMD: the library's probe (64 independent instructions per round on 8 registers)."""
+    import ctypes
+    from deepbind_amd import _lib
+    out = {}
+    for kind, name in enumerate(("v_add_f32", "v_fma_f32", "v_max_f32", "v_max3_f32", "v_add_f32 (VGPR index mode)")):
+        row = {}
+        for waves in (1, 2, 3, 4, 6, 8):
+            r = ctypes.c_double()
+            _lib.call("dbk_probe_valu_issue", kind, waves, iters, ctypes.addressof(r))
+            row["%d waves/SIMD" % waves] = round(r.value, 3)
+        out[name] = row
+    return out
+
+
 def ops_throughput(reps=5):
     """Per-operator figures for the drop-in operators and the general fused kernels on a mid-size batch
     (8192 sequences x 101 nt, 16 models x 16 motifs x width 24: N = 1.02 M rows, F = 256, map = 1.04 GB).
@@ -228,6 +244,7 @@ def main():
     ap.add_argument("--no-train", action="store_true", help="skip the secondary train-step throughput figures")
     ap.add_argument("--ops", action="store_true", help="only the per-operator figures of the drop-in and general fused kernels")
     ap.add_argument("--train-only", action="store_true", help="only the train-step figures (for profiling the training kernels)")
+    ap.add_argument("--issue-rates", action="store_true", help="only the vector-ALU issue rates the kernels' instruction counts are priced with")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain copy kernel over 1 GiB (reference point for the HBM byte counters)")
     args = ap.parse_args()
@@ -240,6 +257,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
 
+    if args.issue_rates:
+        print(json.dumps({"valu_issue": issue_rates()}))
+        return
     if args.train_only:
         print(json.dumps({"train": train_throughput(steps=args.steps, warmup=args.warmup)}))
         return
@@ -309,7 +329,10 @@ def main():
             "frac": adds_per_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS, "traffic": measured_traffic(args.workload),
             "kernel": "fused scan+bias+relu+maxpool (dbk_scanpool_fprop launches)", "kernel_ms": scan_ms,
             "algorithmic_adds_per_launch": adds,
-            "frac_of_unpacked_add_issue_rate": adds_per_s / (256 * 64 * 2.4e9),
+            # algorithmic adds per second over what the SIMDs can issue in plain v_add_f32 lane-operations
+            # (1024 SIMDs x 64 lanes x ~1.0e9 wave-instructions/s each, `--issue-rates`): > 1 because one executed
+            # add of a 3-mer table entry stands for three algorithmic adds
+            "algorithmic_adds_per_issuable_lane_op": adds_per_s / (1024 * 64 * 1.0e9),
             "hbm": {"algorithmic_bytes_per_launch": hbm_bytes, "achieved_GBs": hbm_bytes / (scan_ms * 1e-3) / 1e9,
                     "peak_GBs": HBM_PEAK_GBS, "frac": hbm_bytes / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         },
