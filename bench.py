@@ -82,9 +82,9 @@ def measured_traffic(workload):
 
 def train_throughput(steps=30, warmup=5):
     """Secondary figures: whole train steps (forward + backward + Nesterov update) per second on the
-    three training configurations, fused mode: each step issued natively by one library call per
-    architecture group (the top-level figures; "in_flight" = the groups' streams not joined between
-    steps) and as one captured HIP graph per step ("graphed"). sequences/s = batch rows * steps / wall time."""
+    three training configurations, fused mode: each step issued natively by one library call (the top-level
+    figures; the calibration batch's four architecture groups share every launch) and as one captured HIP
+    graph per step ("graphed"). sequences/s = batch rows * steps / wall time."""
     import torch
     from deepbind_amd import synth
     from deepbind_amd.model import ModelGroup, SequenceNet
@@ -119,8 +119,6 @@ def train_throughput(steps=30, warmup=5):
         net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
     X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
     out["config4_calibration_90_models"] = timed(lambda: grp.train_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
-    out["config4_calibration_90_models"]["in_flight"] = timed(lambda: grp.train_step(X, R, Y, M, join=False), len(cfg["R"]), spec.nmodel)
-    grp.join()
     out["config4_calibration_90_models"]["graphed"] = timed(grp.make_graphed_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
     return out
 

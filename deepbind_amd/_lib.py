@@ -77,6 +77,7 @@ _SIGNATURES = {
     "dbk_l1_decay": [_P, _I, _P, _P, _P, _Z],
     "dbk_head_fprop": [_P, _Z, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
     "dbk_train_step": [_P, _P],
+    "dbk_train_steps": [_P, _Z, _P],
     "dbk_train_step_args_size": [],
     "dbk_probe_valu_issue": [_I, _I, _I, _P],
 }

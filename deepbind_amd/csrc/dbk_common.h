@@ -34,6 +34,37 @@ struct deferred_sums {
 };
 deferred_sums*& deferred();
 
+// One launch per phase for several model groups that step on the same batch (dbk_train_steps): every group
+// keeps the grid, the kernel body and the partial-sum layout it has in a launch of its own, so the results are
+// the same bits; the launch just holds all the grids side by side.
+constexpr unsigned MULTI_MAX = 8;           // groups per launch
+struct scan_group {                         // the scan side of one group
+    const float *W, *bias;                  // look-ahead weights: (4m, F) and (F)
+    unsigned F;                             // filters of all the group's models
+    int ptype;
+    const uint8_t* X;                       // the batch, or the group's own copy after input dropout
+    float *pooled, *dpooled;
+    uint32_t* argmax;
+    unsigned long long* act;                // activity masks (null with max pooling)
+    // filled in by scan_bprop_multi: where the group's partial gradient sums lie
+    float* slabs; size_t slab_stride; unsigned nslab;
+};
+struct head_group {                         // the dense head of one group (arguments of dbk_head_train)
+    int nblock, k, hidden, loss_kind, revcomp;
+    const float *pooled, *rate;
+    uint64_t seed; uint64_t* counter;
+    const float *W1, *b1, *W2, *b2, *Y;
+    const uint8_t* Ymask;
+    float *Z, *dpooled;
+    // filled in by head_train_multi
+    float* partial; unsigned nchunk, pstride;
+};
+// true when every group's shape is one the multi-group launches take (else the groups are stepped one by one)
+bool scan_multi_takes(size_t m, size_t N, size_t P, unsigned n, const scan_group* g);
+int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size_t P, unsigned n, const scan_group* g);
+int scan_bprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size_t P, unsigned n, scan_group* g);
+int head_train_multi(hipStream_t st, size_t nrow, unsigned n, head_group* g);
+
 inline hipStream_t as_stream(dbk_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline unsigned divup(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }

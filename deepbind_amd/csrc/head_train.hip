@@ -36,12 +36,13 @@ struct head_args {
     unsigned nchunk, pstride;
 };
 
-__global__ __launch_bounds__(NT) void k_head_train(head_args a)
+// b: model of the group, chunk: which RB rows
+__device__ __forceinline__ void head_train_body(const head_args& a, const unsigned b, const unsigned chunk)
 {
     extern __shared__ float hs[];
     const int k = a.k, hidden = a.hidden, h1 = hidden > 0 ? hidden : 1;
-    const unsigned b = blockIdx.x, tid = threadIdx.x;
-    const size_t r0 = (size_t)blockIdx.y * RB;
+    const unsigned tid = threadIdx.x;
+    const size_t r0 = (size_t)chunk * RB;
     const int row = tid / NP, part = tid % NP;
     const size_t r = r0 + row;
     const bool live = r < a.n;
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
     }
 
     // ---------------- this chunk's share of the parameter gradients, rows ascending
-    float* part_out = a.partial + ((size_t)blockIdx.y * a.nblock + b) * a.pstride;
+    float* part_out = a.partial + ((size_t)chunk * a.nblock + b) * a.pstride;
     for (int pidx = tid; pidx < k * h1; pidx += NT) {
         const int kk = pidx / h1, h = pidx % h1;
         float s = 0.0f;
@@ -210,6 +211,24 @@ __global__ __launch_bounds__(NT) void k_head_train(head_args a)
     }
 }
 
+__global__ __launch_bounds__(NT) void k_head_train(head_args a) { head_train_body(a, blockIdx.x, blockIdx.y); }
+
+// The heads of several model groups in one launch: workgroups first[g] .. first[g+1]-1 are group g's grid of
+// (models, row chunks), models fastest.
+struct head_multi_args {
+    unsigned n;
+    unsigned first[dbk::MULTI_MAX + 1];
+    head_args g[dbk::MULTI_MAX];
+};
+__global__ __launch_bounds__(NT) void k_head_train_multi(const head_multi_args m)
+{
+    unsigned g = 0;
+    while (g + 1 < m.n && blockIdx.x >= m.first[g + 1]) ++g;
+    const head_args& a = m.g[g];
+    const unsigned local = blockIdx.x - m.first[g];
+    head_train_body(a, local % (unsigned)a.nblock, local / (unsigned)a.nblock);
+}
+
 // Adds the row chunks in ascending order and writes each gradient to its place.
 __global__ void k_head_reduce(head_args a)
 {
@@ -238,7 +257,51 @@ __global__ void k_head_reduce(head_args a)
     if (a.counter && a.counter_advance && blockIdx.x == 0 && threadIdx.x == 0) a.counter[0] += a.counter_advance;
 }
 
+inline size_t head_smem(int k, int h1)
+{
+    return ((size_t)k * h1 + 2 * h1 + (size_t)RB * (k | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
+}
+
 }  // namespace
+
+// The chunk sums are left in the stream's second scratch buffer, group after group, for the step's last kernel.
+int dbk::head_train_multi(hipStream_t st, size_t nrow, unsigned n, dbk::head_group* g)
+{
+    DBK_CHECK(n >= 1 && n <= dbk::MULTI_MAX && nrow >= 1, "ValueError: 1 to %u groups of at least one row", dbk::MULTI_MAX);
+    const size_t nchunk = (nrow + RB - 1) / RB;
+    head_multi_args m;
+    m.n = n;
+    m.first[0] = 0;
+    size_t smem = 0, total = 0;
+    for (unsigned i = 0; i < n; ++i) {
+        const int h1 = g[i].hidden > 0 ? g[i].hidden : 1;
+        DBK_CHECK(g[i].nblock >= 1 && g[i].k >= 1 && g[i].hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, hidden=%d)", g[i].nblock, g[i].k, g[i].hidden);
+        DBK_CHECK(!g[i].revcomp || nrow % 2 == 0, "ValueError: reverse-complement rows come in pairs, got %zu rows", nrow);
+        const size_t need = head_smem(g[i].k, h1);
+        DBK_CHECK(need <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", g[i].k, g[i].hidden, need);
+        smem = need > smem ? need : smem;
+        g[i].nchunk = (unsigned)nchunk;
+        g[i].pstride = (unsigned)(g[i].k * h1 + 2 * h1 + 2);
+        total += nchunk * (size_t)g[i].nblock * g[i].pstride;
+        m.first[i + 1] = m.first[i] + (unsigned)(g[i].nblock * nchunk);
+    }
+    float* partial = (float*)dbk::workspace(total * sizeof(float), st, 1);
+    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", total * sizeof(float));
+    for (unsigned i = 0; i < n; ++i) {
+        g[i].partial = partial;
+        partial += nchunk * (size_t)g[i].nblock * g[i].pstride;
+        head_args& a = m.g[i];
+        a.n = nrow; a.nblock = g[i].nblock; a.k = g[i].k; a.hidden = g[i].hidden; a.loss_kind = g[i].loss_kind; a.revcomp = g[i].revcomp;
+        a.pooled = g[i].pooled; a.rate = g[i].rate; a.U = nullptr; a.seed = g[i].seed; a.offset = 0;
+        a.counter = (unsigned long long*)g[i].counter; a.counter_advance = 0;
+        a.W1 = g[i].W1; a.b1 = g[i].b1; a.W2 = g[i].W2; a.b2 = g[i].b2; a.Y = g[i].Y; a.Ymask = g[i].Ymask;
+        a.Z = g[i].Z; a.dpooled = g[i].dpooled; a.dW1 = a.db1 = a.dW2 = a.db2 = a.loss = nullptr;
+        a.partial = g[i].partial; a.nchunk = g[i].nchunk; a.pstride = g[i].pstride;
+    }
+    DBK_HIP(hipFuncSetAttribute((const void*)k_head_train_multi, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(k_head_train_multi, dim3(m.first[n]), dim3(NT), smem, st, m);
+    DBK_LAUNCH_OK();
+}
 
 extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden, int loss_kind, int reverse_complement,
                               const float* pooled, const float* rate, const float* U, uint64_t seed, uint64_t offset,
@@ -254,7 +317,7 @@ extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, 
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(pooled && W1 && b1 && Y && Z && dpooled && dW1 && db1, "ValueError: null pointer argument");
     DBK_CHECK(hidden == 0 || (W2 && b2 && dW2 && db2), "ValueError: hidden layer requested but W2/b2/dW2/db2 are null");
-    const size_t smem = ((size_t)k * h1 + 2 * h1 + (size_t)RB * (k | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
+    const size_t smem = head_smem(k, h1);
     DBK_CHECK(smem <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", k, hidden, smem);
     const size_t nchunk = (n + RB - 1) / RB;
     DBK_CHECK(nchunk <= 65535, "ValueError: the fused head takes at most %d rows per call (got %zu)", 65535 * RB, n);

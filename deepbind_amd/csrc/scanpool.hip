@@ -24,6 +24,11 @@ using namespace dbk_scan;
 
 constexpr unsigned XCH_SUBS = 4;          // sub-chunks of PSUB positions per wave and staging round
 
+// A workgroup's place in its launch: (x, y) of a grid of gx by gy. The kernels of a training step take it as an
+// argument instead of reading blockIdx / gridDim, so that one launch can hold the grids of several model groups.
+struct wg_t { unsigned x, y, gx, gy; };
+__device__ __forceinline__ wg_t this_wg() { return wg_t{blockIdx.x, blockIdx.y, gridDim.x, gridDim.y}; }
+
 // Scans PSUB positions starting at chunk-relative p0 for this lane's filter.
 __device__ __forceinline__ void scan16(const float* __restrict__ lut, const uint8_t* __restrict__ xl, unsigned m,
                                        unsigned p0, unsigned lane, float acc[PSUB])
@@ -40,12 +45,12 @@ __device__ __forceinline__ void scan16(const float* __restrict__ lut, const uint
 
 // MT > 0: filters of at most MT taps, letters held in scalar registers (scan16_window); MT == 0: any length.
 template <int PT, bool WANT_ARGMAX, int MT>
-__global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __restrict__ W, const float* __restrict__ bias,
-                                                             unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
-                                                             const uint32_t* __restrict__ R, size_t P,
-                                                             float* __restrict__ pooled, uint32_t* __restrict__ argmax,
-                                                             const unsigned* __restrict__ run_if_flag,
-                                                             unsigned long long* __restrict__ act)
+__device__ __forceinline__ void scanpool_fprop_body(const wg_t wg, const float* __restrict__ W, const float* __restrict__ bias,
+                                                    unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                    const uint32_t* __restrict__ R, size_t P,
+                                                    float* __restrict__ pooled, uint32_t* __restrict__ argmax,
+                                                    const unsigned* __restrict__ run_if_flag,
+                                                    unsigned long long* __restrict__ act)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     // when given, the launch only does work if the device flag is set (fallback behind the k-mer kernel)
@@ -62,14 +67,14 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
     uint8_t* xl = reinterpret_cast<uint8_t*>(red + (size_t)nw * 3 * FT);
 
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
+    const unsigned f0 = wg.y * FT, f = f0 + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;    // rows the scan defines; later rows are relu(bias)
     grad_planes<PMT> planes;
     if constexpr (PLANES) weight_planes_load<PMT>(planes, W, m, F, f);
     else build_letter_table(lut, W, m, F, f0, MT);
     const float bf = f < F ? bias[f] : 0.0f;
 
-    for (size_t r = blockIdx.x; r < P; r += gridDim.x) {
+    for (size_t r = wg.x; r < P; r += wg.gx) {
         const size_t a = R[2 * r], b = R[2 * r + 1];
         float mx = -1.0f, sum = 0.0f;
         size_t xi = a;
@@ -104,7 +109,7 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
                         const unsigned long long open = __ballot(((i < n ? acc[p] : 0.0f) + bf) > 0.0f);
                         if (lane == (unsigned)p) mine = open;
                     }
-                    if (lane < (unsigned)PSUB && p0 + lane < rows) act[(c0 + p0 + lane) * gridDim.y + blockIdx.y] = mine;
+                    if (lane < (unsigned)PSUB && p0 + lane < rows) act[(c0 + p0 + lane) * wg.gy + wg.y] = mine;
                 }
 #pragma unroll
                 for (int p = 0; p < PSUB; ++p) {
@@ -143,6 +148,17 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
         }
         __syncthreads();                                         // red[] is reused by the next region
     }
+}
+
+template <int PT, bool WANT_ARGMAX, int MT>
+__global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __restrict__ W, const float* __restrict__ bias,
+                                                             unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                             const uint32_t* __restrict__ R, size_t P,
+                                                             float* __restrict__ pooled, uint32_t* __restrict__ argmax,
+                                                             const unsigned* __restrict__ run_if_flag,
+                                                             unsigned long long* __restrict__ act)
+{
+    scanpool_fprop_body<PT, WANT_ARGMAX, MT>(this_wg(), W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -301,23 +317,24 @@ __device__ __forceinline__ void add_positions4(float* mine, const uint8_t* __res
         }
     }
 }
+// One wave; in a launch of wider workgroups only the first wave of a workgroup may enter.
 template <int PT, int MT>
-__global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
-                                                                   size_t P, const float* __restrict__ pooled,
-                                                                   const uint32_t* __restrict__ argmax, const float* __restrict__ dpooled,
-                                                                   float* __restrict__ slabs, size_t stride)
+__device__ __forceinline__ void scanpool_bprop_sparse_body(const wg_t wg, unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                           size_t P, const float* __restrict__ pooled,
+                                                           const uint32_t* __restrict__ argmax, const float* __restrict__ dpooled,
+                                                           float* __restrict__ slabs, size_t stride)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     float* table = reinterpret_cast<float*>(smem);
     const unsigned lane = threadIdx.x;
-    const unsigned f = blockIdx.y * FT + lane;
+    const unsigned f = wg.y * FT + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
     float* mine = table + lane;                                   // a lane only ever touches its own column: no barriers needed
     for (unsigned row = 0; row < SPARSE_ROWS * m; ++row) mine[row * FT] = 0.0f;
     float db = 0.0f;
     if (f < F) {
-        const size_t gx = gridDim.x;
-        for (size_t r = blockIdx.x; r < P; r += 4 * gx) {
+        const size_t gx = wg.gx;
+        for (size_t r = wg.x; r < P; r += 4 * gx) {
             float g[4];
             size_t pos[4];
 #pragma unroll
@@ -341,7 +358,7 @@ __global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, u
             }
             add_positions4<MT>(mine, X, N, pos, g, on, m);
         }
-        float* out = slabs + (size_t)blockIdx.x * stride;
+        float* out = slabs + (size_t)wg.x * stride;
         for (unsigned j = 0; j < m; ++j) {
             const float* tap = mine + (size_t)j * SPARSE_ROWS * FT;
             const float q = 0.25f * tap[4 * FT];
@@ -353,6 +370,15 @@ __global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, u
         }
         out[(size_t)4 * m * F + f] = db;
     }
+}
+
+template <int PT, int MT>
+__global__ __launch_bounds__(64) void scanpool_bprop_sparse_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                   size_t P, const float* __restrict__ pooled,
+                                                                   const uint32_t* __restrict__ argmax, const float* __restrict__ dpooled,
+                                                                   float* __restrict__ slabs, size_t stride)
+{
+    scanpool_bprop_sparse_body<PT, MT>(this_wg(), m, F, X, N, P, pooled, argmax, dpooled, slabs, stride);
 }
 
 // Dense half of the backward pass (avg and max+avg pooling), filters of at most MT taps: every
@@ -473,12 +499,12 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
 // one window ahead), turns each into this lane's gradient value (davg/count or 0) and adds the window
 // into the register planes, one addition per (position, tap).
 template <int PT, int MT>
-__global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
-                                                                       const uint32_t* __restrict__ R, size_t P,
-                                                                       const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
-                                                                       const float* __restrict__ dpooled,
-                                                                       const unsigned long long* __restrict__ act,
-                                                                       float* __restrict__ slabs, size_t stride)
+__device__ __forceinline__ void scanpool_bprop_dense_act_body(const wg_t wg, unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                              const uint32_t* __restrict__ R, size_t P,
+                                                              const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
+                                                              const float* __restrict__ dpooled,
+                                                              const unsigned long long* __restrict__ act,
+                                                              float* __restrict__ slabs, size_t stride)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const unsigned nw = blockDim.x >> 6;
@@ -490,7 +516,7 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
     uint8_t* xbuf = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT);   // two letter buffers, used in turn
 
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
-    const unsigned f0 = blockIdx.y * FT, f = f0 + lane;
+    const unsigned f0 = wg.y * FT, f = f0 + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
     float db = 0.0f;
     grad_planes<MT> planes;
@@ -532,15 +558,15 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
 
     // activity masks of the 16 rows from p0 of a chunk (lane p takes row p's); rows past the chunk read as "closed"
     auto fetch = [&](size_t c_, unsigned rows_, unsigned p0) -> unsigned long long {
-        return (lane < (unsigned)PSUB && p0 + lane < rows_) ? act[(c_ + p0 + lane) * gridDim.y + blockIdx.y] : 0ull;
+        return (lane < (unsigned)PSUB && p0 + lane < rows_) ? act[(c_ + p0 + lane) * wg.gy + wg.y] : 0ull;
     };
-    size_t r = blockIdx.x;
+    size_t r = wg.x;
     bool valid = r < P;
     size_t a = 0, b = 0, c0 = 0, pa = 0, pb = 0;                   // (pa, pb): bounds of the region after this one
     unsigned long long mk_first = 0ull;                            // this wave's first masks of the current item
     if (valid) {
         a = R[2 * r]; b = R[2 * r + 1]; c0 = a;
-        if (r + gridDim.x < P) { pa = R[2 * (r + gridDim.x)]; pb = R[2 * (r + gridDim.x) + 1]; }
+        if (r + wg.gx < P) { pa = R[2 * (r + wg.gx)]; pb = R[2 * (r + wg.gx) + 1]; }
         mk_first = fetch(c0, rows_of(b, c0), wave * PSUB);
         enter_region(load_pooled(r), a, b);
         unsigned v0, v1;
@@ -554,7 +580,7 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
         // ---- the next item, and its loads
         size_t nr = r, na = a, nb = b, nc0 = c0 + chunk;
         const bool newregion = nc0 >= b;
-        if (newregion) { nr = r + gridDim.x; na = pa; nb = pb; nc0 = na; }
+        if (newregion) { nr = r + wg.gx; na = pa; nb = pb; nc0 = na; }
         const bool nvalid = nr < P;
         unsigned nv0 = 5u, nv1 = 5u;
         pooled_in nq = { 0.0f, 0.0f, 0.0f, 0u };
@@ -563,7 +589,7 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
             load_letters(nc0, rows_of(nb, nc0), nv0, nv1);
             if (newregion) {
                 nq = load_pooled(nr);
-                if (nr + gridDim.x < P) { qa = R[2 * (nr + gridDim.x)]; qb = R[2 * (nr + gridDim.x) + 1]; }
+                if (nr + wg.gx < P) { qa = R[2 * (nr + wg.gx)]; qb = R[2 * (nr + wg.gx) + 1]; }
             }
         }
         const unsigned long long mk_next = nvalid ? fetch(nc0, rows_of(nb, nc0), wave * PSUB) : 0ull;   // the next item's first masks
@@ -622,7 +648,7 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
         }
     }
     __syncthreads();
-    float* out = slabs + (size_t)blockIdx.x * stride;
+    float* out = slabs + (size_t)wg.x * stride;
     for (unsigned e = threadIdx.x; e < m * 4 * FT; e += blockDim.x) {
         const unsigned row = e / FT, fl = e % FT;
         if (f0 + fl < F) out[(size_t)row * F + f0 + fl] = lut[e];
@@ -633,6 +659,58 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
         out[(size_t)4 * m * F + f] = t;
     }
 }
+
+template <int PT, int MT>
+__global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                       const uint32_t* __restrict__ R, size_t P,
+                                                                       const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
+                                                                       const float* __restrict__ dpooled,
+                                                                       const unsigned long long* __restrict__ act,
+                                                                       float* __restrict__ slabs, size_t stride)
+{
+    scanpool_bprop_dense_act_body<PT, MT>(this_wg(), m, F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
+}
+
+// Launch shapes, shared by the single-group launchers and the multi-group ones.
+// forward: as many workgroups as are resident at once (three per CU; two with the register planes of 16 taps);
+// each sets up its filter tile's weights once and then walks its share of the regions
+inline unsigned fprop_grid_x(unsigned mt, unsigned ftiles, size_t P)
+{
+    unsigned gx = (mt == 16 ? 512u : 768u) / ftiles;
+    if (gx < 1) gx = 1;
+    if (gx > P) gx = (unsigned)P;
+    return gx;
+}
+inline size_t fprop_smem(unsigned mt, size_t m)
+{
+    const unsigned nw = 4;
+    const size_t taps = mt ? mt : m;
+    const bool planes = mt == 8 || mt == 16;                     // weights in registers: no table in LDS
+    return (planes ? 0 : taps * NL * FT * sizeof(float)) + nw * 3 * FT * sizeof(float) + ((nw * XCH_SUBS * PSUB + taps - 1 + 7) & ~(size_t)3);
+}
+// sparse half of the backward pass: ~2048 single-wave workgroups, at least four regions each (more regions per
+// workgroup only lengthens its chain of dependent loads)
+inline unsigned sparse_grid_x(unsigned ftiles, size_t P)
+{
+    unsigned gxs = 2048u / ftiles;
+    if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);
+    if (gxs < 1) gxs = 1;
+    return gxs;
+}
+// dense half: four-wave workgroups, as many as are resident at once (its register planes leave room for two per
+// CU, three with 8 taps). A minibatch (a handful of regions per workgroup) takes one workgroup per CU instead:
+// alone the kernel runs as fast (half as many partial sums to write and to reduce), and it leaves half of every
+// CU's registers to whatever else is running, such as the other architectures of a calibration batch.
+inline unsigned dense_grid_x(unsigned mt, unsigned ftiles, size_t P)
+{
+    unsigned gxd = (mt == 8 ? 768u : 512u) / ftiles;
+    if (P < 8 * (size_t)gxd) gxd = 256u / ftiles;
+    if (gxd < 1) gxd = 1;
+    if (gxd > P) gxd = (unsigned)P;
+    return gxd;
+}
+inline size_t sparse_smem(size_t m) { return m * SPARSE_ROWS * FT * sizeof(float); }
+inline size_t dense_smem(unsigned mt) { return ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3); }
 
 template <int PT, int MT>
 int launch_fprop_mt(hipStream_t st, unsigned gx, unsigned ftiles, unsigned nw, size_t smem, const float* W, const float* bias, size_t m,
@@ -656,19 +734,12 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
                     const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, const unsigned* run_if_flag, unsigned long long* act)
 {
     const unsigned nw = 4;
-    const unsigned chunk = nw * XCH_SUBS * PSUB;
     const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 24 ? 24 : (m <= 32 ? 32 : 0)));    // 0: any-length kernel
-    const size_t taps = mt ? mt : m;
-    const bool planes = mt == 8 || mt == 16;                     // weights in registers: no table in LDS
-    size_t smem = (planes ? 0 : taps * NL * FT * sizeof(float)) + nw * 3 * FT * sizeof(float) + ((chunk + taps - 1 + 7) & ~(size_t)3);
+    const size_t smem = fprop_smem(mt, m);
     DBK_CHECK(smem <= lds_limit(), "ValueError: filter length %zu needs %zu bytes of LDS (limit %zu)", m, smem, lds_limit());
     unsigned ftiles = dbk::divup(F, FT);
     DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
-    // as many workgroups as are resident at once (three per CU; two with the register planes of 16 taps); each
-    // sets up its filter tile's weights once and then walks its share of the regions
-    unsigned gx = (mt == 16 ? 512u : 768u) / ftiles;
-    if (gx < 1) gx = 1;
-    if (gx > P) gx = (unsigned)P;
+    const unsigned gx = fprop_grid_x(mt, ftiles, P);
     int rc = 0;
     switch (mt) {
     case 8:  rc = launch_fprop_mt<PT, 8>(st, gx, ftiles, nw, smem, W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act); break;
@@ -728,22 +799,10 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         else hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gx, overwrite);
         DBK_LAUNCH_OK();
     }
-    // sparse half: ~2048 single-wave workgroups, at least four regions each
-    unsigned gxs = 0, gxd = 0;
-    if (PT == DBK_PT_MAX) {                                       // with max+avg pooling the dense half carries the maxima along
-        gxs = 2048u / ftiles;
-        if (gxs > (P + 3) / 4) gxs = (unsigned)((P + 3) / 4);   // more regions per workgroup only lengthens its chain of dependent loads
-        if (gxs < 1) gxs = 1;
-    }
-    // dense half: four-wave workgroups, as many as are resident at once (its register planes leave room for
-    // two per CU, three with 8 taps)
-    if (PT != DBK_PT_MAX) {
-        gxd = (mt == 8 ? 768u : 512u) / ftiles;
-        if (gxd < 1) gxd = 1;
-        if (gxd > P) gxd = (unsigned)P;
-    }
-    const size_t smem_s = m * SPARSE_ROWS * FT * sizeof(float);
-    const size_t smem_d = ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3);
+    // with max+avg pooling the dense half carries the maxima along
+    const unsigned gxs = PT == DBK_PT_MAX ? sparse_grid_x(ftiles, P) : 0u;
+    const unsigned gxd = PT != DBK_PT_MAX ? dense_grid_x(mt, ftiles, P) : 0u;
+    const size_t smem_s = sparse_smem(m), smem_d = dense_smem(mt);
     DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
     float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float), st);
     DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * (gxs + gxd) * sizeof(float));
@@ -778,7 +837,140 @@ int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F,
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// several model groups in one launch
+// ---------------------------------------------------------------------------------------------
+// Workgroups first[g] .. first[g+1]-1 of the launch are group g's grid of gx[g] by ftiles[g], x fastest. The
+// argument block travels by value in the kernel-argument segment.
+struct multi_args {
+    unsigned n, m;
+    size_t N, P;
+    const uint32_t* R;
+    unsigned first[dbk::MULTI_MAX + 1], gx[dbk::MULTI_MAX], ftiles[dbk::MULTI_MAX];
+    dbk::scan_group g[dbk::MULTI_MAX];
+};
+
+__device__ __forceinline__ unsigned multi_locate(const multi_args& a, wg_t& wg)
+{
+    unsigned g = 0;
+    while (g + 1 < a.n && blockIdx.x >= a.first[g + 1]) ++g;
+    const unsigned local = blockIdx.x - a.first[g];
+    wg = wg_t{local % a.gx[g], local / a.gx[g], a.gx[g], a.ftiles[g]};
+    return g;
+}
+
+template <int MT>
+__global__ __launch_bounds__(256) void scanpool_fprop_multi_kernel(const multi_args a)
+{
+    wg_t wg;
+    const dbk::scan_group& j = a.g[multi_locate(a, wg)];
+    if (j.ptype == DBK_PT_MAX)
+        scanpool_fprop_body<DBK_PT_MAX, true, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr, nullptr);
+    else if (j.ptype == DBK_PT_ALL)
+        scanpool_fprop_body<DBK_PT_ALL, true, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr, j.act);
+    else
+        scanpool_fprop_body<DBK_PT_AVG, false, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, nullptr, nullptr, j.act);
+}
+
+// Max pooling: the one-wave sparse kernel in the first wave of the workgroup (the other waves leave at once);
+// otherwise the mask-driven dense kernel.
+template <int MT>
+__global__ __launch_bounds__(256) void scanpool_bprop_multi_kernel(const multi_args a)
+{
+    wg_t wg;
+    const dbk::scan_group& j = a.g[multi_locate(a, wg)];
+    if (j.ptype == DBK_PT_MAX) {
+        if (threadIdx.x < 64)
+            scanpool_bprop_sparse_body<DBK_PT_MAX, MT>(wg, a.m, j.F, j.X, a.N, a.P, j.pooled, j.argmax, j.dpooled, j.slabs, j.slab_stride);
+    } else if (j.ptype == DBK_PT_ALL) {
+        scanpool_bprop_dense_act_body<DBK_PT_ALL, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
+    } else {
+        scanpool_bprop_dense_act_body<DBK_PT_AVG, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
+    }
+}
+
+inline unsigned multi_tier(size_t m) { return m <= 8 ? 8u : (m <= 16 ? 16u : (m <= 24 ? 24u : 0u)); }
+
+template <typename K>
+int launch_multi(K kern, hipStream_t st, size_t smem, const multi_args& a)
+{
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3(a.first[a.n]), dim3(256), smem, st, a);
+    DBK_LAUNCH_OK();
+}
+
 }  // namespace dbk_scanpool_general
+
+namespace dbk_scanpool_kmer {
+bool takes(size_t m, size_t F, size_t N, size_t P);
+}
+
+namespace dbk {
+
+using namespace dbk_scanpool_general;
+
+bool scan_multi_takes(size_t m, size_t N, size_t P, unsigned n, const scan_group* g)
+{
+    if (n < 1 || n > MULTI_MAX || multi_tier(m) == 0 || P == 0 || N == 0) return false;
+    for (unsigned i = 0; i < n; ++i) {
+        if (g[i].F == 0 || dbk::divup(g[i].F, FT) > 65535u) return false;
+        if (g[i].ptype != DBK_PT_MAX && g[i].ptype != DBK_PT_AVG && g[i].ptype != DBK_PT_ALL) return false;
+        if (g[i].ptype != DBK_PT_MAX && !g[i].act) return false;      // the dense backward kernel here is the mask-driven one
+        if (g[i].ptype != DBK_PT_AVG && !g[i].argmax) return false;
+        // a max-pooling group on a batch large enough for the k-mer table goes there when stepped alone (other sums, other bits)
+        if (g[i].ptype == DBK_PT_MAX && dbk_scanpool_kmer::takes(m, g[i].F, N, P)) return false;
+    }
+    return fprop_smem(multi_tier(m), m) <= lds_limit() && sparse_smem(m) <= lds_limit() && dense_smem(multi_tier(m)) <= lds_limit();
+}
+
+int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size_t P, unsigned n, const scan_group* g)
+{
+    const unsigned mt = multi_tier(m);
+    multi_args a;
+    a.n = n; a.m = (unsigned)m; a.N = N; a.P = P; a.R = R;
+    a.first[0] = 0;
+    for (unsigned i = 0; i < n; ++i) {
+        a.g[i] = g[i];
+        a.ftiles[i] = dbk::divup(g[i].F, FT);
+        a.gx[i] = fprop_grid_x(mt, a.ftiles[i], P);
+        a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
+    }
+    const size_t smem = fprop_smem(mt, m);
+    if (mt == 8) return launch_multi(scanpool_fprop_multi_kernel<8>, st, smem, a);
+    if (mt == 16) return launch_multi(scanpool_fprop_multi_kernel<16>, st, smem, a);
+    return launch_multi(scanpool_fprop_multi_kernel<24>, st, smem, a);
+}
+
+int scan_bprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size_t P, unsigned n, scan_group* g)
+{
+    const unsigned mt = multi_tier(m);
+    multi_args a;
+    a.n = n; a.m = (unsigned)m; a.N = N; a.P = P; a.R = R;
+    a.first[0] = 0;
+    size_t total = 0;
+    for (unsigned i = 0; i < n; ++i) {
+        a.ftiles[i] = dbk::divup(g[i].F, FT);
+        a.gx[i] = g[i].ptype == DBK_PT_MAX ? sparse_grid_x(a.ftiles[i], P) : dense_grid_x(mt, a.ftiles[i], P);
+        a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
+        g[i].slab_stride = 4 * m * (size_t)g[i].F + g[i].F;
+        g[i].nslab = a.gx[i];
+        total += g[i].slab_stride * a.gx[i];
+    }
+    float* slabs = (float*)dbk::workspace(total * sizeof(float), st);
+    DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", total * sizeof(float));
+    for (unsigned i = 0; i < n; ++i) {
+        g[i].slabs = slabs;
+        slabs += g[i].slab_stride * a.gx[i];
+        a.g[i] = g[i];
+    }
+    const size_t ss = sparse_smem(m), sd = dense_smem(mt);
+    const size_t smem = ss > sd ? ss : sd;
+    if (mt == 8) return launch_multi(scanpool_bprop_multi_kernel<8>, st, smem, a);
+    if (mt == 16) return launch_multi(scanpool_bprop_multi_kernel<16>, st, smem, a);
+    return launch_multi(scanpool_bprop_multi_kernel<24>, st, smem, a);
+}
+
+}  // namespace dbk
 
 namespace dbk_scanpool_kmer {
 // Fast path (k-mer lookup table); returns -1 when the shape is outside what it handles.

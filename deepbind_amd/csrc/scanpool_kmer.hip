@@ -394,6 +394,14 @@ int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F
 #undef DBK_GO
 }
 
+// Whether a call of this size goes to the table kernel when the choice is left to the library: a filter tile's
+// table costs ~0.1 M position-equivalents to build, which only bulk work repays.
+bool takes(size_t m, size_t F, size_t N, size_t P)
+{
+    if (m > 24 || N == 0 || N > 0x7fffff00u || P > 0x7fff0000u) return false;
+    return (double)N * dbk::divup(F, FTILE) >= 2.0e6;
+}
+
 // force: take the fast path whenever the shape allows, regardless of problem size
 int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, bool force)
@@ -401,8 +409,7 @@ int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size
     if (ptype != DBK_PT_MAX && ptype != DBK_PT_AVG && ptype != DBK_PT_ALL) return -1;
     if (ptype == DBK_PT_AVG && argmax != nullptr) return -1;
     if (m > 24 || N == 0 || N > 0x7fffff00u || P > 0x7fff0000u) return -1;
-    // a filter tile's table costs ~0.1 M position-equivalents to build: only worth it for bulk work
-    if (!force && (double)N * dbk::divup(F, FTILE) < 2.0e6) return -1;
+    if (!force && !takes(m, F, N, P)) return -1;
     const size_t kbytes = (N + KPAD + 255) & ~(size_t)255;
     unsigned char* ws = (unsigned char*)dbk::workspace(256 + kbytes, st);
     if (!ws) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", 256 + kbytes); return 1; }

@@ -58,11 +58,12 @@ __device__ __forceinline__ float chunk_sum(const reduce_update_args& a, unsigned
     return s;
 }
 
-__global__ __launch_bounds__(256) void k_reduce_update(reduce_update_args a)
+// bx of gx: this workgroup's place among those that share the vector
+__device__ __forceinline__ void reduce_update_body(const reduce_update_args& a, const unsigned bx, const unsigned gx)
 {
     const unsigned nW1m = a.k * a.h1;                              // dense weights per model
     const size_t total = a.nparam + (a.loss ? a.nblock : 0);
-    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+    for (size_t e = (size_t)bx * blockDim.x + threadIdx.x; e < total; e += (size_t)gx * blockDim.x) {
         if (e >= a.nparam) {                                       // per-model loss
             const unsigned b = (unsigned)(e - a.nparam);
             const float s = chunk_sum(a, b, nW1m + 2 * a.h1 + 1);
@@ -93,7 +94,38 @@ __global__ __launch_bounds__(256) void k_reduce_update(reduce_update_args a)
         a.L[e] = pn + rm * mom;
     }
     // every workgroup of the head kernel has read the generator position long ago: move it on
-    if (a.counter && a.counter_advance && blockIdx.x == 0 && threadIdx.x == 0) a.counter[0] += a.counter_advance;
+    if (a.counter && a.counter_advance && bx == 0 && threadIdx.x == 0) a.counter[0] += a.counter_advance;
+}
+
+__global__ __launch_bounds__(256) void k_reduce_update(reduce_update_args a) { reduce_update_body(a, blockIdx.x, gridDim.x); }
+
+// The same for several model groups in one launch: workgroups first[g] .. first[g+1]-1 share group g's vector.
+struct reduce_update_multi_args {
+    unsigned n;
+    unsigned first[dbk::MULTI_MAX + 1];
+    reduce_update_args g[dbk::MULTI_MAX];
+};
+__global__ __launch_bounds__(256) void k_reduce_update_multi(const reduce_update_multi_args m)
+{
+    unsigned g = 0;
+    while (g + 1 < m.n && blockIdx.x >= m.first[g + 1]) ++g;
+    reduce_update_body(m.g[g], blockIdx.x - m.first[g], m.first[g + 1] - m.first[g]);
+}
+
+// Look-ahead vectors of several groups in one launch (L = P + mrate*mP, as k_lookahead forms it).
+struct lookahead_multi_args {
+    unsigned n;
+    unsigned first[dbk::MULTI_MAX + 1];
+    struct { size_t nparam; float* L; const float *P, *mP, *mrate; } g[dbk::MULTI_MAX];
+};
+__global__ __launch_bounds__(256) void k_lookahead_multi(const lookahead_multi_args m)
+{
+    unsigned g = 0;
+    while (g + 1 < m.n && blockIdx.x >= m.first[g + 1]) ++g;
+    const auto& a = m.g[g];
+    const size_t gx = m.first[g + 1] - m.first[g];
+    for (size_t e = (size_t)(blockIdx.x - m.first[g]) * blockDim.x + threadIdx.x; e < a.nparam; e += gx * blockDim.x)
+        a.L[e] = a.P[e] + a.mrate[e] * a.mP[e];
 }
 
 __global__ void k_zero_f32(float* p, size_t n)
@@ -103,7 +135,24 @@ __global__ void k_zero_f32(float* p, size_t n)
 
 }  // namespace
 
-extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
+namespace {
+
+// Sizes of a group's parameter blocks.
+struct block_sizes { size_t F, k, nWc, nW1, nb1, nW2, nb2; };
+block_sizes sizes_of(const dbk_train_step_args* a)
+{
+    block_sizes z;
+    z.F = a->nmodel * a->nfilter;                                  // filters of all models, side by side
+    z.k = a->nfilter * (a->ptype == DBK_PT_ALL ? 2 : 1);           // pooled features per model
+    z.nWc = 4 * a->m * z.F;
+    z.nW1 = z.k * a->nmodel * (a->hidden ? a->hidden : 1);
+    z.nb1 = a->nmodel * (a->hidden ? a->hidden : 1);
+    z.nW2 = a->hidden ? a->hidden * a->nmodel : 0;
+    z.nb2 = a->hidden ? a->nmodel : 0;
+    return z;
+}
+
+int check_args(const dbk_train_step_args* a)
 {
     DBK_CHECK(a != nullptr, "ValueError: null argument block");
     DBK_CHECK(a->nmodel >= 1 && a->nfilter >= 1 && a->m >= 1, "ValueError: nmodel, nfilter and m must be >= 1");
@@ -114,21 +163,60 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
     DBK_CHECK(a->ptype == DBK_PT_AVG || a->argmax, "ValueError: max / all pooling needs the argmax work buffer");
     DBK_CHECK(a->input_rate <= 0.0f || (a->Xdrop && a->Mdrop), "ValueError: input dropout needs the Xdrop and Mdrop work buffers");
     DBK_CHECK(!(a->rate || a->input_rate > 0.0f) || a->counter, "ValueError: dropout needs the device generator position");
-    const size_t F = a->nmodel * a->nfilter;                       // filters of all models, side by side
-    const size_t k = a->nfilter * (a->ptype == DBK_PT_ALL ? 2 : 1); // pooled features per model
-    const size_t nWc = 4 * a->m * F;
-    const size_t nW1 = k * a->nmodel * (a->hidden ? a->hidden : 1), nb1 = a->nmodel * (a->hidden ? a->hidden : 1);
-    const size_t nW2 = a->hidden ? a->hidden * a->nmodel : 0, nb2 = a->hidden ? a->nmodel : 0;
-    const size_t need[6] = { a->off_Wc + nWc, a->off_bc + F, a->off_W1 + nW1, a->off_b1 + nb1,
-                             a->off_W2 + nW2, a->off_b2 + nb2 };
+    const block_sizes z = sizes_of(a);
+    const size_t need[6] = { a->off_Wc + z.nWc, a->off_bc + z.F, a->off_W1 + z.nW1, a->off_b1 + z.nb1,
+                             a->off_W2 + z.nW2, a->off_b2 + z.nb2 };
     for (size_t v : need) DBK_CHECK(v <= a->nparam, "ValueError: a parameter block reaches past the flat vector (%zu > %zu)", v, a->nparam);
+    return 0;
+}
+
+// Input dropout of one group (dropoutord.py:50-70): Xdrop = X with dropped letters, mirrored within (fwd, rev) pairs.
+int drop_inputs(dbk_stream_t stream, const dbk_train_step_args* a)
+{
+    int rc = dbk_dropoutord_fp_tr(stream, a->X, a->Xdrop, a->Mdrop, a->N, a->input_rate, a->seed, 0, a->counter);
+    if (rc) return rc;
+    if (a->reverse_complement) {
+        rc = dbk_dropoutord_mirror(stream, a->X, a->Xdrop, a->Mdrop, a->regions, a->nregion, a->m - 1);
+        if (rc) return rc;
+    }
+    return dbk_counter_add(stream, a->counter, (a->N + 3) / 4);
+}
+
+// Arguments of the step's last kernel for one group, given where its partial sums lie.
+int fill_update(reduce_update_args& u, const dbk_train_step_args* a, const block_sizes& z, const float* slabs, size_t slab_stride,
+                unsigned nslab, const float* head_partial, unsigned nchunk, unsigned pstride, uint64_t draws)
+{
+    u.nparam = a->nparam;
+    u.P = a->P; u.L = a->L; u.dP = a->dP; u.mP = a->mP; u.drate = a->drate; u.mrate = a->mrate; u.decay = a->decay;
+    u.off_Wc = a->off_Wc; u.off_bc = a->off_bc; u.off_W1 = a->off_W1; u.off_b1 = a->off_b1;
+    u.off_W2 = a->hidden ? a->off_W2 : a->nparam; u.off_b2 = a->hidden ? a->off_b2 : a->nparam;
+    u.nWc = z.nWc; u.nbc = z.F; u.nW1 = z.nW1; u.nb1 = z.nb1; u.nW2 = z.nW2; u.nb2 = z.nb2;
+    u.slabs = slabs; u.slab_stride = slab_stride; u.nslab = nslab;
+    u.head_partial = head_partial; u.nchunk = nchunk; u.pstride = pstride;
+    u.nblock = (unsigned)a->nmodel; u.k = (unsigned)z.k; u.h1 = (unsigned)(a->hidden ? a->hidden : 1); u.hidden = (unsigned)a->hidden;
+    u.freeze_scan = a->freeze_scan; u.loss_kind = a->loss_kind; u.loss = a->loss; u.nrow = a->nregion;
+    u.counter = (unsigned long long*)a->counter; u.counter_advance = draws;
+    DBK_CHECK(z.nWc + z.F + z.nW1 + z.nb1 + z.nW2 + z.nb2 == a->nparam, "ValueError: the parameter blocks do not tile the flat vector (%zu of %zu elements)",
+              z.nWc + z.F + z.nW1 + z.nb1 + z.nW2 + z.nb2, a->nparam);
+    DBK_CHECK((head_partial != nullptr || a->nregion == 0) && slab_stride == z.nWc + z.F,
+              "RuntimeError: the backward kernels left no partial sums");
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
+{
+    int rc = check_args(a);
+    if (rc) return rc;
+    const block_sizes z = sizes_of(a);
+    const size_t F = z.F, k = z.k, nWc = z.nWc;
 
     // Nesterov with a look-ahead vector: the step's weights are read from L = P + mrate*mP, which the previous
     // step left there (L_ready) or which is formed now; otherwise the look-ahead is applied to P in place.
     const bool beside = a->nesterov && a->L != nullptr;
     float* const P = beside ? a->L : a->P;                         // where this step's weights are read
     float* const dP = a->dP;
-    int rc;
     if (beside) {
         if (!a->L_ready) {
             rc = dbk_gradstep_lookahead(stream, DBK_F32, a->nparam, a->L, a->P, a->mP, a->mrate);
@@ -140,13 +228,7 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
     }
     const uint8_t* X = a->X;
     if (a->input_rate > 0.0f) {
-        rc = dbk_dropoutord_fp_tr(stream, a->X, a->Xdrop, a->Mdrop, a->N, a->input_rate, a->seed, 0, a->counter);
-        if (rc) return rc;
-        if (a->reverse_complement) {
-            rc = dbk_dropoutord_mirror(stream, a->X, a->Xdrop, a->Mdrop, a->regions, a->nregion, a->m - 1);
-            if (rc) return rc;
-        }
-        rc = dbk_counter_add(stream, a->counter, (a->N + 3) / 4);
+        rc = drop_inputs(stream, a);
         if (rc) return rc;
         X = a->Xdrop;
     }
@@ -172,20 +254,8 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
     if (beside) {
         dbk::deferred() = nullptr;
         reduce_update_args u;
-        u.nparam = a->nparam;
-        u.P = a->P; u.L = a->L; u.dP = dP; u.mP = a->mP; u.drate = a->drate; u.mrate = a->mrate; u.decay = a->decay;
-        u.off_Wc = a->off_Wc; u.off_bc = a->off_bc; u.off_W1 = a->off_W1; u.off_b1 = a->off_b1;
-        u.off_W2 = a->hidden ? a->off_W2 : a->nparam; u.off_b2 = a->hidden ? a->off_b2 : a->nparam;
-        u.nWc = nWc; u.nbc = F; u.nW1 = nW1; u.nb1 = nb1; u.nW2 = nW2; u.nb2 = nb2;
-        u.slabs = later.slabs; u.slab_stride = later.slab_stride; u.nslab = later.nslab;
-        u.head_partial = later.head_partial; u.nchunk = later.head_nchunk; u.pstride = later.head_pstride;
-        u.nblock = (unsigned)a->nmodel; u.k = (unsigned)k; u.h1 = (unsigned)(a->hidden ? a->hidden : 1); u.hidden = (unsigned)a->hidden;
-        u.freeze_scan = a->freeze_scan; u.loss_kind = a->loss_kind; u.loss = a->loss; u.nrow = a->nregion;
-        u.counter = (unsigned long long*)a->counter; u.counter_advance = draws;
-        DBK_CHECK(nWc + F + nW1 + nb1 + nW2 + nb2 == a->nparam, "ValueError: the parameter blocks do not tile the flat vector (%zu of %zu elements)",
-                  nWc + F + nW1 + nb1 + nW2 + nb2, a->nparam);
-        DBK_CHECK((later.head_partial != nullptr || a->nregion == 0) && later.slab_stride == nWc + F,
-                  "RuntimeError: the backward kernels left no partial sums");
+        rc = fill_update(u, a, z, later.slabs, later.slab_stride, later.nslab, later.head_partial, later.head_nchunk, later.head_pstride, draws);
+        if (rc) return rc;
         hipLaunchKernelGGL(k_reduce_update, dim3(dbk::ew_grid(a->nparam + a->nmodel)), dim3(256), 0, dbk::as_stream(stream), u);
         DBK_LAUNCH_OK();
     }
@@ -197,6 +267,106 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
     if (a->nesterov) rc = dbk_gradstep_nesterov2(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
     else rc = dbk_gradstep(stream, DBK_F32, a->nparam, P, dP, a->drate, a->mP, a->mrate);
     return rc;
+}
+
+// One step of each of several groups that train on the same batch: every phase of the step is ONE launch holding
+// all the groups' grids, so groups too small to fill the GPU run side by side on one stream. A group's kernels,
+// grids and summation orders are those of its own dbk_train_step, hence the same bits. Taken for up to 8 groups
+// with a look-ahead vector each (Nesterov), filters of at most 24 taps and one shared region table; any other
+// call steps the groups one after the other.
+extern "C" int dbk_train_steps(dbk_stream_t stream, size_t ngroup, const dbk_train_step_args* const* args)
+{
+    DBK_CHECK(ngroup == 0 || args != nullptr, "ValueError: null argument list");
+    for (size_t i = 0; i < ngroup; ++i) {
+        int rc = check_args(args[i]);
+        if (rc) return rc;
+    }
+    if (ngroup == 0) { dbk::clear_error(); return 0; }
+    bool together = ngroup >= 2 && ngroup <= dbk::MULTI_MAX;
+    const dbk_train_step_args* a0 = args[0];
+    for (size_t i = 0; i < ngroup && together; ++i) {
+        const dbk_train_step_args* a = args[i];
+        together = a->nesterov && a->L && a->m == a0->m && a->N == a0->N && a->regions == a0->regions && a->nregion == a0->nregion &&
+                   a->nregion > 0;
+    }
+    // dense (avg / max+avg) groups first: their workgroups run longest
+    const dbk_train_step_args* ord[dbk::MULTI_MAX];
+    dbk::scan_group sg[dbk::MULTI_MAX];
+    if (together) {
+        unsigned n = 0;
+        for (int pass = 0; pass < 2; ++pass)
+            for (size_t i = 0; i < ngroup; ++i)
+                if ((args[i]->ptype == DBK_PT_MAX) == (pass == 1)) ord[n++] = args[i];
+        for (unsigned i = 0; i < n; ++i) {
+            const dbk_train_step_args* a = ord[i];
+            const block_sizes z = sizes_of(a);
+            sg[i].W = a->L + a->off_Wc; sg[i].bias = a->L + a->off_bc;
+            sg[i].F = (unsigned)z.F; sg[i].ptype = a->ptype;
+            sg[i].X = a->input_rate > 0.0f ? a->Xdrop : a->X;
+            sg[i].pooled = a->pooled; sg[i].dpooled = a->dpooled; sg[i].argmax = a->argmax;
+            sg[i].act = a->ptype == DBK_PT_MAX ? nullptr : reinterpret_cast<unsigned long long*>(a->act);
+            sg[i].slabs = nullptr; sg[i].slab_stride = 0; sg[i].nslab = 0;
+        }
+        together = dbk::scan_multi_takes(a0->m, a0->N, a0->nregion, n, sg);
+    }
+    if (!together) {
+        for (size_t i = 0; i < ngroup; ++i) {
+            int rc = dbk_train_step(stream, args[i]);
+            if (rc) return rc;
+        }
+        return 0;
+    }
+    const unsigned n = (unsigned)ngroup;
+    hipStream_t st = dbk::as_stream(stream);
+    int rc;
+    // look-ahead vectors that the previous step did not leave
+    {
+        lookahead_multi_args la;
+        la.n = 0; la.first[0] = 0;
+        for (unsigned i = 0; i < n; ++i)
+            if (!ord[i]->L_ready) {
+                la.g[la.n] = { ord[i]->nparam, ord[i]->L, ord[i]->P, ord[i]->mP, ord[i]->mrate };
+                la.first[la.n + 1] = la.first[la.n] + dbk::ew_grid(ord[i]->nparam);
+                ++la.n;
+            }
+        if (la.n) hipLaunchKernelGGL(k_lookahead_multi, dim3(la.first[la.n]), dim3(256), 0, st, la);
+    }
+    for (unsigned i = 0; i < n; ++i)
+        if (ord[i]->input_rate > 0.0f) {
+            rc = drop_inputs(stream, ord[i]);
+            if (rc) return rc;
+        }
+    rc = dbk::scan_fprop_multi(st, a0->m, a0->N, a0->regions, a0->nregion, n, sg);
+    if (rc) return rc;
+    dbk::head_group hg[dbk::MULTI_MAX];
+    uint64_t draws[dbk::MULTI_MAX];
+    for (unsigned i = 0; i < n; ++i) {
+        const dbk_train_step_args* a = ord[i];
+        const block_sizes z = sizes_of(a);
+        const float* P = a->L;
+        draws[i] = a->rate ? (a->nregion * z.k * a->nmodel + 3) / 4 : 0;
+        hg[i].nblock = (int)a->nmodel; hg[i].k = (int)z.k; hg[i].hidden = (int)a->hidden; hg[i].loss_kind = a->loss_kind;
+        hg[i].revcomp = a->reverse_complement;
+        hg[i].pooled = a->pooled; hg[i].rate = a->rate; hg[i].seed = a->seed; hg[i].counter = a->counter;
+        hg[i].W1 = P + a->off_W1; hg[i].b1 = P + a->off_b1;
+        hg[i].W2 = a->hidden ? P + a->off_W2 : nullptr; hg[i].b2 = a->hidden ? P + a->off_b2 : nullptr;
+        hg[i].Y = a->Y; hg[i].Ymask = a->Ymask; hg[i].Z = a->Z; hg[i].dpooled = a->dpooled;
+        hg[i].partial = nullptr; hg[i].nchunk = 0; hg[i].pstride = 0;
+    }
+    rc = dbk::head_train_multi(st, a0->nregion, n, hg);
+    if (rc) return rc;
+    rc = dbk::scan_bprop_multi(st, a0->m, a0->N, a0->regions, a0->nregion, n, sg);
+    if (rc) return rc;
+    reduce_update_multi_args um;
+    um.n = n; um.first[0] = 0;
+    for (unsigned i = 0; i < n; ++i) {
+        const dbk_train_step_args* a = ord[i];
+        rc = fill_update(um.g[i], a, sizes_of(a), sg[i].slabs, sg[i].slab_stride, sg[i].nslab, hg[i].partial, hg[i].nchunk, hg[i].pstride, draws[i]);
+        if (rc) return rc;
+        um.first[i + 1] = um.first[i] + dbk::ew_grid(a->nparam + a->nmodel);
+    }
+    hipLaunchKernelGGL(k_reduce_update_multi, dim3(um.first[n]), dim3(256), 0, st, um);
+    DBK_LAUNCH_OK();
 }
 
 extern "C" int dbk_train_step_args_size(void) { return (int)sizeof(dbk_train_step_args); }

@@ -59,7 +59,6 @@ class SequenceNet(object):
         # Nesterov look-ahead kept beside the parameters by the natively issued step (each step's update kernel
         # leaves the next step's look-ahead there); valid while nothing else has touched P, mP or mrate
         self._L, self._L_versions = None, None
-        self._busy_stream = None             # side stream a ModelGroup left this net's last step on
         ni, nf = self.ninst, self.nfilter
         self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
         h = self.hidden
@@ -105,7 +104,6 @@ class SequenceNet(object):
 
     def set_rates(self, rate, momentum):
         """Per-model learning and momentum rates spread over the flat vectors."""
-        self.join()
         self.drate.zero_()
         self.mrate.zero_()
         ones = torch.ones_like(self.P)
@@ -115,7 +113,6 @@ class SequenceNet(object):
 
     def set_params(self, params):
         """Copies a dict of NumPy arrays shaped like the layout into the flat parameter vector."""
-        self.join()
         for name, shape, _ in self.layout:
             src = np.asarray(params[name])
             assert tuple(src.shape) == tuple(shape), "%s: expected %s, got %s" % (name, shape, src.shape)
@@ -126,7 +123,6 @@ class SequenceNet(object):
         weights = randn * init (one scale per model, spread with madd_bcast), biases = init_mu.
         init_conv / init_full / init_mu: scalar or one value per model. The normal deviates come from
         the library's generator, so equal seeds give equal parameters."""
-        self.join()
         self.P.zero_()
         offset = 0
         for name, shape, axis in self.layout:
@@ -148,7 +144,6 @@ class SequenceNet(object):
         ni = self.ninst
         if self.weight_decay_start > self.step_count:
             return np.zeros((1, ni))
-        self.join()
         p = self.p
         conv = sm.sum_axis0(sm.mul_sign(p["Wc"], p["Wc"]))                     # |W| summed over taps and channels
         torch.cuda.synchronize()
@@ -163,12 +158,10 @@ class SequenceNet(object):
         return cost.reshape(1, ni)
 
     def get_params(self):
-        self.join()
         torch.cuda.synchronize()
         return {name: self.p[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
     def get_grads(self):
-        self.join()
         torch.cuda.synchronize()
         return {name: self.g[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
@@ -249,7 +242,6 @@ class SequenceNet(object):
     def forward(self, X, R, train=False, U=None, want_argmax=False):
         """Returns the state dict of one forward pass; st["Z"] are the predictions (n x ninst)."""
         p, ni = self.p, self.ninst
-        self.join()
         st = {}
         st["pooled"], st["argmax"], st["A0"] = self._conv_forward(X, R, want_argmax, train=train)
         H0 = st["pooled"]
@@ -280,7 +272,6 @@ class SequenceNet(object):
     def predict(self, X, R):
         """Test-mode predictions through the fused scoring head (dropout rescale folded in)."""
         p = self.p
-        self.join()
         pooled, _, _ = self._conv_forward(X, R, False)
         if self.dtype != torch.float32:
             Z = self.forward(X, R)["Z"]
@@ -299,7 +290,6 @@ class SequenceNet(object):
         (reference: deepity/deepity/node.py:298-341, kangaroo/kangaroo/predict.py:168-193,
         kangaroo/_ext/corr1ord.py:129-133, deepity/std/elemwise.py:148-157)"""
         p, ni = self.p, self.ninst
-        self.join()
         Z0 = sm.zeros((X.numel(), p["Wc"].shape[1]), dtype=self.dtype, device=self.device)
         ks.corr1ord(p["Wc"], X, Z0, 4)
         if self.input_dropout > 0:
@@ -348,7 +338,6 @@ class SequenceNet(object):
     def backward(self, X, R, st, Y, Ymask=None):
         """Fills dP with the gradient of the summed per-model losses (plus L1 decay when active)."""
         p, g, ni = self.p, self.g, self.ninst
-        self.join()
         dA = sm.sub_scale(st["Z"], Y, 1.0 / st["Z"].shape[0])
         if Ymask is not None:
             ds.maskout(Ymask, dA)
@@ -422,17 +411,9 @@ class SequenceNet(object):
         return Z
 
     # ------------------------------------------------------------------ one optimiser step
-    def join(self):
-        """Orders the current stream after this net's last step when a ModelGroup issued it on a side stream."""
-        if self._busy_stream is not None:
-            torch.cuda.current_stream().wait_stream(self._busy_stream)
-            self._busy_stream = None
-
-    def _native_step(self, X, R, Y, Ymask=None, stream=None):
-        """One fused step through dbk_train_step: one library call issues every launch of the step (the
-        scripting host otherwise pays several microseconds per launch, which is what bounds a step on a
-        small minibatch). Same kernels in the same order as gradstep(..., _grad_fused), so the same bits.
-        stream: torch stream to issue on (default: the current one)."""
+    def _prepare_step(self, X, R, Y, Ymask=None):
+        """Fills this net's dbk_train_step_args block for one step on the batch and returns the step's work
+        buffers (made on the current stream, where the step is issued)."""
         ks._u8(X)
         ks._regions(R)
         ni, P = self.ninst, R.shape[0]
@@ -459,15 +440,14 @@ class SequenceNet(object):
             if len(self._step_bufs) >= 4:
                 self._step_bufs.clear()
             dev = self.P.device
-            with torch.cuda.stream(stream if stream is not None else torch.cuda.current_stream()):   # owned by the issuing stream
-                buf = self._step_bufs[key] = dict(
-                    pooled=torch.empty((P, self.k * ni), dtype=torch.float32, device=dev),
-                    dpooled=torch.empty((P, self.k * ni), dtype=torch.float32, device=dev),
-                    argmax=torch.empty((P, self.nfilter * ni), dtype=ks.uindex, device=dev) if self.pool != "avg" else None,
-                    Z=torch.empty((P, ni), dtype=torch.float32, device=dev),
-                    act=ks.activity_words(X, self.p["Wc"]) if self.pool != "max" else None,
-                    Xdrop=torch.empty(X.numel(), dtype=torch.uint8, device=dev) if self.input_dropout > 0 else None,
-                    Mdrop=torch.empty(X.numel(), dtype=torch.bool, device=dev) if self.input_dropout > 0 else None)
+            buf = self._step_bufs[key] = dict(
+                pooled=torch.empty((P, self.k * ni), dtype=torch.float32, device=dev),
+                dpooled=torch.empty((P, self.k * ni), dtype=torch.float32, device=dev),
+                argmax=torch.empty((P, self.nfilter * ni), dtype=ks.uindex, device=dev) if self.pool != "avg" else None,
+                Z=torch.empty((P, ni), dtype=torch.float32, device=dev),
+                act=ks.activity_words(X, self.p["Wc"]) if self.pool != "max" else None,
+                Xdrop=torch.empty(X.numel(), dtype=torch.uint8, device=dev) if self.input_dropout > 0 else None,
+                Mdrop=torch.empty(X.numel(), dtype=torch.bool, device=dev) if self.input_dropout > 0 else None)
         a.nesterov, a.seed = int(bool(self.nesterov)), int(self.rng_seed)
         if self.nesterov:
             if self._L is None:
@@ -489,13 +469,23 @@ class SequenceNet(object):
         a.decay = self.decay_vec.data_ptr() if self.weight_decay_start <= self.step_count else None
         a.freeze_scan = int(self.step_count < self.start_training)
         a.loss = None
-        handle = _lib.stream() if stream is None else ctypes.c_void_p(stream.cuda_stream)
-        _lib.call("dbk_train_step", handle, ctypes.addressof(a))
+        return buf
+
+    def _finish_step(self, X, R):
+        """Host-side mirrors of what a natively issued step moved on the device."""
         if self.input_dropout > 0:
             self._rng_offset += (X.numel() + 3) // 4
         if self.use_dropout:
-            self._rng_offset += (P * self.k * ni + 3) // 4
+            self._rng_offset += (R.shape[0] * self.k * self.ninst + 3) // 4
         self.step_count += 1
+
+    def _native_step(self, X, R, Y, Ymask=None):
+        """One fused step through dbk_train_step: one library call issues every launch of the step (the
+        scripting host otherwise pays several microseconds per launch, which is what bounds a step on a
+        small minibatch). Same kernels in the same order as gradstep(..., _grad_fused), so the same bits."""
+        buf = self._prepare_step(X, R, Y, Ymask)
+        _lib.call("dbk_train_step", _lib.stream(), ctypes.addressof(self._step_args))
+        self._finish_step(X, R)
         return buf["Z"]
 
     def make_graphed_step(self, X, R, Y, Ymask=None):
@@ -511,7 +501,6 @@ class SequenceNet(object):
         """One optimiser step. U / U_input optionally supply the uniforms of the pooled-feature and the
         input dropout (otherwise the library's generator draws them)."""
         fused = self.mode == "fused" and self.dtype == torch.float32 and self.loss is not None
-        self.join()
         if fused and U is None and U_input is None:
             self._native_step(X, R, Y, Ymask)
             return
@@ -529,6 +518,21 @@ class SequenceNet(object):
         self.step_count += 1
 
 
+def _native_steps(jobs):
+    """jobs: list of (net, X, R, Y, Ymask), nets that step on the same batch. One dbk_train_steps call per eight
+    nets on the current stream: every phase of the step is one launch holding all the nets' grids, so nets too
+    small to fill the GPU run side by side without extra streams. Each net gets the bits of its own step."""
+    for i in range(0, len(jobs), 8):
+        chunk = jobs[i:i + 8]
+        blocks = (ctypes.c_void_p * len(chunk))()
+        for j, (net, X, R, Y, Ymask) in enumerate(chunk):
+            net._prepare_step(X, R, Y, Ymask)
+            blocks[j] = ctypes.addressof(net._step_args)
+        _lib.call("dbk_train_steps", _lib.stream(), len(chunk), blocks)
+        for net, X, R, _, _ in chunk:
+            net._finish_step(X, R)
+
+
 def _side_by_side(streams, jobs):
     """Runs job i on streams[i], all forked from the current stream and joined back into it. The nets of
     a group share nothing but read-only inputs, so their small kernels can fill the GPU together.
@@ -542,9 +546,9 @@ def _side_by_side(streams, jobs):
         cur.wait_stream(s)
 
 
-def _graphed_step(jobs, streams=None):
+def _graphed_step(jobs):
     """jobs: list of (net, X, R, Y, Ymask) with static device tensors. Returns step(): one replay of a
-    HIP graph holding one fused training step of every net (as parallel branches when streams are given)."""
+    HIP graph holding one fused training step of every net (several nets share each launch)."""
     for net, *_ in jobs:
         assert net.mode == "fused" and net.dtype == torch.float32 and net.loss is not None
     state = {"graph": None, "decay": None}
@@ -552,19 +556,11 @@ def _graphed_step(jobs, streams=None):
     def decay_flags():
         return tuple((net.weight_decay_start <= net.step_count, net.step_count < net.start_training) for net, *_ in jobs)
 
-    def one(net, X, R, Y, Ymask):
-        def run():
-            # the natively issued step on the capturing stream; the graph always forms its look-ahead itself
-            net._L_versions = None
-            net._native_step(X, R, Y, Ymask)
-        return run
-
     def body():
-        if streams is None:
-            for job in jobs:
-                one(*job)()
-        else:
-            _side_by_side(streams, [one(*job) for job in jobs])
+        # the natively issued step on the capturing stream; the graph always forms its look-ahead itself
+        for net, *_ in jobs:
+            net._L_versions = None
+        _native_steps(jobs)
 
     def capture():
         # The library's scratch buffers belong to a stream and cannot grow under capture: run the step
@@ -593,8 +589,6 @@ def _graphed_step(jobs, streams=None):
         state["graph"], state["decay"] = g, decay_flags()
 
     def step():
-        for net, *_ in jobs:
-            net.join()
         if state["graph"] is None or state["decay"] != decay_flags():
             capture()
         state["graph"].replay()
@@ -630,17 +624,13 @@ class ModelGroup(object):
             self.streams = [torch.cuda.Stream() for _ in self.groups]
         return self.streams
 
-    def train_step(self, X, R, Y, Ymask=None, U=None, join=True):
-        """One step of every architecture group on the shared batch. Each group's step is one native
-        call on the group's own stream (all of default priority), so the host spends a few microseconds
-        per launch and the groups' small kernels overlap on the GPU.
-        join=False leaves the step in flight on the group streams: the next train_step carries on there,
-        and join() - which predict / slice_model / make_graphed_step and every accessor of the nets call -
-        orders the current stream after it. A loop that only steps thereby saves the stream events of a
-        fork and a join per step (about 10 us of host time each).
+    def train_step(self, X, R, Y, Ymask=None, U=None):
+        """One step of every architecture group on the shared batch: one native call whose every launch
+        holds the grids of all the groups (dbk_train_steps), on the current stream. The groups' small
+        kernels thereby run side by side without side streams or events; each group gets the bits of a
+        step of its own.
         U, when given, is a list with one uniforms tensor per architecture group (see self.groups); that
-        path goes through the layer wrappers."""
-        streams = self._streams()
+        path goes through the layer wrappers, one group per side stream."""
         native = U is None and all(net.mode == "fused" and net.dtype == torch.float32 and net.loss is not None
                                    for _, net in self.groups)
         if not native:
@@ -651,54 +641,30 @@ class ModelGroup(object):
                     Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
                     net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
                 return run
-            self.join()
-            _side_by_side(streams, [one(gi, idx, net) for gi, (idx, net) in enumerate(self.groups)])
+            _side_by_side(self._streams(), [one(gi, idx, net) for gi, (idx, net) in enumerate(self.groups)])
             return
         key = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in (X, R, Y, Ymask) if t is not None)
-        in_flight = all(net._busy_stream is s for (_, net), s in zip(self.groups, streams))
-        if key != self._batch_key or not in_flight:
-            # fork: the group streams wait for whatever produced the batch (and for anything the current
-            # stream did to the nets since they were joined)
-            self.join()
-            if key != self._batch_key:
-                self._targets = []
-                for idx, _ in self.groups:
-                    ii = torch.as_tensor(idx, device=Y.device)
-                    self._targets.append((Y.index_select(1, ii).contiguous(),
-                                          Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
-                for t in [X, R, Y, Ymask] + [t for pair in self._targets for t in pair]:
-                    if t is not None:
-                        for s in streams:
-                            t.record_stream(s)
-                self._batch_key, self._batch = key, (X, R, Y, Ymask)
-            ev = torch.cuda.Event()
-            ev.record()
-            for s in streams:
-                s.wait_event(ev)
-        for (idx, net), s, (Yg, Mg) in zip(self.groups, streams, self._targets):
-            net._native_step(X, R, Yg, Mg, stream=s)
-            net._busy_stream = s
-        if join:
-            self.join()
-
-    def join(self):
-        """Orders the current stream after the steps left in flight on the group streams."""
-        for _, net in self.groups:
-            net.join()
+        if key != self._batch_key:
+            # each group's columns of the targets, kept until the batch changes
+            self._targets = []
+            for idx, _ in self.groups:
+                ii = torch.as_tensor(idx, device=Y.device)
+                self._targets.append((Y.index_select(1, ii).contiguous(),
+                                      Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
+            self._batch_key, self._batch = key, (X, R, Y, Ymask)
+        _native_steps([(net, X, R, Yg, Mg) for (_, net), (Yg, Mg) in zip(self.groups, self._targets)])
 
     def make_graphed_step(self, X, R, Y, Ymask=None):
         """One HIP graph holding the fused training step of every architecture group on a static batch."""
         jobs = []
-        self.join()
         for idx, net in self.groups:
             ii = torch.as_tensor(idx, device=Y.device)
             jobs.append((net, X, R, Y.index_select(1, ii).contiguous(),
                          Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
-        return _graphed_step(jobs, self._streams())
+        return _graphed_step(jobs)
 
     def slice_model(self, j):
         """Single-model net for model j of the original ordering."""
-        self.join()
         for idx, net in self.groups:
             if j in idx:
                 return net.slice_model(idx.index(j))
@@ -706,7 +672,6 @@ class ModelGroup(object):
 
     def predict(self, X, R):
         out = torch.empty((R.shape[0], self.nmodel), dtype=torch.float32, device=X.device)
-        self.join()
         for idx, net in self.groups:
             out[:, torch.as_tensor(idx, device=X.device)] = net.predict(X, R)
         return out

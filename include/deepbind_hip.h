@@ -348,6 +348,16 @@ typedef struct dbk_train_step_args {
  * reference: the body of the trainer's loop, deepity/deepity/sgd.py:98-135 (gradstep with the batch
  * gradient as callback, deepity_smat.py:77-117, gradstep.cu:41-72). */
 int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* args);
+/* One step of each of `ngroup` model groups that train on the same batch (same N, regions, nregion and filter
+ * length; architectures may differ: pooling type, hidden units, models per group), e.g. the architectures of
+ * one calibration batch. Every phase of the step is one launch that holds the grids of all the groups, so
+ * groups that are each too small to fill the GPU run side by side on one stream, with no second stream and
+ * no event. Each group's results are the bits its own dbk_train_step gives. Up to 8 groups, each with a
+ * look-ahead vector (Nesterov) and filters of at most 24 taps, are taken together; any other call steps
+ * the groups one after the other on `stream`.
+ * reference: the per-architecture loop over one shared minibatch in the calibration search, which trains
+ * all sampled models on the same batches (deepity/deepity/hpsearch.py:314-330, sgd.py:98-135). */
+int dbk_train_steps(dbk_stream_t stream, size_t ngroup, const dbk_train_step_args* const* args);
 /* sizeof(dbk_train_step_args) as the library was built, for bindings that mirror the block field by field. */
 int dbk_train_step_args_size(void);
 

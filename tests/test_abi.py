@@ -85,6 +85,16 @@ def test_train_step_argument_block_layout_matches_the_header():
     assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"generator position" in lib.dbk_last_error()
     a.rate, a.dpooled = None, None
     assert lib.dbk_train_step(None, ctypes.addressof(a)) != 0 and b"null batch or work buffer" in lib.dbk_last_error()
+    # the several-groups form checks every block of its list the same way, before any launch
+    good = _lib.TrainStepArgs()
+    ctypes.memmove(ctypes.addressof(good), ctypes.addressof(a), ctypes.sizeof(a))
+    good.dpooled = 1
+    blocks = (ctypes.c_void_p * 2)(ctypes.addressof(good), ctypes.addressof(a))
+    assert lib.dbk_train_steps(None, 2, blocks) != 0 and b"null batch or work buffer" in lib.dbk_last_error()
+    assert lib.dbk_train_steps(None, 2, None) != 0 and b"null argument list" in lib.dbk_last_error()
+    blocks[1] = None
+    assert lib.dbk_train_steps(None, 2, blocks) != 0 and b"null argument block" in lib.dbk_last_error()
+    assert lib.dbk_train_steps(None, 0, None) == 0
 
 
 def test_philox_known_answers():

@@ -570,10 +570,10 @@ def test_natively_issued_step_equals_the_step_issued_call_by_call(pool, hidden, 
                 assert np.array_equal(getattr(native, name).cpu().numpy(), getattr(stepwise, name).cpu().numpy()), (change, name)
 
 
-def test_group_steps_left_in_flight_match_joined_steps_across_changing_batches():
-    """ModelGroup.train_step(join=False) keeps the architecture groups running on their own streams from
-    step to step; joined steps, un-joined steps, a change of batch in between and accessors that join
-    implicitly must all give the same bits."""
+def test_groups_stepped_in_shared_launches_match_groups_stepped_alone_across_changing_batches():
+    """ModelGroup.train_step issues one launch per phase for all its architecture groups (dbk_train_steps);
+    every group must end with the bits of its own dbk_train_step, across a change of targets, a smaller batch,
+    the L1 term switching on and an accessor in between."""
     from deepbind_amd import synth
     from deepbind_amd.model import ModelGroup
     cfg = synth.config4()
@@ -587,7 +587,8 @@ def test_group_steps_left_in_flight_match_joined_steps_across_changing_batches()
             net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
         return grp
 
-    joined, flying = make(), make()
+    together, alone = make(), make()
+    assert len(together.groups) == 4 and {net.pool for _, net in together.groups} == {"max", "all"}
     X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
     rng = np.random.default_rng(3)
     Y2 = dev(rng.random(cfg["Y"].shape).astype(np.float32))
@@ -595,16 +596,17 @@ def test_group_steps_left_in_flight_match_joined_steps_across_changing_batches()
     R3, Y3, M3 = dev(cfg["R"][:half]), dev(cfg["Y"][:half]), dev(cfg["Ymask"][:half])
     batches = [(X, R, Y, M)] * 3 + [(X, R, Y2, M)] * 2 + [(X, R3, Y3, M3)] * 2 + [(X, R, Y, M)]
     for i, (bx, br, by, bm) in enumerate(batches):
-        joined.train_step(bx, br, by, bm)
-        flying.train_step(bx, br, by, bm, join=False)
+        together.train_step(bx, br, by, bm)
+        for idx, net in alone.groups:
+            ii = torch.as_tensor(idx, device=by.device)
+            net.train_step(bx, br, by.index_select(1, ii).contiguous(), bm.index_select(1, ii).contiguous())
         if i == 4:
-            # an accessor in the middle joins by itself and the next step forks again
-            pa = flying.predict(X, R)
-            assert np.array_equal(host(pa), host(joined.predict(X, R)))
-    pred_a, pred_b = host(flying.predict(X, R)), host(joined.predict(X, R))      # predict() joins first
-    assert np.array_equal(pred_a, pred_b)
-    for (_, a), (_, b) in zip(joined.groups, flying.groups):
+            assert np.array_equal(host(together.predict(X, R)), host(alone.predict(X, R)))
+    assert np.array_equal(host(together.predict(X, R)), host(alone.predict(X, R)))
+    for (_, a), (_, b) in zip(together.groups, alone.groups):
         pa, pb = a.get_params(), b.get_params()
         for k in pa:
             assert np.array_equal(pa[k], pb[k]), "%s/%d group, %s" % (a.pool, a.hidden, k)
+        assert np.array_equal(host(a.mP), host(b.mP)) and np.array_equal(host(a.dP), host(b.dP))
         assert a.step_count == b.step_count == len(batches) and a._rng_offset == b._rng_offset
+        assert host(a.rng_counter) == host(b.rng_counter)
