@@ -610,3 +610,68 @@ def test_groups_stepped_in_shared_launches_match_groups_stepped_alone_across_cha
         assert np.array_equal(host(a.mP), host(b.mP)) and np.array_equal(host(a.dP), host(b.dP))
         assert a.step_count == b.step_count == len(batches) and a._rng_offset == b._rng_offset
         assert host(a.rng_counter) == host(b.rng_counter)
+
+
+@pytest.mark.parametrize("case", ["mixed_pools_revcomp_input_dropout", "eight_taps", "ten_nets", "different_lengths", "plain_momentum"])
+def test_nets_stepped_through_one_call_end_with_the_bits_of_their_own_steps(case):
+    """dbk_train_steps either runs each phase of the step as one launch for all the nets (same filter-length tier, a
+    look-ahead vector each, at most eight nets) or steps them one after the other; both ways every net must end
+    with the bits of its own dbk_train_step. Covers avg / all / max pooling side by side, reverse-complement
+    pairs, input dropout (each net scans its own dropped copy), mse and nll, 8-, 16- and 24-tap tiers, more nets
+    than one call takes, and the two fallbacks (nets of different tiers, a net without Nesterov momentum)."""
+    from deepbind_amd import data
+    from deepbind_amd.model import SequenceNet, _native_steps
+    rng = np.random.default_rng(11)
+    revcomp = case == "mixed_pools_revcomp_input_dropout"
+    B = 40
+    seqs = ["".join(rng.choice(list("ACGTN"), p=[.24, .24, .24, .24, .04], size=int(rng.integers(18, 45)))) for _ in range(B)]
+    kw = dict(rate=0.05, momentum=0.9, decay_conv=1e-3, decay_full=1e-3, weight_decay_start=1)
+    if case == "mixed_pools_revcomp_input_dropout":
+        m = 16
+        specs = [dict(nmodel=3, pool="avg", hidden=0, loss="mse", reverse_complement=True, dropout=0.25, **kw),
+                 dict(nmodel=5, pool="all", hidden=8, loss="nll", reverse_complement=True, input_dropout=0.2, start_training=2, **kw),
+                 dict(nmodel=2, pool="max", hidden=0, loss="nll", reverse_complement=True, input_dropout=0.1, dropout=0.5, **kw),
+                 dict(nmodel=4, pool="max", hidden=32, loss="mse", reverse_complement=True, **kw)]
+        lens = [m] * 4
+    elif case == "eight_taps":
+        specs = [dict(nmodel=2, pool="all", hidden=0, loss="nll", dropout=0.5, **kw), dict(nmodel=7, pool="max", hidden=4, loss="nll", **kw)]
+        lens = [7, 7]
+    elif case == "ten_nets":
+        specs = [dict(nmodel=1 + i % 3, pool=("max", "all", "avg")[i % 3], hidden=(0, 16)[i % 2], loss="nll", **kw) for i in range(10)]
+        lens = [24] * 10
+    elif case == "different_lengths":
+        specs = [dict(nmodel=2, pool="all", hidden=0, loss="nll", **kw), dict(nmodel=3, pool="max", hidden=8, loss="nll", **kw)]
+        lens = [8, 24]
+    else:
+        specs = [dict(nmodel=2, pool="all", hidden=0, loss="nll", **kw), dict(nmodel=3, pool="max", hidden=8, loss="nll", nesterov=False, **kw)]
+        lens = [16, 16]
+    X, R = data.pack_sequences(seqs, max(lens) - 1, reverse_complement=revcomp)
+    Xd, Rd = dev(X), dev(R)
+    rows = len(R)
+
+    def make():
+        nets, targets = [], []
+        trng = np.random.default_rng(12)
+        for i, (spec, m) in enumerate(zip(specs, lens)):
+            net = SequenceNet(nfilter=16, m=m, **spec)
+            net.init_params(init_conv=0.3, init_full=0.3, init_mu=0.01, seed=40 + i)
+            net.rng_seed = 7 + i
+            Y = (trng.random((rows // (2 if revcomp else 1), net.ninst)) < 0.5).astype(np.float32)
+            Y = np.repeat(Y, 2, axis=0) if revcomp else Y
+            M = trng.random((rows, net.ninst)) < 0.8
+            nets.append(net)
+            targets.append((dev(Y), dev(M)))
+        return nets, targets
+
+    (one_call, t1), (by_itself, t2) = make(), make()
+    for step in range(4):
+        _native_steps([(net, Xd, Rd, Y, M) for net, (Y, M) in zip(one_call, t1)])
+        for net, (Y, M) in zip(by_itself, t2):
+            net.train_step(Xd, Rd, Y, M)
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(zip(one_call, by_itself)):
+        for name in ("P", "mP", "dP"):
+            assert np.array_equal(host(getattr(a, name)), host(getattr(b, name))), (case, i, name)
+        assert np.abs(host(a.mP)).max() > 0
+        assert a.step_count == b.step_count == 4 and a._rng_offset == b._rng_offset
+        assert host(a.rng_counter) == host(b.rng_counter)
