@@ -47,10 +47,11 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
     const size_t r = r0 + row;
     const bool live = r < a.n;
     const size_t ncol = (size_t)k * a.nblock;
-    // per-row strides are odd so that lanes holding different rows hit distinct LDS banks
-    const int ks = k | 1, hst = h1 | 1;
-    float* w1s = hs;                        // [k][h1]
-    float* b1s = w1s + k * h1;              // [h1]
+    // per-row strides are odd so that lanes holding different rows hit distinct LDS banks; the weight rows too:
+    // in the backward pass the eight lanes of a row read eight different inputs' weights for the same hidden unit
+    const int ks = k | 1, hst = h1 | 1, wst = hidden > 0 ? (hidden | 1) : 1;
+    float* w1s = hs;                        // [k][wst]
+    float* b1s = w1s + k * wst;             // [h1]
     float* w2s = b1s + h1;                  // [h1] (unused when hidden == 0)
     float* H0s = w2s + h1;                  // [RB][ks]  inputs after dropout
     float* H1s = H0s + RB * ks;             // [RB][hst] hidden activations (hidden > 0)
@@ -65,8 +66,10 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = e0 + j * NT < k * h1 ? a.W1[(size_t)b * k * h1 + e0 + j * NT] : 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (e0 + j * NT < k * h1) w1s[e0 + j * NT] = v[j];
+        for (int j = 0; j < 4; ++j) {
+            const int e = e0 + j * NT;
+            if (e < k * h1) w1s[(e / h1) * wst + e % h1] = v[j];
+        }
     }
     for (int e = tid; e < h1; e += NT) {                          // both vectors' loads are issued before either is stored
         const float vb = a.b1[(size_t)b * h1 + e];
@@ -117,7 +120,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
         for (int h = part; h < hidden; h += NP) {
             float s = 0.0f;
 #pragma unroll 8
-            for (int kk = 0; kk < k; ++kk) s += x[kk] * w1s[kk * hidden + h];
+            for (int kk = 0; kk < k; ++kk) s += x[kk] * w1s[kk * wst + h];
             s += b1s[h];
             s = s > 0.0f ? s : 0.0f;
             H1s[row * hst + h] = s;
@@ -164,7 +167,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
             if (hidden > 0) {
                 g = 0.0f;
 #pragma unroll 8
-                for (int h = 0; h < hidden; ++h) g += D1s[row * hst + h] * w1s[kk * hidden + h];
+                for (int h = 0; h < hidden; ++h) g += D1s[row * hst + h] * w1s[kk * wst + h];
             } else {
                 g = dA * w1s[kk];
             }
@@ -259,7 +262,7 @@ __global__ void k_head_reduce(head_args a)
 
 inline size_t head_smem(int k, int h1)
 {
-    return ((size_t)k * h1 + 2 * h1 + (size_t)RB * (k | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
+    return ((size_t)k * (h1 | 1) + 2 * h1 + (size_t)RB * (k | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
 }
 
 }  // namespace
