@@ -39,6 +39,7 @@ _SIGNATURES = {
     "dbk_dropoutord_fp_tr_u": [_P, _P, _P, _P, _Z, _F, _P],
     "dbk_scanpool_fprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
     "dbk_scanpool_fprop_general": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
+    "dbk_scanpool_fprop_wide": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
     "dbk_scanpool_fprop_kmer": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
     "dbk_scanpool_bprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P, _P, _P, _I, _P],
     "dbk_blockwise_dot": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],

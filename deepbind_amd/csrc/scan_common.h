@@ -16,7 +16,8 @@ __device__ __forceinline__ unsigned letter_of(unsigned code)
 
 // Builds lut[(j*NL + l)*FT + fl] for filters [f0, f0+FT) from W (4m, F); missing filters read as 0.
 // With mpad > m the table gets all-zero rows for taps m..mpad-1.
-template <typename T>
+// QUAD: a row holds filter fl at element (fl % 16) * 4 + fl / 16, i.e. 16 lanes x 4 filters (16 apart) per lane.
+template <typename T, bool QUAD = false>
 __device__ void build_letter_table(T* lut, const T* __restrict__ W, unsigned m, unsigned F, unsigned f0, unsigned mpad = 0)
 {
     if (mpad < m) mpad = m;
@@ -39,7 +40,7 @@ __device__ void build_letter_table(T* lut, const T* __restrict__ W, unsigned m, 
             z += w[u][1];
             z += w[u][2];
             z += w[u][3];
-            T* row = lut + (size_t)j * NL * FT + fl;
+            T* row = lut + (size_t)j * NL * FT + (QUAD ? (fl & 15u) * 4u + (fl >> 4) : fl);
             row[0 * FT] = w[u][0];
             row[1 * FT] = w[u][1];
             row[2 * FT] = w[u][2];

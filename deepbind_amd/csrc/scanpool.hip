@@ -161,6 +161,169 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
     scanpool_fprop_body<PT, WANT_ARGMAX, MT>(this_wg(), W, bias, m, F, X, N, R, P, pooled, argmax, run_if_flag, act);
 }
 
+// The same forward pass with four filters per lane, for batches of many regions (filters of 17-24 taps).
+//
+// The kernel above spends one 4-byte LDS read per (position, tap, filter): a wave's read moves 256 bytes and the
+// LDS delivers ~104 B/clk/CU of those, which is what bounds it once the GPU is full. Here a lane owns the four
+// filters l, l+16, l+32, l+48 of the tile and the table row is laid out [16 lanes][4 filters], so the 16 lanes
+// of a quarter wave read one aligned 256-byte line with ds_read_b128 (~216 B/clk/CU), and the four quarters of
+// the wave work on four consecutive windows of 16 positions. A wave therefore takes 64 positions of ONE region
+// at a time and the four waves of a workgroup walk four different regions: no workgroup barrier after the
+// table is built. The letters of a quarter's window sit in ten vector registers (they differ between the
+// quarters); one bit-field extract and one address add per letter serve up to 16 (position, tap) reads.
+// Per position the taps are added in ascending order, as everywhere else: maxima and argmax are the bits of
+// the kernel above; averages add the same rectified values in another order (quarter by quarter).
+constexpr unsigned WIDE_SPAN = 64;                                // positions per wave and round
+template <int MT> struct wide_shape {
+    static constexpr unsigned words = (PSUB + MT - 1 + 3) / 4;    // window words per quarter
+    static constexpr unsigned xbytes = (3 * PSUB + 4 * words + 15) & ~15u;   // letters staged per wave and round
+};
+
+template <int PT, bool WANT_ARGMAX, int MT>
+__device__ __forceinline__ void scanpool_fprop_wide_body(const wg_t wg, const float* __restrict__ W, const float* __restrict__ bias,
+                                                         unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                         const uint32_t* __restrict__ R, size_t P,
+                                                         float* __restrict__ pooled, uint32_t* __restrict__ argmax,
+                                                         unsigned long long* __restrict__ act)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr unsigned NWORD = wide_shape<MT>::words, XB = wide_shape<MT>::xbytes;
+    static_assert(XB % 16 == 0 && NWORD == 10, "the window loads below are two 16-byte and one 8-byte read");
+    const unsigned nw = blockDim.x >> 6;
+    float* lut = reinterpret_cast<float*>(smem);                   // [MT*NL][16][4]
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned qd = lane >> 4, l = lane & 15;
+    uint8_t* xw = smem + (size_t)MT * NL * FT * sizeof(float) + (size_t)wave * XB;   // this wave's letters
+    const unsigned f0 = wg.y * FT;
+    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;    // rows the scan defines; later rows are relu(bias)
+    build_letter_table<float, true>(lut, W, m, F, f0, MT);
+    float bf[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bf[c] = f0 + c * 16 + l < F ? bias[f0 + c * 16 + l] : 0.0f;
+    __syncthreads();
+    const float4* lut4 = reinterpret_cast<const float4*>(lut) + l;
+
+    for (size_t r = (size_t)wg.x * nw + wave; r < P; r += (size_t)wg.gx * nw) {
+        const size_t a = R[2 * r], b = R[2 * r + 1];
+        float mx[4] = {-1.0f, -1.0f, -1.0f, -1.0f}, sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        unsigned xi[4] = {0u, 0u, 0u, 0u};                        // row of the maximum, relative to a
+        for (size_t c0 = a; c0 < b; c0 += WIDE_SPAN) {
+            const unsigned rows = (unsigned)((b - c0) < WIDE_SPAN ? (b - c0) : WIDE_SPAN);
+            // ---- letters of positions c0 .. c0 + XB - 1 (two per lane), then this quarter's window words
+            {
+                const size_t g0 = c0 + lane, g1 = g0 + 64;
+                const unsigned v0 = g0 < N ? letter_of(X[g0]) : 5u;
+                const unsigned v1 = (lane + 64 < XB && g1 < N) ? letter_of(X[g1]) : 5u;
+                __builtin_amdgcn_wave_barrier();                   // the previous round's window reads come first
+                xw[lane] = (uint8_t)v0;
+                if (lane + 64 < XB) xw[lane + 64] = (uint8_t)v1;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            }
+            unsigned wq[NWORD];
+            {
+                const uint4 w0 = *reinterpret_cast<const uint4*>(xw + PSUB * qd);
+                const uint4 w1 = *reinterpret_cast<const uint4*>(xw + PSUB * qd + 16);
+                const uint2 w2 = *reinterpret_cast<const uint2*>(xw + PSUB * qd + 32);
+                wq[0] = w0.x; wq[1] = w0.y; wq[2] = w0.z; wq[3] = w0.w;
+                wq[4] = w1.x; wq[5] = w1.y; wq[6] = w1.z; wq[7] = w1.w;
+                wq[8] = w2.x; wq[9] = w2.y;
+            }
+            // ---- the window: 16 positions x MT taps x 4 filters
+            float4 acc[PSUB];
+#pragma unroll
+            for (int p = 0; p < PSUB; ++p) acc[p] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+            for (int q = 0; q < PSUB + MT - 1; ++q) {
+                const unsigned letter = (wq[q >> 2] >> ((q & 3) * 8)) & 0xffu;
+                const float4* col = lut4 + letter * 16u;
+#pragma unroll
+                for (int p = 0; p < PSUB; ++p) {
+                    const int j = q - p;
+                    if (j >= 0 && j < MT) {
+                        const float4 v = col[j * NL * 16];
+                        acc[p].x += v.x; acc[p].y += v.y; acc[p].z += v.z; acc[p].w += v.w;
+                    }
+                }
+                if ((q & 3) == 3) {
+                    // pin the running sums (see scan16_window)
+#pragma unroll
+                    for (int p = 0; p < PSUB; ++p) asm volatile("" : "+v"(acc[p].x), "+v"(acc[p].y), "+v"(acc[p].z), "+v"(acc[p].w));
+                }
+            }
+            // ---- bias, rectifier, pooling; optionally the activity masks of the 64 rows
+            const unsigned pq = PSUB * qd;                         // first position of this quarter's window
+            unsigned long long mine = 0ull;
+#pragma unroll
+            for (int p = 0; p < PSUB; ++p) {
+                const size_t i = c0 + pq + p;
+                const bool defined = i < n;
+                float z[4] = {acc[p].x, acc[p].y, acc[p].z, acc[p].w};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) z[c] = (defined ? z[c] : 0.0f) + bf[c];
+                if (act) {
+                    // ballot c holds, for each quarter, 16 bits: filters 16c .. 16c+15 of that quarter's row p
+                    unsigned lo = 0u, hi = 0u;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const unsigned long long open = __ballot(z[c] > 0.0f);
+                        const unsigned part = (unsigned)(open >> (16u * qd)) & 0xffffu;
+                        if (c < 2) lo |= part << (16 * c);
+                        else hi |= part << (16 * (c - 2));
+                    }
+                    if (l == (unsigned)p) mine = ((unsigned long long)hi << 32) | lo;
+                }
+                if (pq + p < rows) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const float zr = z[c] > 0.0f ? z[c] : 0.0f;
+                        if (PT != DBK_PT_AVG) { if (zr > mx[c]) { mx[c] = zr; xi[c] = (unsigned)(i - a); } }
+                        if (PT != DBK_PT_MAX) sum[c] += zr;
+                    }
+                }
+            }
+            if (act && pq + l < rows) act[(c0 + pq + l) * wg.gy + wg.y] = mine;
+        }
+        // ---- fold the four quarters: larger value wins, equal values keep the earlier row
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+#pragma unroll
+            for (int d = 16; d <= 32; d <<= 1) {
+                const float vm = __shfl_xor(mx[c], d, 64);
+                const unsigned vi = (unsigned)__shfl_xor((int)xi[c], d, 64);
+                const float vs = __shfl_xor(sum[c], d, 64);
+                if (vm > mx[c] || (vm == mx[c] && vi < xi[c])) { mx[c] = vm; xi[c] = vi; }
+                sum[c] += vs;
+            }
+        }
+        if (qd == 0) {
+            const float cnt = (float)(b - a);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const unsigned f = f0 + c * 16 + l;
+                if (f >= F) continue;
+                const size_t j = r * F + f;
+                const float bm = mx[c] > 0.0f ? mx[c] : 0.0f;      // only an empty region gets here with a negative maximum
+                if (PT == DBK_PT_MAX) pooled[j] = bm;
+                else if (PT == DBK_PT_AVG) pooled[j] = sum[c] / cnt;
+                else { pooled[2 * j] = bm; pooled[2 * j + 1] = sum[c] / cnt; }
+                if (WANT_ARGMAX && PT != DBK_PT_AVG) argmax[j] = (uint32_t)((a + xi[c]) * F + f);
+            }
+        }
+    }
+}
+
+template <int PT, bool WANT_ARGMAX, int MT>
+__global__ __launch_bounds__(256) void scanpool_fprop_wide_kernel(const float* __restrict__ W, const float* __restrict__ bias,
+                                                                  unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                  const uint32_t* __restrict__ R, size_t P,
+                                                                  float* __restrict__ pooled, uint32_t* __restrict__ argmax,
+                                                                  unsigned long long* __restrict__ act)
+{
+    scanpool_fprop_wide_body<PT, WANT_ARGMAX, MT>(this_wg(), W, bias, m, F, X, N, R, P, pooled, argmax, act);
+}
+
 // ---------------------------------------------------------------------------------------------
 // backward
 // ---------------------------------------------------------------------------------------------
@@ -709,6 +872,17 @@ inline unsigned dense_grid_x(unsigned mt, unsigned ftiles, size_t P)
     if (gxd > P) gxd = (unsigned)P;
     return gxd;
 }
+// The wide forward kernel (four filters per lane, a wave per region) pays off once there are enough (region, tile)
+// items to keep every CU's LDS busy; a small batch is latency-bound and better off with four waves per region.
+inline bool wide_takes(size_t m, unsigned ftiles, size_t P) { return m > 16 && m <= 24 && P * (size_t)ftiles >= 512; }
+inline unsigned wide_grid_x(unsigned ftiles, size_t P)
+{
+    unsigned gx = 768u / ftiles;                                  // three workgroups per CU are resident (150-160 registers)
+    if (gx < 1) gx = 1;
+    if (gx > (P + 3) / 4) gx = (unsigned)((P + 3) / 4);           // a workgroup walks four regions at a time
+    return gx;
+}
+inline size_t wide_smem() { return (size_t)24 * NL * FT * sizeof(float) + 4 * wide_shape<24>::xbytes; }
 inline size_t sparse_smem(size_t m) { return m * SPARSE_ROWS * FT * sizeof(float); }
 inline size_t dense_smem(unsigned mt) { return ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3); }
 
@@ -730,6 +904,25 @@ int launch_fprop_mt(hipStream_t st, unsigned gx, unsigned ftiles, unsigned nw, s
 }
 
 template <int PT>
+int launch_fprop_wide(hipStream_t st, unsigned ftiles, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+                      const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, unsigned long long* act)
+{
+    const size_t smem = wide_smem();
+    DBK_CHECK(smem <= lds_limit(), "ValueError: the wide forward kernel needs %zu bytes of LDS (limit %zu)", smem, lds_limit());
+    const unsigned gx = wide_grid_x(ftiles, P);
+    if (argmax) {
+        auto kern = scanpool_fprop_wide_kernel<PT, true, 24>;
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, act);
+    } else {
+        auto kern = scanpool_fprop_wide_kernel<PT, false, 24>;
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, act);
+    }
+    DBK_LAUNCH_OK();
+}
+
+template <int PT>
 int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                     const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, const unsigned* run_if_flag, unsigned long long* act)
 {
@@ -739,6 +932,7 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     DBK_CHECK(smem <= lds_limit(), "ValueError: filter length %zu needs %zu bytes of LDS (limit %zu)", m, smem, lds_limit());
     unsigned ftiles = dbk::divup(F, FT);
     DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
+    if (!run_if_flag && wide_takes(m, ftiles, P)) return launch_fprop_wide<PT>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
     const unsigned gx = fprop_grid_x(mt, ftiles, P);
     int rc = 0;
     switch (mt) {
@@ -826,6 +1020,18 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     DBK_LAUNCH_OK();
 }
 
+int fprop_wide(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+               const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, unsigned long long* act)
+{
+    const unsigned ftiles = dbk::divup(F, FT);
+    DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
+    switch (ptype) {
+    case DBK_PT_MAX: return launch_fprop_wide<DBK_PT_MAX>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    case DBK_PT_AVG: return launch_fprop_wide<DBK_PT_AVG>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, nullptr, act);
+    default:         return launch_fprop_wide<DBK_PT_ALL>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    }
+}
+
 int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
           const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, const unsigned* run_if_flag,
           unsigned long long* act)
@@ -847,6 +1053,7 @@ struct multi_args {
     size_t N, P;
     const uint32_t* R;
     unsigned first[dbk::MULTI_MAX + 1], gx[dbk::MULTI_MAX], ftiles[dbk::MULTI_MAX];
+    unsigned wide[dbk::MULTI_MAX];                                 // forward: the group goes through the wide kernel body
     dbk::scan_group g[dbk::MULTI_MAX];
 };
 
@@ -863,7 +1070,19 @@ template <int MT>
 __global__ __launch_bounds__(256) void scanpool_fprop_multi_kernel(const multi_args a)
 {
     wg_t wg;
-    const dbk::scan_group& j = a.g[multi_locate(a, wg)];
+    const unsigned gi = multi_locate(a, wg);
+    const dbk::scan_group& j = a.g[gi];
+    if constexpr (MT == 24) {
+        if (a.wide[gi]) {
+            if (j.ptype == DBK_PT_MAX)
+                scanpool_fprop_wide_body<DBK_PT_MAX, true, 24>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr);
+            else if (j.ptype == DBK_PT_ALL)
+                scanpool_fprop_wide_body<DBK_PT_ALL, true, 24>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.act);
+            else
+                scanpool_fprop_wide_body<DBK_PT_AVG, false, 24>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, nullptr, j.act);
+            return;
+        }
+    }
     if (j.ptype == DBK_PT_MAX)
         scanpool_fprop_body<DBK_PT_MAX, true, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr, nullptr);
     else if (j.ptype == DBK_PT_ALL)
@@ -920,7 +1139,7 @@ bool scan_multi_takes(size_t m, size_t N, size_t P, unsigned n, const scan_group
         // a max-pooling group on a batch large enough for the k-mer table goes there when stepped alone (other sums, other bits)
         if (g[i].ptype == DBK_PT_MAX && dbk_scanpool_kmer::takes(m, g[i].F, N, P)) return false;
     }
-    return fprop_smem(multi_tier(m), m) <= lds_limit() && sparse_smem(m) <= lds_limit() && dense_smem(multi_tier(m)) <= lds_limit();
+    return fprop_smem(multi_tier(m), m) <= lds_limit() && wide_smem() <= lds_limit() && sparse_smem(m) <= lds_limit() && dense_smem(multi_tier(m)) <= lds_limit();
 }
 
 int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size_t P, unsigned n, const scan_group* g)
@@ -929,13 +1148,17 @@ int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
     multi_args a;
     a.n = n; a.m = (unsigned)m; a.N = N; a.P = P; a.R = R;
     a.first[0] = 0;
+    bool any_wide = false;
     for (unsigned i = 0; i < n; ++i) {
         a.g[i] = g[i];
         a.ftiles[i] = dbk::divup(g[i].F, FT);
-        a.gx[i] = fprop_grid_x(mt, a.ftiles[i], P);
+        a.wide[i] = wide_takes(m, a.ftiles[i], P);                 // as the group's own launch would choose
+        a.gx[i] = a.wide[i] ? wide_grid_x(a.ftiles[i], P) : fprop_grid_x(mt, a.ftiles[i], P);
         a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
+        if (a.wide[i]) any_wide = true;
     }
-    const size_t smem = fprop_smem(mt, m);
+    size_t smem = fprop_smem(mt, m);
+    if (any_wide && wide_smem() > smem) smem = wide_smem();
     if (mt == 8) return launch_multi(scanpool_fprop_multi_kernel<8>, st, smem, a);
     if (mt == 16) return launch_multi(scanpool_fprop_multi_kernel<16>, st, smem, a);
     return launch_multi(scanpool_fprop_multi_kernel<24>, st, smem, a);
@@ -950,6 +1173,7 @@ int scan_bprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
     size_t total = 0;
     for (unsigned i = 0; i < n; ++i) {
         a.ftiles[i] = dbk::divup(g[i].F, FT);
+        a.wide[i] = 0;
         a.gx[i] = g[i].ptype == DBK_PT_MAX ? sparse_grid_x(a.ftiles[i], P) : dense_grid_x(mt, a.ftiles[i], P);
         a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
         g[i].slab_stride = 4 * m * (size_t)g[i].F + g[i].F;
@@ -994,6 +1218,21 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream, const float* W, const float*
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
     return dbk_scanpool_general::fprop(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, nullptr,
                                        reinterpret_cast<unsigned long long*>(act));
+}
+
+int dbk_scanpool_fprop_wide(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
+                            const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
+                            float* pooled, uint32_t* argmax, uint64_t* act)
+{
+    DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
+    DBK_CHECK(m > 16 && m <= 24, "NotImplementedError: the wide forward kernel takes filters of 17 to 24 taps (got %zu)", m);
+    DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
+    DBK_CHECK(!argmax || (double)N * (double)nfilter <= 4294967296.0,
+              "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
+    if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
+    return dbk_scanpool_general::fprop_wide(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax,
+                                            reinterpret_cast<unsigned long long*>(act));
 }
 
 int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,

@@ -142,7 +142,8 @@ def activity_words(X, W):
 def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=None):
     """pool(relu(corr1ord(W, X) + b)) per region without storing the (N x P) map.
     Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only.
-    path: "auto" lets the library choose, "general" / "kmer" force one kernel.
+    path: "auto" lets the library choose; "general" / "wide" / "kmer" force the general path (which picks its
+    kernel by size), its many-regions kernel (17-24 taps) or the table kernel.
     act (optional, from activity_words): receives 1 bit per row and filter - rectifier open or not - which
     scanpool_bprop takes in place of recomputing the map (general kernel only)."""
     _u8(X)
@@ -153,7 +154,8 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
     pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
     argmax = torch.empty((P, F), dtype=uindex, device=W.device) if (want_argmax and ptype in ("max", "all")) else None
-    entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "kmer": "dbk_scanpool_fprop_kmer"}[path]
+    entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "wide": "dbk_scanpool_fprop_wide",
+             "kmer": "dbk_scanpool_fprop_kmer"}[path]
     args = [stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax)]
     if path != "kmer":
         args.append(_act(act, X, F))

@@ -134,6 +134,17 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream,
                                const uint32_t* regions, size_t nregion, int ptype,
                                float* pooled, uint32_t* argmax, uint64_t* act);
 
+/* Same contract through the general path's kernel for many regions regardless of problem size: four filters
+ * per lane and one wave per region, for filters of 17 to 24 taps (NotImplementedError otherwise).
+ * dbk_scanpool_fprop_general picks it once regions x filter tiles reach 1024, where the one-filter-per-lane kernel
+ * is bound by the rate of its 4-byte LDS reads. Per position the taps are added in the same order, so maxima,
+ * argmax and activity masks are the same bits; averages add the same values in another order. */
+int dbk_scanpool_fprop_wide(dbk_stream_t stream,
+                            const float* W, const float* bias, size_t m, size_t nfilter,
+                            const uint8_t* X, size_t N,
+                            const uint32_t* regions, size_t nregion, int ptype,
+                            float* pooled, uint32_t* argmax, uint64_t* act);
+
 /* Same contract through the 3-mer lookup-table kernel regardless of problem size; fails with
  * NotImplementedError for shapes that kernel does not take (filter length > 24, avg/all pooling,
  * argmax requested). Inputs it cannot express (code 254, regions outside the sequence) are detected

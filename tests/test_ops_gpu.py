@@ -204,6 +204,56 @@ def test_scanpool_fprop(ks, general, ptype, B, lo, hi, m, F):
         assert np.all(rows >= R[:, :1]) and np.all(rows < R[:, 1:2])
 
 
+@pytest.mark.parametrize("ptype", ["max", "avg", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (40, 20, 40, 24, 144), (23, 0, 300, 17, 70), (300, 30, 70, 20, 64)])
+def test_scanpool_fprop_wide_kernel(ks, ptype, B, lo, hi, m, F):
+    """The many-regions forward kernel (four filters per lane, a wave per region), forced on small inputs: against
+    the unfused chain, and bit for bit against the one-filter-per-lane kernel where the two add in the same order
+    (maxima, argmax, activity masks); regions of 0 to 300 rows, code 254 and N present, filter counts that leave
+    lanes and whole quarters of a tile empty."""
+    rng, W, b, X, R = _fused_case(B + m + F + 1, B, lo, hi, m, F, p254=0.01)
+    A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    act_w, act_n = ks.activity_words(Xd, Wd), ks.activity_words(Xd, Wd)
+    act_w.fill_(-1), act_n.fill_(-1)
+    P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="wide", act=act_w)
+    Pn, In = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="general", act=act_n)   # few regions: the narrow kernel
+    keep = R[:, 1] > R[:, 0]                                          # an empty region's average is 0/0
+    assert_close(host(P)[keep], Pr[keep], ACT, "pooled")
+    got, ref = host(P), host(Pn)
+    if ptype == "max":
+        assert np.array_equal(got, ref)
+    elif ptype == "all":
+        assert np.array_equal(got[:, 0::2], ref[:, 0::2])
+        assert_close(got[keep][:, 1::2], ref[keep][:, 1::2], ACT, "averages, wide vs narrow")
+    if I is not None:
+        assert np.array_equal(host(I), host(In))
+    # masks: the rows inside regions carry the same bits; every other word is left alone
+    aw, an = host(act_w), host(act_n)
+    assert np.array_equal(aw, an)
+    inside = np.zeros(len(X), bool)
+    for a_, b_ in R:
+        inside[a_:b_] = True
+    assert np.all(aw[~inside] == -1)
+    # without argmax and without masks (other template instances)
+    P2, _ = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=False, path="wide")
+    assert np.array_equal(host(P2)[keep], got[keep])
+
+
+def test_scanpool_general_path_picks_the_wide_kernel_for_many_regions(ks):
+    """From 1024 (region, tile) items on, the general path runs the many-regions kernel: same results as forcing it."""
+    rng, W, b, X, R = _fused_case(5, 1100, 18, 40, 24, 40, p254=0.01)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    for ptype in ("max", "avg", "all"):
+        P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="general")
+        Pw, Iw = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="wide")
+        assert np.array_equal(host(P), host(Pw))
+        if I is not None:
+            assert np.array_equal(host(I), host(Iw))
+        A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
+        assert_close(host(P), Pr, ACT, "pooled " + ptype)
+
+
 def test_scanpool_regions_past_the_end_and_gaps(ks):
     """Arbitrary (non-packed) regions, including rows the scan does not define (relu(bias) there)."""
     rng = np.random.default_rng(77)
