@@ -834,6 +834,140 @@ __global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned 
     scanpool_bprop_dense_act_body<PT, MT>(this_wg(), m, F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
 }
 
+// The mask-driven dense backward for many regions: a wave per region. The kernel above spreads the windows of one
+// region over the four waves of a workgroup and meets at a barrier per region chunk; with regions of a few dozen rows
+// that is one window per wave and barrier, and the waves spend half their time waiting for the next chunk's loads.
+// Here every wave walks whole regions on its own (64 rows per round: letters staged in the wave's own LDS bytes, the
+// 64 rows' masks read by the 64 lanes in one load, four windows added into the wave's register planes), with the next
+// region's bounds and pooled gradients requested a region ahead. No barrier until the waves fold their planes into
+// the workgroup's slab at the end, exactly as above. The regions are dealt to waves instead of workgroups, so the
+// partial sums are other (equally fixed) partial sums than the kernel above forms.
+template <int PT, int MT>
+__device__ __forceinline__ void scanpool_bprop_dense_act_wave_body(const wg_t wg, unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                   const uint32_t* __restrict__ R, size_t P,
+                                                                   const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
+                                                                   const float* __restrict__ dpooled,
+                                                                   const unsigned long long* __restrict__ act,
+                                                                   float* __restrict__ slabs, size_t stride)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const unsigned nw = blockDim.x >> 6;
+    constexpr unsigned XB = (3 * PSUB + 4 * window<MT>::words + 15) & ~15u;   // letters behind the four windows of a round
+    static_assert(XB <= 128, "a lane stages at most two letters per round");
+    float* lut = reinterpret_cast<float*>(smem);                   // [MT*4][FT]: only the cross-wave fold at the end uses it
+    float* dbacc = lut + (size_t)MT * 4 * FT;                      // [nw][FT]
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint8_t* xw = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT) + (size_t)wave * XB;
+    const unsigned f0 = wg.y * FT, f = f0 + lane;
+    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
+    float db = 0.0f;
+    grad_planes<MT> planes;
+    planes.clear();
+
+    struct pooled_in { float davg, pmax, dmax; unsigned arg; };
+    auto load_pooled = [&](size_t r_) -> pooled_in {
+        pooled_in q = { 0.0f, 0.0f, 0.0f, 0u };
+        if (f < F) {
+            const size_t j0 = r_ * F + f;
+            q.davg = PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1];
+            if (PT == DBK_PT_ALL) { q.pmax = pooled[2 * j0]; q.dmax = dpooled[2 * j0]; q.arg = argmax[j0]; }
+        }
+        return q;
+    };
+    const size_t step = (size_t)wg.gx * nw;
+    size_t r = (size_t)wg.x * nw + wave;
+    size_t a = 0, b = 0;
+    pooled_in q = { 0.0f, 0.0f, 0.0f, 0u };
+    if (r < P) { a = R[2 * r]; b = R[2 * r + 1]; q = load_pooled(r); }
+    while (r < P) {                                                // uniform over the wave
+        const size_t rn = r + step;
+        size_t na = 0, nb = 0;
+        pooled_in nq = { 0.0f, 0.0f, 0.0f, 0u };
+        if (rn < P) { na = R[2 * rn]; nb = R[2 * rn + 1]; nq = load_pooled(rn); }
+        const float gavg = q.davg / (float)(b - a);
+        float gmax = 0.0f;                                         // max+avg pooling: the winning row also gets the max gradient
+        size_t imax = ~(size_t)0;
+        if (PT == DBK_PT_ALL && q.pmax > 0.0f) { gmax = q.dmax; imax = q.arg / F; }
+        for (size_t c0 = a; c0 < b; c0 += 4 * PSUB) {
+            const unsigned rows = (unsigned)((b - c0) < 4 * PSUB ? (b - c0) : 4 * PSUB);
+            // letters of positions c0 .. c0 + XB - 1 (two per lane) and the masks of the round's rows (lane t: row t)
+            const size_t g0 = c0 + lane, g1 = g0 + 64;
+            const unsigned v0 = g0 < N ? letter_of(X[g0]) : 5u;
+            const unsigned v1 = (lane + 64 < XB && g1 < N) ? letter_of(X[g1]) : 5u;
+            const unsigned long long mkall = lane < rows ? act[(c0 + lane) * wg.gy + wg.y] : 0ull;
+            __builtin_amdgcn_wave_barrier();                       // the previous round's window reads come first
+            xw[lane] = (uint8_t)v0;
+            if (lane + 64 < XB) xw[lane + 64] = (uint8_t)v1;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const unsigned mlo = (unsigned)mkall, mhi = (unsigned)(mkall >> 32);
+#pragma unroll 1
+            for (unsigned p0 = 0; p0 < rows; p0 += PSUB) {
+                unsigned wq[window<MT>::words];
+                load_window<MT>(xw, p0, wq);
+                float g[PSUB];
+                const size_t w0 = c0 + p0;
+                const int relmax = (PT == DBK_PT_ALL && imax >= w0 && imax - w0 < (size_t)PSUB) ? (int)(imax - w0) : -1;
+                const int nrel = n > w0 ? (n - w0 < (size_t)PSUB ? (int)(n - w0) : PSUB) : 0;
+#pragma unroll
+                for (int p = 0; p < PSUB; ++p) {
+                    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)mlo, (int)p0 + p);
+                    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)mhi, (int)p0 + p);
+                    const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
+                    float gg = open ? gavg : 0.0f;
+                    if (PT == DBK_PT_ALL) gg += p == relmax ? gmax : 0.0f;
+                    db += gg;
+                    g[p] = p < nrel ? gg : 0.0f;                   // rows past the scan's end carry bias only
+                }
+                grad_planes_window<MT>(planes, wq, g);
+            }
+        }
+        r = rn; a = na; b = nb; q = nq;
+    }
+    float aw[MT][4];
+    grad_planes_read<MT>(planes, aw);
+    dbacc[wave * FT + lane] = db;
+    float* fold = lut + lane;
+    for (unsigned w = 0; w < nw; ++w) {
+        __syncthreads();
+        if (wave == w) {
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                if ((unsigned)j < m) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float* cell = fold + (j * 4 + c) * FT;
+                        *cell = w == 0 ? aw[j][c] : *cell + aw[j][c];
+                    }
+                }
+        }
+    }
+    __syncthreads();
+    const unsigned f0w = f0;
+    float* out = slabs + (size_t)wg.x * stride;
+    for (unsigned e = threadIdx.x; e < m * 4 * FT; e += blockDim.x) {
+        const unsigned row = e / FT, fl = e % FT;
+        if (f0w + fl < F) out[(size_t)row * F + f0w + fl] = lut[e];
+    }
+    if (wave == 0 && f < F) {
+        float t = dbacc[lane];
+        for (unsigned w = 1; w < nw; ++w) t += dbacc[w * FT + lane];
+        out[(size_t)4 * m * F + f] = t;
+    }
+}
+
+template <int PT, int MT>
+__global__ __launch_bounds__(256) void scanpool_bprop_dense_act_wave_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                            const uint32_t* __restrict__ R, size_t P,
+                                                                            const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
+                                                                            const float* __restrict__ dpooled,
+                                                                            const unsigned long long* __restrict__ act,
+                                                                            float* __restrict__ slabs, size_t stride)
+{
+    scanpool_bprop_dense_act_wave_body<PT, MT>(this_wg(), m, F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
+}
+
 // Launch shapes, shared by the single-group launchers and the multi-group ones.
 // forward: as many workgroups as are resident at once (three per CU; two with the register planes of 16 taps);
 // each sets up its filter tile's weights once and then walks its share of the regions
@@ -883,6 +1017,18 @@ inline unsigned wide_grid_x(unsigned ftiles, size_t P)
     return gx;
 }
 inline size_t wide_smem() { return (size_t)24 * NL * FT * sizeof(float) + 4 * wide_shape<24>::xbytes; }
+// The wave-per-region dense backward: same threshold as the wide forward (enough regions to keep every wave busy
+// with whole regions); the smallest grid that gives every wave the same number of regions as the resident grid would.
+inline bool dense_wave_takes(unsigned ftiles, size_t P) { return P * (size_t)ftiles >= 512; }
+inline unsigned dense_wave_grid_x(unsigned mt, unsigned ftiles, size_t P)
+{
+    unsigned gx = (mt == 8 ? 768u : 512u) / ftiles;                // the resident grid ...
+    if (P < 32 * (size_t)gx) gx = 256u / ftiles;                   // ... or one workgroup per CU when that leaves a wave under 8 regions
+    if (gx < 1) gx = 1;
+    if (gx > (P + 3) / 4) gx = (unsigned)((P + 3) / 4);
+    const size_t per_wave = (P + (size_t)gx * 4 - 1) / ((size_t)gx * 4);
+    return (unsigned)((P + 4 * per_wave - 1) / (4 * per_wave));
+}
 inline size_t sparse_smem(size_t m) { return m * SPARSE_ROWS * FT * sizeof(float); }
 inline size_t dense_smem(unsigned mt) { return ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3); }
 
@@ -951,6 +1097,12 @@ int launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, cons
                   const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* pooled, const uint32_t* argmax,
                   const float* dpooled, const unsigned long long* act, float* slabs, size_t stride)
 {
+    if (act && dense_wave_takes(ftiles, P)) {
+        auto kern = scanpool_bprop_dense_act_wave_kernel<PT, MT>;
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
+        return 0;
+    }
     if (act) {
         auto kern = scanpool_bprop_dense_act_kernel<PT, MT>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -995,7 +1147,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     }
     // with max+avg pooling the dense half carries the maxima along
     const unsigned gxs = PT == DBK_PT_MAX ? sparse_grid_x(ftiles, P) : 0u;
-    const unsigned gxd = PT != DBK_PT_MAX ? dense_grid_x(mt, ftiles, P) : 0u;
+    const unsigned gxd = PT == DBK_PT_MAX ? 0u : (act && dense_wave_takes(ftiles, P)) ? dense_wave_grid_x(mt, ftiles, P) : dense_grid_x(mt, ftiles, P);
     const size_t smem_s = sparse_smem(m), smem_d = dense_smem(mt);
     DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
     float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float), st);
@@ -1053,7 +1205,7 @@ struct multi_args {
     size_t N, P;
     const uint32_t* R;
     unsigned first[dbk::MULTI_MAX + 1], gx[dbk::MULTI_MAX], ftiles[dbk::MULTI_MAX];
-    unsigned wide[dbk::MULTI_MAX];                                 // forward: the group goes through the wide kernel body
+    unsigned wide[dbk::MULTI_MAX];                                 // the group goes through the many-regions kernel body (forward: four filters per lane; backward: a wave per region)
     dbk::scan_group g[dbk::MULTI_MAX];
 };
 
@@ -1097,10 +1249,16 @@ template <int MT>
 __global__ __launch_bounds__(256) void scanpool_bprop_multi_kernel(const multi_args a)
 {
     wg_t wg;
-    const dbk::scan_group& j = a.g[multi_locate(a, wg)];
+    const unsigned gi = multi_locate(a, wg);
+    const dbk::scan_group& j = a.g[gi];
     if (j.ptype == DBK_PT_MAX) {
         if (threadIdx.x < 64)
             scanpool_bprop_sparse_body<DBK_PT_MAX, MT>(wg, a.m, j.F, j.X, a.N, a.P, j.pooled, j.argmax, j.dpooled, j.slabs, j.slab_stride);
+    } else if (a.wide[gi]) {
+        if (j.ptype == DBK_PT_ALL)
+            scanpool_bprop_dense_act_wave_body<DBK_PT_ALL, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
+        else
+            scanpool_bprop_dense_act_wave_body<DBK_PT_AVG, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
     } else if (j.ptype == DBK_PT_ALL) {
         scanpool_bprop_dense_act_body<DBK_PT_ALL, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
     } else {
@@ -1173,8 +1331,9 @@ int scan_bprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
     size_t total = 0;
     for (unsigned i = 0; i < n; ++i) {
         a.ftiles[i] = dbk::divup(g[i].F, FT);
-        a.wide[i] = 0;
-        a.gx[i] = g[i].ptype == DBK_PT_MAX ? sparse_grid_x(a.ftiles[i], P) : dense_grid_x(mt, a.ftiles[i], P);
+        a.wide[i] = g[i].ptype != DBK_PT_MAX && dense_wave_takes(a.ftiles[i], P);     // as the group's own launch would choose
+        a.gx[i] = g[i].ptype == DBK_PT_MAX ? sparse_grid_x(a.ftiles[i], P)
+                  : a.wide[i] ? dense_wave_grid_x(mt, a.ftiles[i], P) : dense_grid_x(mt, a.ftiles[i], P);
         a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
         g[i].slab_stride = 4 * m * (size_t)g[i].F + g[i].F;
         g[i].nslab = a.gx[i];

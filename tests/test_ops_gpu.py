@@ -338,6 +338,44 @@ def test_scanpool_bprop_with_activity_masks_equals_recomputation(ks, ptype, B, l
         ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, path="kmer", act=act)
 
 
+@pytest.mark.parametrize("ptype", ["avg", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(600, 0, 70, 24, 70), (520, 30, 45, 16, 16), (530, 1, 150, 7, 40), (130, 100, 260, 24, 300)])
+def test_scanpool_bprop_many_regions_kernel(ks, ptype, B, lo, hi, m, F):
+    """From 512 (region, filter tile) items on, the mask-driven dense backward deals whole regions to waves (no
+    barrier per region chunk). Its partial sums are other partial sums than the recomputing kernel's, so the two
+    agree to round-off, not bit for bit; it is checked against the float64 chain too, must be deterministic, and
+    must leave alone what lies outside its output. Regions of 0 to 260 rows (several 64-row rounds per region), all
+    three tap tiers, code 254 and N present."""
+    rng, W, b, X, R = _fused_case(7 * B + F, B, lo, hi, m, F, p254=0.02)
+    assert len(R) * ((F + 63) // 64) >= 512
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    act = ks.activity_words(Xd, Wd)
+    P0, I0 = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, act=act)
+    dPh = rng.standard_normal(tuple(P0.shape)).astype(np.float32)
+    dP = dev(dPh)
+    grads = []
+    for kw in (dict(), dict(act=act), dict(act=act)):
+        dW = dev(np.full(W.shape, 7.0, np.float32)); db = dev(np.full((1, F), 7.0, np.float32))
+        ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P0, I0, dP, dW, db, overwrite=True, **kw)
+        grads.append((host(dW), host(db)))
+    assert np.array_equal(grads[1][0], grads[2][0]) and np.array_equal(grads[1][1], grads[2][1])      # deterministic
+    assert_close(grads[1][0], grads[0][0], GRAD, "dW, masks vs recomputation")
+    assert_close(grads[1][1], grads[0][1], GRAD, "db, masks vs recomputation")
+    # against the unfused float64 chain
+    A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
+    dA = np.zeros_like(A)
+    orc.poolrgn_bprop(dA, R, dPh.astype(np.float64), host(I0) if I0 is not None else None, ptype)
+    dZ = orc.relu_bprop(dA, A)
+    dWr = np.zeros(W.shape)
+    orc.corr1ord_bprop_W(dWr, X, dZ)
+    assert_close(grads[1][0], dWr, GRAD, "dW vs float64 chain")
+    assert_close(grads[1][1], dZ.sum(axis=0, keepdims=True), GRAD, "db vs float64 chain")
+    # accumulate mode adds to what is there
+    dW = dev(np.full(W.shape, 0.5, np.float32)); db = dev(np.zeros((1, F), np.float32))
+    ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P0, I0, dP, dW, db, overwrite=False, act=act)
+    assert_close(host(dW) - 0.5, grads[1][0], GRAD, "accumulating call")
+
+
 @pytest.mark.parametrize("ptype", ["max", "all"])
 def test_scanpool_bprop_bulk_is_linear_and_independent_of_region_order(ks, ptype):
     """Size-independent properties of the fused backward at a bulk size (4096 sequences x 101 nt, 128 filters of
