@@ -268,6 +268,52 @@ __global__ __launch_bounds__(256) void corr1ord_planes_kernel(const float* __res
     }
 }
 
+// forward, float32, 17 to 24 taps, many rows: four filters per lane (4l .. 4l+3: the table's ordinary row layout read
+// as float4), ds_read_b128 on aligned 256-byte lines, a wave on its own 64 rows per round (no workgroup barrier after
+// the table is built), one 16-byte store per lane and row: a quarter wave writes a whole 256-byte row segment.
+// The register-plane kernel above is bound by the half-rate index-mode adds (0.36 ms for 6.24e9 adds); here the
+// adds are plain and the LDS delivers twice the bytes per clock of the one-filter-per-lane table kernel.
+// Same additions in the same order as above.
+template <int MT>
+__global__ __launch_bounds__(256) void corr1ord_wide_kernel(const float* __restrict__ W, unsigned m, unsigned F,
+                                                            const uint8_t* __restrict__ X, size_t n, float* __restrict__ Z)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* lut = reinterpret_cast<float*>(smem);                   // [MT*NL][FT]
+    const unsigned nw = blockDim.x >> 6;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned qd = lane >> 4, l = lane & 15;
+    uint8_t* xw = smem + (size_t)MT * NL * FT * sizeof(float) + (size_t)wave * wide_shape<MT>::xbytes;
+    const unsigned f0 = blockIdx.y * FT, f = f0 + 4 * l;
+    const size_t N = n + m - 1;
+    build_letter_table(lut, W, m, F, f0, MT);
+    __syncthreads();
+    const float4* lut4 = reinterpret_cast<const float4*>(lut) + l;
+    const bool vec = (F & 3u) == 0 && (reinterpret_cast<uintptr_t>(Z) & 15u) == 0;   // 16-byte stores allowed
+    const size_t span = 4 * PSUB;
+    for (size_t c0 = ((size_t)blockIdx.x * nw + wave) * span; c0 < n; c0 += (size_t)gridDim.x * nw * span) {
+        unsigned wq[wide_shape<MT>::words];
+        wide_stage<MT>(xw, X, N, c0, lane, wq);
+        float4 acc[PSUB];
+        scan16_wide<MT>(lut4, wq, acc);
+        const size_t i0 = c0 + PSUB * qd;
+#pragma unroll
+        for (int p = 0; p < PSUB; ++p) {
+            const size_t i = i0 + p;
+            if (i >= n) break;
+            float* dst = Z + i * F + f;
+            if (vec) {
+                if (f < F) *reinterpret_cast<float4*>(dst) = acc[p];
+            } else {
+                if (f + 0 < F) dst[0] = acc[p].x;
+                if (f + 1 < F) dst[1] = acc[p].y;
+                if (f + 2 < F) dst[2] = acc[p].z;
+                if (f + 3 < F) dst[3] = acc[p].w;
+            }
+        }
+    }
+}
+
 // filter gradient, pass 1: a lane keeps its filter's whole [letter][tap] column in registers; the window's
 // letters (scalars) pick the register plane each gradient value is added into through the register index
 // mode: one addition per (position, tap). "Mean of the four" letters collect in a plane of their own that
@@ -431,6 +477,20 @@ int launch_fprop(hipStream_t st, const T* W, size_t m, size_t F, const uint8_t* 
 {
     const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 24 ? 24 : (m <= 32 ? 32 : 0)));
     if constexpr (sizeof(T) == 4) {
+        // many rows of 17-24 taps: four filters per lane (enough waves of 64 rows to fill the GPU's 3072 wave slots)
+        if (mt == 24 && (n + 63) / 64 * dbk::divup(F, FT) >= 4096) {
+            const unsigned ftiles = dbk::divup(F, FT);
+            DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
+            const size_t smem_q = (size_t)24 * NL * FT * sizeof(float) + 4 * wide_shape<24>::xbytes;
+            if (smem_q <= lds_limit()) {
+                unsigned gx = 768u / ftiles;                       // three workgroups per CU are resident
+                if (gx < 1) gx = 1;
+                if (gx > dbk::divup(n, 256)) gx = dbk::divup(n, 256);
+                DBK_HIP(hipFuncSetAttribute((const void*)corr1ord_wide_kernel<24>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q));
+                hipLaunchKernelGGL(corr1ord_wide_kernel<24>, dim3(gx, ftiles), dim3(256), smem_q, st, (const float*)W, (unsigned)m, (unsigned)F, X, n, (float*)Z);
+                DBK_LAUNCH_OK();
+            }
+        }
         if (mt && mt <= 24) {
             const unsigned ftiles = dbk::divup(F, FT), chunk = 4 * WSUBS_W * PSUB;
             DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);

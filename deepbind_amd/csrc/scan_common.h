@@ -99,6 +99,67 @@ __device__ __forceinline__ void scan16_window(const T* __restrict__ lut, const u
     }
 }
 
+// ---- four filters per lane ---------------------------------------------------------------------------
+// A lane owns four filters and a table row holds [16 lanes][4 filters], so the 16 lanes of a quarter wave read one
+// aligned 256-byte line per ds_read_b128 (about twice the bytes per clock of 4-byte reads); the four quarters of a
+// wave work on four consecutive windows of PSUB positions. The letters of a quarter's window sit in vector
+// registers (they differ between the quarters).
+template <int MT> struct wide_shape {
+    static constexpr unsigned words = (PSUB + MT - 1 + 3) / 4;               // window words per quarter
+    static constexpr unsigned xbytes = (3 * PSUB + 4 * words + 15) & ~15u;   // letters a wave stages per round of 4 x PSUB positions
+    static_assert(xbytes <= 128, "a lane stages at most two letters per round");
+};
+
+// Letters of positions c0 .. c0 + xbytes - 1 into the wave's own LDS bytes (two per lane; past the end of X:
+// "nothing"), then this quarter's window words. A wave's LDS accesses execute in program order, so only the
+// compiler has to be kept from reordering them.
+template <int MT>
+__device__ __forceinline__ void wide_stage(uint8_t* xw, const uint8_t* __restrict__ X, size_t N, size_t c0, unsigned lane,
+                                           unsigned (&wq)[wide_shape<MT>::words])
+{
+    constexpr unsigned XB = wide_shape<MT>::xbytes;
+    const size_t g0 = c0 + lane, g1 = g0 + 64;
+    const unsigned v0 = g0 < N ? letter_of(X[g0]) : 5u;
+    const unsigned v1 = (lane + 64 < XB && g1 < N) ? letter_of(X[g1]) : 5u;
+    __builtin_amdgcn_wave_barrier();                               // the previous round's window reads come first
+    xw[lane] = (uint8_t)v0;
+    if (lane + 64 < XB) xw[lane + 64] = (uint8_t)v1;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const unsigned* src = reinterpret_cast<const unsigned*>(xw + PSUB * (lane >> 4));
+#pragma unroll
+    for (unsigned t = 0; t < wide_shape<MT>::words; ++t) wq[t] = src[t];
+}
+
+// acc[p] = sum over taps j < MT of the table row (j, letter at window position p + j), four filters at a time,
+// taps in ascending order per position. lut4: the table as float4, already offset by this lane's place in a row.
+// One bit-field extract and one address add per letter serve up to PSUB reads with immediate offsets.
+template <int MT>
+__device__ __forceinline__ void scan16_wide(const float4* __restrict__ lut4, const unsigned (&wq)[wide_shape<MT>::words], float4 (&acc)[PSUB])
+{
+#pragma unroll
+    for (int p = 0; p < PSUB; ++p) acc[p] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+    for (int q = 0; q < PSUB + MT - 1; ++q) {
+        const unsigned letter = (wq[q >> 2] >> ((q & 3) * 8)) & 0xffu;
+        const float4* col = lut4 + letter * 16u;
+#pragma unroll
+        for (int p = 0; p < PSUB; ++p) {
+            const int j = q - p;
+            if (j >= 0 && j < MT) {
+                const float4 v = col[j * NL * 16];
+                acc[p].x += v.x; acc[p].y += v.y; acc[p].z += v.z; acc[p].w += v.w;
+            }
+        }
+        if ((q & 3) == 3) {
+            // pin the running sums (see scan16_window)
+#pragma unroll
+            for (int p = 0; p < PSUB; ++p) asm volatile("" : "+v"(acc[p].x), "+v"(acc[p].y), "+v"(acc[p].z), "+v"(acc[p].w));
+        }
+    }
+}
+
 // ---- filter-gradient accumulation through the VGPR index mode -------------------------------------
 // dW[tap j][letter c][filter] += g[position p] for every (p, j) of a window whose letter at p + j is c.
 // The letter is the same for all lanes (a scalar), the filter is the lane. Spelled with ordinary

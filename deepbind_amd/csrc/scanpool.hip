@@ -173,11 +173,7 @@ __global__ __launch_bounds__(256) void scanpool_fprop_kernel(const float* __rest
 // quarters); one bit-field extract and one address add per letter serve up to 16 (position, tap) reads.
 // Per position the taps are added in ascending order, as everywhere else: maxima and argmax are the bits of
 // the kernel above; averages add the same rectified values in another order (quarter by quarter).
-constexpr unsigned WIDE_SPAN = 64;                                // positions per wave and round
-template <int MT> struct wide_shape {
-    static constexpr unsigned words = (PSUB + MT - 1 + 3) / 4;    // window words per quarter
-    static constexpr unsigned xbytes = (3 * PSUB + 4 * words + 15) & ~15u;   // letters staged per wave and round
-};
+constexpr unsigned WIDE_SPAN = 4 * PSUB;                          // positions per wave and round
 
 template <int PT, bool WANT_ARGMAX, int MT>
 __device__ __forceinline__ void scanpool_fprop_wide_body(const wg_t wg, const float* __restrict__ W, const float* __restrict__ bias,
@@ -188,7 +184,6 @@ __device__ __forceinline__ void scanpool_fprop_wide_body(const wg_t wg, const fl
 {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr unsigned NWORD = wide_shape<MT>::words, XB = wide_shape<MT>::xbytes;
-    static_assert(XB % 16 == 0 && NWORD == 10, "the window loads below are two 16-byte and one 8-byte read");
     const unsigned nw = blockDim.x >> 6;
     float* lut = reinterpret_cast<float*>(smem);                   // [MT*NL][16][4]
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -209,49 +204,11 @@ __device__ __forceinline__ void scanpool_fprop_wide_body(const wg_t wg, const fl
         unsigned xi[4] = {0u, 0u, 0u, 0u};                        // row of the maximum, relative to a
         for (size_t c0 = a; c0 < b; c0 += WIDE_SPAN) {
             const unsigned rows = (unsigned)((b - c0) < WIDE_SPAN ? (b - c0) : WIDE_SPAN);
-            // ---- letters of positions c0 .. c0 + XB - 1 (two per lane), then this quarter's window words
-            {
-                const size_t g0 = c0 + lane, g1 = g0 + 64;
-                const unsigned v0 = g0 < N ? letter_of(X[g0]) : 5u;
-                const unsigned v1 = (lane + 64 < XB && g1 < N) ? letter_of(X[g1]) : 5u;
-                __builtin_amdgcn_wave_barrier();                   // the previous round's window reads come first
-                xw[lane] = (uint8_t)v0;
-                if (lane + 64 < XB) xw[lane + 64] = (uint8_t)v1;
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            }
+            // ---- the round's letters, then this quarter's window: 16 positions x MT taps x 4 filters
             unsigned wq[NWORD];
-            {
-                const uint4 w0 = *reinterpret_cast<const uint4*>(xw + PSUB * qd);
-                const uint4 w1 = *reinterpret_cast<const uint4*>(xw + PSUB * qd + 16);
-                const uint2 w2 = *reinterpret_cast<const uint2*>(xw + PSUB * qd + 32);
-                wq[0] = w0.x; wq[1] = w0.y; wq[2] = w0.z; wq[3] = w0.w;
-                wq[4] = w1.x; wq[5] = w1.y; wq[6] = w1.z; wq[7] = w1.w;
-                wq[8] = w2.x; wq[9] = w2.y;
-            }
-            // ---- the window: 16 positions x MT taps x 4 filters
+            wide_stage<MT>(xw, X, N, c0, lane, wq);
             float4 acc[PSUB];
-#pragma unroll
-            for (int p = 0; p < PSUB; ++p) acc[p] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-#pragma unroll
-            for (int q = 0; q < PSUB + MT - 1; ++q) {
-                const unsigned letter = (wq[q >> 2] >> ((q & 3) * 8)) & 0xffu;
-                const float4* col = lut4 + letter * 16u;
-#pragma unroll
-                for (int p = 0; p < PSUB; ++p) {
-                    const int j = q - p;
-                    if (j >= 0 && j < MT) {
-                        const float4 v = col[j * NL * 16];
-                        acc[p].x += v.x; acc[p].y += v.y; acc[p].z += v.z; acc[p].w += v.w;
-                    }
-                }
-                if ((q & 3) == 3) {
-                    // pin the running sums (see scan16_window)
-#pragma unroll
-                    for (int p = 0; p < PSUB; ++p) asm volatile("" : "+v"(acc[p].x), "+v"(acc[p].y), "+v"(acc[p].z), "+v"(acc[p].w));
-                }
-            }
+            scan16_wide<MT>(lut4, wq, acc);
             // ---- bias, rectifier, pooling; optionally the activity masks of the 64 rows
             const unsigned pq = PSUB * qd;                         // first position of this quarter's window
             unsigned long long mine = 0ull;

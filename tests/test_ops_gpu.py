@@ -33,7 +33,10 @@ def sm():
 
 
 # ------------------------------------------------------------------------------------------ scan
-@pytest.mark.parametrize("N,m,F", [(300, 24, 16), (1000, 16, 64), (777, 5, 70), (24, 24, 3), (5000, 24, 200), (130, 32, 17)])
+@pytest.mark.parametrize("N,m,F", [(300, 24, 16), (1000, 16, 64), (777, 5, 70), (24, 24, 3), (5000, 24, 200), (130, 32, 17),
+                                   # many rows of 17-24 taps: the four-filters-per-lane kernel (16-byte stores; scalar stores when
+                                   # the filter count is no multiple of four; a last tile with one filter)
+                                   (70400, 24, 256), (140100, 19, 70), (263000, 24, 17)])
 def test_corr1ord_bit_exact(ks, N, m, F):
     rng = np.random.default_rng(N + m + F)
     X = random_codes(rng, N, 0.05, 0.03)
