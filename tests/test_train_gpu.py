@@ -612,18 +612,20 @@ def test_groups_stepped_in_shared_launches_match_groups_stepped_alone_across_cha
         assert host(a.rng_counter) == host(b.rng_counter)
 
 
-@pytest.mark.parametrize("case", ["mixed_pools_revcomp_input_dropout", "eight_taps", "ten_nets", "different_lengths", "plain_momentum"])
+@pytest.mark.parametrize("case", ["mixed_pools_revcomp_input_dropout", "eight_taps", "ten_nets", "different_lengths", "plain_momentum",
+                                  "many_regions", "many_regions_16_taps"])
 def test_nets_stepped_through_one_call_end_with_the_bits_of_their_own_steps(case):
     """dbk_train_steps either runs each phase of the step as one launch for all the nets (same filter-length tier, a
     look-ahead vector each, at most eight nets) or steps them one after the other; both ways every net must end
     with the bits of its own dbk_train_step. Covers avg / all / max pooling side by side, reverse-complement
     pairs, input dropout (each net scans its own dropped copy), mse and nll, 8-, 16- and 24-tap tiers, more nets
-    than one call takes, and the two fallbacks (nets of different tiers, a net without Nesterov momentum)."""
+    than one call takes, the two fallbacks (nets of different tiers, a net without Nesterov momentum), and batches
+    of enough regions for the many-regions kernel bodies (four filters per lane forward, a wave per region backward)."""
     from deepbind_amd import data
     from deepbind_amd.model import SequenceNet, _native_steps
     rng = np.random.default_rng(11)
     revcomp = case == "mixed_pools_revcomp_input_dropout"
-    B = 40
+    B = 600 if case.startswith("many_regions") else 40
     seqs = ["".join(rng.choice(list("ACGTN"), p=[.24, .24, .24, .24, .04], size=int(rng.integers(18, 45)))) for _ in range(B)]
     kw = dict(rate=0.05, momentum=0.9, decay_conv=1e-3, decay_full=1e-3, weight_decay_start=1)
     if case == "mixed_pools_revcomp_input_dropout":
@@ -639,6 +641,10 @@ def test_nets_stepped_through_one_call_end_with_the_bits_of_their_own_steps(case
     elif case == "ten_nets":
         specs = [dict(nmodel=1 + i % 3, pool=("max", "all", "avg")[i % 3], hidden=(0, 16)[i % 2], loss="nll", **kw) for i in range(10)]
         lens = [24] * 10
+    elif case.startswith("many_regions"):
+        specs = [dict(nmodel=3, pool="avg", hidden=0, loss="mse", dropout=0.25, **kw), dict(nmodel=5, pool="all", hidden=8, loss="nll", **kw),
+                 dict(nmodel=4, pool="max", hidden=0, loss="nll", input_dropout=0.1, **kw)]
+        lens = [24 if case == "many_regions" else 16] * 3
     elif case == "different_lengths":
         specs = [dict(nmodel=2, pool="all", hidden=0, loss="nll", **kw), dict(nmodel=3, pool="max", hidden=8, loss="nll", **kw)]
         lens = [8, 24]
