@@ -24,6 +24,7 @@ if ROOT not in sys.path:
 
 FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published FP32 vector peak (FMA = 2 FLOP)
 HBM_PEAK_GBS = 8000.0
+LDS_PEAK_TBS = 216 * 256 * 2.4e9 / 1e12     # aligned ds_read_b128 as measured: 216 B/clk/CU x 256 CUs x 2.4 GHz
 
 
 def cpu_baseline(cfg, nseq_c, nseq_np):
@@ -305,6 +306,7 @@ def main():
     adds_per_s = adds / (scan_ms * 1e-3)
     # algorithmic HBM bytes of the scan+pool launch: sequence bytes in, filters in, pooled features out
     hbm_bytes = cfg["X"].size + p["Wc"].nbytes + p["bc"].nbytes + nseq * spec.F * 4
+    lds_bytes = positions * spec.F * ((spec.m + 2) // 3 + ((spec.m + 2) // 3) % 2) * 4     # an even number of 3-tap groups
     out = {
         "metric": "seq_positions_per_sec_fwd_scan_pool",
         "value": positions * args.steps / elapsed,
@@ -333,6 +335,10 @@ def main():
             "algorithmic_adds_per_issuable_lane_op": adds_per_s / (1024 * 64 * 1.0e9),
             "hbm": {"algorithmic_bytes_per_launch": hbm_bytes, "achieved_GBs": hbm_bytes / (scan_ms * 1e-3) / 1e9,
                     "peak_GBs": HBM_PEAK_GBS, "frac": hbm_bytes / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+            # what the table kernel is bound by: every executed add consumes one 4-byte table entry from LDS
+            # (ceil(m/3) entries per position and filter); measured rate of aligned ds_read_b128: 216 B/clk/CU
+            "lds": {"bytes_per_launch": lds_bytes, "achieved_TBs": lds_bytes / (scan_ms * 1e-3) / 1e12,
+                    "measured_peak_TBs": LDS_PEAK_TBS, "frac": lds_bytes / (scan_ms * 1e-3) / 1e12 / LDS_PEAK_TBS},
         },
     }
     if not args.no_train:
