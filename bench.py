@@ -81,7 +81,7 @@ def measured_traffic(workload):
     return None
 
 
-def train_throughput(steps=30, warmup=5):
+def train_throughput(steps=100, warmup=10):
     """Secondary figures: whole train steps (forward + backward + Nesterov update) per second on the
     three training configurations, fused mode: each step issued natively by one library call (the top-level
     figures; the calibration batch's four architecture groups share every launch) and as one captured HIP
