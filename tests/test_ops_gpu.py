@@ -244,7 +244,7 @@ def test_scanpool_fprop_wide_kernel(ks, ptype, B, lo, hi, m, F):
 
 
 def test_scanpool_general_path_picks_the_wide_kernel_for_many_regions(ks):
-    """From 1024 (region, tile) items on, the general path runs the many-regions kernel: same results as forcing it."""
+    """From 512 (region, tile) items on, the general path runs the many-regions kernel: same results as forcing it."""
     rng, W, b, X, R = _fused_case(5, 1100, 18, 40, 24, 40, p254=0.01)
     Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
     for ptype in ("max", "avg", "all"):
