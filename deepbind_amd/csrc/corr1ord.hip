@@ -268,7 +268,7 @@ __global__ __launch_bounds__(256) void corr1ord_planes_kernel(const float* __res
     }
 }
 
-// forward, float32, 17 to 24 taps, many rows: four filters per lane (4l .. 4l+3: the table's ordinary row layout read
+// forward, float32, 9 to 24 taps, many rows: four filters per lane (4l .. 4l+3: the table's ordinary row layout read
 // as float4), ds_read_b128 on aligned 256-byte lines, a wave on its own 64 rows per round (no workgroup barrier after
 // the table is built), one 16-byte store per lane and row: a quarter wave writes a whole 256-byte row segment.
 // The register-plane kernel above is bound by the half-rate index-mode adds (0.36 ms for 6.24e9 adds); here the
@@ -477,17 +477,18 @@ int launch_fprop(hipStream_t st, const T* W, size_t m, size_t F, const uint8_t* 
 {
     const unsigned mt = m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 24 ? 24 : (m <= 32 ? 32 : 0)));
     if constexpr (sizeof(T) == 4) {
-        // many rows of 17-24 taps: four filters per lane (enough waves of 64 rows to fill the GPU's 3072 wave slots)
-        if (mt == 24 && (n + 63) / 64 * dbk::divup(F, FT) >= 4096) {
+        // many rows of 9-24 taps: four filters per lane (enough waves of 64 rows to fill the GPU's 3072 wave slots)
+        if ((mt == 16 || mt == 24) && (n + 63) / 64 * dbk::divup(F, FT) >= 4096) {
             const unsigned ftiles = dbk::divup(F, FT);
             DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
-            const size_t smem_q = (size_t)24 * NL * FT * sizeof(float) + 4 * wide_shape<24>::xbytes;
+            const size_t smem_q = (size_t)mt * NL * FT * sizeof(float) + 4 * (mt == 16 ? wide_shape<16>::xbytes : wide_shape<24>::xbytes);
             if (smem_q <= lds_limit()) {
                 unsigned gx = 768u / ftiles;                       // three workgroups per CU are resident
                 if (gx < 1) gx = 1;
                 if (gx > dbk::divup(n, 256)) gx = dbk::divup(n, 256);
-                DBK_HIP(hipFuncSetAttribute((const void*)corr1ord_wide_kernel<24>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q));
-                hipLaunchKernelGGL(corr1ord_wide_kernel<24>, dim3(gx, ftiles), dim3(256), smem_q, st, (const float*)W, (unsigned)m, (unsigned)F, X, n, (float*)Z);
+                auto kq = mt == 16 ? corr1ord_wide_kernel<16> : corr1ord_wide_kernel<24>;
+                DBK_HIP(hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q));
+                hipLaunchKernelGGL(kq, dim3(gx, ftiles), dim3(256), smem_q, st, (const float*)W, (unsigned)m, (unsigned)F, X, n, (float*)Z);
                 DBK_LAUNCH_OK();
             }
         }

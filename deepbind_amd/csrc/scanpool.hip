@@ -965,7 +965,8 @@ inline unsigned dense_grid_x(unsigned mt, unsigned ftiles, size_t P)
 }
 // The wide forward kernel (four filters per lane, a wave per region) pays off once there are enough (region, tile)
 // items to keep every CU's LDS busy; a small batch is latency-bound and better off with four waves per region.
-inline bool wide_takes(size_t m, unsigned ftiles, size_t P) { return m > 16 && m <= 24 && P * (size_t)ftiles >= 512; }
+inline bool wide_takes(size_t m, unsigned ftiles, size_t P) { return m > 8 && m <= 24 && P * (size_t)ftiles >= 512; }
+inline unsigned wide_tier(size_t m) { return m <= 16 ? 16u : 24u; }
 inline unsigned wide_grid_x(unsigned ftiles, size_t P)
 {
     unsigned gx = 768u / ftiles;                                  // three workgroups per CU are resident (150-160 registers)
@@ -973,7 +974,7 @@ inline unsigned wide_grid_x(unsigned ftiles, size_t P)
     if (gx > (P + 3) / 4) gx = (unsigned)((P + 3) / 4);           // a workgroup walks four regions at a time
     return gx;
 }
-inline size_t wide_smem() { return (size_t)24 * NL * FT * sizeof(float) + 4 * wide_shape<24>::xbytes; }
+inline size_t wide_smem(unsigned mt) { return (size_t)mt * NL * FT * sizeof(float) + 4 * (mt == 16 ? wide_shape<16>::xbytes : wide_shape<24>::xbytes); }
 // The wave-per-region dense backward: same threshold as the wide forward (enough regions to keep every wave busy
 // with whole regions); the smallest grid that gives every wave the same number of regions as the resident grid would.
 inline bool dense_wave_takes(unsigned ftiles, size_t P) { return P * (size_t)ftiles >= 512; }
@@ -1010,18 +1011,14 @@ template <int PT>
 int launch_fprop_wide(hipStream_t st, unsigned ftiles, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                       const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, unsigned long long* act)
 {
-    const size_t smem = wide_smem();
+    const unsigned mt = wide_tier(m);
+    const size_t smem = wide_smem(mt);
     DBK_CHECK(smem <= lds_limit(), "ValueError: the wide forward kernel needs %zu bytes of LDS (limit %zu)", smem, lds_limit());
     const unsigned gx = wide_grid_x(ftiles, P);
-    if (argmax) {
-        auto kern = scanpool_fprop_wide_kernel<PT, true, 24>;
-        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, act);
-    } else {
-        auto kern = scanpool_fprop_wide_kernel<PT, false, 24>;
-        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, act);
-    }
+    auto kern = argmax ? (mt == 16 ? scanpool_fprop_wide_kernel<PT, true, 16> : scanpool_fprop_wide_kernel<PT, true, 24>)
+                       : (mt == 16 ? scanpool_fprop_wide_kernel<PT, false, 16> : scanpool_fprop_wide_kernel<PT, false, 24>);
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, act);
     DBK_LAUNCH_OK();
 }
 
@@ -1181,14 +1178,14 @@ __global__ __launch_bounds__(256) void scanpool_fprop_multi_kernel(const multi_a
     wg_t wg;
     const unsigned gi = multi_locate(a, wg);
     const dbk::scan_group& j = a.g[gi];
-    if constexpr (MT == 24) {
+    if constexpr (MT == 16 || MT == 24) {
         if (a.wide[gi]) {
             if (j.ptype == DBK_PT_MAX)
-                scanpool_fprop_wide_body<DBK_PT_MAX, true, 24>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr);
+                scanpool_fprop_wide_body<DBK_PT_MAX, true, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr);
             else if (j.ptype == DBK_PT_ALL)
-                scanpool_fprop_wide_body<DBK_PT_ALL, true, 24>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.act);
+                scanpool_fprop_wide_body<DBK_PT_ALL, true, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.act);
             else
-                scanpool_fprop_wide_body<DBK_PT_AVG, false, 24>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, nullptr, j.act);
+                scanpool_fprop_wide_body<DBK_PT_AVG, false, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, nullptr, j.act);
             return;
         }
     }
@@ -1254,7 +1251,7 @@ bool scan_multi_takes(size_t m, size_t N, size_t P, unsigned n, const scan_group
         // a max-pooling group on a batch large enough for the k-mer table goes there when stepped alone (other sums, other bits)
         if (g[i].ptype == DBK_PT_MAX && dbk_scanpool_kmer::takes(m, g[i].F, N, P)) return false;
     }
-    return fprop_smem(multi_tier(m), m) <= lds_limit() && wide_smem() <= lds_limit() && sparse_smem(m) <= lds_limit() && dense_smem(multi_tier(m)) <= lds_limit();
+    return fprop_smem(multi_tier(m), m) <= lds_limit() && wide_smem(24) <= lds_limit() && sparse_smem(m) <= lds_limit() && dense_smem(multi_tier(m)) <= lds_limit();
 }
 
 int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size_t P, unsigned n, const scan_group* g)
@@ -1273,7 +1270,7 @@ int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
         if (a.wide[i]) any_wide = true;
     }
     size_t smem = fprop_smem(mt, m);
-    if (any_wide && wide_smem() > smem) smem = wide_smem();
+    if (any_wide && wide_smem(wide_tier(m)) > smem) smem = wide_smem(wide_tier(m));
     if (mt == 8) return launch_multi(scanpool_fprop_multi_kernel<8>, st, smem, a);
     if (mt == 16) return launch_multi(scanpool_fprop_multi_kernel<16>, st, smem, a);
     return launch_multi(scanpool_fprop_multi_kernel<24>, st, smem, a);
@@ -1341,7 +1338,7 @@ int dbk_scanpool_fprop_wide(dbk_stream_t stream, const float* W, const float* bi
                             float* pooled, uint32_t* argmax, uint64_t* act)
 {
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
-    DBK_CHECK(m > 16 && m <= 24, "NotImplementedError: the wide forward kernel takes filters of 17 to 24 taps (got %zu)", m);
+    DBK_CHECK(m > 8 && m <= 24, "NotImplementedError: the wide forward kernel takes filters of 9 to 24 taps (got %zu)", m);
     DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
     DBK_CHECK(!argmax || (double)N * (double)nfilter <= 4294967296.0,
               "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);

@@ -135,7 +135,7 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream,
                                float* pooled, uint32_t* argmax, uint64_t* act);
 
 /* Same contract through the general path's kernel for many regions regardless of problem size: four filters
- * per lane and one wave per region, for filters of 17 to 24 taps (NotImplementedError otherwise).
+ * per lane and one wave per region, for filters of 9 to 24 taps (NotImplementedError otherwise).
  * dbk_scanpool_fprop_general picks it once regions x filter tiles reach 512, where the one-filter-per-lane kernel
  * is bound by the rate of its 4-byte LDS reads. Per position the taps are added in the same order, so maxima,
  * argmax and activity masks are the same bits; averages add the same values in another order. */

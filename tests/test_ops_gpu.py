@@ -36,7 +36,7 @@ def sm():
 @pytest.mark.parametrize("N,m,F", [(300, 24, 16), (1000, 16, 64), (777, 5, 70), (24, 24, 3), (5000, 24, 200), (130, 32, 17),
                                    # many rows of 17-24 taps: the four-filters-per-lane kernel (16-byte stores; scalar stores when
                                    # the filter count is no multiple of four; a last tile with one filter)
-                                   (70400, 24, 256), (140100, 19, 70), (263000, 24, 17)])
+                                   (70400, 24, 256), (140100, 19, 70), (263000, 24, 17), (70400, 16, 256), (140100, 9, 70)])
 def test_corr1ord_bit_exact(ks, N, m, F):
     rng = np.random.default_rng(N + m + F)
     X = random_codes(rng, N, 0.05, 0.03)
@@ -208,11 +208,12 @@ def test_scanpool_fprop(ks, general, ptype, B, lo, hi, m, F):
 
 
 @pytest.mark.parametrize("ptype", ["max", "avg", "all"])
-@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (40, 20, 40, 24, 144), (23, 0, 300, 17, 70), (300, 30, 70, 20, 64)])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (40, 20, 40, 24, 144), (23, 0, 300, 17, 70), (300, 30, 70, 20, 64),
+                                          (128, 38, 41, 16, 16), (50, 0, 200, 9, 130), (200, 30, 70, 13, 64)])
 def test_scanpool_fprop_wide_kernel(ks, ptype, B, lo, hi, m, F):
     """The many-regions forward kernel (four filters per lane, a wave per region), forced on small inputs: against
     the unfused chain, and bit for bit against the one-filter-per-lane kernel where the two add in the same order
-    (maxima, argmax, activity masks); regions of 0 to 300 rows, code 254 and N present, filter counts that leave
+    (maxima, argmax, activity masks); regions of 0 to 300 rows, both tap tiers (9-16, 17-24), code 254 and N present, filter counts that leave
     lanes and whole quarters of a tile empty."""
     rng, W, b, X, R = _fused_case(B + m + F + 1, B, lo, hi, m, F, p254=0.01)
     A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
@@ -243,9 +244,10 @@ def test_scanpool_fprop_wide_kernel(ks, ptype, B, lo, hi, m, F):
     assert np.array_equal(host(P2)[keep], got[keep])
 
 
-def test_scanpool_general_path_picks_the_wide_kernel_for_many_regions(ks):
+@pytest.mark.parametrize("m", [24, 16])
+def test_scanpool_general_path_picks_the_wide_kernel_for_many_regions(ks, m):
     """From 512 (region, tile) items on, the general path runs the many-regions kernel: same results as forcing it."""
-    rng, W, b, X, R = _fused_case(5, 1100, 18, 40, 24, 40, p254=0.01)
+    rng, W, b, X, R = _fused_case(5, 1100, 18, 40, m, 40, p254=0.01)
     Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
     for ptype in ("max", "avg", "all"):
         P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="general")
