@@ -186,7 +186,8 @@ __device__ __forceinline__ void scanpool_fprop_wide_body(const wg_t wg, const fl
     constexpr unsigned NWORD = wide_shape<MT>::words, XB = wide_shape<MT>::xbytes;
     const unsigned nw = blockDim.x >> 6;
     float* lut = reinterpret_cast<float*>(smem);                   // [MT*NL][16][4]
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave's index, region bounds and loop control are wave-uniform: kept in scalar registers
+    const unsigned lane = threadIdx.x & 63, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const unsigned qd = lane >> 4, l = lane & 15;
     uint8_t* xw = smem + (size_t)MT * NL * FT * sizeof(float) + (size_t)wave * XB;   // this wave's letters
     const unsigned f0 = wg.y * FT;
@@ -199,7 +200,7 @@ __device__ __forceinline__ void scanpool_fprop_wide_body(const wg_t wg, const fl
     const float4* lut4 = reinterpret_cast<const float4*>(lut) + l;
 
     for (size_t r = (size_t)wg.x * nw + wave; r < P; r += (size_t)wg.gx * nw) {
-        const size_t a = R[2 * r], b = R[2 * r + 1];
+        const size_t a = (unsigned)__builtin_amdgcn_readfirstlane((int)R[2 * r]), b = (unsigned)__builtin_amdgcn_readfirstlane((int)R[2 * r + 1]);
         float mx[4] = {-1.0f, -1.0f, -1.0f, -1.0f}, sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         unsigned xi[4] = {0u, 0u, 0u, 0u};                        // row of the maximum, relative to a
         for (size_t c0 = a; c0 < b; c0 += WIDE_SPAN) {
