@@ -814,7 +814,8 @@ __device__ __forceinline__ void scanpool_bprop_dense_act_wave_body(const wg_t wg
     static_assert(XB <= 128, "a lane stages at most two letters per round");
     float* lut = reinterpret_cast<float*>(smem);                   // [MT*4][FT]: only the cross-wave fold at the end uses it
     float* dbacc = lut + (size_t)MT * 4 * FT;                      // [nw][FT]
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave's index, region bounds and loop control are wave-uniform: kept in scalar registers
+    const unsigned lane = threadIdx.x & 63, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     uint8_t* xw = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT) + (size_t)wave * XB;
     const unsigned f0 = wg.y * FT, f = f0 + lane;
     const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
@@ -836,12 +837,13 @@ __device__ __forceinline__ void scanpool_bprop_dense_act_wave_body(const wg_t wg
     size_t r = (size_t)wg.x * nw + wave;
     size_t a = 0, b = 0;
     pooled_in q = { 0.0f, 0.0f, 0.0f, 0u };
-    if (r < P) { a = R[2 * r]; b = R[2 * r + 1]; q = load_pooled(r); }
+    auto bound = [&](size_t idx) -> size_t { return (unsigned)__builtin_amdgcn_readfirstlane((int)R[idx]); };
+    if (r < P) { a = bound(2 * r); b = bound(2 * r + 1); q = load_pooled(r); }
     while (r < P) {                                                // uniform over the wave
         const size_t rn = r + step;
         size_t na = 0, nb = 0;
         pooled_in nq = { 0.0f, 0.0f, 0.0f, 0u };
-        if (rn < P) { na = R[2 * rn]; nb = R[2 * rn + 1]; nq = load_pooled(rn); }
+        if (rn < P) { na = bound(2 * rn); nb = bound(2 * rn + 1); nq = load_pooled(rn); }
         const float gavg = q.davg / (float)(b - a);
         float gmax = 0.0f;                                         // max+avg pooling: the winning row also gets the max gradient
         size_t imax = ~(size_t)0;
