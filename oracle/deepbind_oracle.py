@@ -21,6 +21,10 @@ checks live in tests/test_oracle_pins.py):
                         (closed form only): PARITY UNPINNED beyond the per-block np.dot identity
   weight_cost         - scalar loops over each model's own weights
   gradstep*           - three-line closed form (gradstep.cu:41-72) vs. an unrolled scalar loop
+  train_step          - (tests/test_oracle_train_step.py) models stepped together == each model stepped alone
+                        with scalar rates; two Nesterov steps written out from the docstring recurrence with
+                        central-finite-difference gradients of loss + L1 cost; a hand-written worked case of
+                        the decay block lengths rows/ninst and size/ninst; both gates at start-1 and start
   dropout masks       - the reference draws them from cuRAND (not reproducible without the
                         CUDA SDK): masks are INPUTS here (uniforms U supplied by the caller);
                         the random stream itself is PARITY UNPINNED
