@@ -124,22 +124,6 @@ def train_throughput(steps=100, warmup=10):
     return out
 
 
-def issue_rates(iters=4000):
-    """Sustained issue rate of one SIMD (1e9 wave-instructions/s) for the instructions the scan kernels are made of,
-    at 1-8 resident waves per SIMD: the library's probe (64 independent instructions per round on 8 registers)."""
-    import ctypes
-    from deepbind_amd import _lib
-    out = {}
-    for kind, name in enumerate(("v_add_f32", "v_fma_f32", "v_max_f32", "v_max3_f32", "v_add_f32 (VGPR index mode)")):
-        row = {}
-        for waves in (1, 2, 3, 4, 6, 8):
-            r = ctypes.c_double()
-            _lib.call("dbk_probe_valu_issue", kind, waves, iters, ctypes.addressof(r))
-            row["%d waves/SIMD" % waves] = round(r.value, 3)
-        out[name] = row
-    return out
-
-
 def ops_throughput(reps=5):
     """Per-operator figures for the drop-in operators and the general fused kernels on a mid-size batch
     (8192 sequences x 101 nt, 16 models x 16 motifs x width 24: N = 1.02 M rows, F = 256, map = 1.04 GB).
@@ -243,7 +227,6 @@ def main():
     ap.add_argument("--no-train", action="store_true", help="skip the secondary train-step throughput figures")
     ap.add_argument("--ops", action="store_true", help="only the per-operator figures of the drop-in and general fused kernels")
     ap.add_argument("--train-only", action="store_true", help="only the train-step figures (for profiling the training kernels)")
-    ap.add_argument("--issue-rates", action="store_true", help="only the vector-ALU issue rates the kernels' instruction counts are priced with")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain copy kernel over 1 GiB (reference point for the HBM byte counters)")
     args = ap.parse_args()
@@ -256,9 +239,6 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
 
-    if args.issue_rates:
-        print(json.dumps({"valu_issue": issue_rates()}))
-        return
     if args.train_only:
         print(json.dumps({"train": train_throughput(steps=args.steps, warmup=args.warmup)}))
         return

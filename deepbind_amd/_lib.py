@@ -80,7 +80,6 @@ _SIGNATURES = {
     "dbk_train_step": [_P, _P],
     "dbk_train_steps": [_P, _Z, _P],
     "dbk_train_step_args_size": [],
-    "dbk_probe_valu_issue": [_I, _I, _I, _P],
 }
 
 

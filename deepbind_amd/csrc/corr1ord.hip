@@ -541,7 +541,7 @@ inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, 
     if (gy > nchunk) gy = nchunk;
     const size_t nelem = 4 * m * F;
     float* partial = (float*)dbk::workspace(nelem * gy * sizeof(float), st);
-    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", nelem * gy * sizeof(float));
+    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", nelem * gy * sizeof(float), dbk::workspace_error());
     const size_t smem = (size_t)mt * 4 * FT * sizeof(float) + ((chunk + mt - 1 + 7) & ~(size_t)3);
     auto kern = mt == 8 ? corr1ord_bprop_W_window_kernel<8> : mt == 16 ? corr1ord_bprop_W_window_kernel<16> : corr1ord_bprop_W_window_kernel<24>;
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -578,7 +578,7 @@ int launch_bprop_W(hipStream_t st, T* dW, size_t m, size_t F, const uint8_t* X, 
     if (gy > nchunk) gy = nchunk;
     size_t nelem = 4 * m * F;
     T* partial = (T*)dbk::workspace(nelem * gy * sizeof(T), st);
-    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", nelem * gy * sizeof(T));
+    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", nelem * gy * sizeof(T), dbk::workspace_error());
     auto kern = corr1ord_bprop_W_partial_kernel<T>;
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3(ftiles, gy), dim3(nw * 64), smem, st, partial, (unsigned)m, (unsigned)F, X, n, dZ, chunk, nchunk);

@@ -16,11 +16,14 @@ void clear_error();
 
 // Device scratch that grows on demand and lives until the process ends. One buffer per (device, stream):
 // launches are ordered within a stream, so consecutive calls on it can share the buffer, and calls on
-// different streams never do. At most 64 distinct streams per device; null when that is exceeded or
-// when memory runs out. Growing a buffer synchronises the device (and so cannot happen under capture).
+// different streams never do. 64 stream slots per device; when all are taken the slot used longest ago
+// passes to the new stream (after draining the device). Growing a buffer or recycling a slot synchronises
+// the device, which a stream under capture does not allow: null then, and when memory runs out, with the
+// reason in workspace_error().
 // `which` selects one of two independent buffers of the stream (a call that must keep one kernel's partial
 // results while another kernel fills its own uses the second).
 void* workspace(size_t bytes, hipStream_t stream, int which = 0);
+const char* workspace_error();
 
 // While dbk_train_step runs, dbk_head_train and dbk_scanpool_bprop leave their partial results unreduced and
 // describe them here instead: the step's last kernel adds them up (in the order the stand-alone reduction

@@ -544,7 +544,7 @@ int launch_bdot_tn_tile(hipStream_t st, int nblock, int n, int m, int k, int p, 
     const unsigned nchunk = dbk::divup((size_t)n, TN_CHUNK);
     const size_t nout = (size_t)k * m * nblock;
     T* partial = (T*)dbk::workspace(nout * nchunk * sizeof(T), st);
-    if (!partial) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", nout * nchunk * sizeof(T)); return 1; }
+    if (!partial) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch (%s)", nout * nchunk * sizeof(T), dbk::workspace_error()); return 1; }
     const size_t smem = (size_t)TN_ROWS * ((k | 1) + (m | 1)) * sizeof(T);
     auto kern = k_bdot_tn_tile<T>;
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));

@@ -381,7 +381,7 @@ int launch_colsum(hipStream_t st, const T* X, T* out, size_t n, size_t m)
         return 0;
     }
     T* partial = (T*)dbk::workspace(nslice * m * sizeof(T), st);
-    if (!partial) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", nslice * m * sizeof(T)); return 1; }
+    if (!partial) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch (%s)", nslice * m * sizeof(T), dbk::workspace_error()); return 1; }
     hipLaunchKernelGGL(k_colsum<T>, dim3(tiles, (unsigned)nslice), dim3(256), 0, st, X, partial, n, m, rows_per);
     hipLaunchKernelGGL(k_colsum_fold<T>, dim3(dbk::ew_grid(m)), dim3(256), 0, st, (const T*)partial, out, m, (unsigned)nslice);
     return 0;

@@ -289,7 +289,7 @@ int dbk::head_train_multi(hipStream_t st, size_t nrow, unsigned n, dbk::head_gro
         m.first[i + 1] = m.first[i] + (unsigned)(g[i].nblock * nchunk);
     }
     float* partial = (float*)dbk::workspace(total * sizeof(float), st, 1);
-    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", total * sizeof(float));
+    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", total * sizeof(float), dbk::workspace_error());
     for (unsigned i = 0; i < n; ++i) {
         g[i].partial = partial;
         partial += nchunk * (size_t)g[i].nblock * g[i].pstride;
@@ -334,7 +334,7 @@ extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, 
     const size_t pbytes = nchunk * (size_t)nblock * a.pstride * sizeof(float);
     dbk::deferred_sums* later = dbk::deferred();                   // inside dbk_train_step: the chunk sums are taken by its last kernel
     a.partial = (float*)dbk::workspace(pbytes, dbk::as_stream(stream), later ? 1 : 0);
-    DBK_CHECK(a.partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch", pbytes);
+    DBK_CHECK(a.partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", pbytes, dbk::workspace_error());
     DBK_HIP(hipFuncSetAttribute((const void*)k_head_train, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(k_head_train, dim3(nblock, (unsigned)nchunk), dim3(NT), smem, dbk::as_stream(stream), a);
     if (later) {

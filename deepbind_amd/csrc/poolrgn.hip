@@ -107,9 +107,16 @@ __global__ __launch_bounds__(256) void poolrgn_bprop_kernel(T* __restrict__ dU, 
     if (f >= F || r >= P) return;
     const region_t g = load_region(R, r, per_step);
     const size_t j = r * F + f;
-    // the argmax scatter is always atomic: the index is caller data and may point anywhere in the map
+    // The argmax index is caller data. One that lies in this thread's own column and region (what the forward
+    // pass produces) has this thread as its only writer when regions are disjoint: a plain add. Any other index
+    // may point anywhere in the map and is added atomically.
+    auto scatter = [&](T v) {
+        const size_t ai = argmax[j], row = ai / F;
+        if (!ATOMIC && ai - row * F == f && row >= g.a && row < g.b) dU[ai] += v;
+        else atomicAdd(&dU[ai], v);
+    };
     if (PT == DBK_PT_MAX) {
-        atomicAdd(&dU[argmax[j]], dP[j]);
+        scatter(dP[j]);
         return;
     }
     T dy;
@@ -128,7 +135,7 @@ __global__ __launch_bounds__(256) void poolrgn_bprop_kernel(T* __restrict__ dU, 
         }
     }
     for (; i < g.b; i += g.step) accumulate<ATOMIC>(&dU[i * F + f], dy);
-    if (PT == DBK_PT_ALL) atomicAdd(&dU[argmax[j]], dP[2 * j]);
+    if (PT == DBK_PT_ALL) scatter(dP[2 * j]);
 }
 
 template <typename T>
@@ -161,7 +168,7 @@ int launch_bwd(hipStream_t st, T* dU, size_t F, const uint32_t* R, size_t P, boo
 {
     DBK_CHECK(dbk::divup(F, 64) <= 65535u, "ValueError: too many feature maps (%zu) for one launch", F);
     unsigned* flag = (unsigned*)dbk::workspace(256, st);
-    DBK_CHECK(flag != nullptr, "MemoryError: could not allocate scratch");
+    DBK_CHECK(flag != nullptr, "MemoryError: could not allocate scratch (%s)", dbk::workspace_error());
     hipLaunchKernelGGL(regions_disjoint_kernel, dim3(1), dim3(1024), 0, st, R, P, per_step, flag);
     switch (ptype) {
     case DBK_PT_MAX: launch_bwd_pt<T, DBK_PT_MAX>(st, dU, F, R, P, per_step, dP, argmax, flag); break;

@@ -17,35 +17,81 @@ void set_error(const char* fmt, ...)
 
 void clear_error() { g_err[0] = 0; }
 
-struct ws_t { hipStream_t stream = nullptr; void* ptr[2] = {nullptr, nullptr}; size_t bytes[2] = {0, 0}; bool used = false; };
+struct ws_t { hipStream_t stream = nullptr; void* ptr[2] = {nullptr, nullptr}; size_t bytes[2] = {0, 0}; bool used = false; uint64_t tick = 0; };
 constexpr int WS_DEVICES = 64, WS_STREAMS = 64;
 static ws_t g_ws[WS_DEVICES][WS_STREAMS];
+static uint64_t g_ws_tick = 0;
 static std::mutex g_ws_mutex;
+static thread_local char g_ws_why[160] = {0};
+
+const char* workspace_error() { return g_ws_why; }
+
+static bool capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return status != hipStreamCaptureStatusNone;
+}
 
 void* workspace(size_t bytes, hipStream_t stream, int which)
 {
     int dev = 0;
+    g_ws_why[0] = 0;
     if (which < 0 || which > 1) return nullptr;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= WS_DEVICES) return nullptr;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= WS_DEVICES) {
+        snprintf(g_ws_why, sizeof(g_ws_why), "no current device below %d", WS_DEVICES);
+        return nullptr;
+    }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    ws_t* w = nullptr;
+    ws_t *w = nullptr, *vacant = nullptr, *oldest = nullptr;
     for (int i = 0; i < WS_STREAMS && !w; ++i) {
         ws_t& c = g_ws[dev][i];
-        if (c.used ? c.stream == stream : true) w = &c;        // this stream's slot, or the first free one
+        if (c.used && c.stream == stream) w = &c;
+        else if (!c.used) { if (!vacant) vacant = &c; }
+        else if (!oldest || c.tick < oldest->tick) oldest = &c;
     }
-    if (!w) return nullptr;
+    if (!w) w = vacant;
+    if (!w) {
+        // Every slot belongs to some stream: the one used longest ago changes hands, buffers included. Its stream
+        // may have been destroyed (a graph capture's) or may still run work that reads the buffers, so the whole
+        // device is drained first, which a capture in progress does not allow.
+        if (capturing(stream)) {
+            snprintf(g_ws_why, sizeof(g_ws_why), "all %d stream slots are taken and one cannot be recycled while the stream is capturing", WS_STREAMS);
+            return nullptr;
+        }
+        if (hipDeviceSynchronize() != hipSuccess) {
+            (void)hipGetLastError();
+            snprintf(g_ws_why, sizeof(g_ws_why), "could not drain the device to recycle a stream slot");
+            return nullptr;
+        }
+        w = oldest;
+    }
     w->used = true;
     w->stream = stream;
+    w->tick = ++g_ws_tick;
     if (w->bytes[which] >= bytes && w->ptr[which]) return w->ptr[which];
+    if (capturing(stream)) {
+        snprintf(g_ws_why, sizeof(g_ws_why), "scratch cannot grow while the stream is capturing: run the call once eagerly on this stream first");
+        return nullptr;
+    }
     if (w->ptr[which]) {
         // earlier launches may still be reading the old buffer
-        if (hipDeviceSynchronize() != hipSuccess) return nullptr;
+        if (hipDeviceSynchronize() != hipSuccess) {
+            (void)hipGetLastError();
+            snprintf(g_ws_why, sizeof(g_ws_why), "could not drain the device before growing the buffer");
+            return nullptr;
+        }
         (void)hipFree(w->ptr[which]);
         w->ptr[which] = nullptr;
         w->bytes[which] = 0;
     }
     size_t want = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes + bytes / 4;
-    if (hipMalloc(&w->ptr[which], want) != hipSuccess) { w->ptr[which] = nullptr; return nullptr; }
+    if (hipMalloc(&w->ptr[which], want) != hipSuccess) {
+        (void)hipGetLastError();
+        w->ptr[which] = nullptr;
+        snprintf(g_ws_why, sizeof(g_ws_why), "hipMalloc of %zu bytes failed", want);
+        return nullptr;
+    }
     w->bytes[which] = want;
     return w->ptr[which];
 }

@@ -223,16 +223,18 @@ template <int MT> struct grad_planes {
                  : [idx] "s"(idx), [q] "n"(Q), [mt] "n"(MT), [g0] "v"(g[0]), [g1] "v"(g[1]), [g2] "v"(g[2]),        \
                    [g3] "v"(g[3]), [g4] "v"(g[4]), [g5] "v"(g[5]), [g6] "v"(g[6]), [g7] "v"(g[7]), [g8] "v"(g[8]),  \
                    [g9] "v"(g[9]), [g10] "v"(g[10]), [g11] "v"(g[11]), [g12] "v"(g[12]), [g13] "v"(g[13]),          \
-                   [g14] "v"(g[14]), [g15] "v"(g[15]))
+                   [g14] "v"(g[14]), [g15] "v"(g[15])                                                               \
+                 : "m0")
 
 // All (p, j) pairs of the window that meet letter position Q: tap j = Q - p of position p.
 template <int Q, int MT>
 __device__ __forceinline__ void grad_planes_add(grad_planes<MT>& A, unsigned letter, const float (&g)[PSUB])
 {
     static_assert(PSUB == 16, "the instruction text lists 16 positions");
-    // M0 (which the index lives in while the mode is on) is left changed: the compiler never carries a value
-    // in M0 across other code - it writes M0 immediately before each instruction that reads it - and saving
-    // and restoring it here costs more than the sixteen additions (measured: +48 %).
+    // M0 (which the index lives in while the mode is on) is left changed and declared as clobbered, so the
+    // compiler re-establishes any value of its own in M0 after the block; saving and restoring it here would
+    // cost more than the sixteen additions (measured: +48 %). The planes are pinned to v96..v239 because the
+    // instruction text under the index mode names its registers relative to v96.
     const unsigned idx = letter * (unsigned)MT;          // first register of the letter's plane, relative to v96
     if constexpr (MT == 8) DBK_GP_ASM(DBK_GP_LIST("+{v[96:127]}"(A.t0), "+{v[128:143]}"(A.u0)));
     else if constexpr (MT == 16) DBK_GP_ASM(DBK_GP_LIST("+{v[96:127]}"(A.t0), "+{v[128:159]}"(A.t1), "+{v[160:191]}"(A.t2)));
@@ -316,13 +318,14 @@ __device__ __forceinline__ void weight_planes_load(grad_planes<MT>& A, const flo
                    [a5] "+v"(acc[5]), [a6] "+v"(acc[6]), [a7] "+v"(acc[7]), [a8] "+v"(acc[8]), [a9] "+v"(acc[9]),   \
                    [a10] "+v"(acc[10]), [a11] "+v"(acc[11]), [a12] "+v"(acc[12]), [a13] "+v"(acc[13]),              \
                    [a14] "+v"(acc[14]), [a15] "+v"(acc[15])                                                         \
-                 : PLANES, [idx] "s"(idx), [q] "n"(Q), [mt] "n"(MT))
+                 : PLANES, [idx] "s"(idx), [q] "n"(Q), [mt] "n"(MT)                                                 \
+                 : "m0")
 
 template <int Q, int MT>
 __device__ __forceinline__ void weight_planes_add(const grad_planes<MT>& A, unsigned letter, float (&acc)[PSUB])
 {
     static_assert(PSUB == 16, "the instruction text lists 16 positions");
-    const unsigned idx = letter * (unsigned)MT;          // (M0 is left changed: see grad_planes_add)
+    const unsigned idx = letter * (unsigned)MT;          // (M0 is clobbered: see grad_planes_add)
     if constexpr (MT == 8) DBK_WP_ASM(DBK_GP_LIST("{v[96:127]}"(A.t0), "{v[128:143]}"(A.u0)));
     else if constexpr (MT == 16) DBK_WP_ASM(DBK_GP_LIST("{v[96:127]}"(A.t0), "{v[128:159]}"(A.t1), "{v[160:191]}"(A.t2)));
     else DBK_WP_ASM(DBK_GP_LIST("{v[96:127]}"(A.t0), "{v[128:159]}"(A.t1), "{v[160:191]}"(A.t2), "{v[192:223]}"(A.t3), "{v[224:239]}"(A.u0)));
@@ -371,16 +374,17 @@ __device__ __forceinline__ float slab_sum(const float* __restrict__ slabs, size_
 
 inline size_t lds_limit()
 {
-    static size_t cached = 0;
-    if (!cached) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && v > 0)
-            cached = (size_t)v;
+    // LDS bytes a workgroup may use on the current device (asked once per device)
+    static size_t cached[64] = {0};
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 65536;
+    if (!cached[dev]) {
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && v > 0)
+            cached[dev] = (size_t)v;
         else
-            cached = 65536;
+            cached[dev] = 65536;
     }
-    return cached;
+    return cached[dev];
 }
 
 

@@ -1093,7 +1093,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         if (gx < 1) gx = 1;
         if (gx > P) gx = (unsigned)P;
         float* slabs = (float*)dbk::workspace(stride * gx * sizeof(float), st);
-        DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * gx * sizeof(float));
+        DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", stride * gx * sizeof(float), dbk::workspace_error());
         auto kern = scanpool_bprop_kernel<PT>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(nw * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P,
@@ -1108,7 +1108,7 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     const size_t smem_s = sparse_smem(m), smem_d = dense_smem(mt);
     DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
     float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float), st);
-    DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", stride * (gxs + gxd) * sizeof(float));
+    DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", stride * (gxs + gxd) * sizeof(float), dbk::workspace_error());
     if (gxs) {
         constexpr int PS = PT == DBK_PT_AVG ? DBK_PT_MAX : PT;
         auto kern = mt == 8 ? scanpool_bprop_sparse_kernel<PS, 8> : mt == 16 ? scanpool_bprop_sparse_kernel<PS, 16> : scanpool_bprop_sparse_kernel<PS, 24>;
@@ -1297,7 +1297,7 @@ int scan_bprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
         total += g[i].slab_stride * a.gx[i];
     }
     float* slabs = (float*)dbk::workspace(total * sizeof(float), st);
-    DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch", total * sizeof(float));
+    DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", total * sizeof(float), dbk::workspace_error());
     for (unsigned i = 0; i < n; ++i) {
         g[i].slabs = slabs;
         slabs += g[i].slab_stride * a.gx[i];

@@ -360,11 +360,7 @@ int launch_mode(hipStream_t st, unsigned nwave, unsigned grid, size_t smem, cons
                 const uint8_t* K, size_t N, const uint32_t* R, size_t P, unsigned nsplit, const unsigned* flag, float* pooled,
                 uint32_t* argmax)
 {
-    // the plain max kernel exists for 8, 12 and 16 waves (tuning knob); the other modes for 12
     auto kern = scanpool_kmer_kernel<G, 768, MODE>;
-    if (MODE == M_MAX && nwave == 8) kern = scanpool_kmer_kernel<G, 512, M_MAX>;
-    if (MODE == M_MAX && nwave == 16) kern = scanpool_kmer_kernel<G, 1024, M_MAX>;
-    if (MODE != M_MAX) nwave = 12;
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3(grid), dim3(nwave * 64), smem, st, W, bias, (unsigned)m, (unsigned)F, K, N, R,
                        (unsigned)P, nsplit, flag, pooled, argmax);
@@ -381,10 +377,7 @@ int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F
     unsigned nsplit = 256u / ntile;
     if (nsplit < 1) nsplit = 1;
     // 12 waves (3 per SIMD) measured fastest on MI355X: 8 leave LDS latency exposed, 16 add nothing.
-    unsigned nwave = 12;
-    if (const char* e = getenv("DBK_KMER_WAVES")) nwave = (unsigned)atoi(e);     // tuning knob
-    if (nwave != 8 && nwave != 12 && nwave != 16) nwave = 12;
-    if (ptype != DBK_PT_MAX || argmax) nwave = 12;
+    const unsigned nwave = 12;
     while (nsplit > 1 && (size_t)(nsplit - 1) * nwave * 4 >= P) --nsplit;       // no more streams than regions
     const unsigned grid = ntile * nsplit;
 #define DBK_GO(MODE) return launch_mode<G, MODE>(st, nwave, grid, smem, W, bias, m, F, K, N, R, P, nsplit, flag, pooled, argmax)
@@ -412,7 +405,7 @@ int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size
     if (!force && !takes(m, F, N, P)) return -1;
     const size_t kbytes = (N + KPAD + 255) & ~(size_t)255;
     unsigned char* ws = (unsigned char*)dbk::workspace(256 + kbytes, st);
-    if (!ws) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch", 256 + kbytes); return 1; }
+    if (!ws) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch (%s)", 256 + kbytes, dbk::workspace_error()); return 1; }
     unsigned* flag = (unsigned*)ws;
     uint8_t* K = ws + 256;
     const size_t ndef = N + 1 >= m + 1 ? N - m + 1 : 0;          // rows the scan defines

@@ -372,15 +372,6 @@ int dbk_train_steps(dbk_stream_t stream, size_t ngroup, const dbk_train_step_arg
 /* sizeof(dbk_train_step_args) as the library was built, for bindings that mirror the block field by field. */
 int dbk_train_step_args_size(void);
 
-/* ------------------------------------------------------------------ diagnostics */
-
-/* Sustained issue rate of one SIMD, in 1e9 wave-instructions per second, for kind 0 v_add_f32, 1 v_fma_f32,
- * 2 v_max_f32, 3 v_max3_f32, 4 v_add_f32 under the VGPR index mode, with waves_per_simd (1..8) resident waves
- * each issuing iters x 64 independent instructions. Synchronous; allocates and frees its own buffers; uses the
- * null stream. Prices the scan kernels' instruction counts (what bounds them: see the kernel sources).
- * reference: the autotuner's micro-benchmarks, kangaroo/kangaroo_smat/autotune.cu (no call of its own there). */
-int dbk_probe_valu_issue(int kind, int waves_per_simd, int iters, double* ginstr_per_s_per_simd);
-
 #ifdef __cplusplus
 }
 #endif

@@ -29,6 +29,47 @@ def assert_close(got, ref, rel, what=""):
         what, int(bad.sum()), bad.size, float(err.max()), float(bound.flat[err.argmax()]))
 
 
+def model_blocks(a, nmodel, axis):
+    """The per-model blocks of an array whose models are laid out along `axis`."""
+    return np.split(np.asarray(a), nmodel, axis=axis)
+
+
+def assert_close_per_model(got, ref, rel, nmodel, axis, what=""):
+    """assert_close on every model's own block, with that block's own scale: a model whose values are
+    orders of magnitude below its neighbours' is still checked to `rel` of ITS largest magnitude."""
+    for b, (g, r) in enumerate(zip(model_blocks(got, nmodel, axis), model_blocks(ref, nmodel, axis))):
+        assert_close(g, r, rel, "%s [model %d]" % (what, b))
+
+
+# Worst elementwise relative errors seen by the parity tests, printed in the run's summary
+# (tests/conftest.py) and written to gpurun_out/parity_elementwise.json when that folder exists.
+# err_rel = |got - ref| / max(|ref|, FLOOR_FRAC * max|ref| of the compared block): a pure elementwise ratio
+# is meaningless where a sum of signed terms cancels to ~0, so magnitudes below a thousandth of the block's
+# largest are measured against that floor; `share_within` is the share of elements inside the stated
+# tolerance with NO floor at all.
+FLOOR_FRAC = 1e-3
+REPORT = {}
+
+
+def record_error(config, kind, got, ref, tol):
+    got = np.asarray(got, dtype=np.float64).ravel()
+    ref = np.asarray(ref, dtype=np.float64).ravel()
+    if ref.size == 0:
+        return
+    scale = np.abs(ref).max()
+    if scale == 0:
+        return
+    err = np.abs(got - ref)
+    floored = float((err / np.maximum(np.abs(ref), FLOOR_FRAC * scale)).max())
+    nz = np.abs(ref) > 0
+    within = float(((err[nz] / np.abs(ref[nz])) <= tol).mean()) if nz.any() else 1.0
+    e = REPORT.setdefault((config, kind), {"worst_rel_err": 0.0, "share_within": 1.0, "tol": tol, "elements": 0,
+                                            "floor": "%g x block max" % FLOOR_FRAC})
+    e["worst_rel_err"] = max(e["worst_rel_err"], floored)
+    e["share_within"] = (e["share_within"] * e["elements"] + within * ref.size) / (e["elements"] + ref.size)
+    e["elements"] += int(ref.size)
+
+
 def random_codes(rng, N, pn=0.05, p254=0.0):
     X = rng.integers(0, 4, size=N).astype(np.uint8)
     u = rng.random(N)

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import deepbind_oracle as orc
-from tests.gpu_util import assert_close, dev, host
+from tests.gpu_util import assert_close, assert_close_per_model, dev, host, model_blocks, record_error
 
 pytestmark = pytest.mark.gpu
 
@@ -16,7 +16,7 @@ def _f64(d):
     return {k: np.asarray(v, dtype=np.float64).copy() for k, v in d.items()}
 
 
-def _run_config(cfg, mode, nsteps, dropout_rate=0.0, decay=(0.0, 0.0), weight_decay_start=100, bias_jitter=0.01):
+def _run_config(cfg, mode, nsteps, dropout_rate=0.0, decay=(0.0, 0.0), weight_decay_start=100, bias_jitter=0.01, name=None):
     from deepbind_amd.model import SequenceNet
     spec = cfg["spec"]
     rng = np.random.default_rng(99)
@@ -41,23 +41,34 @@ def _run_config(cfg, mode, nsteps, dropout_rate=0.0, decay=(0.0, 0.0), weight_de
         got_g = net.get_grads()
         for k in g:
             assert_close(got_g[k], g[k], GRAD, "step %d grad %s (%s)" % (step, k, mode))
+            if name:
+                record_error(name, "gradients", got_g[k], g[k], GRAD)
     got = net.get_params()
     for k in ref_p:
         assert_close(got[k], ref_p[k], GRAD, "params %s after %d steps (%s)" % (k, nsteps, mode))
+        if name:
+            record_error(name, "parameters", got[k], ref_p[k], GRAD)
+    if name:
+        st = orc.model_forward(ref_p, cfg["X"], cfg["R"], spec.nmodel, spec.pool[0], spec.hidden[0],
+                               out="logistic" if spec.loss == "nll" else "linear")
+        net.use_dropout, keep = False, net.use_dropout
+        record_error(name, "activations", host(net.predict(X, R)), st["Zout"], ACT)
+        record_error(name, "activations", host(net.forward(X, R)["pooled"]), st["Pl"], ACT)
+        net.use_dropout = keep
     return net, got
 
 
 @pytest.mark.parametrize("mode", ["fused", "unfused"])
 def test_config2_rna_regression_train_steps(mode):
     from deepbind_amd import synth
-    _run_config(synth.config2(), mode, nsteps=3)
+    _run_config(synth.config2(), mode, nsteps=3, name="config2 (%s)" % mode)
 
 
 @pytest.mark.parametrize("mode", ["fused", "unfused"])
 def test_config3_classification_train_steps_with_dropout_and_decay(mode):
     from deepbind_amd import synth
     cfg = synth.config3()
-    _run_config(cfg, mode, nsteps=3, dropout_rate=0.5, decay=(1e-4, 1e-3), weight_decay_start=1)
+    _run_config(cfg, mode, nsteps=3, dropout_rate=0.5, decay=(1e-4, 1e-3), weight_decay_start=1, name="config3 (%s)" % mode)
 
 
 def test_train_step_is_bit_stable_and_modes_agree():
@@ -83,43 +94,81 @@ def test_config1_forward_scores():
     got = host(net.predict(dev(cfg["X"]), dev(cfg["R"])))
     assert got.shape == (64, 1)
     assert_close(got, st["A"], ACT, "config 1 scores")
+    record_error("config1", "activations", got, st["A"], ACT)
     assert_close(host(net.forward(dev(cfg["X"]), dev(cfg["R"]))["Z"]), st["A"], ACT, "config 1 scores (layer by layer)")
 
 
 def test_config4_calibration_batch_mixed_architectures():
-    """90 models (30 hyper-parameter draws x 3 folds), pool and hidden size chosen per model, shared batch."""
+    """90 models (30 hyper-parameter draws x 3 folds), pool and hidden size chosen per model, shared batch,
+    stepped through the shared launches (one native call for all architecture groups) with every model's own
+    drawn dropout rate. The oracle gets the uniforms the library's generator draws at each group's stream
+    position. Every model is compared on its OWN block of every array, with that block's own scale: the
+    models' initial scales span four orders of magnitude."""
     from deepbind_amd import synth
+    from deepbind_amd import deepity_smat as ds
     from deepbind_amd.model import ModelGroup
     cfg = synth.config4()
     spec, hp = cfg["spec"], cfg["hp"]
+    assert (hp["dropout"] > 0).sum() >= 20 and (hp["dropout"] == 0).sum() >= 20
     grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
-                     decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=0.0, weight_decay_start=0)
+                     decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"], weight_decay_start=1)
     assert len(grp.groups) <= 4 and sum(len(i) for i, _ in grp.groups) == 90
-    for idx, net in grp.groups:
-        stacked = {}
-        for name, shape, axis in net.layout:
-            parts = [cfg["models"][j][name] for j in idx]
-            stacked[name] = np.concatenate(parts, axis=axis)
+    init, ref, mom = [], [], []
+    for gi, (idx, net) in enumerate(grp.groups):
+        net.rng_seed = 40 + gi
+        stacked = {name: np.concatenate([cfg["models"][j][name] for j in idx], axis=axis) for name, _, axis in net.layout}
         net.set_params(stacked)
+        init.append(stacked)
+        ref.append(_f64(stacked))
+        mom.append({k: np.zeros(v.shape) for k, v in stacked.items()})
     X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
-    nsteps = 2
-    for _ in range(nsteps):
+    nsteps = 3
+    for step in range(nsteps):
+        # the uniforms each group's head will draw in this step: its generator at (seed, position)
+        Us = [host(ds.uniform_like(torch.empty((R.shape[0], net.k * net.ninst), device="cuda"), net.rng_seed, net._rng_offset))
+              if net.use_dropout else None for _, net in grp.groups]
         grp.train_step(X, R, Y, M)
-    # the oracle steps each architecture group with the same model-axis layout (the reference's
-    # scan-filter decay indexing depends on the number of models sharing a graph, so the grouping is part of the semantics)
-    for idx, net in grp.groups:
-        pool, hid = net.pool, net.hidden
-        p = {name: np.concatenate([cfg["models"][j][name] for j in idx], axis=axis).astype(np.float64) for name, _, axis in net.layout}
-        mom = {k: np.zeros(v.shape) for k, v in p.items()}
-        for step in range(nsteps):
-            orc.train_step(p, mom, cfg["X"], cfg["R"], cfg["Y"][:, idx].astype(np.float64), len(idx), pool, hid, "nll",
-                           hp["rate"][idx], hp["momentum"][idx], Ymask=cfg["Ymask"][:, idx],
-                           decay_conv=hp["decay_conv"][idx], decay_full=hp["decay_full"][idx], step=step, weight_decay_start=0)
+        # the oracle steps each architecture group with the same model-axis layout (the reference's scan-filter
+        # decay indexing depends on the number of models sharing a graph, so the grouping is part of the semantics)
+        for gi, (idx, net) in enumerate(grp.groups):
+            drop = (hp["dropout"][idx].astype(np.float64), Us[gi]) if net.use_dropout else None
+            _, g = orc.train_step(ref[gi], mom[gi], cfg["X"], cfg["R"], cfg["Y"][:, idx].astype(np.float64), len(idx), net.pool,
+                                  net.hidden, "nll", hp["rate"][idx], hp["momentum"][idx], Ymask=cfg["Ymask"][:, idx], dropout=drop,
+                                  decay_conv=hp["decay_conv"][idx], decay_full=hp["decay_full"][idx], step=step, weight_decay_start=1)
+            got_g = net.get_grads()
+            for name, _, axis in net.layout:
+                what = "step %d %s/%d gradient %s" % (step, net.pool, net.hidden, name)
+                assert_close_per_model(got_g[name], g[name], GRAD, len(idx), axis, what)
+                for a, b in zip(model_blocks(got_g[name], len(idx), axis), model_blocks(g[name], len(idx), axis)):
+                    record_error("config4 (shared launches)", "gradients", a, b, GRAD)
+    nmoved = 0
+    for gi, (idx, net) in enumerate(grp.groups):
         got = net.get_params()
-        for k in p:
-            assert_close(got[k], p[k], GRAD, "%s/%d group %s" % (pool, hid, k))
+        for name, _, axis in net.layout:
+            assert_close_per_model(got[name], ref[gi][name], GRAD, len(idx), axis, "%s/%d parameters %s" % (net.pool, net.hidden, name))
+            for a, b in zip(model_blocks(got[name], len(idx), axis), model_blocks(ref[gi][name], len(idx), axis)):
+                record_error("config4 (shared launches)", "parameters", a, b, GRAD)
+        # every model trained: its filters changed by what the reference's update changes them by (compared as
+        # CHANGES, so a model whose filters were left alone, or stepped with a neighbour's rate, fails even
+        # when the change is far below the weights' own size); float32 storage rounds each of the steps
+        for b, (w0, w1, wr) in enumerate(zip(model_blocks(init[gi]["Wc"], len(idx), 1), model_blocks(got["Wc"], len(idx), 1),
+                                             model_blocks(ref[gi]["Wc"], len(idx), 1))):
+            d_ref, d_got = wr - w0, w1.astype(np.float64) - w0
+            slack = (nsteps + 1) * np.spacing(np.abs(w0)).astype(np.float64)
+            bad = np.abs(d_got - d_ref) > 2e-2 * np.abs(d_ref).max() + slack
+            assert not bad.any(), "model %d of group %d: filter update differs from the reference's" % (b, gi)
+            if np.abs(d_ref).max() > 100 * np.spacing(np.float32(np.abs(w0).max())):     # a change float32 can hold
+                assert (w1 != w0).mean() > 0.5, "model %d of group %d: filters did not move" % (b, gi)
+                nmoved += 1
+    assert nmoved >= 80, nmoved
     scores = host(grp.predict(X, R))
     assert scores.shape == (256, 90) and np.isfinite(scores).all() and scores.min() >= 0 and scores.max() <= 1
+    col = 0
+    for gi, (idx, net) in enumerate(grp.groups):
+        st = orc.model_forward(ref[gi], cfg["X"], cfg["R"], len(idx), net.pool, net.hidden, out="logistic",
+                               dropout=(hp["dropout"][idx].astype(np.float64), None) if net.use_dropout else None, train=False)
+        assert_close(scores[:, idx], st["Zout"], 1e-4, "scores of group %d" % gi)
+        record_error("config4 (shared launches)", "activations", scores[:, idx], st["Zout"], ACT)
 
 
 def test_reverse_complement_mode_train_and_predict():
