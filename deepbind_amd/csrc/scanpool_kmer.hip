@@ -43,7 +43,7 @@
 #include "dbk_common.h"
 #include "scan_common.h"
 #include <cmath>
-#include <cstdlib>
+#include <mutex>
 
 namespace dbk_scanpool_general {
 int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
@@ -395,17 +395,22 @@ bool takes(size_t m, size_t F, size_t N, size_t P)
     return (double)N * dbk::divup(F, FTILE) >= 2.0e6;
 }
 
-// force: take the fast path whenever the shape allows, regardless of problem size
+// Bytes of device scratch a call over N sequence bytes needs: the flag word's 256-byte line, then the index bytes.
+inline size_t scratch_bytes(size_t N) { return 256 + ((N + KPAD + 255) & ~(size_t)255); }
+
+// force: take the fast path whenever the shape allows, regardless of problem size.
+// ws: device scratch of scratch_bytes(N) bytes the caller provides, or null to take the stream's grow-on-demand buffer.
 int fprop_impl(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
-               const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, bool force)
+               const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, bool force, unsigned char* ws = nullptr)
 {
     if (ptype != DBK_PT_MAX && ptype != DBK_PT_AVG && ptype != DBK_PT_ALL) return -1;
     if (ptype == DBK_PT_AVG && argmax != nullptr) return -1;
     if (m > 24 || N == 0 || N > 0x7fffff00u || P > 0x7fff0000u) return -1;
     if (!force && !takes(m, F, N, P)) return -1;
-    const size_t kbytes = (N + KPAD + 255) & ~(size_t)255;
-    unsigned char* ws = (unsigned char*)dbk::workspace(256 + kbytes, st);
-    if (!ws) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch (%s)", 256 + kbytes, dbk::workspace_error()); return 1; }
+    if (!ws) {
+        ws = (unsigned char*)dbk::workspace(scratch_bytes(N), st);
+        if (!ws) { dbk::set_error("MemoryError: could not allocate %zu bytes of scratch (%s)", scratch_bytes(N), dbk::workspace_error()); return 1; }
+    }
     unsigned* flag = (unsigned*)ws;
     uint8_t* K = ws + 256;
     const size_t ndef = N + 1 >= m + 1 ? N - m + 1 : 0;          // rows the scan defines
@@ -433,7 +438,58 @@ int fprop(hipStream_t st, const float* W, const float* bias, size_t m, size_t F,
     return fprop_impl(st, W, bias, m, F, X, N, R, P, ptype, pooled, argmax, false);
 }
 
+// ---- scratch that is part of the loaded code object, for callers that must not allocate ------------------
+// Every device the library runs on holds its own copy of this array, at its own address, from the moment the code
+// object is loaded there until the process ends. The array's name is a host-side handle, not a device address:
+// host code asks the runtime for the address once per device and passes that pointer to the kernels.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t(64) << 20) + 512;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+static unsigned char* g_static_scratch[64] = {nullptr};
+static std::mutex g_static_scratch_mutex;
+
+// Address of the current device's copy of `scratch` (looked up on the first call per device); null on failure.
+static unsigned char* static_scratch()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { dbk::set_error("RuntimeError: no current device below 64"); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (!g_static_scratch[dev]) {
+        unsigned char* p = nullptr;
+        hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            dbk::set_error("RuntimeError: hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_static_scratch[dev] = p;
+    }
+    return g_static_scratch[dev];
+}
+
 }  // namespace dbk_scanpool_kmer
+
+extern "C" int dbk_scanpool_fprop_kmer_static(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
+                                              const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
+                                              float* pooled, uint32_t* argmax)
+{
+    using namespace dbk_scanpool_kmer;
+    DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
+    if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
+    DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
+    DBK_CHECK(!argmax || (double)N * (double)nfilter <= 4294967296.0,
+              "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
+    DBK_CHECK(scratch_bytes(N) <= STATIC_SCRATCH_BYTES,
+              "ValueError: %zu sequence bytes need %zu bytes of scratch, the built-in buffer holds %zu (at most %zu sequence bytes per call); "
+              "score in smaller batches or call dbk_scanpool_fprop_kmer", N, scratch_bytes(N), STATIC_SCRATCH_BYTES,
+              STATIC_SCRATCH_BYTES - 256 - KPAD - 255);
+    unsigned char* ws = static_scratch();
+    if (!ws) return 2;
+    // The flag word and the index bytes are rewritten from the inputs by the call's first two launches, so
+    // nothing of an earlier call's contents is read.
+    int rc = fprop_impl(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax, true, ws);
+    DBK_CHECK(rc >= 0, "NotImplementedError: the k-mer table path takes max / avg / all pooling and filter length <= 24");
+    return rc;
+}
 
 extern "C" int dbk_scanpool_fprop_kmer(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
                                        const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,

@@ -139,11 +139,14 @@ def activity_words(X, W):
     return torch.empty((X.numel(), (W.shape[1] + 63) // 64), dtype=torch.int64, device=W.device)
 
 
-def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=None):
+def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=None, out=None):
     """pool(relu(corr1ord(W, X) + b)) per region without storing the (N x P) map.
     Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only.
     path: "auto" lets the library choose; "general" / "wide" / "kmer" force the general path (which picks its
-    kernel by size), its many-regions kernel (17-24 taps) or the table kernel.
+    kernel by size), its many-regions kernel (17-24 taps) or the table kernel; "kmer_static" is the table kernel
+    with the scratch buffer that is built into the library (no allocation inside the call; at most 64 MiB of
+    sequence bytes; calls that overlap on one GPU must not use it together).
+    out (optional): (pooled, argmax|None) tensors to write into instead of new ones, so that the call allocates nothing.
     act (optional, from activity_words): receives 1 bit per row and filter - rectifier open or not - which
     scanpool_bprop takes in place of recomputing the map (general kernel only)."""
     _u8(X)
@@ -152,12 +155,20 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=
     require(W.dtype == torch.float32 and b.dtype == torch.float32, "TypeError: the fused path is float32 only")
     require(W.shape[0] % 4 == 0 and b.numel() == W.shape[1], "ValueError: W must be (4m x P) and b must have P entries")
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
-    pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
-    argmax = torch.empty((P, F), dtype=uindex, device=W.device) if (want_argmax and ptype in ("max", "all")) else None
+    want_argmax = want_argmax and ptype in ("max", "all")
+    if out is not None:
+        pooled, argmax = out
+        require(pooled.dtype == torch.float32 and tuple(pooled.shape) == (P, F * (2 if ptype == "all" else 1)),
+                "ValueError: out[0] must be float32 (regions x pooled features)")
+        require((argmax is not None) == bool(want_argmax), "ValueError: out[1] must be given exactly when argmax is wanted")
+        require(argmax is None or (argmax.dtype == uindex and tuple(argmax.shape) == (P, F)), "ValueError: out[1] must be (regions x filters) indices")
+    else:
+        pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
+        argmax = torch.empty((P, F), dtype=uindex, device=W.device) if want_argmax else None
     entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "wide": "dbk_scanpool_fprop_wide",
-             "kmer": "dbk_scanpool_fprop_kmer"}[path]
+             "kmer": "dbk_scanpool_fprop_kmer", "kmer_static": "dbk_scanpool_fprop_kmer_static"}[path]
     args = [stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax)]
-    if path != "kmer":
+    if path not in ("kmer", "kmer_static"):
         args.append(_act(act, X, F))
     else:
         require(act is None, "ValueError: the table kernel does not write activity masks")

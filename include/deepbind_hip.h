@@ -155,6 +155,20 @@ int dbk_scanpool_fprop_kmer(dbk_stream_t stream,
                             const uint32_t* regions, size_t nregion, int ptype,
                             float* pooled, uint32_t* argmax);
 
+/* dbk_scanpool_fprop_kmer for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid allocation): same arguments, same kernels, same results, but the call's
+ * scratch (a flag word and one index byte per sequence byte) lies in a buffer that is part of the loaded
+ * library instead of a grow-on-demand allocation, so the call never allocates, frees or synchronises.
+ * Limit: N <= 64 MiB of sequence bytes per call (ValueError beyond; the buffer's 64.0005 MiB are held on every
+ * GPU the library runs on until the process ends). All calls on one GPU share the buffer: calls that overlap
+ * on one GPU (different streams, different host threads) race; calls ordered on one stream do not.
+ * No counterpart in the reference (its wrappers allocate per call, kangaroo/_ext/kangaroo_smat.py:121-132). */
+int dbk_scanpool_fprop_kmer_static(dbk_stream_t stream,
+                                   const float* W, const float* bias, size_t m, size_t nfilter,
+                                   const uint8_t* X, size_t N,
+                                   const uint32_t* regions, size_t nregion, int ptype,
+                                   float* pooled, uint32_t* argmax);
+
 /* Backward of the fused chain: given dpooled (same layout as pooled), the forward's pooled and
  * argmax, accumulates dW (C*m, F) += (as corr1ord_bprop_W does; with overwrite != 0 it is written
  * instead, which saves the caller a fill) and writes dbias (1, F) =. Deterministic (no float atomics).
