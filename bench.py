@@ -23,46 +23,113 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published FP32 vector peak (FMA = 2 FLOP)
+FP32_ADD_ISSUE_PEAK_TADDS = 78.6    # the same peak for a stream of plain adds (1 FLOP per lane-operation)
 HBM_PEAK_GBS = 8000.0
-LDS_PEAK_TBS = 216 * 256 * 2.4e9 / 1e12     # aligned ds_read_b128 as measured: 216 B/clk/CU x 256 CUs x 2.4 GHz
 
 
-def cpu_baseline(cfg, nseq_c, nseq_np):
-    """Times the CPU restatement (the checker's plain-C port, OpenMP over all host cores) and the
-    NumPy float32 formulation on a bounded subsample of the same workload; returns positions/s."""
-    from oracle import oracle_c, deepbind_oracle as orc
+def _numpy_scanpool(Wc, bc, X, R, m, chunk=4):
+    """The NumPy float32 formulation of scan + bias + ReLU + max pool (what the reference's array library falls back
+    to on host arrays): m gathers from a per-tap letter table, np.maximum, np.maximum.reduceat over region starts;
+    `chunk` sequences at a time so that a chunk's map stays in the host's caches (3x faster than whole-batch maps)."""
+    from oracle import deepbind_oracle as orc
+    F = Wc.shape[1]
+    out = np.empty((len(R), F), np.float32)
+    for i in range(0, len(R), chunk):
+        Rc = R[i:i + chunk].astype(np.int64)
+        a, b = int(Rc[0, 0]), int(Rc[-1, 1])
+        Xc = X[a:b + m - 1]
+        Z = np.zeros((Xc.size, F), np.float32)
+        orc.corr1ord(Wc, Xc, Z)
+        A = np.maximum(Z + bc, 0)
+        out[i:i + chunk] = np.maximum.reduceat(A[:b - a], Rc[:, 0] - a, axis=0)
+    return out
+
+
+def cpu_baseline(cfg, nseq, budget_s=30.0):
+    """Times the reference's CPU path - the NumPy float32 semantics its array library's tests compare against - on a
+    bounded subsample of the same workload, after one warm-up: best of up to 5 runs within `budget_s` seconds.
+    The checker's plain-C port (OpenMP over all host cores) is timed beside it as a secondary figure."""
+    from oracle import oracle_c
     spec, p = cfg["spec"], cfg["params"]
     m = spec.m
-
-    def sample(nseq):
-        R = cfg["R"][:nseq]
-        end = int(R[-1, 1])
-        X = np.ascontiguousarray(cfg["X"][:end + m - 1])
-        return X, np.ascontiguousarray(R), end
-
+    R = np.ascontiguousarray(cfg["R"][:nseq])
+    pos = int(R[-1, 1])
+    X = np.ascontiguousarray(cfg["X"][:pos + m - 1]).ravel()
     cores = len(os.sched_getaffinity(0))
-    X, R, pos = sample(nseq_c)
+    _numpy_scanpool(p["Wc"], p["bc"], X, R[:48], m)                    # warm-up
+    best, runs, spent = float("inf"), 0, 0.0
+    while runs < 5 and (runs == 0 or spent + best <= budget_s):
+        t0 = time.perf_counter()
+        _numpy_scanpool(p["Wc"], p["bc"], X, R, m)
+        dt = time.perf_counter() - t0
+        best, runs, spent = min(best, dt), runs + 1, spent + dt
+    np_rate = pos / best
     oracle_c.scanpool(p["Wc"], p["bc"], X[:2000 + m], R[:2], 0)       # warm-up (thread pool, page-in)
-    best = float("inf")
+    cbest = float("inf")
     for _ in range(3):
         t0 = time.perf_counter()
         oracle_c.scanpool(p["Wc"], p["bc"], X, R, 0)
-        best = min(best, time.perf_counter() - t0)
-    c_rate = pos / best
-    Xn, Rn, posn = sample(nseq_np)
-    t0 = time.perf_counter()
-    Z = np.zeros((Xn.size, spec.F), np.float32)
-    orc.corr1ord(p["Wc"], Xn, Z)
-    A = np.maximum(Z + p["bc"], 0)
-    np.maximum.reduceat(A, Rn[:, 0].astype(np.int64), axis=0)
-    np_rate = posn / (time.perf_counter() - t0)
+        cbest = min(cbest, time.perf_counter() - t0)
+    try:
+        from threadpoolctl import threadpool_info
+        blas = max([t.get("num_threads", 1) for t in threadpool_info() if t.get("user_api") == "blas"] or [1])
+    except Exception:
+        blas = None
     return {
-        "value": c_rate, "unit": "positions/s", "cores": cores, "kind": "port",
-        "sample": "plain-C port of the reference scan+bias+relu+maxpool (OpenMP, %d threads), %d of the %d sequences x all %d filters, best of 3"
-                  % (cores, nseq_c, len(cfg["R"]), spec.F),
-        "numpy_f32_positions_per_s": np_rate,
-        "numpy_sample": "NumPy float32 LUT-gather formulation, single process, %d sequences x all %d filters, 1 run" % (nseq_np, spec.F),
+        "value": np_rate, "unit": "positions/s", "cores": 1, "kind": "port",
+        "sample": "NumPy float32 restatement of the reference's CPU path (per-tap letter-table gathers, np.maximum, np.maximum.reduceat; "
+                  "one thread: these NumPy calls do not use BLAS), first %d of the %d sequences x all %d filters = %d positions, "
+                  "best of %d runs after a warm-up; scale linearly for the full batch" % (nseq, len(cfg["R"]), spec.F, pos, runs),
+        "host": {"os_cpu_count": os.cpu_count(), "sched_affinity": cores, "blas_threads": blas},
+        "c_port_positions_per_s": pos / cbest,
+        "c_port_sample": "plain-C port of the same chain (OpenMP, %d threads), same sample, best of 3" % cores,
     }
+
+
+def train_cpu_baseline(cfg, groups, nsteps=2, budget_s=12.0):
+    """One optimiser step of the NumPy float32 restatement of the reference's train step on the same batch:
+    sequences per second, best of up to `nsteps` timed steps after one warm-up step. groups: list of
+    (model indices, pool, hidden, stacked float32 parameter dict) - one entry for a single net, one per
+    architecture for the calibration batch (each architecture is one graph in the reference too)."""
+    from oracle import deepbind_oracle as orc
+    spec = cfg["spec"]
+    hp = cfg.get("hp")
+    state = []
+    for idx, pool, hidden, params in groups:
+        p = {k: np.array(v, dtype=np.float32) for k, v in params.items()}
+        state.append((idx, pool, hidden, p, {k: np.zeros_like(v) for k, v in p.items()}))
+    Y = cfg["Y"].astype(np.float32)
+    Ymask = cfg.get("Ymask")
+    rng = np.random.default_rng(0)
+
+    def one_step(step):
+        for idx, pool, hidden, p, mom in state:
+            k = spec.nfilter * (2 if pool == "all" else 1)
+            if hp is not None:
+                rate, mu = hp["rate"][idx], hp["momentum"][idx]
+                drop = (hp["dropout"][idx], rng.random((len(cfg["R"]), k * len(idx)), dtype=np.float32)) if (hp["dropout"][idx] > 0).any() else None
+                dc, df = hp["decay_conv"][idx], hp["decay_full"][idx]
+            else:
+                rate, mu, dc, df = cfg["rate"], cfg["momentum"], 0.0, 0.0
+                dr = cfg.get("dropout_rate", 0.0)
+                drop = (np.full(1, dr, np.float32), rng.random((len(cfg["R"]), k), dtype=np.float32)) if dr > 0 else None
+            orc.train_step(p, mom, cfg["X"], cfg["R"], Y[:, idx], len(idx), pool, hidden, spec.loss, rate, mu,
+                           Ymask=None if Ymask is None else Ymask[:, idx], dropout=drop, decay_conv=dc, decay_full=df,
+                           step=step, weight_decay_start=0)
+
+    one_step(0)
+    best, runs, spent = float("inf"), 0, 0.0
+    while runs < nsteps and (runs == 0 or spent + best <= budget_s):
+        t0 = time.perf_counter()
+        one_step(1 + runs)
+        dt = time.perf_counter() - t0
+        best, runs, spent = min(best, dt), runs + 1, spent + dt
+    nseq = len(cfg["R"])
+    return {"value": nseq / best, "unit": "sequences/s", "ms_per_step": best * 1e3, "cores": 1, "kind": "port",
+            "model_sequences_per_s": nseq * spec.nmodel / best,
+            "sample": "NumPy float32 restatement of the reference's train step (forward, backward, L1 term, Nesterov update) on the "
+                      "same batch, all %d models, best of %d steps after a warm-up step; the dense products go through NumPy's BLAS"
+                      % (spec.nmodel, runs)}
 
 
 def measured_traffic(workload):
@@ -81,11 +148,27 @@ def measured_traffic(workload):
     return None
 
 
-def train_throughput(steps=100, warmup=10):
-    """Secondary figures: whole train steps (forward + backward + Nesterov update) per second on the
-    three training configurations, fused mode: each step issued natively by one library call (the top-level
-    figures; the calibration batch's four architecture groups share every launch) and as one captured HIP
-    graph per step ("graphed"). sequences/s = batch rows * steps / wall time."""
+def profiled_kernels(tag):
+    """Dominant kernel of a training configuration and its average duration from the committed rocprofv3 kernel
+    trace (profiles/train_step_kernel_trace.md, lines 'dominant[<tag>]: <kernel> <avg_us>'); None when not on file."""
+    path = os.path.join(ROOT, "profiles", "train_step_kernel_trace.md")
+    try:
+        for line in open(path):
+            if line.startswith("dominant[%s]:" % tag):
+                name, us = line.split(":", 1)[1].rsplit(None, 1)
+                return {"kernel": name.strip(), "rocprof_avg_us": float(us)}
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def train_throughput(steps=100, warmup=10, cpu=True):
+    """Whole train steps (forward + backward + Nesterov update) per second on the three training configurations,
+    fused mode: each step issued natively by one library call (the top-level figures; the calibration batch's
+    architecture groups share every launch) and as one captured HIP graph per step ("graphed").
+    sequences/s = batch rows * steps / wall time. Roofline: algorithmic adds per step = 2 * positions * filters *
+    taps (the scan and the filter gradient cost the same count; bias, ReLU, pooling and the dense head are not
+    counted) over the step time, against the FP32 vector peak (FMA-counted) and against the add-issue peak."""
     import torch
     from deepbind_amd import synth
     from deepbind_amd.model import ModelGroup, SequenceNet
@@ -96,14 +179,31 @@ def train_throughput(steps=100, warmup=10):
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        e0.record()
         for _ in range(steps):
             fn()
+        e1.record()
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) / steps
-        return {"ms_per_step": dt * 1e3, "sequences_per_s": nseq / dt, "model_sequences_per_s": nseq * nmodel / dt}
+        return {"ms_per_step": dt * 1e3, "gpu_ms_per_step": e0.elapsed_time(e1) / steps, "sequences_per_s": nseq / dt,
+                "model_sequences_per_s": nseq * nmodel / dt}
 
-    for name, cfg, drop in (("config2_rna_regression", synth.config2(), 0.0), ("config3_classification", synth.config3(), 0.5)):
+    def roofline(tag, cfg, rec):
+        spec = cfg["spec"]
+        adds = 2.0 * synth.positions(cfg["R"]) * spec.F * spec.m
+        rate = adds / (rec["ms_per_step"] * 1e-3) / 1e12
+        r = {"bound": "fp32_valu", "algorithmic_adds_per_step": adds, "achieved": rate, "unit": "T adds/s",
+             "peak": FP32_VECTOR_PEAK_TFLOPS, "frac": rate / FP32_VECTOR_PEAK_TFLOPS,
+             "frac_vs_add_issue_peak": rate / FP32_ADD_ISSUE_PEAK_TADDS}
+        dom = profiled_kernels(tag)
+        if dom:
+            r["dominant_kernel"] = dom
+        return r
+
+    for tag, name, cfg, drop in (("config2", "config2_rna_regression", synth.config2(), 0.0),
+                                 ("config3", "config3_classification", synth.config3(), 0.5)):
         spec = cfg["spec"]
         net = SequenceNet(1, spec.nfilter, spec.m, pool=spec.pool[0], hidden=spec.hidden[0], loss=spec.loss,
                           rate=cfg["rate"], momentum=cfg["momentum"], dropout=drop)
@@ -111,16 +211,27 @@ def train_throughput(steps=100, warmup=10):
         X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
         out[name] = timed(lambda: net.train_step(X, R, Y), len(cfg["R"]), 1)
         out[name]["graphed"] = timed(net.make_graphed_step(X, R, Y), len(cfg["R"]), 1)
+        out[name]["roofline"] = roofline(tag, cfg, out[name])
+        if cpu:
+            cfg["dropout_rate"] = drop
+            out[name]["cpu_baseline"] = train_cpu_baseline(cfg, [([0], spec.pool[0], spec.hidden[0], cfg["params"])], nsteps=5)
     cfg = synth.config4()
     spec, hp = cfg["spec"], cfg["hp"]
     grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
                      decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"],
                      weight_decay_start=0)       # the L1 term is on in every timed step (steady state; a captured graph is re-captured when it switches on)
+    stacked = []
     for idx, net in grp.groups:
-        net.set_params({n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout})
+        params = {n: np.concatenate([cfg["models"][j][n] for j in idx], axis=ax) for n, _, ax in net.layout}
+        net.set_params(params)
+        stacked.append((idx, net.pool, net.hidden, params))
     X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
-    out["config4_calibration_90_models"] = timed(lambda: grp.train_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
-    out["config4_calibration_90_models"]["graphed"] = timed(grp.make_graphed_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
+    name = "config4_calibration_90_models"
+    out[name] = timed(lambda: grp.train_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
+    out[name]["graphed"] = timed(grp.make_graphed_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
+    out[name]["roofline"] = roofline("config4", cfg, out[name])
+    if cpu:
+        out[name]["cpu_baseline"] = train_cpu_baseline(cfg, stacked, nsteps=2)
     return out
 
 
@@ -240,7 +351,7 @@ def main():
     torch.cuda.set_device(0)
 
     if args.train_only:
-        print(json.dumps({"train": train_throughput(steps=args.steps, warmup=args.warmup)}))
+        print(json.dumps({"train": train_throughput(steps=args.steps, warmup=args.warmup, cpu=not args.no_cpu_baseline)}))
         return
     if args.ops:
         print(json.dumps({"ops": ops_throughput()}))
@@ -286,7 +397,6 @@ def main():
     adds_per_s = adds / (scan_ms * 1e-3)
     # algorithmic HBM bytes of the scan+pool launch: sequence bytes in, filters in, pooled features out
     hbm_bytes = cfg["X"].size + p["Wc"].nbytes + p["bc"].nbytes + nseq * spec.F * 4
-    lds_bytes = positions * spec.F * ((spec.m + 2) // 3 + ((spec.m + 2) // 3) % 2) * 4     # an even number of 3-tap groups
     out = {
         "metric": "seq_positions_per_sec_fwd_scan_pool",
         "value": positions * args.steps / elapsed,
@@ -302,29 +412,23 @@ def main():
         "sequences_per_s": nseq * args.steps / elapsed,
         "model_sequences_per_s": nseq * spec.nmodel * args.steps / elapsed,
         "roofline": {
-            # compute-bound, priced against the published FP32 peak (the schema's compute label is "mfma";
-            # the kernel itself issues vector adds only, see bound_detail)
-            "bound": "mfma", "bound_detail": "FP32 vector ALU gather-add, no MFMA instruction issued; peak = published 157.3 TFLOP/s FP32 (FMA-counted)",
+            # compute-bound on the FP32 vector ALUs (a gather-add: no matrix instruction is issued)
+            "bound": "fp32_valu", "bound_detail": "FP32 vector ALU gather-add, no MFMA instruction issued; peak = published 157.3 TFLOP/s FP32 vector "
+                                                  "(FMA-counted); a stream of plain adds tops out at 78.6 T adds/s",
             "achieved": adds_per_s / 1e12, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": adds_per_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS, "traffic": measured_traffic(args.workload),
+            "frac": adds_per_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+            "frac_vs_add_issue_peak": adds_per_s / 1e12 / FP32_ADD_ISSUE_PEAK_TADDS,
+            "traffic": measured_traffic(args.workload),
             "kernel": "fused scan+bias+relu+maxpool (dbk_scanpool_fprop launches)", "kernel_ms": scan_ms,
             "algorithmic_adds_per_launch": adds,
-            # algorithmic adds per second over what the SIMDs can issue in plain v_add_f32 lane-operations
-            # (1024 SIMDs x 64 lanes x ~1.0e9 wave-instructions/s each, `--issue-rates`): > 1 because one executed
-            # add of a 3-mer table entry stands for three algorithmic adds
-            "algorithmic_adds_per_issuable_lane_op": adds_per_s / (1024 * 64 * 1.0e9),
             "hbm": {"algorithmic_bytes_per_launch": hbm_bytes, "achieved_GBs": hbm_bytes / (scan_ms * 1e-3) / 1e9,
                     "peak_GBs": HBM_PEAK_GBS, "frac": hbm_bytes / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
-            # what the table kernel is bound by: every executed add consumes one 4-byte table entry from LDS
-            # (ceil(m/3) entries per position and filter); measured rate of aligned ds_read_b128: 216 B/clk/CU
-            "lds": {"bytes_per_launch": lds_bytes, "achieved_TBs": lds_bytes / (scan_ms * 1e-3) / 1e12,
-                    "measured_peak_TBs": LDS_PEAK_TBS, "frac": lds_bytes / (scan_ms * 1e-3) / 1e12 / LDS_PEAK_TBS},
         },
     }
     if not args.no_train:
-        out["train"] = train_throughput()
+        out["train"] = train_throughput(cpu=not args.no_cpu_baseline)
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, nseq_c=min(nseq, 1000), nseq_np=min(nseq, 300))
+        out["cpu_baseline"] = cpu_baseline(cfg, nseq=min(nseq, 1000))
     print(json.dumps(out))
 
 
