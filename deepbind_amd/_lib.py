@@ -35,6 +35,7 @@ _SIGNATURES = {
     "dbk_poolrgn": [_P, _I, _P, _Z, _P, _Z, _I, _P, _P, _I],
     "dbk_poolrgn_bprop": [_P, _I, _P, _Z, _P, _Z, _I, _P, _P, _I],
     "dbk_dropoutord_fp_tr": [_P, _P, _P, _P, _Z, _F, _U64, _U64, _P],
+    "dbk_corr1ord_constraint": [_P, _I, _P, _Z, _Z, _I, _D, _D],
     "dbk_dropoutord_mirror": [_P, _P, _P, _P, _P, _Z, _Z],
     "dbk_dropoutord_fp_tr_u": [_P, _P, _P, _P, _Z, _F, _P],
     "dbk_scanpool_fprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
@@ -74,10 +75,10 @@ _SIGNATURES = {
     "dbk_logistic": [_P, _I, _P, _P, _Z],
     "dbk_loss_terms": [_P, _I, _I, _P, _P, _P, _Z],
     "dbk_sub_scale": [_P, _I, _P, _P, _D, _P, _Z],
-    "dbk_head_train": [_P, _Z, _I, _I, _I, _I, _I, _P, _P, _P, _U64, _U64, _P, _U64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
+    "dbk_head_train": [_P, _Z, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _U64, _U64, _P, _U64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "dbk_counter_add": [_P, _P, _U64],
     "dbk_l1_decay": [_P, _I, _P, _P, _P, _Z],
-    "dbk_head_fprop": [_P, _Z, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
+    "dbk_head_fprop": [_P, _Z, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _P],
     "dbk_train_step": [_P, _P],
     "dbk_train_steps": [_P, _Z, _P],
     "dbk_train_step_args_size": [],
@@ -98,6 +99,7 @@ class TrainStepArgs(ctypes.Structure):
         ("decay", _P), ("freeze_scan", _I),
         ("pooled", _P), ("argmax", _P), ("Z", _P), ("dpooled", _P), ("loss", _P), ("act", _P),
         ("L", _P), ("L_ready", _I),
+        ("nfeat", _Z), ("feats", _P),
     ]
 
 _dll = None

@@ -53,8 +53,8 @@ struct scan_group {                         // the scan side of one group
     float* slabs; size_t slab_stride; unsigned nslab;
 };
 struct head_group {                         // the dense head of one group (arguments of dbk_head_train)
-    int nblock, k, hidden, loss_kind, revcomp;
-    const float *pooled, *rate;
+    int nblock, k, kf, hidden, loss_kind, revcomp;   // kf: feature columns shared by all models (after each model's k inputs)
+    const float *pooled, *feats, *rate;
     uint64_t seed; uint64_t* counter;
     const float *W1, *b1, *W2, *b2, *Y;
     const uint8_t* Ymask;

@@ -315,7 +315,8 @@ __global__ void k_bdot_tn_fold(int nblock, int m, int k, int p, int off, unsigne
 // in registers (one contiguous k*4-byte read of HBM per thread) and writes one score.
 constexpr int HEAD_MAXK = 64;
 template <int KMAX>
-__global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int hidden, const float* __restrict__ pooled,
+__global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int kf, int kw, int hidden, const float* __restrict__ pooled,
+                                              const float* __restrict__ feats,
                                               const float* __restrict__ in_scale, const float* __restrict__ W1,
                                               const float* __restrict__ b1, const float* __restrict__ W2,
                                               const float* __restrict__ b2, bool apply_logistic, float* __restrict__ scores)
@@ -324,11 +325,13 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
     // models vary fastest over the grid: the workgroups that share a tile of rows run together, so each
     // 4 KB row of the feature matrix is pulled from HBM once and served to its 64 models from L2
     const unsigned b = blockIdx.x;
-    const int h1 = hidden > 0 ? hidden : 1;
-    float* w1s = hsm;                       // [k][h1]
-    float* b1s = w1s + (size_t)k * h1;      // [h1]
+    // a model's block of W1 has kw rows: k for its own inputs, then the shared feature columns, of which the
+    // first kf are read here (kf = 0 when the features are all zeros: their weights then play no part)
+    const int h1 = hidden > 0 ? hidden : 1, kt = k + kf;
+    float* w1s = hsm;                       // [kt][h1]
+    float* b1s = w1s + (size_t)kt * h1;     // [h1]
     float* w2s = b1s + h1;                  // [hidden]
-    for (int e = threadIdx.x; e < k * h1; e += blockDim.x) w1s[e] = W1[(size_t)b * k * h1 + e];
+    for (int e = threadIdx.x; e < kt * h1; e += blockDim.x) w1s[e] = W1[(size_t)b * kw * h1 + e];
     for (int e = threadIdx.x; e < h1; e += blockDim.x) b1s[e] = b1[(size_t)b * h1 + e];
     for (int e = threadIdx.x; e < hidden; e += blockDim.x) w2s[e] = W2[(size_t)b * hidden + e];
     __syncthreads();
@@ -336,9 +339,10 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
     const float bias2 = hidden > 0 ? b2[b] : 0.0f;
     for (size_t r = (size_t)blockIdx.y * blockDim.x + threadIdx.x; r < n; r += (size_t)gridDim.y * blockDim.x) {
         const float* x = pooled + r * (size_t)k * nblock + (size_t)b * k;
+        const float* xf = feats + r * (size_t)kf;                    // (only read when kf > 0)
         float xr[KMAX];
 #pragma unroll
-        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = kk < k ? x[kk] * sc : 0.0f;
+        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = kk < k ? x[kk] * sc : (kk < kt ? xf[kk - k] : 0.0f);
         float out;
         if (hidden > 0) {
             out = 0.0f;
@@ -350,7 +354,7 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
                     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
 #pragma unroll
                     for (int kk = 0; kk < KMAX; ++kk)
-                        if (kk < k) {
+                        if (kk < kt) {
                             const float4 w = *reinterpret_cast<const float4*>(w1s + kk * hidden + h);
                             // fused multiply-add, as the reference's GEMM library issues them
                             a0 = __builtin_fmaf(xr[kk], w.x, a0);
@@ -371,7 +375,7 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
                 float a = 0.0f;
 #pragma unroll
                 for (int kk = 0; kk < KMAX; ++kk)
-                    if (kk < k) a += xr[kk] * w1s[kk * hidden + h];
+                    if (kk < kt) a += xr[kk] * w1s[kk * hidden + h];
                 a += b1s[h];
                 a = a > 0.0f ? a : 0.0f;
                 out += a * w2s[h];
@@ -381,7 +385,7 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
             out = 0.0f;
 #pragma unroll
             for (int kk = 0; kk < KMAX; ++kk)
-                if (kk < k) out += xr[kk] * w1s[kk];
+                if (kk < kt) out += xr[kk] * w1s[kk];
             out += b1s[0];
         }
         if (apply_logistic) out = 1.0f / (1.0f + expf(-out));
@@ -396,23 +400,24 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int h
 // and the four rows of a wave read the same line.
 constexpr int HG = 16;
 template <int KMAX>
-__global__ __launch_bounds__(256) void k_head16(size_t n, int nblock, int k, int hidden, const float* __restrict__ pooled,
+__global__ __launch_bounds__(256) void k_head16(size_t n, int nblock, int k, int kf, int kw, int hidden, const float* __restrict__ pooled,
+                                                const float* __restrict__ feats,
                                                 const float* __restrict__ in_scale, const float* __restrict__ W1,
                                                 const float* __restrict__ b1, const float* __restrict__ W2,
                                                 const float* __restrict__ b2, bool apply_logistic, float* __restrict__ scores)
 {
     extern __shared__ __align__(16) float hsm[];
-    const int hq = hidden >> 2;
-    float* w1s = hsm;                                   // [k][hq][HG][4]
-    float* b1s = w1s + (size_t)k * hidden * HG;         // [hq][HG][4]
+    const int hq = hidden >> 2, kt = k + kf;            // inputs read: the model's own k, then kf shared feature columns
+    float* w1s = hsm;                                   // [kt][hq][HG][4]
+    float* b1s = w1s + (size_t)kt * hidden * HG;        // [hq][HG][4]
     float* w2s = b1s + (size_t)hidden * HG;             // [hq][HG][4]
     const unsigned g = threadIdx.x & (HG - 1), rl = threadIdx.x >> 4;
     const unsigned m0 = blockIdx.x * HG;                // first model of this workgroup
-    for (int e = threadIdx.x; e < k * hidden * HG; e += blockDim.x) {
+    for (int e = threadIdx.x; e < kt * hidden * HG; e += blockDim.x) {
         // destination order: e = ((kk*hq + h4)*HG + gg)*4 + c
         const int c = e & 3, gg = (e >> 2) & (HG - 1), rest = e >> 6, h4 = rest % hq, kk = rest / hq;
         const unsigned mdl = m0 + gg;
-        w1s[e] = mdl < (unsigned)nblock ? W1[((size_t)mdl * k + kk) * hidden + h4 * 4 + c] : 0.0f;
+        w1s[e] = mdl < (unsigned)nblock ? W1[((size_t)mdl * kw + kk) * hidden + h4 * 4 + c] : 0.0f;
     }
     for (int e = threadIdx.x; e < hidden * HG; e += blockDim.x) {
         const int c = e & 3, gg = (e >> 2) & (HG - 1), h4 = e >> 6;
@@ -433,20 +438,22 @@ __global__ __launch_bounds__(256) void k_head16(size_t n, int nblock, int k, int
     size_t r = (size_t)blockIdx.y * 16 + rl;
     float xn[KMAX];                                      // next row's inputs, fetched while this row is computed
 #pragma unroll
-    for (int kk = 0; kk < KMAX; ++kk) xn[kk] = (kk < k && r < n) ? pooled[r * rowlen + (size_t)mdl * k + kk] : 0.0f;
+    for (int kk = 0; kk < KMAX; ++kk)
+        xn[kk] = r < n ? (kk < k ? pooled[r * rowlen + (size_t)mdl * k + kk] : (kk < kt ? feats[r * (size_t)kf + (kk - k)] : 0.0f)) : 0.0f;
     for (; r < n; r += rstep) {
         float xr[KMAX];
 #pragma unroll
-        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = xn[kk] * sc;
+        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = kk < k ? xn[kk] * sc : xn[kk];
         const size_t rn = r + rstep;
 #pragma unroll
-        for (int kk = 0; kk < KMAX; ++kk) xn[kk] = (kk < k && rn < n) ? pooled[rn * rowlen + (size_t)mdl * k + kk] : 0.0f;
+        for (int kk = 0; kk < KMAX; ++kk)
+            xn[kk] = rn < n ? (kk < k ? pooled[rn * rowlen + (size_t)mdl * k + kk] : (kk < kt ? feats[rn * (size_t)kf + (kk - k)] : 0.0f)) : 0.0f;
         float out = 0.0f;
         for (int h4 = 0; h4 < hq; ++h4) {
             float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
 #pragma unroll
             for (int kk = 0; kk < KMAX; ++kk)
-                if (kk < k) {
+                if (kk < kt) {
                     const float4 w = w1v[(kk * hq + h4) * HG];
                     a0 = __builtin_fmaf(xr[kk], w.x, a0);
                     a1 = __builtin_fmaf(xr[kk], w.y, a1);
@@ -656,32 +663,34 @@ int dbk_blockwise_dot_tn(dbk_stream_t stream, int dtype, int nblock, int n, int 
 }
 
 int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
-                   const float* pooled, const float* in_scale,
+                   const float* pooled, int nfeat, const float* feats, const float* in_scale,
                    const float* W1, const float* b1, const float* W2, const float* b2,
                    int apply_logistic, float* scores)
 {
-    DBK_CHECK(nblock >= 1 && k >= 1 && hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, hidden=%d)", nblock, k, hidden);
+    DBK_CHECK(nblock >= 1 && k >= 1 && nfeat >= 0 && hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, nfeat=%d, hidden=%d)", nblock, k, nfeat, hidden);
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(pooled && W1 && b1 && scores, "ValueError: null pointer argument");
     DBK_CHECK(hidden == 0 || (W2 && b2), "ValueError: hidden layer requested but W2/b2 are null");
-    DBK_CHECK(k <= HEAD_MAXK, "ValueError: the fused head takes at most %d inputs per model (got %d)", HEAD_MAXK, k);
+    // all-zero feature columns (feats == NULL) add nothing: their weight rows are stepped over, not read
+    const int kw = k + nfeat, kf = feats ? nfeat : 0, kk_all = k + kf;
+    DBK_CHECK(kk_all <= HEAD_MAXK, "ValueError: the fused head takes at most %d inputs per model (got %d)", HEAD_MAXK, kk_all);
     const int h1 = hidden > 0 ? hidden : 1;
-    size_t smem = ((size_t)k * h1 + h1 + hidden) * sizeof(float);
+    size_t smem = ((size_t)kk_all * h1 + h1 + hidden) * sizeof(float);
     DBK_CHECK(smem <= 65536, "ValueError: head weights (%zu bytes per model) do not fit in LDS", smem);
     unsigned gx = dbk::divup(n, 256);
     if (gx > 2048u) gx = 2048u;
-    const size_t smem16 = ((size_t)k * hidden + 2 * (size_t)hidden) * HG * sizeof(float);
+    const size_t smem16 = ((size_t)kk_all * hidden + 2 * (size_t)hidden) * HG * sizeof(float);
     if (hidden > 0 && (hidden & 3) == 0 && smem16 <= 65536 && n >= 4096) {
         // bulk scoring: 16 models per workgroup, coalesced reads of the feature matrix
         const unsigned gy = row_slices(n, 16, dbk::divup(nblock, HG));
-        auto kern16 = k <= 16 ? k_head16<16> : (k <= 32 ? k_head16<32> : k_head16<64>);
+        auto kern16 = kk_all <= 16 ? k_head16<16> : (kk_all <= 32 ? k_head16<32> : k_head16<64>);
         DBK_HIP(hipFuncSetAttribute((const void*)kern16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem16));
-        hipLaunchKernelGGL(kern16, dim3(dbk::divup(nblock, HG), gy), dim3(256), smem16, dbk::as_stream(stream), n, nblock, k, hidden, pooled,
-                           in_scale, W1, b1, W2, b2, apply_logistic != 0, scores);
+        hipLaunchKernelGGL(kern16, dim3(dbk::divup(nblock, HG), gy), dim3(256), smem16, dbk::as_stream(stream), n, nblock, k, kf, kw, hidden, pooled,
+                           feats, in_scale, W1, b1, W2, b2, apply_logistic != 0, scores);
         DBK_LAUNCH_OK();
     }
-    auto kern = k <= 16 ? k_head<16> : (k <= 32 ? k_head<32> : k_head<64>);
-    hipLaunchKernelGGL(kern, dim3(nblock, gx), dim3(256), smem, dbk::as_stream(stream), n, nblock, k, hidden, pooled, in_scale,
+    auto kern = kk_all <= 16 ? k_head<16> : (kk_all <= 32 ? k_head<32> : k_head<64>);
+    hipLaunchKernelGGL(kern, dim3(nblock, gx), dim3(256), smem, dbk::as_stream(stream), n, nblock, k, kf, kw, hidden, pooled, feats, in_scale,
                        W1, b1, W2, b2, apply_logistic != 0, scores);
     DBK_LAUNCH_OK();
 }

@@ -356,6 +356,37 @@ template <typename T> __global__ void k_sub_scale(const T* Z, const T* Y, T scal
 #define CF64(p) ((const double*)(p))
 
 // The typed pointer casts differ per dtype, so each entry point spells out both launches.
+// The scan filters' constraint, applied to W (4m, F) in place after every update (kangaroo/_ext/corr1ord.py:60-77):
+// kind 0 "pfm": each filter tap's four letter weights become log(e / sum(e)), e = exp(w), letters added A,C,G,T;
+// kind 1 "psam": log(e / max(e)); kind 2: clipped to [lo, hi] (minimum with hi first, then maximum with lo).
+// One thread per (tap, filter); a wave reads four 256-byte row segments.
+template <typename T> __global__ void k_scan_constraint(T* W, size_t m, size_t F, int kind, T lo, T hi)
+{
+    GRID_STRIDE(i, m * F) {
+        const size_t tap = i / F, f = i % F;
+        T* w = W + tap * 4 * F + f;
+        T v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = w[(size_t)c * F];
+        if (kind == 2) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const T a = v[c] < hi ? v[c] : hi;
+                w[(size_t)c * F] = a > lo ? a : lo;
+            }
+        } else {
+            T e[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) e[c] = exp(v[c]);
+            T d;
+            if (kind == 0) { d = e[0]; d += e[1]; d += e[2]; d += e[3]; }
+            else { d = e[0]; d = e[1] > d ? e[1] : d; d = e[2] > d ? e[2] : d; d = e[3] > d ? e[3] : d; }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) w[(size_t)c * F] = log(e[c] / d);
+        }
+    }
+}
+
 #define EW2(kernel, n, ARGS32, ARGS64)                                                                     \
     do {                                                                                                   \
         DBK_DTYPE_OK(dtype);                                                                               \
@@ -511,6 +542,12 @@ int dbk_colsum(dbk_stream_t stream, int dtype, const void* X, void* out, size_t 
                               : launch_colsum<double>(dbk::as_stream(stream), CF64(X), F64(out), n, m);
     if (rc) return rc;
     DBK_LAUNCH_OK();
+}
+int dbk_corr1ord_constraint(dbk_stream_t stream, int dtype, void* W, size_t m, size_t nfilter, int kind, double lo, double hi)
+{
+    DBK_CHECK(kind >= 0 && kind <= 2, "NotImplementedError: constraint kind %d (0 = pfm, 1 = psam, 2 = clip to [lo, hi])", kind);
+    DBK_CHECK(W || m * nfilter == 0, "ValueError: null pointer argument");
+    EW2(k_scan_constraint, m * nfilter, A(F32(W), m, nfilter, kind, (float)lo, (float)hi), A(F64(W), m, nfilter, kind, lo, hi));
 }
 int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
 {

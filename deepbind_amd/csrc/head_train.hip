@@ -24,8 +24,8 @@ constexpr int NT = RB * NP;        // threads per workgroup
 
 struct head_args {
     size_t n;
-    int nblock, k, hidden, loss_kind, revcomp;
-    const float *pooled, *rate, *U;
+    int nblock, k, kf, hidden, loss_kind, revcomp;   // k pooled features per model + kf feature columns shared by all models
+    const float *pooled, *feats, *rate, *U;
     unsigned long long seed, offset;
     unsigned long long* counter;
     unsigned long long counter_advance;
@@ -40,7 +40,8 @@ struct head_args {
 __device__ __forceinline__ void head_train_body(const head_args& a, const unsigned b, const unsigned chunk)
 {
     extern __shared__ float hs[];
-    const int k = a.k, hidden = a.hidden, h1 = hidden > 0 ? hidden : 1;
+    // kt inputs per model: its k pooled features, then the kf shared feature columns (no dropout, no gradient back)
+    const int k = a.k, kt = a.k + a.kf, hidden = a.hidden, h1 = hidden > 0 ? hidden : 1;
     const unsigned tid = threadIdx.x;
     const size_t r0 = (size_t)chunk * RB;
     const int row = tid / NP, part = tid % NP;
@@ -49,9 +50,9 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
     const size_t ncol = (size_t)k * a.nblock;
     // per-row strides are odd so that lanes holding different rows hit distinct LDS banks; the weight rows too:
     // in the backward pass the eight lanes of a row read eight different inputs' weights for the same hidden unit
-    const int ks = k | 1, hst = h1 | 1, wst = hidden > 0 ? (hidden | 1) : 1;
-    float* w1s = hs;                        // [k][wst]
-    float* b1s = w1s + k * wst;             // [h1]
+    const int ks = kt | 1, hst = h1 | 1, wst = hidden > 0 ? (hidden | 1) : 1;
+    float* w1s = hs;                        // [kt][wst]
+    float* b1s = w1s + kt * wst;            // [h1]
     float* w2s = b1s + h1;                  // [h1] (unused when hidden == 0)
     float* H0s = w2s + h1;                  // [RB][ks]  inputs after dropout
     float* H1s = H0s + RB * ks;             // [RB][hst] hidden activations (hidden > 0)
@@ -61,14 +62,14 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
     unsigned char* kept = reinterpret_cast<unsigned char*>(lss + RB);   // [RB][k] dropout keep flags
 
     // four loads in flight per thread and round (a plain strided loop waits for each load before the next)
-    for (int e0 = tid; e0 < k * h1; e0 += 4 * NT) {
+    for (int e0 = tid; e0 < kt * h1; e0 += 4 * NT) {
         float v[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = e0 + j * NT < k * h1 ? a.W1[(size_t)b * k * h1 + e0 + j * NT] : 0.0f;
+        for (int j = 0; j < 4; ++j) v[j] = e0 + j * NT < kt * h1 ? a.W1[(size_t)b * kt * h1 + e0 + j * NT] : 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int e = e0 + j * NT;
-            if (e < k * h1) w1s[(e / h1) * wst + e % h1] = v[j];
+            if (e < kt * h1) w1s[(e / h1) * wst + e % h1] = v[j];
         }
     }
     for (int e = tid; e < h1; e += NT) {                          // both vectors' loads are issued before either is stored
@@ -111,6 +112,12 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
             kept[e] = kp;
         }
     }
+    // the shared feature columns follow the model's own inputs in the row (a null pointer stands for all zeros)
+    for (int e = tid; e < RB * a.kf; e += NT) {
+        const int er = e / a.kf, kk = e % a.kf;
+        const size_t rr = r0 + er;
+        H0s[er * ks + k + kk] = (a.feats && rr < a.n) ? a.feats[rr * a.kf + kk] : 0.0f;
+    }
     __syncthreads();
 
     // ---------------- forward: the row's eight lanes split the hidden units (or, without a hidden layer, the inputs)
@@ -120,7 +127,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
         for (int h = part; h < hidden; h += NP) {
             float s = 0.0f;
 #pragma unroll 8
-            for (int kk = 0; kk < k; ++kk) s += x[kk] * w1s[kk * wst + h];
+            for (int kk = 0; kk < kt; ++kk) s += x[kk] * w1s[kk * wst + h];
             s += b1s[h];
             s = s > 0.0f ? s : 0.0f;
             H1s[row * hst + h] = s;
@@ -128,7 +135,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
         }
     } else {
 #pragma unroll 4
-        for (int kk = part; kk < k; kk += NP) outp += x[kk] * w1s[kk];
+        for (int kk = part; kk < kt; kk += NP) outp += x[kk] * w1s[kk];
     }
     // butterfly over the row's lanes: every lane ends with the same bits
     outp += __shfl_xor(outp, 1, 64);
@@ -177,7 +184,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
 
     // ---------------- this chunk's share of the parameter gradients, rows ascending
     float* part_out = a.partial + ((size_t)chunk * a.nblock + b) * a.pstride;
-    for (int pidx = tid; pidx < k * h1; pidx += NT) {
+    for (int pidx = tid; pidx < kt * h1; pidx += NT) {
         const int kk = pidx / h1, h = pidx % h1;
         float s = 0.0f;
         if (hidden > 0) {
@@ -200,8 +207,8 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
         } else {
             for (int rr = 0; rr < RB; ++rr) gb1 += dAs[rr];
         }
-        part_out[k * h1 + h] = gb1;
-        part_out[k * h1 + h1 + h] = gW2;
+        part_out[kt * h1 + h] = gb1;
+        part_out[kt * h1 + h1 + h] = gW2;
     }
     if (tid == NT - 1) {
         float gb2 = 0.0f, ls = 0.0f;
@@ -209,8 +216,8 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
             gb2 += dAs[rr];
             ls += lss[rr];
         }
-        part_out[k * h1 + 2 * h1] = gb2;
-        part_out[k * h1 + 2 * h1 + 1] = ls;
+        part_out[kt * h1 + 2 * h1] = gb2;
+        part_out[kt * h1 + 2 * h1 + 1] = ls;
     }
 }
 
@@ -235,8 +242,8 @@ __global__ __launch_bounds__(NT) void k_head_train_multi(const head_multi_args m
 // Adds the row chunks in ascending order and writes each gradient to its place.
 __global__ void k_head_reduce(head_args a)
 {
-    const int k = a.k, hidden = a.hidden, h1 = hidden > 0 ? hidden : 1;
-    const unsigned nW1 = k * h1;
+    const int kt = a.k + a.kf, hidden = a.hidden, h1 = hidden > 0 ? hidden : 1;
+    const unsigned nW1 = kt * h1;
     const size_t total = (size_t)a.nblock * a.pstride;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
         const unsigned b = (unsigned)(e / a.pstride), idx = (unsigned)(e % a.pstride);
@@ -260,9 +267,10 @@ __global__ void k_head_reduce(head_args a)
     if (a.counter && a.counter_advance && blockIdx.x == 0 && threadIdx.x == 0) a.counter[0] += a.counter_advance;
 }
 
-inline size_t head_smem(int k, int h1)
+inline size_t head_smem(int k, int kf, int h1)
 {
-    return ((size_t)k * (h1 | 1) + 2 * h1 + (size_t)RB * (k | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
+    const int kt = k + kf;
+    return ((size_t)kt * (h1 | 1) + 2 * h1 + (size_t)RB * (kt | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
 }
 
 }  // namespace
@@ -278,13 +286,13 @@ int dbk::head_train_multi(hipStream_t st, size_t nrow, unsigned n, dbk::head_gro
     size_t smem = 0, total = 0;
     for (unsigned i = 0; i < n; ++i) {
         const int h1 = g[i].hidden > 0 ? g[i].hidden : 1;
-        DBK_CHECK(g[i].nblock >= 1 && g[i].k >= 1 && g[i].hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, hidden=%d)", g[i].nblock, g[i].k, g[i].hidden);
+        DBK_CHECK(g[i].nblock >= 1 && g[i].k >= 1 && g[i].kf >= 0 && g[i].hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, nfeat=%d, hidden=%d)", g[i].nblock, g[i].k, g[i].kf, g[i].hidden);
         DBK_CHECK(!g[i].revcomp || nrow % 2 == 0, "ValueError: reverse-complement rows come in pairs, got %zu rows", nrow);
-        const size_t need = head_smem(g[i].k, h1);
-        DBK_CHECK(need <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", g[i].k, g[i].hidden, need);
+        const size_t need = head_smem(g[i].k, g[i].kf, h1);
+        DBK_CHECK(need <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", g[i].k + g[i].kf, g[i].hidden, need);
         smem = need > smem ? need : smem;
         g[i].nchunk = (unsigned)nchunk;
-        g[i].pstride = (unsigned)(g[i].k * h1 + 2 * h1 + 2);
+        g[i].pstride = (unsigned)((g[i].k + g[i].kf) * h1 + 2 * h1 + 2);
         total += nchunk * (size_t)g[i].nblock * g[i].pstride;
         m.first[i + 1] = m.first[i] + (unsigned)(g[i].nblock * nchunk);
     }
@@ -294,7 +302,7 @@ int dbk::head_train_multi(hipStream_t st, size_t nrow, unsigned n, dbk::head_gro
         g[i].partial = partial;
         partial += nchunk * (size_t)g[i].nblock * g[i].pstride;
         head_args& a = m.g[i];
-        a.n = nrow; a.nblock = g[i].nblock; a.k = g[i].k; a.hidden = g[i].hidden; a.loss_kind = g[i].loss_kind; a.revcomp = g[i].revcomp;
+        a.n = nrow; a.nblock = g[i].nblock; a.k = g[i].k; a.kf = g[i].kf; a.feats = g[i].feats; a.hidden = g[i].hidden; a.loss_kind = g[i].loss_kind; a.revcomp = g[i].revcomp;
         a.pooled = g[i].pooled; a.rate = g[i].rate; a.U = nullptr; a.seed = g[i].seed; a.offset = 0;
         a.counter = (unsigned long long*)g[i].counter; a.counter_advance = 0;
         a.W1 = g[i].W1; a.b1 = g[i].b1; a.W2 = g[i].W2; a.b2 = g[i].b2; a.Y = g[i].Y; a.Ymask = g[i].Ymask;
@@ -307,30 +315,30 @@ int dbk::head_train_multi(hipStream_t st, size_t nrow, unsigned n, dbk::head_gro
 }
 
 extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden, int loss_kind, int reverse_complement,
-                              const float* pooled, const float* rate, const float* U, uint64_t seed, uint64_t offset,
+                              const float* pooled, int nfeat, const float* feats, const float* rate, const float* U, uint64_t seed, uint64_t offset,
                               uint64_t* counter, uint64_t counter_advance,
                               const float* W1, const float* b1, const float* W2, const float* b2,
                               const float* Y, const uint8_t* Ymask,
                               float* Z, float* dpooled, float* dW1, float* db1, float* dW2, float* db2, float* loss)
 {
-    DBK_CHECK(nblock >= 1 && k >= 1 && hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, hidden=%d)", nblock, k, hidden);
+    DBK_CHECK(nblock >= 1 && k >= 1 && nfeat >= 0 && hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, nfeat=%d, hidden=%d)", nblock, k, nfeat, hidden);
     DBK_CHECK(loss_kind == 0 || loss_kind == 1, "ValueError: loss kind must be 0 (logistic + nll) or 1 (linear + mse), got %d", loss_kind);
     const int h1 = hidden > 0 ? hidden : 1;
     DBK_CHECK(!reverse_complement || n % 2 == 0, "ValueError: reverse-complement rows come in pairs, got %zu rows", n);
     if (n == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(pooled && W1 && b1 && Y && Z && dpooled && dW1 && db1, "ValueError: null pointer argument");
     DBK_CHECK(hidden == 0 || (W2 && b2 && dW2 && db2), "ValueError: hidden layer requested but W2/b2/dW2/db2 are null");
-    const size_t smem = head_smem(k, h1);
-    DBK_CHECK(smem <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", k, hidden, smem);
+    const size_t smem = head_smem(k, nfeat, h1);
+    DBK_CHECK(smem <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", k + nfeat, hidden, smem);
     const size_t nchunk = (n + RB - 1) / RB;
     DBK_CHECK(nchunk <= 65535, "ValueError: the fused head takes at most %d rows per call (got %zu)", 65535 * RB, n);
     head_args a;
-    a.n = n; a.nblock = nblock; a.k = k; a.hidden = hidden; a.loss_kind = loss_kind; a.revcomp = reverse_complement;
+    a.n = n; a.nblock = nblock; a.k = k; a.kf = nfeat; a.feats = feats; a.hidden = hidden; a.loss_kind = loss_kind; a.revcomp = reverse_complement;
     a.pooled = pooled; a.rate = rate; a.U = U; a.seed = seed; a.offset = offset; a.counter = (unsigned long long*)counter; a.counter_advance = counter_advance;
     a.W1 = W1; a.b1 = b1; a.W2 = W2; a.b2 = b2; a.Y = Y; a.Ymask = Ymask;
     a.Z = Z; a.dpooled = dpooled; a.dW1 = dW1; a.db1 = db1; a.dW2 = dW2; a.db2 = db2; a.loss = loss;
     a.nchunk = (unsigned)nchunk;
-    a.pstride = (unsigned)(k * h1 + 2 * h1 + 2);
+    a.pstride = (unsigned)((k + nfeat) * h1 + 2 * h1 + 2);
     const size_t pbytes = nchunk * (size_t)nblock * a.pstride * sizeof(float);
     dbk::deferred_sums* later = dbk::deferred();                   // inside dbk_train_step: the chunk sums are taken by its last kernel
     a.partial = (float*)dbk::workspace(pbytes, dbk::as_stream(stream), later ? 1 : 0);

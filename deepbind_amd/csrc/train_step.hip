@@ -38,7 +38,7 @@ struct reduce_update_args {
     size_t nWc, nbc, nW1, nb1, nW2, nb2;
     const float* slabs; size_t slab_stride; unsigned nslab;
     const float* head_partial; unsigned nchunk, pstride;
-    unsigned nblock, k, h1, hidden;
+    unsigned nblock, k, h1, hidden;                                // k: rows of a model's block of W1
     int freeze_scan, loss_kind;
     float* loss; size_t nrow;
     unsigned long long* counter; unsigned long long counter_advance;
@@ -138,14 +138,15 @@ __global__ void k_zero_f32(float* p, size_t n)
 namespace {
 
 // Sizes of a group's parameter blocks.
-struct block_sizes { size_t F, k, nWc, nW1, nb1, nW2, nb2; };
+struct block_sizes { size_t F, k, kt, nWc, nW1, nb1, nW2, nb2; };
 block_sizes sizes_of(const dbk_train_step_args* a)
 {
     block_sizes z;
     z.F = a->nmodel * a->nfilter;                                  // filters of all models, side by side
     z.k = a->nfilter * (a->ptype == DBK_PT_ALL ? 2 : 1);           // pooled features per model
     z.nWc = 4 * a->m * z.F;
-    z.nW1 = z.k * a->nmodel * (a->hidden ? a->hidden : 1);
+    z.kt = z.k + a->nfeat;                                         // rows of a model's block of W1: its inputs, then the shared feature columns
+    z.nW1 = z.kt * a->nmodel * (a->hidden ? a->hidden : 1);
     z.nb1 = a->nmodel * (a->hidden ? a->hidden : 1);
     z.nW2 = a->hidden ? a->hidden * a->nmodel : 0;
     z.nb2 = a->hidden ? a->nmodel : 0;
@@ -193,7 +194,7 @@ int fill_update(reduce_update_args& u, const dbk_train_step_args* a, const block
     u.nWc = z.nWc; u.nbc = z.F; u.nW1 = z.nW1; u.nb1 = z.nb1; u.nW2 = z.nW2; u.nb2 = z.nb2;
     u.slabs = slabs; u.slab_stride = slab_stride; u.nslab = nslab;
     u.head_partial = head_partial; u.nchunk = nchunk; u.pstride = pstride;
-    u.nblock = (unsigned)a->nmodel; u.k = (unsigned)z.k; u.h1 = (unsigned)(a->hidden ? a->hidden : 1); u.hidden = (unsigned)a->hidden;
+    u.nblock = (unsigned)a->nmodel; u.k = (unsigned)z.kt; u.h1 = (unsigned)(a->hidden ? a->hidden : 1); u.hidden = (unsigned)a->hidden;
     u.freeze_scan = a->freeze_scan; u.loss_kind = a->loss_kind; u.loss = a->loss; u.nrow = a->nregion;
     u.counter = (unsigned long long*)a->counter; u.counter_advance = draws;
     DBK_CHECK(z.nWc + z.F + z.nW1 + z.nb1 + z.nW2 + z.nb2 == a->nparam, "ValueError: the parameter blocks do not tile the flat vector (%zu of %zu elements)",
@@ -242,7 +243,7 @@ extern "C" int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* a)
     if (rc) return rc;
     const uint64_t draws = a->rate ? (a->nregion * k * a->nmodel + 3) / 4 : 0;
     rc = dbk_head_train(stream, a->nregion, (int)a->nmodel, (int)k, (int)a->hidden, a->loss_kind, a->reverse_complement,
-                        a->pooled, a->rate, nullptr, a->seed, 0, a->counter, draws,
+                        a->pooled, (int)a->nfeat, a->feats, a->rate, nullptr, a->seed, 0, a->counter, draws,
                         P + a->off_W1, P + a->off_b1, a->hidden ? P + a->off_W2 : nullptr, a->hidden ? P + a->off_b2 : nullptr,
                         a->Y, a->Ymask, a->Z, a->dpooled,
                         dP + a->off_W1, dP + a->off_b1, a->hidden ? dP + a->off_W2 : nullptr, a->hidden ? dP + a->off_b2 : nullptr,
@@ -345,7 +346,7 @@ extern "C" int dbk_train_steps(dbk_stream_t stream, size_t ngroup, const dbk_tra
         const block_sizes z = sizes_of(a);
         const float* P = a->L;
         draws[i] = a->rate ? (a->nregion * z.k * a->nmodel + 3) / 4 : 0;
-        hg[i].nblock = (int)a->nmodel; hg[i].k = (int)z.k; hg[i].hidden = (int)a->hidden; hg[i].loss_kind = a->loss_kind;
+        hg[i].nblock = (int)a->nmodel; hg[i].k = (int)z.k; hg[i].kf = (int)a->nfeat; hg[i].feats = a->feats; hg[i].hidden = (int)a->hidden; hg[i].loss_kind = a->loss_kind;
         hg[i].revcomp = a->reverse_complement;
         hg[i].pooled = a->pooled; hg[i].rate = a->rate; hg[i].seed = a->seed; hg[i].counter = a->counter;
         hg[i].W1 = P + a->off_W1; hg[i].b1 = P + a->off_b1;

@@ -223,36 +223,44 @@ def uniform_like(X, seed, offset):
     return U
 
 
-def head_fprop(pooled, W1, b1, W2=None, b2=None, nblock=1, in_scale=None, apply_logistic=False):
+def head_fprop(pooled, W1, b1, W2=None, b2=None, nblock=1, in_scale=None, apply_logistic=False, nfeat=0, feats=None):
     """Scores (n x nblock) of nblock independent heads on pooled (n x k*nblock): one dense layer
-    (W2 is None) or dense -> bias -> ReLU -> dense -> bias, optional logistic. float32 only."""
+    (W2 is None) or dense -> bias -> ReLU -> dense -> bias, optional logistic. float32 only.
+    nfeat: feature columns shared by all models, entering after each model's own inputs (W1 has k + nfeat
+    rows per model); feats (n, nfeat) or None for all zeros."""
     require(pooled.dtype == torch.float32, "TypeError: the fused head is float32 only")
     n = pooled.shape[0]
     k = pooled.shape[1] // nblock
     hidden = 0 if W2 is None else W1.shape[1]
-    require(W1.shape[0] == k * nblock, "ValueError: W1 must have k*nblock rows")
+    require(W1.shape[0] == (k + nfeat) * nblock, "ValueError: W1 must have (k + nfeat) * nblock rows")
+    require(feats is None or (feats.dtype == torch.float32 and tuple(feats.shape) == (n, nfeat)), "ValueError: feats must be float32 (n, nfeat)")
     scores = torch.empty((n, nblock), dtype=torch.float32, device=pooled.device)
     sc = None if in_scale is None else _vec(in_scale, pooled)
-    call("dbk_head_fprop", stream(), n, nblock, k, hidden, ptr(pooled), ptr(sc), ptr(W1), ptr(b1), ptr(W2), ptr(b2),
+    call("dbk_head_fprop", stream(), n, nblock, k, hidden, ptr(pooled), int(nfeat), ptr(feats), ptr(sc), ptr(W1), ptr(b1), ptr(W2), ptr(b2),
          int(bool(apply_logistic)), ptr(scores))
     return scores
 
 
 def head_train(pooled, W1, b1, W2, b2, Y, nblock, loss, dW1, db1, dW2=None, db2=None, Ymask=None, rate=None, U=None,
-               seed=0, offset=0, counter=None, counter_advance=0, reverse_complement=False, want_loss=False):
+               seed=0, offset=0, counter=None, counter_advance=0, reverse_complement=False, want_loss=False,
+               nfeat=0, feats=None):
     """Forward and backward of nblock dense heads. Returns (Z, dpooled, loss|None); the weight gradients
     are written into dW1, db1, dW2, db2. With `counter` (device int64) the dropout generator position is
-    read from it and moved on by `counter_advance` once the masks are drawn. float32 only."""
+    read from it and moved on by `counter_advance` once the masks are drawn. float32 only.
+    nfeat: feature columns shared by all models that enter the first layer after each model's pooled
+    features (W1 has k + nfeat rows per model); feats (n, nfeat) or None for all zeros."""
     require(pooled.dtype == torch.float32, "TypeError: the fused head is float32 only")
     n = pooled.shape[0]
     k = pooled.shape[1] // nblock
     hidden = 0 if W2 is None else W1.shape[1]
+    require(W1.shape[0] == (k + nfeat) * nblock, "ValueError: W1 must have (k + nfeat) * nblock = %d rows, got %d" % ((k + nfeat) * nblock, W1.shape[0]))
+    require(feats is None or (feats.dtype == torch.float32 and tuple(feats.shape) == (n, nfeat)), "ValueError: feats must be float32 (n, nfeat)")
     Z = torch.empty((n, nblock), dtype=torch.float32, device=pooled.device)
     dpooled = torch.empty_like(pooled)
     L = torch.empty((1, nblock), dtype=torch.float32, device=pooled.device) if want_loss else None
     r = None if rate is None else _vec(rate, pooled)
     call("dbk_head_train", stream(), n, nblock, k, hidden, {"nll": 0, "mse": 1}[loss], int(bool(reverse_complement)),
-         ptr(pooled), ptr(r), ptr(U), int(seed), int(offset), ptr(counter), int(counter_advance), ptr(W1), ptr(b1), ptr(W2), ptr(b2), ptr(Y), ptr(Ymask),
+         ptr(pooled), int(nfeat), ptr(feats), ptr(r), ptr(U), int(seed), int(offset), ptr(counter), int(counter_advance), ptr(W1), ptr(b1), ptr(W2), ptr(b2), ptr(Y), ptr(Ymask),
          ptr(Z), ptr(dpooled), ptr(dW1), ptr(db1), ptr(dW2), ptr(db2), ptr(L))
     return Z, dpooled, L
 

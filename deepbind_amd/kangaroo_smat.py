@@ -131,6 +131,23 @@ def dropoutord_fp_train(X, rate, U=None, regions=None, padding=None, seed=None, 
     return Z, M
 
 
+def corr1ord_enforce_constraints(W, constraint, nchannel=4):
+    """Applies the scan filters' constraint to W (4*m, nfilter) in place: "pfm" (each tap's letter weights become
+    log-probabilities), "psam" (log of the weights relative to the tap's largest), a (lo, hi) tuple (clip), or
+    None (nothing). reference: corr1ord.enforce_constraints, kangaroo/_ext/corr1ord.py:60-77"""
+    if constraint is None:
+        return
+    require(nchannel == 4, "NotImplementedError: only the 4-letter alphabet is supported")
+    require(W.dim() == 2 and W.shape[0] % 4 == 0 and W.is_contiguous(), "ValueError: W must be a contiguous (4*m, nfilter) matrix")
+    if constraint in ("pfm", "psam"):
+        kind, lo, hi = (0 if constraint == "pfm" else 1), 0.0, 0.0
+    elif type(constraint) == tuple:
+        kind, (lo, hi) = 2, constraint
+    else:
+        raise NotImplementedError("constraint \"%s\" not implemented" % str(constraint))
+    call("dbk_corr1ord_constraint", stream(), dtype_code(W), ptr(W), W.shape[0] // 4, W.shape[1], kind, float(lo), float(hi))
+
+
 # ------------------------------------------------------------------------------------------------
 # fused scan + bias + ReLU + pool
 # ------------------------------------------------------------------------------------------------

@@ -37,7 +37,7 @@ class SequenceNet(object):
     def __init__(self, nmodel, nfilter, m, pool="max", hidden=32, loss="nll", dtype=torch.float32,
                  rate=0.01, momentum=0.9, decay_conv=0.0, decay_full=0.0, dropout=0.0,
                  weight_decay_start=100, nesterov=True, mode="fused", reverse_complement=False, input_dropout=0.0,
-                 start_training=0, device="cuda"):
+                 start_training=0, feature_columns=0, constraint=None, device="cuda"):
         assert pool in ("max", "avg", "all") and loss in ("nll", "mse", None)
         self.ninst, self.nfilter, self.m = int(nmodel), int(nfilter), int(m)
         self.pool, self.hidden, self.loss = pool, int(hidden), loss
@@ -53,6 +53,9 @@ class SequenceNet(object):
         self.input_dropout = float(input_dropout)
         # the scan filters' gradient is zeroed while step < start_training (reference: kangaroo/_ext/corr1ord.py:135-136)
         self.start_training = int(start_training)
+        # constraint on the scan filters, enforced before the first step and after every update:
+        # "pfm", "psam", a (lo, hi) tuple or None (reference: kangaroo/_ext/corr1ord.py:60-77, deepity/sgd.py:103-107,137)
+        self.constraint = constraint
         self.step_count = 0
         self._step_args = None               # argument block and work buffers of the natively issued step
         self._step_bufs = {}
@@ -61,13 +64,20 @@ class SequenceNet(object):
         self._L, self._L_versions = None, None
         ni, nf = self.ninst, self.nfilter
         self.k = nf * (2 if pool == "all" else 1)          # pooled features per model
+        # the reference's first dense layer (its "combiner") has a second input: a feature matrix with
+        # feature_columns columns (16 in its models) that all models share. Each model's block of W1 then has
+        # k + feature_columns rows, and the L1 cost and decay cover those rows too. The reference's data source
+        # fills that matrix with zeros, which is what a batch without `F` means here.
+        # (reference: kangaroo/kangaroo/model.py:101-112, data.py:59-69, deepity/std/full.py:137-178)
+        self.nfeat = int(feature_columns)
+        kw = self.k + self.nfeat                           # rows of one model's block of W1
         h = self.hidden
         # (name, shape, axis along which models are laid out)
         layout = [("Wc", (4 * m, nf * ni), 1), ("bc", (1, nf * ni), 1)]
         if h > 0:
-            layout += [("W1", (self.k * ni, h), 0), ("b1", (1, h * ni), 1), ("W2", (h * ni, 1), 0), ("b2", (1, ni), 1)]
+            layout += [("W1", (kw * ni, h), 0), ("b1", (1, h * ni), 1), ("W2", (h * ni, 1), 0), ("b2", (1, ni), 1)]
         else:
-            layout += [("W1", (self.k * ni, 1), 0), ("b1", (1, ni), 1)]
+            layout += [("W1", (kw * ni, 1), 0), ("b1", (1, ni), 1)]
         self.layout = layout
         sizes = [int(np.prod(shape)) for _, shape, _ in layout]
         self.offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
@@ -157,6 +167,14 @@ class SequenceNet(object):
                 cost = cost + rows.cpu().numpy().astype(np.float64).ravel() * self.decay_full.cpu().numpy().ravel()
         return cost.reshape(1, ni)
 
+    def enforce_constraints(self):
+        """Applies the scan filters' constraint to the parameters in place. The trainer calls it once before the
+        first step (after the parameters are set) and train_step calls it after every update."""
+        if self.constraint is None:
+            return
+        ks.corr1ord_enforce_constraints(self.p["Wc"], self.constraint)
+        self._L_versions = None              # the look-ahead kept beside the parameters no longer matches them
+
     def get_params(self):
         torch.cuda.synchronize()
         return {name: self.p[name].cpu().numpy().copy() for name, _, _ in self.layout}
@@ -168,7 +186,7 @@ class SequenceNet(object):
     # ------------------------------------------------------------------ export
     def _config(self):
         return dict(nfilter=self.nfilter, m=self.m, pool=self.pool, hidden=self.hidden, loss=self.loss or "",
-                    reverse_complement=self.reverse_complement, input_dropout=self.input_dropout)
+                    reverse_complement=self.reverse_complement, input_dropout=self.input_dropout, feature_columns=self.nfeat)
 
     def slice_model(self, i):
         """A single-model net holding model i's parameters and dropout rate, for export and prediction
@@ -176,7 +194,7 @@ class SequenceNet(object):
         assert 0 <= i < self.ninst
         one = SequenceNet(1, self.nfilter, self.m, pool=self.pool, hidden=self.hidden, loss=self.loss, dtype=self.dtype,
                           dropout=float(self.dropout[i].item()), mode=self.mode, reverse_complement=self.reverse_complement,
-                          input_dropout=self.input_dropout, device=self.device)
+                          input_dropout=self.input_dropout, feature_columns=self.nfeat, device=self.device)
         src = self.get_params()
         picked = {}
         for name, shape, axis in self.layout:
@@ -201,7 +219,8 @@ class SequenceNet(object):
             params = {k[2:]: f[k] for k in f.files if k.startswith("p_")}
         net = SequenceNet(1, int(cfg["nfilter"]), int(cfg["m"]), pool=str(cfg["pool"]), hidden=int(cfg["hidden"]),
                           loss=(str(cfg["loss"]) or None), dropout=float(cfg["dropout"]), mode=mode,
-                          reverse_complement=bool(cfg["reverse_complement"]), input_dropout=float(cfg["input_dropout"]), device=device)
+                          reverse_complement=bool(cfg["reverse_complement"]), input_dropout=float(cfg["input_dropout"]),
+                          feature_columns=int(cfg.get("feature_columns", 0)), device=device)
         net.set_params(params)
         return net
 
@@ -239,7 +258,30 @@ class SequenceNet(object):
         pooled, amax = ks.poolrgn(A, R, self.pool, want_argmax=want_argmax)
         return pooled, amax, A
 
-    def forward(self, X, R, train=False, U=None, want_argmax=False):
+    def _features(self, F, n):
+        """The batch's shared feature matrix (n, feature_columns); None means the reference's all-zero one."""
+        if F is None:
+            return torch.zeros((n, self.nfeat), dtype=self.dtype, device=self.device)
+        _lib.require(F.dtype == self.dtype and tuple(F.shape) == (n, self.nfeat), "ValueError: F must be (rows, feature_columns) of the net's dtype")
+        return F
+
+    def _dense1(self, H0, F):
+        """First dense layer: the pooled features, or [pooled features | shared feature columns] stacked along
+        each model's rows of W1 (reference: deepity/std/full.py:154-160)."""
+        if self.nfeat == 0:
+            return ds.blockwise_dot(H0, self.p["W1"], self.ninst)
+        return ds.blockwise_dot_combined([H0, self._features(F, H0.shape[0])], self.p["W1"], self.ninst, [False, True])
+
+    def _dense1_back(self, H0, F, dA1, want_dW=True):
+        """(dW1, dH0) of the first dense layer (reference: deepity/std/full.py:162-178)."""
+        W1, ni = self.p["W1"], self.ninst
+        if self.nfeat == 0:
+            return (ds.blockwise_dot_tn(H0, dA1, ni, W1) if want_dW else None), ds.blockwise_dot_nt(dA1, W1, ni)
+        Xs = [H0, self._features(F, H0.shape[0])]
+        dW = ds.blockwise_dot_tn_combined(Xs, dA1, W1, ni, [False, True]) if want_dW else None
+        return dW, ds.blockwise_dot_nt_combined(Xs, dA1, W1, ni, [False, True])[0]
+
+    def forward(self, X, R, train=False, U=None, want_argmax=False, F=None):
         """Returns the state dict of one forward pass; st["Z"] are the predictions (n x ninst)."""
         p, ni = self.p, self.ninst
         st = {}
@@ -255,8 +297,8 @@ class SequenceNet(object):
                 H0, st["M"] = ds.dropout_fp_train(H0, self.dropout, self.reverse_complement, U=U)
             else:
                 H0 = ds.dropout_fp_test(H0, self.dropout)
-        st["H0"] = H0
-        A1 = sm.add_rowvec(ds.blockwise_dot(H0, p["W1"], ni), p["b1"])
+        st["H0"], st["F"] = H0, F
+        A1 = sm.add_rowvec(self._dense1(H0, F), p["b1"])
         if self.hidden > 0:
             st["H1"] = sm.relu(A1)
             A2 = sm.add_rowvec(ds.blockwise_dot(st["H1"], p["W2"], ni), p["b2"])
@@ -269,19 +311,21 @@ class SequenceNet(object):
             ds.calc_Zmask(st["Z"], st["Zmask"])
         return st
 
-    def predict(self, X, R):
+    def predict(self, X, R, F=None):
         """Test-mode predictions through the fused scoring head (dropout rescale folded in)."""
         p = self.p
         pooled, _, _ = self._conv_forward(X, R, False)
         if self.dtype != torch.float32:
-            Z = self.forward(X, R)["Z"]
+            Z = self.forward(X, R, F=F)["Z"]
             return ds.pair_max(Z) if self.reverse_complement else Z
         scale = (1.0 - self.dropout) if self.use_dropout else None
+        if F is not None:
+            self._features(F, pooled.shape[0])
         Z = ds.head_fprop(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), nblock=self.ninst,
-                          in_scale=scale, apply_logistic=(self.loss == "nll"))
+                          in_scale=scale, apply_logistic=(self.loss == "nll"), nfeat=self.nfeat, feats=F)
         return ds.pair_max(Z) if self.reverse_complement else Z
 
-    def input_gradients(self, X, R):
+    def input_gradients(self, X, R, F=None):
         """Test-mode predictions plus the gradient map used for sequence logos / mutation maps:
         returns (Z (rows, ninst), dX (N, 4)) where dX is the back-propagated gradient w.r.t. the
         one-hot inputs of dA = Z (targets 0, no batch mean, output column 0 only, and with
@@ -297,7 +341,7 @@ class SequenceNet(object):
         A0 = sm.relu(sm.add_rowvec(Z0, p["bc"]))
         pooled, amax = ks.poolrgn(A0, R, self.pool, want_argmax=True)
         H0 = ds.dropout_fp_test(pooled, self.dropout) if self.use_dropout else pooled
-        A1 = sm.add_rowvec(ds.blockwise_dot(H0, p["W1"], ni), p["b1"])
+        A1 = sm.add_rowvec(self._dense1(H0, F), p["b1"])
         if self.hidden > 0:
             H1 = sm.relu(A1)
             A2 = sm.add_rowvec(ds.blockwise_dot(H1, p["W2"], ni), p["b2"])
@@ -312,7 +356,7 @@ class SequenceNet(object):
         if dA.shape[1] > 1:
             dA[:, 1:] = 0
         dA1 = sm.mul_sign(ds.blockwise_dot_nt(dA, p["W2"], ni), H1) if self.hidden > 0 else dA
-        dH0 = ds.blockwise_dot_nt(dA1, p["W1"], ni)
+        dH0 = self._dense1_back(H0, F, dA1, want_dW=False)[1]
         if self.use_dropout:
             dH0 = ds.dropout_bp_te(dH0, self.dropout)
         dA0 = sm.zeros_like(A0)
@@ -350,8 +394,8 @@ class SequenceNet(object):
         else:
             dA1 = dA
         g["b1"].copy_(sm.sum_axis0(dA1))
-        g["W1"].copy_(ds.blockwise_dot_tn(st["H0"], dA1, ni, p["W1"]))
-        dH0 = ds.blockwise_dot_nt(dA1, p["W1"], ni)
+        dW1, dH0 = self._dense1_back(st["H0"], st.get("F"), dA1)
+        g["W1"].copy_(dW1)
         if self.use_dropout:
             dH0 = ds.dropout_bp_tr(dH0, st["M"]) if "M" in st else ds.dropout_bp_te(dH0, self.dropout)
         if self.mode == "fused":
@@ -388,7 +432,7 @@ class SequenceNet(object):
     def _add_decay(self):
         ds.l1_decay(self.P, self.decay_vec, self.dP)
 
-    def _grad_fused(self, X, R, Y, Ymask, U, U_input=None):
+    def _grad_fused(self, X, R, Y, Ymask, U, U_input=None, F=None):
         """Gradient of one batch in a handful of launches: fused scan+pool forward, the whole dense head
         forward+backward (+ chunk reduction), fused scan+pool backward (+ slab reduction)."""
         p, g = self.p, self.g
@@ -401,7 +445,7 @@ class SequenceNet(object):
         Z, dpooled, _ = ds.head_train(pooled, p["W1"], p["b1"], p.get("W2"), p.get("b2"), Y, self.ninst, self.loss,
                                       g["W1"], g["b1"], g.get("W2"), g.get("b2"), Ymask=Ymask, rate=rate, U=U,
                                       seed=self.rng_seed, counter=self.rng_counter, counter_advance=draws,
-                                      reverse_complement=self.reverse_complement)
+                                      reverse_complement=self.reverse_complement, nfeat=self.nfeat, feats=F)
         self._rng_offset += draws
         ks.scanpool_bprop(p["Wc"], p["bc"], X, R, self.pool, pooled, amax, dpooled, g["Wc"], g["bc"], overwrite=True, act=act)
         if self.weight_decay_start <= self.step_count:
@@ -411,7 +455,7 @@ class SequenceNet(object):
         return Z
 
     # ------------------------------------------------------------------ one optimiser step
-    def _prepare_step(self, X, R, Y, Ymask=None):
+    def _prepare_step(self, X, R, Y, Ymask=None, F=None):
         """Fills this net's dbk_train_step_args block for one step on the batch and returns the step's work
         buffers (made on the current stream, where the step is issued)."""
         ks._u8(X)
@@ -463,6 +507,8 @@ class SequenceNet(object):
         pv = lambda t: None if t is None else _lib.ptr(t).value          # checks device + contiguity
         a.X, a.N, a.regions, a.nregion = pv(X), X.numel(), pv(R), P
         a.Y, a.Ymask = pv(Y), pv(Ymask)
+        _lib.require(F is None or (F.dtype == torch.float32 and tuple(F.shape) == (P, self.nfeat)), "ValueError: F must be float32 (rows x feature_columns)")
+        a.nfeat, a.feats = self.nfeat, pv(F)
         a.input_rate = self.input_dropout
         for name, t in buf.items():
             setattr(a, name, None if t is None else t.data_ptr())
@@ -479,58 +525,62 @@ class SequenceNet(object):
             self._rng_offset += (R.shape[0] * self.k * self.ninst + 3) // 4
         self.step_count += 1
 
-    def _native_step(self, X, R, Y, Ymask=None):
+    def _native_step(self, X, R, Y, Ymask=None, F=None):
         """One fused step through dbk_train_step: one library call issues every launch of the step (the
         scripting host otherwise pays several microseconds per launch, which is what bounds a step on a
         small minibatch). Same kernels in the same order as gradstep(..., _grad_fused), so the same bits."""
-        buf = self._prepare_step(X, R, Y, Ymask)
+        buf = self._prepare_step(X, R, Y, Ymask, F)
         _lib.call("dbk_train_step", _lib.stream(), ctypes.addressof(self._step_args))
         self._finish_step(X, R)
+        self.enforce_constraints()
         return buf["Z"]
 
-    def make_graphed_step(self, X, R, Y, Ymask=None):
+    def make_graphed_step(self, X, R, Y, Ymask=None, F=None):
         """Captures one fused training step on the given (static) batch tensors into a HIP graph and
         returns a function that replays it: for launch-bound batch sizes the step then costs one
         graph launch instead of ~10 kernel launches. Dropout masks stay fresh on every replay because
         the generator position lives in device memory. The graph bakes in whether L1 decay is
         active and whether the scan filters are still frozen, so it is re-captured when the step
         counter crosses weight_decay_start or start_training."""
-        return _graphed_step([(self, X, R, Y, Ymask)])
+        return _graphed_step([(self, X, R, Y, Ymask, F)])
 
-    def train_step(self, X, R, Y, Ymask=None, U=None, U_input=None):
+    def train_step(self, X, R, Y, Ymask=None, U=None, U_input=None, F=None):
         """One optimiser step. U / U_input optionally supply the uniforms of the pooled-feature and the
-        input dropout (otherwise the library's generator draws them)."""
+        input dropout (otherwise the library's generator draws them). F: the batch's shared feature matrix
+        (rows x feature_columns), None for all zeros."""
         fused = self.mode == "fused" and self.dtype == torch.float32 and self.loss is not None
         if fused and U is None and U_input is None:
-            self._native_step(X, R, Y, Ymask)
+            self._native_step(X, R, Y, Ymask, F)
             return
 
         self._L_versions = None                 # the step below updates P and mP in place
 
         def grad():
             if fused:
-                self._grad_fused(X, R, Y, Ymask, U, U_input)
+                self._grad_fused(X, R, Y, Ymask, U, U_input, F)
             else:
                 Xd = self._drop_inputs(X, R, U_input)
-                st = self.forward(Xd, R, train=True, U=U, want_argmax=True)
+                st = self.forward(Xd, R, train=True, U=U, want_argmax=True, F=F)
                 self.backward(Xd, R, st, Y, Ymask)
         ds.gradstep(self.P, self.dP, self.drate, self.mP, self.mrate, grad, nesterov=self.nesterov)
         self.step_count += 1
+        self.enforce_constraints()
 
 
 def _native_steps(jobs):
-    """jobs: list of (net, X, R, Y, Ymask), nets that step on the same batch. One dbk_train_steps call per eight
+    """jobs: list of (net, X, R, Y, Ymask[, F]), nets that step on the same batch. One dbk_train_steps call per eight
     nets on the current stream: every phase of the step is one launch holding all the nets' grids, so nets too
     small to fill the GPU run side by side without extra streams. Each net gets the bits of its own step."""
     for i in range(0, len(jobs), 8):
         chunk = jobs[i:i + 8]
         blocks = (ctypes.c_void_p * len(chunk))()
-        for j, (net, X, R, Y, Ymask) in enumerate(chunk):
-            net._prepare_step(X, R, Y, Ymask)
+        for j, (net, X, R, Y, Ymask, *rest) in enumerate(chunk):
+            net._prepare_step(X, R, Y, Ymask, rest[0] if rest else None)
             blocks[j] = ctypes.addressof(net._step_args)
         _lib.call("dbk_train_steps", _lib.stream(), len(chunk), blocks)
-        for net, X, R, _, _ in chunk:
+        for net, X, R, *_ in chunk:
             net._finish_step(X, R)
+            net.enforce_constraints()
 
 
 def _side_by_side(streams, jobs):
@@ -547,7 +597,7 @@ def _side_by_side(streams, jobs):
 
 
 def _graphed_step(jobs):
-    """jobs: list of (net, X, R, Y, Ymask) with static device tensors. Returns step(): one replay of a
+    """jobs: list of (net, X, R, Y, Ymask, F) with static device tensors. Returns step(): one replay of a
     HIP graph holding one fused training step of every net (several nets share each launch)."""
     for net, *_ in jobs:
         assert net.mode == "fused" and net.dtype == torch.float32 and net.loss is not None
@@ -592,7 +642,7 @@ def _graphed_step(jobs):
         if state["graph"] is None or state["decay"] != decay_flags():
             capture()
         state["graph"].replay()
-        for net, X, R, Y, Ymask in jobs:
+        for net, X, R, *_ in jobs:
             net._L_versions = None              # (a step issued natively after this one forms its look-ahead afresh)
             if net.input_dropout > 0:
                 net._rng_offset += (X.numel() + 3) // 4
@@ -624,7 +674,7 @@ class ModelGroup(object):
             self.streams = [torch.cuda.Stream() for _ in self.groups]
         return self.streams
 
-    def train_step(self, X, R, Y, Ymask=None, U=None):
+    def train_step(self, X, R, Y, Ymask=None, U=None, F=None):
         """One step of every architecture group on the shared batch: one native call whose every launch
         holds the grids of all the groups (dbk_train_steps), on the current stream. The groups' small
         kernels thereby run side by side without side streams or events; each group gets the bits of a
@@ -639,7 +689,7 @@ class ModelGroup(object):
                     ii = torch.as_tensor(idx, device=Y.device)
                     Yg = Y.index_select(1, ii).contiguous()
                     Mg = Ymask.index_select(1, ii).contiguous() if Ymask is not None else None
-                    net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi])
+                    net.train_step(X, R, Yg, Mg, U=None if U is None else U[gi], F=F)
                 return run
             _side_by_side(self._streams(), [one(gi, idx, net) for gi, (idx, net) in enumerate(self.groups)])
             return
@@ -652,15 +702,15 @@ class ModelGroup(object):
                 self._targets.append((Y.index_select(1, ii).contiguous(),
                                       Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
             self._batch_key, self._batch = key, (X, R, Y, Ymask)
-        _native_steps([(net, X, R, Yg, Mg) for (_, net), (Yg, Mg) in zip(self.groups, self._targets)])
+        _native_steps([(net, X, R, Yg, Mg, F) for (_, net), (Yg, Mg) in zip(self.groups, self._targets)])
 
-    def make_graphed_step(self, X, R, Y, Ymask=None):
+    def make_graphed_step(self, X, R, Y, Ymask=None, F=None):
         """One HIP graph holding the fused training step of every architecture group on a static batch."""
         jobs = []
         for idx, net in self.groups:
             ii = torch.as_tensor(idx, device=Y.device)
             jobs.append((net, X, R, Y.index_select(1, ii).contiguous(),
-                         Ymask.index_select(1, ii).contiguous() if Ymask is not None else None))
+                         Ymask.index_select(1, ii).contiguous() if Ymask is not None else None, F))
         return _graphed_step(jobs)
 
     def slice_model(self, j):
@@ -670,8 +720,8 @@ class ModelGroup(object):
                 return net.slice_model(idx.index(j))
         raise IndexError(j)
 
-    def predict(self, X, R):
+    def predict(self, X, R, F=None):
         out = torch.empty((R.shape[0], self.nmodel), dtype=torch.float32, device=X.device)
         for idx, net in self.groups:
-            out[:, torch.as_tensor(idx, device=X.device)] = net.predict(X, R)
+            out[:, torch.as_tensor(idx, device=X.device)] = net.predict(X, R, F)
         return out

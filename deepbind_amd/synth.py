@@ -11,8 +11,8 @@ are (rows_per_model * nmodel, ncol) with model-major rows
 
 The combiner of the reference's sequence model has 16 extra, always-zero
 "dinucleotide feature" input columns (reference: code/libs/kangaroo/kangaroo/data.py:59-69);
-they multiply zeros and never change the output, so the synthetic models here
-leave them out.
+they multiply zeros and never change the output, so the synthetic benchmark models here
+leave them out (SequenceNet(feature_columns=16) builds the reference-shaped layer).
 """
 import numpy as np
 

@@ -296,16 +296,27 @@ int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, cons
 /* dZ = (Z - Y) * scale. reference: deepity/std/loss.py:98-112 */
 int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n);
 
+/* The scan filters' constraint, applied to W (4m, nfilter) in place after every parameter update:
+ * kind 0 ("pfm"): the four letter weights of every (tap, filter) become log(exp(w) / sum of the four exp(w));
+ * kind 1 ("psam"): log(exp(w) / max of the four exp(w)); kind 2: w clipped to [lo, hi].
+ * reference: corr1ord.enforce_constraints, kangaroo/kangaroo/_ext/corr1ord.py:60-77, called by the trainer
+ * before the first and after every step (deepity/deepity/sgd.py:103-107,137). */
+int dbk_corr1ord_constraint(dbk_stream_t stream, int dtype, void* W, size_t m, size_t nfilter, int kind, double lo, double hi);
+
 /* ------------------------------------------------------------------ fused dense head for scoring */
 
 /* scores[r, b] = head_b(pooled[r, b*k:(b+1)*k]) for nblock models with k inputs each:
  * hidden > 0: relu(x.W1_b + b1_b).W2_b + b2_b ; hidden == 0: x.W1_b + b1_b ; then logistic if
  * apply_logistic. W1 (k*nblock, hidden|1), b1 (1, hidden*nblock | nblock), W2 (hidden*nblock, 1), b2 (1, nblock).
  * in_scale multiplies the inputs (test-time dropout rescale, one value per model, may be NULL).
+ * nfeat > 0: every model's block of W1 has k + nfeat rows, the last nfeat of them weighting the columns of
+ * feats (n, nfeat), a feature matrix shared by all models and not scaled by in_scale (the reference's
+ * combiner input X1, kangaroo/kangaroo/model.py:101-112); feats == NULL stands for all zeros, which is what
+ * the reference's data source supplies (kangaroo/kangaroo/data.py:59-69).
  * Replaces blockwise_dot_combined -> bias -> relu -> blockwise_dot -> bias (-> logistic)
  * (reference: deepity/std/full.py:78-83,154-160, softmax.py:58-61). float32 only. */
 int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
-                   const float* pooled, const float* in_scale,
+                   const float* pooled, int nfeat, const float* feats, const float* in_scale,
                    const float* W1, const float* b1, const float* W2, const float* b2,
                    int apply_logistic, float* scores);
 
@@ -319,10 +330,12 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
  * Writes Z (n, nblock), dpooled (n, k*nblock), dW1, db1, dW2, db2 (overwritten, not accumulated) and,
  * if loss is not NULL, the per-model mean loss (nblock). Masks drawn here equal those of
  * dbk_dropout_fp_tr for the same (seed, offset). float32. Deterministic.
+ * nfeat, feats: shared feature columns as in dbk_head_fprop (no dropout on them, no gradient back to them;
+ * W1 and dW1 then have k + nfeat rows per model).
  * Replaces the reference's layer-by-layer head in a training step (deepity/std/elemwise.py:71-180,
  * full.py:78-119, softmax.py:58-77, loss.py:98-119). */
 int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden, int loss_kind, int reverse_complement,
-                   const float* pooled, const float* rate, const float* U, uint64_t seed, uint64_t offset,
+                   const float* pooled, int nfeat, const float* feats, const float* rate, const float* U, uint64_t seed, uint64_t offset,
                    uint64_t* counter, uint64_t counter_advance,
                    const float* W1, const float* b1, const float* W2, const float* b2,
                    const float* Y, const uint8_t* Ymask,
@@ -362,6 +375,9 @@ typedef struct dbk_train_step_args {
     uint64_t* act;                          /* activity masks (see dbk_scanpool_fprop), N * ceil(nmodel*nfilter/64) words; may be NULL */
     float* L;                               /* look-ahead vector (nparam), may be NULL: see dbk_gradstep_lookahead */
     int L_ready;                            /* L already holds P + mrate*mP (left there by the previous step) */
+    size_t nfeat; const float* feats;       /* shared feature columns (nregion, nfeat) entering the first dense layer after each model's
+                                               pooled features: W1 is ((k+nfeat)*nmodel, hidden|1); feats NULL = all zeros
+                                               (reference: kangaroo/kangaroo/model.py:101-112, data.py:59-69) */
 } dbk_train_step_args;
 
 /* One optimiser step, all launches issued from native code on `stream`:

@@ -25,6 +25,12 @@ checks live in tests/test_oracle_pins.py):
                         with scalar rates; two Nesterov steps written out from the docstring recurrence with
                         central-finite-difference gradients of loss + L1 cost; a hand-written worked case of
                         the decay block lengths rows/ninst and size/ninst; both gates at start-1 and start
+  model_forward/_backward/train_step with features= (the combiner's second, broadcast input) - equal to the same
+                        functions without it on a model whose pooled features are widened by the feature columns
+                        (block-concatenation identity) and finite differences of the loss w.r.t. the extra W1 rows
+  enforce_constraints - pfm: each tap's four exp(w) sum to one and differences of w across letters are kept
+                        (softmax shift invariance); psam: the largest of the four becomes 0, differences kept;
+                        clip: np.clip; all three idempotent
   dropout masks       - the reference draws them from cuRAND (not reproducible without the
                         CUDA SDK): masks are INPUTS here (uniforms U supplied by the caller);
                         the random stream itself is PARITY UNPINNED
@@ -479,9 +485,13 @@ def madd_bcast(A, b, k, dst):
 # whole-model forward / backward for a homogeneous batch of models on the model axis
 # layer order: kangaroo/kangaroo/model.py:45-132 ; deepity/_io_/load.py:51-72 ; cfg/*/M{1,2}.cfg
 # ----------------------------------------------------------------------------------------------
-def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None, train=False, matchrows=False, input_keep=1.0):
+def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None, train=False, matchrows=False, input_keep=1.0,
+                  features=None):
     """scan (-> * input_keep: the test-time side of input dropout, kangaroo/_ext/corr1ord.py:104-109) -> bias ->
-    relu -> pool -> dropout -> dense(+bias[,relu,dense,bias]) -> (logistic)."""
+    relu -> pool -> dropout -> dense(+bias[,relu,dense,bias]) -> (logistic).
+    features: the (rows, nfeat) matrix that the reference's first dense layer (its "combiner") takes as a second,
+    broadcast input after the pooled features (kangaroo/kangaroo/model.py:101-112, deepity/std/full.py:154-160);
+    W1 then has k + nfeat rows per model. None = a model built without that input."""
     m = params["Wc"].shape[0] // 4
     N = np.asarray(X).size
     st = {}
@@ -499,7 +509,12 @@ def model_forward(params, X, R, nmodel, pool, hidden, out="linear", dropout=None
         else:
             H = dropout_fp_test(H, rate)
     st["H0"] = H
-    A1 = bias_fprop(blockwise_dot(H, params["W1"], nmodel), params["b1"])
+    st["F"] = features
+    if features is None:
+        A1 = blockwise_dot(H, params["W1"], nmodel)
+    else:
+        A1 = blockwise_dot_combined([H, features], params["W1"], nmodel, [False, True])
+    A1 = bias_fprop(A1, params["b1"])
     if hidden:
         st["H1"] = relu_fprop(A1)
         A2 = bias_fprop(blockwise_dot(st["H1"], params["W2"], nmodel), params["b2"])
@@ -521,8 +536,13 @@ def model_backward(params, X, R, st, dA, nmodel, pool, hidden, dropout=None, tra
     else:
         dA1 = dA
     g["b1"] = bias_bprop(dA1)[1]
-    g["W1"] = blockwise_dot_tn(st["H0"], dA1, nmodel, params["W1"])
-    dH0 = blockwise_dot_nt(dA1, params["W1"], nmodel)
+    if st.get("F") is None:
+        g["W1"] = blockwise_dot_tn(st["H0"], dA1, nmodel, params["W1"])
+        dH0 = blockwise_dot_nt(dA1, params["W1"], nmodel)
+    else:                                                          # deepity/std/full.py:162-178
+        Xs = [st["H0"], st["F"]]
+        g["W1"] = blockwise_dot_tn_combined(Xs, dA1, params["W1"], nmodel, [False, True])
+        dH0 = blockwise_dot_nt_combined(Xs, dA1, params["W1"], nmodel, [False, True])[0]
     if dropout is not None:
         dH0 = dropout_bp_tr(dH0, st["M"]) if train else dropout_bp_te(dH0, dropout[0])
     dA0 = np.zeros_like(st["A0"])
@@ -556,15 +576,18 @@ PARAM_AXIS = {"Wc": 1, "bc": 1, "W1": 0, "b1": 1, "W2": 0, "b2": 1}
 
 
 def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum, Ymask=None, dropout=None,
-               decay_conv=0.0, decay_full=0.0, step=0, weight_decay_start=100, reverse_complement=False, start_training=0):
-    """Nesterov step in place on params / mom (dicts of arrays). dropout = (rates, U) or None."""
+               decay_conv=0.0, decay_full=0.0, step=0, weight_decay_start=100, reverse_complement=False, start_training=0,
+               features=None, constraint=None):
+    """Nesterov step in place on params / mom (dicts of arrays). dropout = (rates, U) or None.
+    features: see model_forward. constraint: enforced on the scan filters after the update (deepity/sgd.py:137)."""
     names = [n for n in ("Wc", "bc", "W1", "b1", "W2", "b2") if n in params]
     eta = {n: _per_element(rate, params[n].shape, nmodel, PARAM_AXIS[n]).astype(params[n].dtype) for n in names}
     mu = {n: _per_element(momentum, params[n].shape, nmodel, PARAM_AXIS[n]).astype(params[n].dtype) for n in names}
     for n in names:
         gradstep_nesterov1(params[n], mom[n], mu[n])
     out = "logistic" if loss == "nll" else "linear"
-    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=True, matchrows=reverse_complement)
+    st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=True, matchrows=reverse_complement,
+                       features=features)
     Zmask = calc_zmask(st["Zout"]) if reverse_complement else None      # deepity/std/loss.py:114-119
     dA = loss_bprop(st["Zout"], Y, Ymask=Ymask, Zmask=Zmask)
     g = model_backward(params, X, R, st, dA, nmodel, pool, hidden, dropout=dropout, train=True)
@@ -582,7 +605,30 @@ def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum,
         g["Wc"] = g["Wc"] * 0                                      # kangaroo/_ext/corr1ord.py:135-136
     for n in names:
         gradstep_nesterov2(params[n], g[n].astype(params[n].dtype), eta[n], mom[n], mu[n])
+    enforce_constraints(params["Wc"], constraint)
     return st, g
+
+
+def enforce_constraints(W, constraint):
+    """corr1ord.enforce_constraints (kangaroo/_ext/corr1ord.py:60-77), in place on W (4*fsize, filters)."""
+    if constraint is None:
+        return W
+    if constraint in ("pfm", "psam"):
+        F = np.exp(W)
+        for i in range(W.shape[0] // 4):
+            Fi = F[i * 4:(i + 1) * 4, :]
+            if constraint == "pfm":
+                Fi[:] = Fi / np.sum(Fi, axis=0)
+            else:
+                Fi[:] = Fi / np.max(Fi, axis=0)
+        W[:] = np.log(F)
+    elif type(constraint) == tuple:
+        lo, hi = constraint
+        W[:] = np.minimum(W, hi)
+        W[:] = np.maximum(W, lo)
+    else:
+        raise NotImplementedError("constraint \"%s\" not implemented" % str(constraint))
+    return W
 
 
 def weight_cost(params, nmodel, decay_conv, decay_full):
