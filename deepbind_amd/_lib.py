@@ -76,6 +76,7 @@ _SIGNATURES = {
     "dbk_loss_terms": [_P, _I, _I, _P, _P, _P, _Z],
     "dbk_sub_scale": [_P, _I, _P, _P, _D, _P, _Z],
     "dbk_head_train": [_P, _Z, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _U64, _U64, _P, _U64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
+    "dbk_softmax": [_P, _I, _P, _P, _Z, _Z],
     "dbk_counter_add": [_P, _P, _U64],
     "dbk_l1_decay": [_P, _I, _P, _P, _P, _Z],
     "dbk_head_fprop": [_P, _Z, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _P],

@@ -295,10 +295,27 @@ template <typename T> __global__ void k_loss_terms(int kind, const T* Z, const T
             T a = z > (T)1e-15 ? z : (T)1e-15;
             T b = ((T)1 - z) > (T)1e-15 ? ((T)1 - z) : (T)1e-15;
             L[i] = log(a) * y + log(b) * ((T)1 - y);
+        } else if (kind == 2) {                                    // several columns per output: multiclass term
+            T a = z > (T)1e-15 ? z : (T)1e-15;
+            L[i] = log(a) * y;
         } else {
             T d = z - y;
             L[i] = d * d;
         }
+    }
+}
+// Softmax over groups of g consecutive elements (a row of a (rows x ncol) matrix holds ncol/g groups):
+// z = exp(x - max) / sum(exp(x - max)), maximum and sum taken left to right. One thread per group.
+template <typename T> __global__ void k_softmax_groups(const T* X, T* Z, size_t ngroups, size_t g)
+{
+    GRID_STRIDE(i, ngroups) {
+        const T* x = X + i * g;
+        T* z = Z + i * g;
+        T mx = x[0];
+        for (size_t c = 1; c < g; ++c) mx = x[c] > mx ? x[c] : mx;
+        T s = (T)0;
+        for (size_t c = 0; c < g; ++c) { const T e = exp(x[c] - mx); z[c] = e; s += e; }
+        for (size_t c = 0; c < g; ++c) z[c] = z[c] / s;
     }
 }
 __global__ void k_uniform_fill(float* U, size_t n, uint64_t seed, uint64_t offset)
@@ -567,8 +584,14 @@ int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t 
 }
 int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, const void* Y, void* L, size_t n)
 {
-    DBK_CHECK(kind == 0 || kind == 1, "ValueError: loss kind must be 0 (nll) or 1 (mse), got %d", kind);
+    DBK_CHECK(kind >= 0 && kind <= 2, "ValueError: loss kind must be 0 (nll), 1 (mse) or 2 (multiclass nll), got %d", kind);
     EW2(k_loss_terms, n, A(kind, CF32(Z), CF32(Y), F32(L), n), A(kind, CF64(Z), CF64(Y), F64(L), n));
+}
+int dbk_softmax(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n, size_t group)
+{
+    DBK_CHECK(group >= 1 && n % group == 0, "ValueError: %zu elements do not split into groups of %zu", n, group);
+    const size_t ngroups = n / group;
+    EW2(k_softmax_groups, ngroups, A(CF32(X), F32(Z), ngroups, group), A(CF64(X), F64(Z), ngroups, group));
 }
 int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n)
 {

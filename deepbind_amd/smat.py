@@ -99,10 +99,20 @@ def logistic(X):
     return Z
 
 
+def softmax(X, nchunk=1):
+    """Row-wise softmax of a 2-D matrix; with nchunk > 1 every row is split into nchunk equal chunks that are
+    normalised separately (reference: deepity/std/softmax.py:58-71 with nchunk = ngroup * ninst)."""
+    require(X.dim() == 2 and X.shape[1] % nchunk == 0, "ValueError: the number of columns must be divisible by nchunk")
+    Z = torch.empty_like(X)
+    call("dbk_softmax", stream(), dtype_code(X), ptr(X), ptr(Z), X.numel(), X.shape[1] // nchunk)
+    return Z
+
+
 def loss_terms(Z, Y, kind):
-    """Elementwise loss terms before masking / averaging; kind is "nll" or "mse"."""
+    """Elementwise loss terms before masking / averaging; kind is "nll", "mse" or "nll_multiclass"
+    (several columns per output: log(max(1e-15, Z)) * Y, reference: deepity/std/loss.py:147-151)."""
     L = torch.empty_like(Z)
-    call("dbk_loss_terms", stream(), dtype_code(Z), {"nll": 0, "mse": 1}[kind], ptr(Z), ptr(Y), ptr(L), Z.numel())
+    call("dbk_loss_terms", stream(), dtype_code(Z), {"nll": 0, "mse": 1, "nll_multiclass": 2}[kind], ptr(Z), ptr(Y), ptr(L), Z.numel())
     return L
 
 

@@ -290,8 +290,13 @@ int dbk_mul_sign(dbk_stream_t stream, int dtype, const void* dZ, const void* Z, 
 int dbk_sign(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n);
 /* Z = 1/(1+exp(-X)). reference: smat_cuda/elemwise2.cu:46,68 */
 int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n);
+/* Z = softmax of every group of `group` consecutive elements of X (n elements, row-major, group divides the
+ * row length): exp(x - max) / sum. The output node of a model with several columns per output.
+ * reference: deepity/std/softmax.py:58-71 (rows split into ngroup * ninst chunks), smat softmax checked by
+ * smat/py/smat/tests/unittest.py:601-603 */
+int dbk_softmax(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n, size_t group);
 /* Elementwise loss terms L (n rows, m cols): kind 0 = log(max(1e-15,Z))*Y + log(max(1e-15,1-Z))*(1-Y),
- * kind 1 = (Z-Y)^2. reference: deepity/std/loss.py:131-145 */
+ * kind 1 = (Z-Y)^2, kind 2 = log(max(1e-15,Z))*Y (multiclass). reference: deepity/std/loss.py:131-151 */
 int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, const void* Y, void* L, size_t n);
 /* dZ = (Z - Y) * scale. reference: deepity/std/loss.py:98-112 */
 int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n);

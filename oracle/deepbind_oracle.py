@@ -17,6 +17,8 @@ checks live in tests/test_oracle_pins.py):
   poolrgn / _bprop    - np.max / np.argmax / np.mean per slice; scatter / uniform-spread adjoints
   bias/relu/logistic/nll/mse/maskout/calc_zmask - NumPy closed forms the reference's own
                         unit tests compare against (smat/tests/unittest.py:425-471,531-623)
+  softmax             - scipy.special.softmax per chunk (the reference's own test compares with a NumPy softmax,
+                        smat/py/smat/tests/unittest.py:601-603); rows sum to one per chunk
   blockwise_dot*      - np.dot per block; no reference test exists at that boundary
                         (closed form only): PARITY UNPINNED beyond the per-block np.dot identity
   weight_cost         - scalar loops over each model's own weights
@@ -409,6 +411,19 @@ def blockwise_dot_tn_combined(Xs, dZ, W, nblock, Xbroadcast, dWmask=None):
 # ----------------------------------------------------------------------------------------------
 def logistic(A):
     return (1 / (1 + np.exp(-A.astype(np.float64)))).astype(A.dtype)
+
+
+def softmax(X, nchunk=1):
+    """deepity/std/softmax.py:58-71: rows split into nchunk = ngroup * ninst chunks, each normalised on its own."""
+    A = X.reshape((-1, X.shape[1] // nchunk))
+    Z = np.exp(A - A.max(axis=1, keepdims=True))
+    Z = Z / Z.sum(axis=1, keepdims=True)
+    return Z.reshape(X.shape)
+
+
+def nll_multiclass_terms(Z, Y):
+    """deepity/std/loss.py:147-151."""
+    return np.log(np.maximum(Z.dtype.type(1e-15), Z)) * Y
 
 
 def maskout(M, A):

@@ -845,3 +845,24 @@ def test_config5_full_size_against_subsampled_checkers(ks):
     perm = rng.permutation(100000)
     Pp, _ = ks.scanpool_fprop(W, b, X, dev(np.ascontiguousarray(cfg["R"][perm])), "max")
     assert torch.equal(Pp, P[torch.as_tensor(perm, device="cuda")])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_softmax_chunks_and_multiclass_loss_terms(dtype):
+    """Output node of a model with several columns per output (deepity/std/softmax.py:58-71, loss.py:147-151)."""
+    from deepbind_amd import smat as sm
+    rng = np.random.default_rng(13)
+    X = (rng.standard_normal((300, 24)) * 4).astype(dtype)
+    tol = 1e-6 if dtype == np.float32 else 1e-14
+    for nchunk in (1, 3, 24):
+        got = host(sm.softmax(dev(X), nchunk))
+        ref = orc.softmax(X.astype(np.float64), nchunk)
+        assert np.abs(got - ref).max() <= tol
+    with pytest.raises(Exception):
+        sm.softmax(dev(X), 5)
+    Z = orc.softmax(X.astype(np.float64), 3).astype(dtype)
+    Z[0, 0] = 0                                                     # log(max(1e-15, 0))
+    Y = (rng.random(Z.shape) < 0.3).astype(dtype)
+    got = host(sm.loss_terms(dev(Z), dev(Y), "nll_multiclass"))
+    ref = orc.nll_multiclass_terms(Z.astype(np.float64), Y.astype(np.float64))
+    assert np.abs(got - ref).max() <= (1e-5 if dtype == np.float32 else 1e-13) * np.abs(ref).max()

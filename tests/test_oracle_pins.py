@@ -391,3 +391,27 @@ def test_weight_cost_is_the_per_model_l1_norm_times_decay():
         full = sum(abs(v) for v in p["W1"][nf * b:nf * (b + 1)].ravel()) + sum(abs(v) for v in p["W2"][hid * b:hid * (b + 1)].ravel())
         want[b] = dc[b] * conv + df[b] * full
     np.testing.assert_allclose(orc.weight_cost(p, nm, dc, df).ravel(), want, rtol=1e-12)
+
+
+def test_softmax_chunks_and_multiclass_terms():
+    """softmax per chunk == scipy's softmax on each chunk; the multiclass term's sum is the cross entropy, whose
+    gradient w.r.t. the pre-activations is Z - Y (what the loss node back-propagates, deepity/std/loss.py:98-112)."""
+    from scipy.special import softmax as sp_softmax
+    rng = np.random.default_rng(12)
+    X = rng.standard_normal((7, 12)) * 3
+    for nchunk in (1, 3, 4):
+        Z = orc.softmax(X, nchunk)
+        w = 12 // nchunk
+        for c in range(nchunk):
+            np.testing.assert_allclose(Z[:, c * w:(c + 1) * w], sp_softmax(X[:, c * w:(c + 1) * w], axis=1), rtol=1e-12)
+    Y = np.eye(4)[rng.integers(0, 4, 7)]
+    A = rng.standard_normal((7, 4))
+    cost = lambda a: -orc.nll_multiclass_terms(orc.softmax(a), Y).sum()
+    g = np.zeros_like(A)
+    for i in range(7):
+        for j in range(4):
+            up, dn = A.copy(), A.copy()
+            up[i, j] += 1e-6
+            dn[i, j] -= 1e-6
+            g[i, j] = (cost(up) - cost(dn)) / 2e-6
+    np.testing.assert_allclose(g, orc.softmax(A) - Y, atol=1e-8)
