@@ -82,6 +82,8 @@ _SIGNATURES = {
     "dbk_head_fprop": [_P, _Z, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _P],
     "dbk_train_step": [_P, _P],
     "dbk_train_steps": [_P, _Z, _P],
+    "dbk_train_step_single_workspace": [_P, _P],
+    "dbk_train_step_single": [_P, _P, _P, _Z],
     "dbk_train_step_args_size": [],
 }
 

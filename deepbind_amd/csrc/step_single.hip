@@ -1,0 +1,718 @@
+// One whole optimiser step of a SMALL model group in ONE launch.
+//
+// A training step on a minibatch of a hundred short sequences and one to four models is a few million
+// additions: issued as forward / head / backward / update launches it costs what four dependent launches
+// cost (30-40 us), and a 64-filter tile leaves most lanes of a wave idle when the group has 16 filters.
+// Here a workgroup takes a few regions (sequences) of the batch through the WHOLE step without leaving the
+// CU - scan + bias + ReLU + pooling, the dense head forward and backward, the filter gradients - writes its
+// share of every parameter's gradient to a partial-sum buffer, and after ONE grid-wide barrier all
+// workgroups together add up the shares in a fixed order and apply the Nesterov update. Nothing but the
+// partial sums and the predictions goes through HBM.
+//
+//   lanes        a wave's 64 lanes are (64 / Fp) position groups x Fp filters (Fp = 16, 32 or 64 = the
+//                group's filters rounded up), so a single 16-filter model keeps all lanes busy: every
+//                position group scans its own contiguous block of a region's positions, four positions at a
+//                time, the block's letters sliding through registers (one LDS word per four positions)
+//   forward      z[p][f] = sum over taps of table[tap][letter(p + tap)][f], taps ascending (the order of the
+//                reference kernel, kangaroo_smat/corr1ord.cuh:139-157), + bias, ReLU, running max / first
+//                argmax / sum per lane, folded over position groups and waves (poolrgn.cuh:44-160)
+//   head         dropout (the library generator, same element numbering as dbk_dropout_fp_tr) -> dense
+//                (+ shared feature columns) -> bias [-> ReLU -> dense -> bias] -> logistic | identity ->
+//                dA = (Z - Y) / n with Ymask and the reverse-complement pair rule -> gradients
+//                (deepity/std/full.py:78-178, loss.py:98-119, dropout.cu:41-109)
+//   backward     a thread owns (tap, filter) pairs and keeps their five letter accumulators (A, C, G, T,
+//                "mean of the four") in registers over the workgroup's regions. The average-pooling part
+//                needs no pass over the positions: the gradient is the same number c = dpooled / rows at every
+//                position whose rectifier is open, so dW[tap][letter][f] += c * popcount(open(f) & letters
+//                (letter) >> tap) with one bit per position (the rectifier bits are left by the forward pass,
+//                the letter bits by the staging). The max-pooling part adds the pooled gradient at the argmax
+//                row's letters (corr1ord_bprop.cuh:91-137, poolrgn_bprop.cuh:45-127)
+//   update       g = sum of the workgroups' shares, eight lanes per parameter (each adds a contiguous run of
+//                workgroups in ascending order, then a fixed butterfly), + L1 term, frozen filters zeroed,
+//                Nesterov step from the look-ahead P + mrate * mP (gradstep.cu:41-72, full.py:111-119,
+//                corr1ord.py:120-138)
+//
+// The barrier is a ticket counter in the caller's workspace; every workgroup of the grid must be resident, so
+// the grid never exceeds 128 workgroups of 256 threads (a CU holds at least one), and the wait is bounded:
+// a workgroup that gives up sets the workspace's status word and leaves without touching the parameters.
+// Results are deterministic (no float atomics; LDS atomics only OR bits), within the tolerances of the
+// multi-launch step but not its bits (other summation orders).
+#include "dbk_common.h"
+#include "rng.h"
+#include "scan_common.h"
+
+namespace {
+
+using dbk_scan::NL;
+using dbk_scan::letter_of;
+
+constexpr int NTMIN = 256, NTMAX = 512, NWMAX = NTMAX / 64;    // threads of a workgroup: 256, or 512 when it has a single region
+constexpr unsigned MAXROWS = 256;                 // rows of one region
+constexpr unsigned AW = MAXROWS / 32;             // words of rectifier bits per (region, filter)
+constexpr unsigned LW = AW + 2;                   // words of letter bits per (region, letter): rows + taps - 1 positions
+constexpr unsigned TXTB = 384;                    // staged letters per region (a dword-aligned copy, padded with "nothing")
+constexpr unsigned LPE = 8;                       // lanes that share one parameter in the update
+constexpr unsigned MAXG = 128;                    // workgroups of a launch
+constexpr size_t WORK_HEADER = 16384;              // bytes of the workspace before the shares: launch number, status, "go", flags
+constexpr unsigned GO_AT = 32, FLAGS_AT = 64;     // words of the workspace: the "go" word; the first workgroup flag
+constexpr unsigned FLAG_STRIDE = 16;              // words from one workgroup's flag to the next (a 64-byte line each)
+constexpr unsigned SPIN_LIMIT = 400000;           // polls of the barrier before a workgroup gives up (~0.2 s)
+
+struct single_args {
+    unsigned nmodel, nfilter, F, Fp, lgFp, m, hidden, h1, k, kt, kf, ptype, loss_kind, revcomp;
+    unsigned RC, G;                               // regions per workgroup, workgroups
+    size_t nparam, pstride;                       // parameters; floats of one workgroup's share (nparam + nmodel, padded)
+    float *P, *dP, *mP;
+    const float *drate, *mrate, *decay;
+    size_t off_Wc, off_bc, off_W1, off_b1, off_W2, off_b2;
+    const uint8_t* X; size_t N;
+    const uint32_t* R; unsigned nregion;
+    const float* Y; const uint8_t* Ymask; const float* feats;
+    const float* rate; unsigned long long seed; unsigned long long* counter; unsigned long long draws;
+    int freeze_scan;
+    float *Z, *loss;
+    unsigned* sync;                               // [0] number of the last launch, [1] status (non-zero: see grid_barrier), [64..] flags
+    float* partial;                               // [G][pstride]
+};
+
+// LDS carve-up (all offsets in 4-byte words), computed identically on the host for the launch size.
+struct lds_map {
+    unsigned wt, look, Y, Ym, misc, text, lmask, amask, PL, arg, gmax, cavg, rows, red, H0, H1, D1, dA, ls, zs, kept, total;
+};
+__host__ __device__ inline lds_map make_map(unsigned MT, unsigned Fp, unsigned nm, unsigned kt, unsigned k, unsigned h1, unsigned nparam,
+                                            unsigned RC, bool dense)
+{
+    lds_map o;
+    unsigned at = 0;
+    auto take = [&](unsigned n) { const unsigned r = at; at += (n + 3u) & ~3u; return r; };
+    o.wt = take(MT * NL * Fp);
+    o.look = take(nparam);                        // the whole look-ahead vector: the dense layers are read from it in place
+    o.Y = take(RC * nm);
+    o.Ym = take(RC * nm);
+    o.misc = take(8 + nm);                        // generator position (2 words), barrier target, dropout rates
+    o.text = take(RC * TXTB / 4);
+    o.lmask = take(RC * 5 * LW);
+    o.amask = take(dense ? RC * Fp * AW : 0);
+    o.PL = take(RC * nm * k);
+    o.arg = take(RC * Fp);
+    o.gmax = take(RC * Fp);
+    o.cavg = take(RC * Fp);
+    o.rows = take(RC * 2);
+    o.red = take(NWMAX * 3 * Fp);
+    o.H0 = take(RC * nm * kt);
+    o.H1 = take(RC * nm * h1);
+    o.D1 = take(RC * nm * h1);
+    o.dA = take(RC * nm);
+    o.ls = take(RC * nm);
+    o.zs = take(RC * nm);
+    o.kept = take((RC * nm * k + 3) / 4);
+    o.total = at;
+    return o;
+}
+
+// Scans this lane's block of positions [start, start + Bq) of a region whose letters are staged at tw (dword view,
+// dword 0 = the region's first row), four positions per round. rows: positions of the region; row0: the region's
+// first row in X; nscan: rows of X the scan defines (later rows read as bias only).
+template <int MT>
+__device__ __forceinline__ void scan_block(const float* __restrict__ wt, const unsigned* __restrict__ tw, unsigned start, unsigned Bq,
+                                           unsigned rows, size_t row0, size_t nscan, unsigned f, unsigned lgFp, float bf, bool want_bits,
+                                           unsigned* __restrict__ abits, float& mx, unsigned& xi, float& sum)
+{
+    constexpr int WN = (MT + 6) / 4;                              // dwords covering the letters of four positions
+    const unsigned Fp4 = 4u << lgFp;                              // bytes of one table row
+    const char* lane_row = reinterpret_cast<const char*>(wt) + 4u * f;
+    unsigned w[WN];
+    const unsigned* src = tw + (start >> 2);
+#pragma unroll
+    for (int i = 0; i < WN; ++i) w[i] = src[i];
+    for (unsigned j = 0; j < Bq; j += 4) {
+        float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+#pragma unroll
+            for (int ph = 0; ph < 4; ++ph) {
+                const int q = ph + t;
+                const unsigned letter = (w[q >> 2] >> ((q & 3) * 8)) & 0xffu;
+                z[ph] += *reinterpret_cast<const float*>(lane_row + letter * Fp4 + (unsigned)t * NL * Fp4);
+            }
+        }
+#pragma unroll
+        for (int ph = 0; ph < 4; ++ph) {
+            const unsigned p = start + j + ph;
+            if (p < rows) {
+                float v = (row0 + p < nscan ? z[ph] : 0.0f) + bf;
+                const bool open = v > 0.0f;
+                v = open ? v : 0.0f;
+                if (v > mx) { mx = v; xi = p; }
+                sum += v;
+                if (want_bits && open) atomicOr(&abits[p >> 5], 1u << (p & 31));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i + 1 < WN; ++i) w[i] = w[i + 1];
+        w[WN - 1] = src[(j >> 2) + WN];
+    }
+}
+
+// All workgroups of the grid meet here once. Accesses of many workgroups to ONE address at device scope are served
+// one after the other (measured: ~50 ns per read-modify-write, 6.5 us for a counter that 128 workgroups increment;
+// ~3 us when every workgroup reads every other's flag), so no word is shared more than it must be: each workgroup
+// raises a flag in a 64-byte line of its own - the number of this launch, one more than the number the workspace
+// held when the kernel started; workgroup 0 alone reads all the flags (two per lane of its first wave) and, when
+// they all show the number, writes it to the "go" word; every other workgroup polls that one word with one lane.
+// Returns 0 when the step may go on, else the status to leave with (1: this workgroup gave up waiting; otherwise
+// what another workgroup flagged before it arrived).
+__device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, unsigned launch, float* dbg = nullptr)
+{
+    __shared__ unsigned verdict;
+    unsigned* flags = sync + FLAGS_AT;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const unsigned lane = threadIdx.x;
+        if (lane == 0) {
+            __threadfence();                                       // this workgroup's shares are visible device-wide
+            if (dbg) dbg[0] = (float)(wall_clock64() & 0xffffff);
+            __hip_atomic_store(&flags[blockIdx.x * FLAG_STRIDE], launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        unsigned tries = 0;
+        bool done = false;
+        if (blockIdx.x == 0) {
+            for (;;) {
+                const unsigned v0 = lane < G ? __hip_atomic_load(&flags[lane * FLAG_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : launch;
+                const unsigned v1 = lane + 64 < G ? __hip_atomic_load(&flags[(lane + 64) * FLAG_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : launch;
+                done = __all(v0 == launch && v1 == launch);
+                if (dbg && tries == 0 && lane == 0) dbg[1] = (float)(wall_clock64() & 0xffffff);
+                if (done || ++tries >= SPIN_LIMIT) break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (lane == 0 && done) __hip_atomic_store(&sync[GO_AT], launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (lane == 0) {
+            for (;;) {
+                done = __hip_atomic_load(&sync[GO_AT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == launch;
+                if (dbg && tries == 0) dbg[1] = (float)(wall_clock64() & 0xffffff);
+                if (done || ++tries >= SPIN_LIMIT) break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        if (lane == 0) {
+            unsigned status = __hip_atomic_load(&sync[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (!done) { atomicExch(&sync[1], 1u); status = 1u; }
+            if (dbg) { dbg[2] = (float)(wall_clock64() & 0xffffff); dbg[3] = (float)tries; }
+            __threadfence();
+            verdict = status;
+        }
+    }
+    __syncthreads();
+    return verdict;
+}
+
+#ifdef DBK_STEP_PROF
+#define STAMP(i) do { if (threadIdx.x == 0) { const long long now_ = wall_clock64(); if (blockIdx.x == 0) reinterpret_cast<long long*>(a.sync + 3072)[i] = now_; \
+    if ((i) == 0 || (i) == 5 || (i) == 6) a.partial[(size_t)blockIdx.x * a.pstride + a.nparam + a.nmodel + ((i) == 0 ? 0 : (i) - 4)] = (float)(now_ & 0xffffff); } } while (0)
+#else
+#define STAMP(i) do {} while (0)
+#endif
+
+template <int MT>
+__global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
+{
+    extern __shared__ __align__(16) unsigned smem[];
+    const bool dense = a.ptype != DBK_PT_MAX, sparse = a.ptype != DBK_PT_AVG;
+    const lds_map L = make_map(MT, a.Fp, a.nmodel, a.kt, a.k, a.h1, (unsigned)a.nparam, a.RC, dense);
+    float* wt = reinterpret_cast<float*>(smem + L.wt);
+    float* Lk = reinterpret_cast<float*>(smem + L.look);
+    const float* W1s = Lk + a.off_W1;
+    const float* b1s = Lk + a.off_b1;
+    const float* W2s = Lk + a.off_W2;
+    const float* b2s = Lk + a.off_b2;
+    float* Ys = reinterpret_cast<float*>(smem + L.Y);
+    unsigned* Yms = smem + L.Ym;
+    unsigned* misc = smem + L.misc;
+    float* rates = reinterpret_cast<float*>(smem + L.misc + 8);
+    uint8_t* text = reinterpret_cast<uint8_t*>(smem + L.text);
+    unsigned* lmask = smem + L.lmask;
+    unsigned* amask = smem + L.amask;
+    float* PL = reinterpret_cast<float*>(smem + L.PL);
+    unsigned* argp = smem + L.arg;
+    float* gmax = reinterpret_cast<float*>(smem + L.gmax);
+    float* cavg = reinterpret_cast<float*>(smem + L.cavg);
+    unsigned* rinfo = smem + L.rows;                               // [RC][2]: rows, first row (low 32 bits are enough: N < 2^32 checked)
+    float* red = reinterpret_cast<float*>(smem + L.red);
+    float* H0 = reinterpret_cast<float*>(smem + L.H0);
+    float* H1 = reinterpret_cast<float*>(smem + L.H1);
+    float* D1 = reinterpret_cast<float*>(smem + L.D1);
+    float* dAs = reinterpret_cast<float*>(smem + L.dA);
+    float* lss = reinterpret_cast<float*>(smem + L.ls);
+    float* zs = reinterpret_cast<float*>(smem + L.zs);
+    uint8_t* kept = reinterpret_cast<uint8_t*>(smem + L.kept);
+
+    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, NT = blockDim.x, NW = NT >> 6;
+    const unsigned F = a.F, Fp = a.Fp, nm = a.nmodel, k = a.k, kt = a.kt, h1 = a.h1, hidden = a.hidden, m = a.m, RC = a.RC;
+    const unsigned r0 = blockIdx.x * RC;                           // first region of this workgroup
+    const unsigned nreg = r0 < a.nregion ? (a.nregion - r0 < RC ? a.nregion - r0 : RC) : 0u;
+    const unsigned kpf = a.ptype == DBK_PT_ALL ? 2u : 1u;          // pooled features per filter
+
+    STAMP(0);
+    // ---------------- everything this workgroup reads from global memory before the barrier, requested in ONE round:
+    // the look-ahead vector P + mrate * mP (gradstep.cu:41-51), its regions' bounds, targets, masks, dropout rates and
+    // the generator position. (Dependent round trips, not arithmetic, are what a step of this size costs.)
+    {
+        constexpr unsigned UN = 4;
+        for (size_t e0 = tid; e0 < a.nparam; e0 += UN * NT) {
+            float vp[UN], vr[UN], vm[UN];
+#pragma unroll
+            for (unsigned u = 0; u < UN; ++u) {
+                const size_t e = e0 + u * NT;
+                const bool in = e < a.nparam;
+                vp[u] = in ? a.P[e] : 0.0f;
+                vr[u] = in ? a.mrate[e] : 0.0f;
+                vm[u] = in ? a.mP[e] : 0.0f;
+            }
+#pragma unroll
+            for (unsigned u = 0; u < UN; ++u)
+                if (e0 + u * NT < a.nparam) Lk[e0 + u * NT] = vp[u] + vr[u] * vm[u];
+        }
+    }
+    {
+        unsigned ra = 0, rb = 0;
+        float y = 0.0f, dr = 0.0f;
+        unsigned ym = 1u, c_lo = 0u, c_hi = 0u, tickets = 0u;
+        if (tid < RC && r0 + tid < a.nregion) { ra = a.R[2 * (r0 + tid)]; rb = a.R[2 * (r0 + tid) + 1]; }
+        if (tid < RC * nm && r0 + tid / nm < a.nregion) {
+            const size_t i = (size_t)(r0 + tid / nm) * nm + tid % nm;
+            y = a.Y[i];
+            if (a.Ymask) ym = a.Ymask[i];
+        }
+        if (tid < nm && a.rate) dr = a.rate[tid];
+        if (tid == 0) {
+            if (a.counter) { const unsigned long long c = a.counter[0]; c_lo = (unsigned)c; c_hi = (unsigned)(c >> 32); }
+            tickets = __hip_atomic_load(&a.sync[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (tid < RC) {
+            unsigned rows = rb > ra ? rb - ra : 0u;
+            if (rows > MAXROWS) {                                  // not a shape this kernel takes: flag it, touch nothing of the region
+                atomicExch(&a.sync[1], 2u);
+                rows = 0u;
+            }
+            rinfo[2 * tid] = rows;
+            rinfo[2 * tid + 1] = ra;
+        }
+        if (tid < RC * nm) { Ys[tid] = y; Yms[tid] = ym; }
+        if (tid < nm) rates[tid] = dr;
+        if (tid == 0) {
+            misc[0] = c_lo; misc[1] = c_hi;
+            misc[2] = tickets + 1u;                                // this launch's number (see grid_barrier)
+        }
+    }
+    for (unsigned e = tid; e < RC * 5 * LW; e += NT) lmask[e] = 0u;
+    if (dense)
+        for (unsigned e = tid; e < RC * Fp * AW; e += NT) amask[e] = 0u;
+    __syncthreads();
+    STAMP(1);
+    // ---------------- the regions' letters are requested; the letter table [tap][letter][filter] (zero rows past m) is
+    // built from the look-ahead meanwhile; then the letters land dword-aligned per region, with one bit per (letter, position)
+    constexpr unsigned TXN = (4 * TXTB + NTMIN - 1) / NTMIN;       // letters per thread when the workgroup has up to four regions
+    const bool few = RC * TXTB <= TXN * NT;
+    unsigned lt[TXN];
+    auto letter_at = [&](unsigned e) -> unsigned {
+        const unsigned rl = e / TXTB, q = e % TXTB;
+        const unsigned rows = rinfo[2 * rl];
+        const size_t g = (size_t)rinfo[2 * rl + 1] + q;
+        return (rows && q < rows + MT - 1 && g < a.N) ? (unsigned)a.X[g] : 254u;
+    };
+    auto put_letter = [&](unsigned e, unsigned code) {
+        const unsigned rl = e / TXTB, q = e % TXTB;
+        const unsigned l = letter_of(code);
+        text[e] = (uint8_t)l;
+        if (l < 5u) atomicOr(&lmask[(rl * 5 + l) * LW + (q >> 5)], 1u << (q & 31));
+    };
+    if (few) {
+#pragma unroll
+        for (unsigned i = 0; i < TXN; ++i) lt[i] = tid + i * NT < RC * TXTB ? letter_at(tid + i * NT) : 254u;
+    }
+    for (unsigned e = tid; e < MT * Fp; e += NT) {
+        const unsigned t = e / Fp, f = e % Fp;
+        float w0 = 0.0f, w1 = 0.0f, w2 = 0.0f, w3 = 0.0f;
+        if (t < m && f < F) {
+            const float* w = Lk + a.off_Wc + (size_t)(4 * t) * F + f;
+            w0 = w[0]; w1 = w[F]; w2 = w[2 * F]; w3 = w[3 * F];
+        }
+        float z = w0;
+        z += w1;
+        z += w2;
+        z += w3;
+        float* row = wt + (size_t)t * NL * Fp + f;
+        row[0 * Fp] = w0; row[1 * Fp] = w1; row[2 * Fp] = w2; row[3 * Fp] = w3;
+        row[4 * Fp] = z * 0.25f;
+        row[5 * Fp] = 0.0f;
+    }
+    // which pooled features the dropout keeps (element numbering of the stand-alone kernels): drawn now, while the letters travel
+    {
+        const size_t ncol = (size_t)k * nm;
+        const unsigned long long off = (unsigned long long)misc[1] << 32 | misc[0];
+        for (unsigned e = tid; e < RC * nm * k; e += NT) {
+            const unsigned rl = e / (nm * k), col = e % (nm * k), b = col / k;
+            const size_t rr = (size_t)r0 + rl;
+            bool kp = true;
+            if (rl < nreg && a.rate) kp = dbk_rng::uniform_at(a.seed, off, (a.revcomp ? (rr >> 1) : rr) * ncol + col) >= rates[b];
+            kept[e] = kp;
+        }
+    }
+    if (few) {
+#pragma unroll
+        for (unsigned i = 0; i < TXN; ++i)
+            if (tid + i * NT < RC * TXTB) put_letter(tid + i * NT, lt[i]);
+    } else {
+        for (unsigned e = tid; e < RC * TXTB; e += NT) put_letter(e, letter_at(e));
+    }
+    __syncthreads();
+
+    STAMP(2);
+    // ---------------- forward: scan + bias + ReLU + pooling, region by region, all four waves on one region
+    const unsigned PG = 64u >> a.lgFp, NG = NW * PG;               // position groups per wave / per workgroup
+    const unsigned f = lane & (Fp - 1), gidx = wave * PG + (lane >> a.lgFp);
+    const float bf = f < F ? Lk[a.off_bc + f] : 0.0f;
+    const size_t nscan = a.N + 1 >= (size_t)m + 1 ? a.N - m + 1 : 0;
+    for (unsigned rl = 0; rl < nreg; ++rl) {
+        const unsigned rows = rinfo[2 * rl];
+        const unsigned Bq = 4u * ((rows + 4u * NG - 1u) / (4u * NG));
+        const unsigned start = gidx * Bq;
+        float mx = -1.0f, sum = 0.0f;
+        unsigned xi = 0xffffffffu;
+        if (start < rows)
+            scan_block<MT>(wt, reinterpret_cast<const unsigned*>(text + rl * TXTB), start, Bq, rows, rinfo[2 * rl + 1], nscan, f, a.lgFp, bf,
+                           dense, amask + (rl * Fp + f) * AW, mx, xi, sum);
+        // fold the position groups of the wave (lanes f, f + Fp, ...): larger value wins, equal values keep the earlier row
+        for (unsigned d = Fp; d < 64u; d <<= 1) {
+            const float om = __shfl_xor(mx, (int)d, 64), os = __shfl_xor(sum, (int)d, 64);
+            const unsigned oi = (unsigned)__shfl_xor((int)xi, (int)d, 64);
+            if (om > mx || (om == mx && oi < xi)) { mx = om; xi = oi; }
+            sum = (lane & d) ? os + sum : sum + os;               // lower group first, on both sides of the exchange
+        }
+        if (lane < Fp) {
+            red[(wave * 3 + 0) * Fp + f] = mx;
+            red[(wave * 3 + 1) * Fp + f] = __uint_as_float(xi);
+            red[(wave * 3 + 2) * Fp + f] = sum;
+        }
+        __syncthreads();
+        if (tid < Fp) {
+            float bm = red[tid], bs = red[2 * Fp + tid];
+            unsigned bi = __float_as_uint(red[Fp + tid]);
+            for (unsigned w = 1; w < NW; ++w) {
+                const float vm = red[(w * 3 + 0) * Fp + tid];
+                const unsigned vi = __float_as_uint(red[(w * 3 + 1) * Fp + tid]);
+                if (vm > bm || (vm == bm && vi < bi)) { bm = vm; bi = vi; }
+                bs += red[(w * 3 + 2) * Fp + tid];
+            }
+            bm = bm > 0.0f ? bm : 0.0f;
+            if (bi == 0xffffffffu) bi = 0u;
+            argp[rl * Fp + tid] = bi;
+            if (tid < F) {
+                float* out = PL + (size_t)rl * nm * k + (size_t)tid * kpf;
+                const float mean = rows ? bs / (float)rows : 0.0f;
+                if (a.ptype == DBK_PT_MAX) out[0] = bm;
+                else if (a.ptype == DBK_PT_AVG) out[0] = mean;
+                else { out[0] = bm; out[1] = mean; }
+            }
+        }
+        __syncthreads();
+    }
+
+    STAMP(3);
+    // ---------------- dense head, forward and backward, for this workgroup's rows
+    const float inv_n = 1.0f / (float)a.nregion;
+    for (unsigned e = tid; e < RC * nm * k; e += NT) {             // inputs after dropout
+        const unsigned rl = e / (nm * k), col = e % (nm * k), b = col / k, kk = col % k;
+        H0[((size_t)rl * nm + b) * kt + kk] = (rl < nreg && kept[e]) ? PL[e] : 0.0f;
+    }
+    for (unsigned e = tid; e < RC * nm * a.kf; e += NT) {          // the shared feature columns follow each model's own inputs
+        const unsigned rl = e / (nm * a.kf), rest = e % (nm * a.kf), b = rest / a.kf, j = rest % a.kf;
+        H0[((size_t)rl * nm + b) * kt + k + j] = (a.feats && rl < nreg) ? a.feats[((size_t)r0 + rl) * a.kf + j] : 0.0f;
+    }
+    __syncthreads();
+    STAMP(8);
+    if (hidden) {
+        for (unsigned e = tid; e < RC * nm * hidden; e += NT) {
+            const unsigned rb = e / hidden, h = e % hidden, b = rb % nm;
+            const float* x = H0 + (size_t)rb * kt;
+            const float* wcol = W1s + (size_t)b * kt * hidden + h;
+            float s = 0.0f;
+#pragma unroll 8
+            for (unsigned kk = 0; kk < kt; ++kk) s += x[kk] * wcol[kk * hidden];
+            s += b1s[b * hidden + h];
+            H1[e] = s > 0.0f ? s : 0.0f;
+        }
+        __syncthreads();
+    }
+    STAMP(9);
+    // output pre-activation and prediction of (row, model): one wave per output, a lane per input, summed by a fixed butterfly
+    for (unsigned e = wave; e < RC * nm; e += NW) {
+        const unsigned b = e % nm;
+        float part = 0.0f;
+        if (hidden) {
+            for (unsigned h = lane; h < hidden; h += 64) part += H1[(size_t)e * hidden + h] * W2s[b * hidden + h];
+        } else {
+            for (unsigned kk = lane; kk < kt; kk += 64) part += H0[(size_t)e * kt + kk] * W1s[(size_t)b * kt + kk];
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
+        if (lane == 0) {
+            const float out = part + (hidden ? b2s[b] : b1s[b]);
+            zs[e] = a.loss_kind == 0 ? 1.0f / (1.0f + expf(-out)) : out;
+        }
+    }
+    __syncthreads();
+    STAMP(10);
+    // loss gradient of (row, model), formed by every thread that needs it; the hidden units' gradients with it
+    for (unsigned e = tid; e < RC * nm * h1; e += NT) {
+        const unsigned rb = e / h1, h = e % h1, rl = rb / nm, b = rb % nm;
+        const size_t rr = (size_t)r0 + rl;
+        float dA = 0.0f, lterm = 0.0f;
+        if (rl < nreg) {
+            const float z = zs[rb], y = Ys[rb];
+            bool use = Yms[rb] != 0u;
+            if (a.revcomp) {                                       // of a (fwd, rev) pair only the larger prediction trains; ties keep the first
+                const float zo = zs[(rl ^ 1u) * nm + b];
+                use = use && ((rr & 1) ? !(zo >= z) : (z >= zo));
+            }
+            if (use) {
+                dA = (z - y) * inv_n;
+                if (h == 0)
+                    lterm = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
+            }
+            if (h == 0) a.Z[rr * nm + b] = z;
+        }
+        if (h == 0) { dAs[rb] = dA; lss[rb] = lterm; }
+        if (hidden) D1[e] = H1[e] > 0.0f ? dA * W2s[b * hidden + h] : 0.0f;
+    }
+    __syncthreads();
+    STAMP(12);
+    for (unsigned e = tid; e < RC * nm * k; e += NT) {             // gradient at the pooled features -> what the scan's backward pass needs
+        const unsigned rl = e / (nm * k), col = e % (nm * k), b = col / k, kk = col % k, rb = rl * nm + b;
+        float g;
+        if (hidden) {
+            g = 0.0f;
+            const float* wrow = W1s + ((size_t)b * kt + kk) * hidden;
+#pragma unroll 8
+            for (unsigned h = 0; h < hidden; ++h) g += D1[(size_t)rb * hidden + h] * wrow[h];
+        } else {
+            g = dAs[rb] * W1s[(size_t)b * kt + kk];
+        }
+        if (!kept[e]) g = 0.0f;
+        const unsigned fl = b * a.nfilter + kk / kpf;             // filter of the group
+        const bool is_avg = a.ptype == DBK_PT_AVG || (a.ptype == DBK_PT_ALL && (kk & 1u));
+        if (is_avg) cavg[rl * Fp + fl] = (rl < nreg && rinfo[2 * rl]) ? g / (float)rinfo[2 * rl] : 0.0f;
+        else gmax[rl * Fp + fl] = (rl < nreg && PL[e] > 0.0f) ? g : 0.0f;
+    }
+    STAMP(13);
+    // this workgroup's share of the dense layers' gradients and of the loss, rows ascending
+    float* share = a.partial + (size_t)blockIdx.x * a.pstride;
+    for (unsigned e = tid; e < nm * kt * h1; e += NT) {
+        const unsigned b = e / (kt * h1), kk = (e / h1) % kt, h = e % h1;
+        float s = 0.0f;
+        for (unsigned rl = 0; rl < RC; ++rl) {
+            const unsigned rb = rl * nm + b;
+            s += H0[(size_t)rb * kt + kk] * (hidden ? D1[(size_t)rb * hidden + h] : dAs[rb]);
+        }
+        share[a.off_W1 + e] = s;
+    }
+    for (unsigned e = tid; e < nm * h1; e += NT) {
+        const unsigned b = e / h1, h = e % h1;
+        float gb1 = 0.0f, gW2 = 0.0f;
+        for (unsigned rl = 0; rl < RC; ++rl) {
+            const unsigned rb = rl * nm + b;
+            if (hidden) { gb1 += D1[(size_t)rb * hidden + h]; gW2 += H1[(size_t)rb * hidden + h] * dAs[rb]; }
+            else gb1 += dAs[rb];
+        }
+        share[a.off_b1 + e] = gb1;
+        if (hidden) share[a.off_W2 + e] = gW2;
+    }
+    for (unsigned b = tid; b < nm; b += NT) {
+        float gb2 = 0.0f, ls = 0.0f;
+        for (unsigned rl = 0; rl < RC; ++rl) { gb2 += dAs[rl * nm + b]; ls += lss[rl * nm + b]; }
+        if (hidden) share[a.off_b2 + b] = gb2;
+        share[a.nparam + b] = ls;
+    }
+    __syncthreads();
+
+    STAMP(4);
+    // ---------------- scan filters: a thread's (tap, filter) pairs, five letter accumulators each, regions ascending
+    constexpr unsigned MAXPAIR = (MT * 64 + NTMIN - 1) / NTMIN;
+#pragma unroll
+    for (unsigned i = 0; i < MAXPAIR; ++i) {
+        const unsigned e = tid + i * NT;
+        if (e >= MT * Fp) break;
+        const unsigned t = e >> a.lgFp, fl = e & (Fp - 1);
+        float acc[5] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f}, accb = 0.0f;
+        for (unsigned rl = 0; rl < nreg; ++rl) {
+            const unsigned rows = rinfo[2 * rl];
+            if (dense) {
+                const float c = cavg[rl * Fp + fl];
+                const unsigned* am = amask + (rl * Fp + fl) * AW;
+                const unsigned nw = (rows + 31u) >> 5;
+                unsigned cnt[5] = {0u, 0u, 0u, 0u, 0u}, open = 0u;
+                for (unsigned w = 0; w < nw; ++w) {
+                    const unsigned bits = am[w];
+                    open += __popc(bits);
+#pragma unroll
+                    for (int l = 0; l < 5; ++l) {
+                        const unsigned* lm = lmask + (rl * 5 + l) * LW + w;
+                        const unsigned shifted = (unsigned)(((unsigned long long)lm[1] << 32 | lm[0]) >> t);   // letter bits of positions p + t
+                        cnt[l] += __popc(bits & shifted);
+                    }
+                }
+#pragma unroll
+                for (int l = 0; l < 5; ++l) acc[l] += c * (float)cnt[l];
+                accb += c * (float)open;
+            }
+            if (sparse) {
+                const float g = gmax[rl * Fp + fl];
+                const unsigned l = text[rl * TXTB + argp[rl * Fp + fl] + t];
+#pragma unroll
+                for (int c = 0; c < 5; ++c) acc[c] += l == (unsigned)c ? g : 0.0f;
+                accb += g;
+            }
+        }
+        if (t < m && fl < F) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) share[a.off_Wc + (size_t)(4 * t + c) * F + fl] = acc[c] + 0.25f * acc[4];
+        }
+        if (t == 0 && fl < F) share[a.off_bc + fl] = accb;
+    }
+
+    STAMP(5);
+    // ---------------- every workgroup's share is written: meet, then add them up and step the parameters.
+    // What the update reads of the parameter vectors is requested before the wait (nothing changes it until then).
+    const size_t total = a.nparam + nm, estep = (size_t)a.G * NT / LPE, efirst = ((size_t)blockIdx.x * NT + tid) / LPE;
+    const unsigned sub = tid & (LPE - 1);
+    float q_p = 0.0f, q_rm = 0.0f, q_mp = 0.0f, q_dr = 0.0f, q_dec = 0.0f;
+    if (sub == 0 && efirst < a.nparam) {
+        q_p = a.P[efirst]; q_rm = a.mrate[efirst]; q_mp = a.mP[efirst]; q_dr = a.drate[efirst];
+        if (a.decay) q_dec = a.decay[efirst];
+    }
+#ifdef DBK_STEP_PROF
+    if (grid_barrier(a.sync, a.G, misc[2], a.partial + (size_t)blockIdx.x * a.pstride + a.nparam + a.nmodel + 3) != 0u) return;
+#else
+    if (grid_barrier(a.sync, a.G, misc[2]) != 0u) return;
+#endif
+    // (every workgroup read the launch number before it raised its flag, so it can move on now)
+    if (blockIdx.x == 0 && tid == 0) __hip_atomic_store(&a.sync[0], misc[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);              // flagged (by any workgroup, before the barrier) or gave up: no update
+    STAMP(6);
+    const unsigned per = (a.G + LPE - 1) / LPE;                    // workgroups each of the eight lanes adds, ascending
+    const unsigned g0 = sub * per, g1 = g0 + per < a.G ? g0 + per : a.G;
+    for (size_t e = efirst; e < total; e += estep) {
+        float s = 0.0f;
+        for (unsigned c0 = g0; c0 < g1; c0 += 8) {
+            float v[8];
+#pragma unroll
+            for (unsigned u = 0; u < 8; ++u) v[u] = c0 + u < g1 ? a.partial[(size_t)(c0 + u) * a.pstride + e] : 0.0f;
+#pragma unroll
+            for (unsigned u = 0; u < 8; ++u)
+                if (c0 + u < g1) s += v[u];
+        }
+        s += __shfl_xor(s, 1, 64);                                 // fixed butterfly: every lane of the eight ends with the same bits
+        s += __shfl_xor(s, 2, 64);
+        s += __shfl_xor(s, 4, 64);
+        if (sub) continue;
+        if (e >= a.nparam) {
+            if (a.loss) a.loss[e - a.nparam] = a.loss_kind == 0 ? -s / (float)a.nregion : 0.5f * s / (float)a.nregion;
+            continue;
+        }
+        if (e != efirst) {
+            q_p = a.P[e]; q_rm = a.mrate[e]; q_mp = a.mP[e]; q_dr = a.drate[e];
+            if (a.decay) q_dec = a.decay[e];
+        }
+        float g = s;
+        const float lk = q_p + q_rm * q_mp;
+        if (a.decay) g += (float)((lk > 0.0f) - (lk < 0.0f)) * q_dec;
+        if (a.freeze_scan && e - a.off_Wc < (size_t)4 * m * F) g = 0.0f;
+        a.dP[e] = g;
+        const float delta = g * q_dr;
+        a.mP[e] = q_mp * q_rm - delta;
+        a.P[e] = lk - delta;
+    }
+    STAMP(7);
+    if (a.counter && a.draws && blockIdx.x == 0 && tid == 0) a.counter[0] += a.draws;
+}
+
+unsigned ilog2(unsigned v) { unsigned l = 0; while ((1u << l) < v) ++l; return l; }
+
+// Fills the launch shape for a group; false when the single-launch step does not take it.
+bool plan(const dbk_train_step_args* a, single_args& s, unsigned& MT, size_t& lds_bytes)
+{
+    if (!a || a->nmodel < 1 || a->nmodel > 4 || a->nfilter < 1 || a->m < 1 || a->m > 32) return false;
+    const size_t F = a->nmodel * a->nfilter;
+    if (F > 64 || a->hidden > 64 || !a->nesterov || a->input_rate > 0.0f || a->nregion < 1 || a->N >= 0xffffff00ull) return false;
+    if (a->ptype != DBK_PT_MAX && a->ptype != DBK_PT_AVG && a->ptype != DBK_PT_ALL) return false;
+    if (a->reverse_complement && (a->nregion & 1)) return false;
+    s.nmodel = (unsigned)a->nmodel; s.nfilter = (unsigned)a->nfilter; s.F = (unsigned)F;
+    s.Fp = F <= 16 ? 16u : (F <= 32 ? 32u : 64u);
+    s.lgFp = ilog2(s.Fp);
+    s.m = (unsigned)a->m; s.hidden = (unsigned)a->hidden; s.h1 = s.hidden ? s.hidden : 1u;
+    s.k = (unsigned)a->nfilter * (a->ptype == DBK_PT_ALL ? 2u : 1u);
+    s.kf = (unsigned)a->nfeat; s.kt = s.k + s.kf;
+    if (s.kt > 160) return false;
+    s.ptype = (unsigned)a->ptype; s.loss_kind = (unsigned)a->loss_kind; s.revcomp = a->reverse_complement ? 1u : 0u;
+    MT = a->m <= 16 ? 16u : (a->m <= 24 ? 24u : 32u);
+    // regions per workgroup: as few as keep the grid within MAXG workgroups (one region: eight waves share it),
+    // an even number with reverse-complement pairs (a pair's two rows meet in one workgroup)
+    unsigned RC = (unsigned)((a->nregion + MAXG - 1) / MAXG);
+    if (a->reverse_complement) RC += RC & 1u;
+    if (RC > 16) return false;
+    s.RC = RC;
+    s.G = (unsigned)((a->nregion + RC - 1) / RC);
+    if (s.G > MAXG) return false;
+    s.nparam = a->nparam;
+    s.pstride = (a->nparam + a->nmodel + 63) & ~(size_t)63;
+    if (a->nparam > 24576) return false;
+    const lds_map L = make_map(MT, s.Fp, s.nmodel, s.kt, s.k, s.h1, (unsigned)a->nparam, s.RC, a->ptype != DBK_PT_MAX);
+    lds_bytes = (size_t)L.total * 4;
+    return lds_bytes <= dbk_scan::lds_limit();
+}
+
+}  // namespace
+
+extern "C" int dbk_train_step_single_workspace(const dbk_train_step_args* a, size_t* work_bytes)
+{
+    DBK_CHECK(a && work_bytes, "ValueError: null pointer argument");
+    single_args s;
+    unsigned MT;
+    size_t lds;
+    *work_bytes = plan(a, s, MT, lds) ? WORK_HEADER + (size_t)s.G * s.pstride * sizeof(float) : 0;
+    dbk::clear_error();
+    return 0;
+}
+
+extern "C" int dbk_train_step_single(dbk_stream_t stream, const dbk_train_step_args* a, void* work, size_t work_bytes)
+{
+    single_args s;
+    unsigned MT = 0;
+    size_t lds = 0;
+    DBK_CHECK(plan(a, s, MT, lds), "NotImplementedError: the single-launch step takes 1-4 models with at most 64 filters of at most 32 taps, "
+              "Nesterov momentum, no input dropout and at most %u x 16 regions of at most %u rows", MAXG, MAXROWS);
+    DBK_CHECK(a->P && a->dP && a->mP && a->drate && a->mrate, "ValueError: null parameter vector");
+    DBK_CHECK(a->X && a->regions && a->Y && a->Z, "ValueError: null batch or work buffer");
+    DBK_CHECK(!a->rate || a->counter, "ValueError: dropout needs the device generator position");
+    DBK_CHECK(work && work_bytes >= WORK_HEADER + (size_t)s.G * s.pstride * sizeof(float) && ((uintptr_t)work & 15) == 0,
+              "ValueError: the workspace must hold dbk_train_step_single_workspace() bytes, 16-byte aligned");
+    const size_t F = s.F, h1 = s.h1;
+    const size_t nWc = 4 * a->m * F, nW1 = (size_t)s.kt * a->nmodel * h1, nb1 = a->nmodel * h1;
+    const size_t nW2 = s.hidden ? s.hidden * a->nmodel : 0, nb2 = s.hidden ? a->nmodel : 0;
+    DBK_CHECK(nWc + F + nW1 + nb1 + nW2 + nb2 == a->nparam, "ValueError: the parameter blocks do not tile the flat vector (%zu of %zu elements)",
+              nWc + F + nW1 + nb1 + nW2 + nb2, a->nparam);
+    const size_t need[6] = { a->off_Wc + nWc, a->off_bc + F, a->off_W1 + nW1, a->off_b1 + nb1, a->off_W2 + nW2, a->off_b2 + nb2 };
+    for (size_t v : need) DBK_CHECK(v <= a->nparam, "ValueError: a parameter block reaches past the flat vector (%zu > %zu)", v, a->nparam);
+    s.P = a->P; s.dP = a->dP; s.mP = a->mP; s.drate = a->drate; s.mrate = a->mrate; s.decay = a->decay;
+    s.off_Wc = a->off_Wc; s.off_bc = a->off_bc; s.off_W1 = a->off_W1; s.off_b1 = a->off_b1; s.off_W2 = a->off_W2; s.off_b2 = a->off_b2;
+    s.X = a->X; s.N = a->N; s.R = a->regions; s.nregion = (unsigned)a->nregion;
+    s.Y = a->Y; s.Ymask = a->Ymask; s.feats = a->feats;
+    s.rate = a->rate; s.seed = a->seed; s.counter = (unsigned long long*)a->counter;
+    s.draws = a->rate ? (a->nregion * s.k * a->nmodel + 3) / 4 : 0;
+    s.freeze_scan = a->freeze_scan; s.Z = a->Z; s.loss = a->loss;
+    s.sync = (unsigned*)work;
+    s.partial = (float*)((char*)work + WORK_HEADER);
+    auto kern = MT == 16 ? k_step_single<16> : (MT == 24 ? k_step_single<24> : k_step_single<32>);
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(s.G), dim3(s.RC == 1 ? NTMAX : NTMIN), lds, dbk::as_stream(stream), s);
+    DBK_LAUNCH_OK();
+}

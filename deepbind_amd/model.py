@@ -37,7 +37,7 @@ class SequenceNet(object):
     def __init__(self, nmodel, nfilter, m, pool="max", hidden=32, loss="nll", dtype=torch.float32,
                  rate=0.01, momentum=0.9, decay_conv=0.0, decay_full=0.0, dropout=0.0,
                  weight_decay_start=100, nesterov=True, mode="fused", reverse_complement=False, input_dropout=0.0,
-                 start_training=0, feature_columns=0, constraint=None, device="cuda"):
+                 start_training=0, feature_columns=0, constraint=None, single_launch=True, device="cuda"):
         assert pool in ("max", "avg", "all") and loss in ("nll", "mse", None)
         self.ninst, self.nfilter, self.m = int(nmodel), int(nfilter), int(m)
         self.pool, self.hidden, self.loss = pool, int(hidden), loss
@@ -56,9 +56,14 @@ class SequenceNet(object):
         # constraint on the scan filters, enforced before the first step and after every update:
         # "pfm", "psam", a (lo, hi) tuple or None (reference: kangaroo/_ext/corr1ord.py:60-77, deepity/sgd.py:103-107,137)
         self.constraint = constraint
+        # small groups (1-4 models, at most 64 filters, regions of at most 256 rows) step in ONE launch
+        # (dbk_train_step_single) unless this is switched off; same numbers within tolerance, other summation orders
+        self.single_launch = bool(single_launch)
+        self._single_rows = {}               # longest region of the region tables seen, by (pointer, version, regions)
         self.step_count = 0
         self._step_args = None               # argument block and work buffers of the natively issued step
         self._step_bufs = {}
+        self._step_sig, self._step_buf, self._step_nesterov = None, None, None
         # Nesterov look-ahead kept beside the parameters by the natively issued step (each step's update kernel
         # leaves the next step's look-ahead there); valid while nothing else has touched P, mP or mrate
         self._L, self._L_versions = None, None
@@ -175,7 +180,36 @@ class SequenceNet(object):
         ks.corr1ord_enforce_constraints(self.p["Wc"], self.constraint)
         self._L_versions = None              # the look-ahead kept beside the parameters no longer matches them
 
+    def _single_work(self, buf, R):
+        """Workspace of the single-launch step for this batch shape, or None when the step does not take it."""
+        if "work" not in buf:
+            need = ctypes.c_size_t(0)
+            _lib.call("dbk_train_step_single_workspace", ctypes.addressof(self._step_args), ctypes.addressof(need))
+            buf["work"] = torch.zeros(need.value, dtype=torch.uint8, device=self.P.device) if need.value else None
+        if buf["work"] is None:
+            return None
+        key = (R.data_ptr(), R._version, R.shape[0])
+        rows = self._single_rows.get(key)
+        if rows is None:                     # one read-back per region table: the kernel keeps whole regions in LDS
+            if len(self._single_rows) >= 256:
+                self._single_rows.clear()
+            Rl = R.to(torch.int64)
+            rows = self._single_rows[key] = int((Rl[:, 1] - Rl[:, 0]).max().item()) if R.shape[0] else 0
+        return buf["work"] if rows <= 256 else None
+
+    def _check_single_status(self):
+        """Raises when a single-launch step flagged its workspace (the step then left the parameters untouched)."""
+        for buf in self._step_bufs.values():
+            work = buf.get("work")
+            if work is not None:
+                status = int(work[4:8].view(torch.int32).item())
+                if status:
+                    work[4:8].zero_()
+                    raise _lib.DeepbindError("RuntimeError: a single-launch training step was abandoned (%s)" %
+                                             ("a workgroup waited too long at the barrier" if status == 1 else "a region has more than 256 rows"))
+
     def get_params(self):
+        self._check_single_status()
         torch.cuda.synchronize()
         return {name: self.p[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
@@ -458,13 +492,24 @@ class SequenceNet(object):
     def _prepare_step(self, X, R, Y, Ymask=None, F=None):
         """Fills this net's dbk_train_step_args block for one step on the batch and returns the step's work
         buffers (made on the current stream, where the step is issued)."""
+        a = self._step_args
+        # the same batch tensors as in the previous step (a training loop over resident batches): only the switches move
+        sig = (X.data_ptr(), X.numel(), R.data_ptr(), R.shape[0], R._version, Y.data_ptr(), Y.numel(),
+               None if Ymask is None else Ymask.data_ptr(), None if F is None else F.data_ptr())
+        if a is not None and sig == self._step_sig and not self.nesterov_changed():
+            if self.nesterov:
+                versions = (self.P._version, self.mP._version, self.mrate._version)
+                a.L_ready = int(self._L_versions == versions)
+                self._L_versions = versions
+            a.decay = self.decay_vec.data_ptr() if self.weight_decay_start <= self.step_count else None
+            a.freeze_scan = int(self.step_count < self.start_training)
+            return self._step_buf
         ks._u8(X)
         ks._regions(R)
         ni, P = self.ninst, R.shape[0]
         _lib.require(R.shape[1] == 2, "ValueError: the fused path takes 2-column regions")
         _lib.require(Y.dtype == torch.float32 and tuple(Y.shape) == (P, ni), "ValueError: Y must be float32 (rows x models)")
         _lib.require(Ymask is None or (Ymask.dtype == torch.bool and tuple(Ymask.shape) == (P, ni)), "ValueError: Ymask must be bool (rows x models)")
-        a = self._step_args
         if a is None:
             a = self._step_args = _lib.TrainStepArgs()
             off = {name: int(o) for (name, _, _), o in zip(self.layout, self.offsets[:-1])}
@@ -511,11 +556,16 @@ class SequenceNet(object):
         a.nfeat, a.feats = self.nfeat, pv(F)
         a.input_rate = self.input_dropout
         for name, t in buf.items():
-            setattr(a, name, None if t is None else t.data_ptr())
+            if name != "work":
+                setattr(a, name, None if t is None else t.data_ptr())
         a.decay = self.decay_vec.data_ptr() if self.weight_decay_start <= self.step_count else None
         a.freeze_scan = int(self.step_count < self.start_training)
         a.loss = None
+        self._step_sig, self._step_buf, self._step_nesterov = sig, buf, (bool(self.nesterov), int(self.rng_seed))
         return buf
+
+    def nesterov_changed(self):
+        return self._step_nesterov != (bool(self.nesterov), int(self.rng_seed))
 
     def _finish_step(self, X, R):
         """Host-side mirrors of what a natively issued step moved on the device."""
@@ -530,7 +580,12 @@ class SequenceNet(object):
         scripting host otherwise pays several microseconds per launch, which is what bounds a step on a
         small minibatch). Same kernels in the same order as gradstep(..., _grad_fused), so the same bits."""
         buf = self._prepare_step(X, R, Y, Ymask, F)
-        _lib.call("dbk_train_step", _lib.stream(), ctypes.addressof(self._step_args))
+        work = self._single_work(buf, R) if self.single_launch else None
+        if work is not None:
+            _lib.call("dbk_train_step_single", _lib.stream(), ctypes.addressof(self._step_args), _lib.ptr(work), work.numel())
+            self._L_versions = None          # (this kernel forms the look-ahead itself and leaves none behind)
+        else:
+            _lib.call("dbk_train_step", _lib.stream(), ctypes.addressof(self._step_args))
         self._finish_step(X, R)
         self.enforce_constraints()
         return buf["Z"]
@@ -571,6 +626,10 @@ def _native_steps(jobs):
     """jobs: list of (net, X, R, Y, Ymask[, F]), nets that step on the same batch. One dbk_train_steps call per eight
     nets on the current stream: every phase of the step is one launch holding all the nets' grids, so nets too
     small to fill the GPU run side by side without extra streams. Each net gets the bits of its own step."""
+    if len(jobs) == 1:
+        net, X, R, Y, Ymask, *rest = jobs[0]
+        net._native_step(X, R, Y, Ymask, rest[0] if rest else None)
+        return
     for i in range(0, len(jobs), 8):
         chunk = jobs[i:i + 8]
         blocks = (ctypes.c_void_p * len(chunk))()

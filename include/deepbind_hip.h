@@ -404,6 +404,21 @@ int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* args);
  * reference: the per-architecture loop over one shared minibatch in the calibration search, which trains
  * all sampled models on the same batches (deepity/deepity/hpsearch.py:314-330, sgd.py:98-135). */
 int dbk_train_steps(dbk_stream_t stream, size_t ngroup, const dbk_train_step_args* const* args);
+/* The same step for a SMALL group in ONE launch: 1-4 models with at most 64 filters (of at most 32 taps) between
+ * them, Nesterov momentum, no input dropout, at most 2048 regions of at most 256 rows each. A workgroup takes a few
+ * regions through forward, dense head and backward without leaving the CU, and after one grid-wide barrier
+ * (bounded wait) all workgroups add up their shares of the gradient in a fixed order and apply the update.
+ * Reads pooled / argmax / dpooled / act / L of the block not at all (weights come from P + mrate * mP); writes Z,
+ * dP, mP, P, loss and advances the generator position. Deterministic; within the tolerances of dbk_train_step,
+ * not its bits (other summation orders).
+ * work: caller-owned device memory of dbk_train_step_single_workspace() bytes, 16-byte aligned, ZERO before its
+ * first use and from then on passed unchanged to every call with the same nregion (word 0 is the barrier's ticket
+ * counter; word 1 a status the kernel sets: 1 = a workgroup gave up waiting at the barrier, 2 = a region had more
+ * than 256 rows; with a non-zero status the parameters are left untouched). Calls that share a workspace must not
+ * overlap. *work_bytes = 0 from the query means the shape is not taken (use dbk_train_step).
+ * reference: the body of the trainer's loop, deepity/deepity/sgd.py:98-135, as dbk_train_step. */
+int dbk_train_step_single_workspace(const dbk_train_step_args* args, size_t* work_bytes);
+int dbk_train_step_single(dbk_stream_t stream, const dbk_train_step_args* args, void* work, size_t work_bytes);
 /* sizeof(dbk_train_step_args) as the library was built, for bindings that mirror the block field by field. */
 int dbk_train_step_args_size(void);
 

@@ -130,7 +130,7 @@ def test_group_of_architectures_with_feature_columns_shared_launches_and_graph()
 
     def make():
         grp = ModelGroup(pools, hiddens, nf, m, loss="nll", rate=0.05, momentum=0.9, dropout=0.25, decay_full=1e-2,
-                         weight_decay_start=1, feature_columns=NFEAT)
+                         weight_decay_start=1, feature_columns=NFEAT, single_launch=False)
         for gi, (_, net) in enumerate(grp.groups):
             net.init_params(init_conv=0.1, init_full=0.1, seed=gi)
             net.rng_seed = 7 + gi

@@ -1,0 +1,182 @@
+"""GPU parity of the single-launch training step (dbk_train_step_single: forward, dense head, backward and the
+Nesterov update of a small model group in one kernel) against the CPU oracle's whole step, run-to-run bit
+stability, agreement with the multi-launch step, graph replays, and the shapes it hands back to the multi-launch step."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import deepbind_oracle as orc
+from tests.gpu_util import assert_close_per_model, dev, host, record_error
+
+pytestmark = pytest.mark.gpu
+
+ACT, GRAD = 1e-5, 1e-4
+
+
+def _f64(d):
+    return {k: np.asarray(v, dtype=np.float64).copy() for k, v in d.items()}
+
+
+def _batch(rng, B, m, lo, hi, pn=0.03, reverse_complement=False):
+    from deepbind_amd import data
+    seqs = ["".join("ACGTN"[c] for c in rng.choice(5, size=int(rng.integers(lo, hi + 1)), p=[(1 - pn) / 4] * 4 + [pn])) for _ in range(B)]
+    return data.pack_sequences(seqs, m - 1, reverse_complement=reverse_complement)
+
+
+def _net(rng, nm, nf, m, pool, hidden, loss, scale=0.3, **kw):
+    from deepbind_amd.model import SequenceNet
+    net = SequenceNet(nm, nf, m, pool=pool, hidden=hidden, loss=loss, **kw)
+    params = {name: (rng.standard_normal(shape) * (scale if name.startswith("W") else 0.05)).astype(np.float32) for name, shape, _ in net.layout}
+    net.set_params(params)
+    return net, params
+
+
+def _used_single(net):
+    return any(buf.get("work") is not None for buf in net._step_bufs.values())
+
+
+CASES = [
+    # pool, hidden, loss, nm, nf, m, B, lengths, rc, nfeat
+    ("max", 32, "nll", 1, 16, 24, 128, (101, 101), False, 0),      # config 3's shape
+    ("all", 0, "mse", 1, 16, 16, 128, (38, 41), False, 0),         # config 2's shape
+    ("avg", 8, "nll", 2, 16, 11, 60, (12, 70), False, 0),
+    ("all", 32, "nll", 4, 16, 24, 50, (20, 40), False, 16),
+    ("max", 0, "mse", 3, 12, 9, 33, (5, 30), False, 0),            # 36 filters: padded to 64 lanes
+    ("all", 16, "nll", 2, 16, 20, 64, (30, 200), True, 0),         # reverse-complement pairs, regions up to 219 rows
+    ("max", 32, "nll", 1, 16, 32, 300, (20, 60), False, 16),       # four regions per workgroup
+]
+
+
+@pytest.mark.parametrize("pool,hidden,loss,nm,nf,m,B,lengths,rc,nfeat", CASES)
+def test_single_launch_step_matches_the_oracle(pool, hidden, loss, nm, nf, m, B, lengths, rc, nfeat):
+    from deepbind_amd import deepity_smat as ds
+    rng = np.random.default_rng(17)
+    X, R = _batch(rng, B, m, lengths[0], lengths[1], reverse_complement=rc)
+    rows = len(R)
+    rate, mu = rng.uniform(0.01, 0.1, nm), rng.uniform(0.5, 0.95, nm)
+    drop = np.where(np.arange(nm) % 2 == 0, 0.5, 0.0) if nm > 1 else np.array([0.5])
+    dfull, dconv = rng.uniform(0, 1e-2, nm), 1e-3
+    net, params = _net(rng, nm, nf, m, pool, hidden, loss, rate=rate, momentum=mu, dropout=drop, decay_conv=dconv, decay_full=dfull,
+                       weight_decay_start=1, reverse_complement=rc, feature_columns=nfeat, start_training=1)
+    Y = rng.random((rows, nm)).astype(np.float32) if loss == "mse" else (rng.random((rows, nm)) < 0.5).astype(np.float32)
+    Ymask = rng.random((rows, nm)) < 0.85
+    F = rng.standard_normal((rows, nfeat)).astype(np.float32) if nfeat else None
+    Xd, Rd, Yd, Md, Fd = dev(X), dev(R), dev(Y), dev(Ymask), (dev(F) if nfeat else None)
+    ref_p, ref_m = _f64(params), {n: np.zeros(v.shape) for n, v in params.items()}
+    name = "single launch (%s/%d, %d x %d filters x %d taps)" % (pool, hidden, nm, nf, m)
+    for step in range(3):
+        U = host(ds.uniform_like(torch.empty((rows // (2 if rc else 1), net.k * nm), device="cuda"), net.rng_seed, net._rng_offset))
+        if rc:
+            U = np.repeat(U, 2, axis=0)                            # a (fwd, rev) pair shares its draw
+        net.train_step(Xd, Rd, Yd, Md, F=Fd)
+        st, g = orc.train_step(ref_p, ref_m, X, R, Y.astype(np.float64), nm, pool, hidden, loss, rate, mu, Ymask=Ymask, dropout=(drop, U),
+                               decay_conv=dconv, decay_full=dfull, step=step, weight_decay_start=1, reverse_complement=rc, start_training=1,
+                               features=None if F is None else F.astype(np.float64))
+        got = net.get_grads()
+        for pname, _, axis in net.layout:
+            assert_close_per_model(got[pname], g[pname], GRAD, nm, axis, "step %d gradient %s" % (step, pname))
+            record_error(name, "gradients", got[pname], g[pname], GRAD)
+        Z = host(net._step_bufs[(Xd.numel(), rows)]["Z"])
+        assert_close_per_model(Z, st["Zout"], ACT, nm, 1, "step %d predictions" % step)
+        record_error(name, "activations", Z, st["Zout"], ACT)
+    assert _used_single(net), "the step did not go through the single-launch kernel"
+    got = net.get_params()
+    for pname, _, axis in net.layout:
+        assert_close_per_model(got[pname], ref_p[pname], GRAD, nm, axis, "parameters %s" % pname)
+        record_error(name, "parameters", got[pname], ref_p[pname], GRAD)
+
+
+@pytest.mark.parametrize("pool,hidden,loss", [("max", 32, "nll"), ("all", 0, "mse")])
+def test_single_launch_step_is_bit_stable_and_agrees_with_the_multi_launch_step(pool, hidden, loss):
+    rng = np.random.default_rng(5)
+    m, B = 24, 128
+    X, R = _batch(rng, B, m, 30, 101)
+    Y = rng.random((B, 2)).astype(np.float32)
+    Xd, Rd, Yd = dev(X), dev(R), dev(Y)
+    outs = []
+    for single in (True, True, False):
+        r2 = np.random.default_rng(6)
+        net, _ = _net(r2, 2, 16, m, pool, hidden, loss, rate=0.05, momentum=0.9, dropout=0.4, decay_full=1e-3, weight_decay_start=0,
+                      single_launch=single)
+        losses = []
+        for _ in range(4):
+            net.train_step(Xd, Rd, Yd)
+        assert _used_single(net) == single
+        outs.append(net.get_params())
+    for pname in outs[0]:
+        assert np.array_equal(outs[0][pname], outs[1][pname]), "run-to-run difference in %s" % pname
+        assert_close_per_model(outs[0][pname], outs[2][pname], GRAD, 1, 0, "single vs multi launch %s" % pname)
+
+
+def test_single_launch_step_in_a_graph_and_loss_output():
+    rng = np.random.default_rng(8)
+    m, B = 16, 128
+    X, R = _batch(rng, B, m, 38, 41)
+    Y = rng.standard_normal((B, 1)).astype(np.float32)
+    Xd, Rd, Yd = dev(X), dev(R), dev(Y)
+    nets = []
+    for _ in range(2):
+        r2 = np.random.default_rng(9)
+        nets.append(_net(r2, 1, 16, m, "all", 0, "mse", rate=0.02, momentum=0.9, dropout=0.25)[0])
+    eager, graphed = nets
+    step = graphed.make_graphed_step(Xd, Rd, Yd)
+    for i in range(4):
+        eager.train_step(Xd, Rd, Yd)
+        step()
+        torch.cuda.synchronize()
+        a, b = eager.get_params(), graphed.get_params()
+        for pname in a:
+            assert np.array_equal(a[pname], b[pname]), "replay %d differs from the eager step in %s" % (i, pname)
+    assert _used_single(eager) and _used_single(graphed)
+    assert eager.step_count == graphed.step_count == 4 and eager._rng_offset == graphed._rng_offset
+
+
+def test_shapes_the_single_launch_step_does_not_take_fall_back():
+    """A region longer than 256 rows, or more than four models: the multi-launch step runs (same bits as with the
+    single-launch step switched off); calling the entry point directly on an unsupported shape is refused."""
+    from deepbind_amd import _lib
+    rng = np.random.default_rng(10)
+    m = 12
+    X, R = _batch(rng, 16, m, 280, 300)
+    Y = rng.random((16, 1)).astype(np.float32)
+    outs = []
+    for single in (True, False):
+        net, _ = _net(np.random.default_rng(11), 1, 16, m, "max", 8, "nll", rate=0.05, single_launch=single)
+        net.train_step(dev(X), dev(R), dev(Y))
+        assert not _used_single(net) or single
+        outs.append(net.get_params())
+    for pname in outs[0]:
+        assert np.array_equal(outs[0][pname], outs[1][pname])
+    X, R = _batch(rng, 16, m, 20, 30)
+    net, _ = _net(np.random.default_rng(12), 6, 16, m, "max", 8, "nll", rate=0.05)
+    net.train_step(dev(X), dev(R), dev(rng.random((16, 6)).astype(np.float32)))
+    assert not _used_single(net)
+    work = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    with pytest.raises(_lib.DeepbindError, match="NotImplementedError"):
+        _lib.call("dbk_train_step_single", _lib.stream(), ctypes.addressof(net._step_args), _lib.ptr(work), work.numel())
+
+
+def test_region_longer_than_the_kernel_takes_is_flagged_and_leaves_the_parameters_alone():
+    """The kernel's own guard (the Python side normally never lets such a batch through)."""
+    from deepbind_amd import _lib
+    rng = np.random.default_rng(13)
+    m = 12
+    X, R = _batch(rng, 16, m, 280, 300)
+    net, _ = _net(np.random.default_rng(14), 1, 16, m, "max", 8, "nll", rate=0.05)
+    before = net.get_params()
+    Xd, Rd, Yd = dev(X), dev(R), dev(rng.random((16, 1)).astype(np.float32))
+    buf = net._prepare_step(Xd, Rd, Yd)
+    need = ctypes.c_size_t(0)
+    _lib.call("dbk_train_step_single_workspace", ctypes.addressof(net._step_args), ctypes.addressof(need))
+    assert need.value > 0
+    buf["work"] = torch.zeros(need.value, dtype=torch.uint8, device="cuda")
+    _lib.call("dbk_train_step_single", _lib.stream(), ctypes.addressof(net._step_args), _lib.ptr(buf["work"]), need.value)
+    torch.cuda.synchronize()
+    assert int(buf["work"][4:8].view(torch.int32).item()) == 2
+    with pytest.raises(_lib.DeepbindError, match="256 rows"):
+        net.get_params()
+    after = net.get_params()
+    for pname in before:
+        assert np.array_equal(before[pname], after[pname])
