@@ -614,144 +614,168 @@ __global__ void reduce_slabs_kernel(float* __restrict__ dW, float* __restrict__ 
     }
 }
 
-// Dense half of the backward pass when the forward pass left its activity masks (one 64-bit lane mask per
-// row and filter tile: bit l set = the rectifier of filter tile*64 + l is open at that row): nothing is
-// recomputed and no table is needed. Per window of 16 positions a wave reads 16 masks (lane p reads row p's,
-// one window ahead), turns each into this lane's gradient value (davg/count or 0) and adds the window
-// into the register planes, one addition per (position, tap).
+// The mask-driven backward through bit counts. At every row of a region whose rectifier is open the average-pooling
+// gradient is the SAME number c = dpooled / rows, so the filter gradient needs no pass over the rows:
+//     dW[tap][letter][f] += c * popcount(open_f & (is_letter >> tap))
+// with one bit per row: open_f from the forward pass's activity masks (stored one 64-bit lane mask per row; turned
+// into one row mask per lane = filter with a six-stage butterfly of lane exchanges), is_letter from five ballots over the chunk's
+// letters (wave-uniform, shifted in scalar registers). A wave walks whole regions in chunks of 64 rows: per chunk
+// ~7 vector instructions per (tap, letter) whatever the number of rows, against one half-rate index-mode add per
+// (row, tap) in the kernels above: a third of their issue slots at 53 rows, a fifth at 64. The max-pooling gradient
+// lands on one row per (region, filter): that row's letters are cut out of the same letter bits, once per region.
+// A lane keeps the 5 x MT sums of its filter in registers over all its regions (ascending), the waves fold them
+// into the workgroup's slab as above. Deterministic; c * count is rounded once where the kernels above add c count
+// times, so the sums agree with theirs to rounding, not bit for bit.
+// PT: DBK_PT_AVG / ALL read the masks; DBK_PT_MAX needs none.
+// Transposes the 64 x 64 bit matrix whose row i is lane i's (lo, hi): afterwards bit i of lane j is what bit j of
+// lane i was. Six butterfly stages (block sizes 32 ... 1): a lane and its partner lane ^ d swap the off-diagonal
+// d x d blocks they hold between them.
+__device__ __forceinline__ void transpose_masks(unsigned& lo, unsigned& hi, unsigned lane)
+{
+    {   // d = 32: whole words change places
+        const unsigned plo = (unsigned)__shfl_xor((int)lo, 32, 64), phi = (unsigned)__shfl_xor((int)hi, 32, 64);
+        if (lane & 32u) lo = phi; else hi = plo;
+    }
+#pragma unroll
+    for (unsigned d = 16; d >= 1; d >>= 1) {
+        // bits whose index has bit d clear, within a word
+        const unsigned keep = d == 16 ? 0x0000ffffu : d == 8 ? 0x00ff00ffu : d == 4 ? 0x0f0f0f0fu : d == 2 ? 0x33333333u : 0x55555555u;
+        const unsigned plo = (unsigned)__shfl_xor((int)lo, (int)d, 64), phi = (unsigned)__shfl_xor((int)hi, (int)d, 64);
+        if (lane & d) {
+            lo = ((plo >> d) & keep) | (lo & ~keep);
+            hi = ((phi >> d) & keep) | (hi & ~keep);
+        } else {
+            lo = (lo & keep) | ((plo & keep) << d);
+            hi = (hi & keep) | ((phi & keep) << d);
+        }
+    }
+}
 template <int PT, int MT>
-__device__ __forceinline__ void scanpool_bprop_dense_act_body(const wg_t wg, unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
-                                                              const uint32_t* __restrict__ R, size_t P,
-                                                              const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
-                                                              const float* __restrict__ dpooled,
-                                                              const unsigned long long* __restrict__ act,
-                                                              float* __restrict__ slabs, size_t stride)
+__device__ __forceinline__ void scanpool_bprop_bits_body(const wg_t wg, unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                         const uint32_t* __restrict__ R, size_t P,
+                                                         const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
+                                                         const float* __restrict__ dpooled,
+                                                         const unsigned long long* __restrict__ act,
+                                                         float* __restrict__ slabs, size_t stride)
 {
     extern __shared__ __align__(16) unsigned char smem[];
+    constexpr bool DENSE = PT != DBK_PT_MAX, PEAK = PT != DBK_PT_AVG;
     const unsigned nw = blockDim.x >> 6;
-    const unsigned chunk = nw * XCH_SUBS * PSUB;
-    constexpr unsigned XBUF = (4 * XCH_SUBS * PSUB + MT - 1 + 7) & ~3u;   // bytes of one letter buffer (>= window_span of a full chunk)
-    static_assert(XBUF <= 512, "a thread stages at most two letters per chunk");
-    float* lut = reinterpret_cast<float*>(smem);                   // [MT*4][FT]: only the cross-wave fold at the end uses it
+    float* lut = reinterpret_cast<float*>(smem);                   // [MT*4][FT]: the cross-wave fold at the end
     float* dbacc = lut + (size_t)MT * 4 * FT;                      // [nw][FT]
-    uint8_t* xbuf = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT);   // two letter buffers, used in turn
-
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+    const unsigned lane = threadIdx.x & 63, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const unsigned f0 = wg.y * FT, f = f0 + lane;
-    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
+    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;      // rows the scan defines; later rows carry bias only
+    float acc[5][MT];
+#pragma unroll
+    for (int l = 0; l < 5; ++l)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[l][t] = 0.0f;
     float db = 0.0f;
-    grad_planes<MT> planes;
-    planes.clear();
 
-    // The work is a sequence of items (region, chunk of up to 256 rows). While an item is being added into the
-    // planes, everything the next item needs is already on its way: its letters (two per thread, parked in
-    // registers and put into the other LDS buffer afterwards), the next region's pooled gradients and the
-    // bounds of the region after that. One barrier per item.
-    auto rows_of = [&](size_t b_, size_t c_) -> unsigned { return c_ < b_ ? (unsigned)((b_ - c_) < chunk ? (b_ - c_) : chunk) : 0u; };
-    auto load_letters = [&](size_t c_, unsigned rows_, unsigned& v0, unsigned& v1) {
-        const unsigned cnt = window_span<MT>(rows_);
-        const size_t g0 = c_ + tid, g1 = g0 + 256;
-        v0 = (tid < cnt && g0 < N) ? letter_of(X[g0]) : 5u;
-        v1 = (tid + 256 < cnt && g1 < N) ? letter_of(X[g1]) : 5u;
-    };
-    auto store_letters = [&](uint8_t* buf, unsigned v0, unsigned v1) {
-        buf[tid] = (uint8_t)v0;
-        if (tid + 256 < XBUF) buf[tid + 256] = (uint8_t)v1;
-    };
     struct pooled_in { float davg, pmax, dmax; unsigned arg; };
     auto load_pooled = [&](size_t r_) -> pooled_in {
         pooled_in q = { 0.0f, 0.0f, 0.0f, 0u };
-        if (f < F) {
+        if (f < F && r_ < P) {
             const size_t j0 = r_ * F + f;
-            q.davg = PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1];
-            if (PT == DBK_PT_ALL) { q.pmax = pooled[2 * j0]; q.dmax = dpooled[2 * j0]; q.arg = argmax[j0]; }
+            if (PT == DBK_PT_AVG) q.davg = dpooled[j0];
+            else if (PT == DBK_PT_ALL) { q.davg = dpooled[2 * j0 + 1]; q.pmax = pooled[2 * j0]; q.dmax = dpooled[2 * j0]; q.arg = argmax[j0]; }
+            else { q.pmax = pooled[j0]; q.dmax = dpooled[j0]; q.arg = argmax[j0]; }
         }
         return q;
     };
-    float gavg = 0.0f, gmax = 0.0f;                                // max+avg pooling: see the recomputing kernel
-    size_t imax = ~(size_t)0;
-    auto enter_region = [&](const pooled_in& q, size_t a_, size_t b_) {
-        gavg = q.davg / (float)(b_ - a_);
-        gmax = 0.0f;
-        imax = ~(size_t)0;
-        if (PT == DBK_PT_ALL && q.pmax > 0.0f) { gmax = q.dmax; imax = q.arg / F; }
+    auto bound = [&](size_t r_, unsigned which) -> size_t { return r_ < P ? (unsigned)__builtin_amdgcn_readfirstlane((int)R[2 * r_ + which]) : 0u; };
+    struct raw { unsigned x0, x1; unsigned long long mk; };       // a chunk as loaded: two letters per lane, the row's mask
+    auto load_chunk = [&](size_t c0, size_t bend) -> raw {
+        raw w = { 254u, 254u, 0ull };
+        const size_t g0 = c0 + lane, g1 = g0 + 64;
+        if (g0 < N) w.x0 = X[g0];
+        if (lane < (unsigned)MT - 1 && g1 < N) w.x1 = X[g1];
+        if (DENSE && g0 < bend) w.mk = act[g0 * wg.gy + wg.y];
+        return w;
     };
 
-    // activity masks of the 16 rows from p0 of a chunk (lane p takes row p's); rows past the chunk read as "closed"
-    auto fetch = [&](size_t c_, unsigned rows_, unsigned p0) -> unsigned long long {
-        return (lane < (unsigned)PSUB && p0 + lane < rows_) ? act[(c_ + p0 + lane) * wg.gy + wg.y] : 0ull;
-    };
-    size_t r = wg.x;
-    bool valid = r < P;
-    size_t a = 0, b = 0, c0 = 0, pa = 0, pb = 0;                   // (pa, pb): bounds of the region after this one
-    unsigned long long mk_first = 0ull;                            // this wave's first masks of the current item
-    if (valid) {
-        a = R[2 * r]; b = R[2 * r + 1]; c0 = a;
-        if (r + wg.gx < P) { pa = R[2 * (r + wg.gx)]; pb = R[2 * (r + wg.gx) + 1]; }
-        mk_first = fetch(c0, rows_of(b, c0), wave * PSUB);
-        enter_region(load_pooled(r), a, b);
-        unsigned v0, v1;
-        load_letters(c0, rows_of(b, c0), v0, v1);
-        store_letters(xbuf, v0, v1);
-    }
-    __syncthreads();
-    unsigned cur = 0;
-    while (valid) {                                                // uniform over the workgroup
-        const unsigned rows = rows_of(b, c0);
-        // ---- the next item, and its loads
-        size_t nr = r, na = a, nb = b, nc0 = c0 + chunk;
-        const bool newregion = nc0 >= b;
-        if (newregion) { nr = r + wg.gx; na = pa; nb = pb; nc0 = na; }
-        const bool nvalid = nr < P;
-        unsigned nv0 = 5u, nv1 = 5u;
-        pooled_in nq = { 0.0f, 0.0f, 0.0f, 0u };
-        size_t qa = 0, qb = 0;
-        if (nvalid) {
-            load_letters(nc0, rows_of(nb, nc0), nv0, nv1);
-            if (newregion) {
-                nq = load_pooled(nr);
-                if (nr + wg.gx < P) { qa = R[2 * (nr + wg.gx)]; qb = R[2 * (nr + wg.gx) + 1]; }
-            }
-        }
-        const unsigned long long mk_next = nvalid ? fetch(nc0, rows_of(nb, nc0), wave * PSUB) : 0ull;   // the next item's first masks
-        // ---- this item
-        const uint8_t* xl = xbuf + cur * XBUF;
-        unsigned long long mk = mk_first;
-#pragma unroll 1
-        for (unsigned s = 0; s < XCH_SUBS; ++s) {
-            const unsigned p0 = (s * nw + wave) * PSUB;
-            if (p0 >= rows) break;
-            const unsigned long long mkn = fetch(c0, rows, p0 + nw * PSUB);
-            unsigned wq[window<MT>::words];
-            load_window<MT>(xl, p0, wq);
-            float g[PSUB];
-            // window-relative 32-bit positions of the winning row (this lane's; -1 when it lies elsewhere: it is always
-            // inside the region) and of the scan's end, so that the per-position tests are one 32-bit compare each
-            const size_t w0 = c0 + p0;
-            const int relmax = (PT == DBK_PT_ALL && imax >= w0 && imax - w0 < (size_t)PSUB) ? (int)(imax - w0) : -1;
-            const int nrel = n > w0 ? (n - w0 < (size_t)PSUB ? (int)(n - w0) : PSUB) : 0;
+    const size_t step = (size_t)wg.gx * nw;
+    size_t r = (size_t)wg.x * nw + wave;
+    size_t a = bound(r, 0), b = bound(r, 1), na = bound(r + step, 0), nb = bound(r + step, 1);
+    size_t nna = bound(r + 2 * step, 0), nnb = bound(r + 2 * step, 1);
+    pooled_in q = load_pooled(r), nq = load_pooled(r + step);
+    size_t c0 = a;
+    raw cur = r < P ? load_chunk(c0, b) : raw{ 254u, 254u, 0ull };
+    float gavg = 0.0f, gmax = 0.0f;
+    size_t imax = ~(size_t)0;
+    unsigned tm[5] = { 0u, 0u, 0u, 0u, 0u };                        // letters of the taps at the winning row: bit t of tm[l]
+    while (r < P) {                                                // uniform over the wave
+        // ---- the chunk after this one is requested before this one is worked on
+        const bool last = c0 + 64 >= b;
+        const size_t nc0 = last ? na : c0 + 64, nend = last ? nb : b;
+        const bool more = last ? r + step < P : true;
+        raw nxt = { 254u, 254u, 0ull };
+        if (more) nxt = load_chunk(nc0, nend);
+        if (c0 == a) {
+            if (DENSE) gavg = b > a ? q.davg / (float)(b - a) : 0.0f;
+            if (PEAK) {
+                gmax = 0.0f; imax = ~(size_t)0;
+                if (q.pmax > 0.0f) { gmax = q.dmax; imax = q.arg / F; }
 #pragma unroll
-            for (int p = 0; p < PSUB; ++p) {
-                const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)mk, p);
-                const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(mk >> 32), p);
-                const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
-                float gg = open ? gavg : 0.0f;
-                if (PT == DBK_PT_ALL) gg += p == relmax ? gmax : 0.0f;
-                db += gg;
-                g[p] = p < nrel ? gg : 0.0f;                       // rows past the scan's end carry bias only
+                for (int l = 0; l < 5; ++l) tm[l] = 0u;
             }
-            grad_planes_window<MT>(planes, wq, g);
-            mk = mkn;
         }
-        // ---- hand over
-        if (nvalid) store_letters(xbuf + (cur ^ 1u) * XBUF, nv0, nv1);
-        __syncthreads();
-        if (newregion && nvalid) { enter_region(nq, na, nb); pa = qa; pb = qb; }
-        r = nr; a = na; b = nb; c0 = nc0; valid = nvalid; cur ^= 1u;
-        mk_first = mk_next;
+        // ---- one bit per (letter, position) of the chunk: positions c0 .. c0 + 63 and the MT - 1 behind them
+        const unsigned v0 = letter_of(cur.x0), v1 = letter_of(cur.x1);
+        unsigned long long L0[5], L1[5];
+#pragma unroll
+        for (int l = 0; l < 5; ++l) { L0[l] = __ballot(v0 == (unsigned)l); L1[l] = __ballot(v1 == (unsigned)l); }
+        const size_t nrel = n > c0 ? n - c0 : 0;                   // rows of the chunk the scan defines
+        if (DENSE) {
+            // ---- one bit per row for this lane's filter: bit i of lane f = bit f of row i's mask
+            const unsigned mlo = (unsigned)cur.mk, mhi = (unsigned)(cur.mk >> 32);
+            unsigned tlo = mlo, thi = mhi;
+            transpose_masks(tlo, thi, lane);
+            db += gavg * (float)(__popc(tlo) + __popc(thi));
+            const unsigned long long keep = nrel >= 64 ? ~0ull : ((1ull << nrel) - 1ull);
+            tlo &= (unsigned)keep;
+            thi &= (unsigned)(keep >> 32);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+#pragma unroll
+                for (int l = 0; l < 5; ++l) {
+                    const unsigned long long sh = t == 0 ? L0[l] : (L0[l] >> t) | (L1[l] << (64 - t));   // is_letter at row + t
+                    const unsigned cnt = __popc(tlo & (unsigned)sh) + __popc(thi & (unsigned)(sh >> 32));
+                    acc[l][t] = __builtin_fmaf(gavg, (float)cnt, acc[l][t]);
+                }
+            }
+        }
+        if (PEAK) {
+            // ---- the winning row of this lane's filter, if it lies in the chunk: its taps' letters
+            const bool here = imax >= c0 && imax - c0 < 64;
+            const unsigned rel = here ? (unsigned)(imax - c0) : 0u;
+            if (here) db += gmax;
+            const bool counts = here && imax < n;
+#pragma unroll
+            for (int l = 0; l < 5; ++l) {
+                const unsigned long long cut = rel == 0 ? L0[l] : (L0[l] >> rel) | (L1[l] << (64 - rel));
+                tm[l] |= counts ? (unsigned)cut : 0u;              // (MT <= 32 taps: the low word is all that is looked at)
+            }
+            if (last) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+#pragma unroll
+                    for (int l = 0; l < 5; ++l) acc[l][t] = __builtin_fmaf(gmax, (float)((tm[l] >> t) & 1u), acc[l][t]);
+                }
+            }
+        }
+        // ---- on to the next chunk / region
+        if (last) {
+            r += step;
+            a = na; b = nb; q = nq;
+            na = nna; nb = nnb;
+            nna = bound(r + 2 * step, 0); nnb = bound(r + 2 * step, 1);
+            nq = load_pooled(r + step);
+        }
+        c0 = nc0;
+        cur = nxt;
     }
-    float aw[MT][4];
-    grad_planes_read<MT>(planes, aw);
     dbacc[wave * FT + lane] = db;
     float* fold = lut + lane;
     for (unsigned w = 0; w < nw; ++w) {
@@ -762,8 +786,9 @@ __device__ __forceinline__ void scanpool_bprop_dense_act_body(const wg_t wg, uns
                 if ((unsigned)j < m) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
+                        const float v = acc[c][j] + 0.25f * acc[4][j];
                         float* cell = fold + (j * 4 + c) * FT;
-                        *cell = w == 0 ? aw[j][c] : *cell + aw[j][c];
+                        *cell = w == 0 ? v : *cell + v;
                     }
                 }
         }
@@ -782,150 +807,14 @@ __device__ __forceinline__ void scanpool_bprop_dense_act_body(const wg_t wg, uns
 }
 
 template <int PT, int MT>
-__global__ __launch_bounds__(256) void scanpool_bprop_dense_act_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
-                                                                       const uint32_t* __restrict__ R, size_t P,
-                                                                       const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
-                                                                       const float* __restrict__ dpooled,
-                                                                       const unsigned long long* __restrict__ act,
-                                                                       float* __restrict__ slabs, size_t stride)
+__global__ __launch_bounds__(256) void scanpool_bprop_bits_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
+                                                                  const uint32_t* __restrict__ R, size_t P,
+                                                                  const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
+                                                                  const float* __restrict__ dpooled,
+                                                                  const unsigned long long* __restrict__ act,
+                                                                  float* __restrict__ slabs, size_t stride)
 {
-    scanpool_bprop_dense_act_body<PT, MT>(this_wg(), m, F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
-}
-
-// The mask-driven dense backward for many regions: a wave per region. The kernel above spreads the windows of one
-// region over the four waves of a workgroup and meets at a barrier per region chunk; with regions of a few dozen rows
-// that is one window per wave and barrier, and the waves spend half their time waiting for the next chunk's loads.
-// Here every wave walks whole regions on its own (64 rows per round: letters staged in the wave's own LDS bytes, the
-// 64 rows' masks read by the 64 lanes in one load, four windows added into the wave's register planes), with the next
-// region's bounds and pooled gradients requested a region ahead. No barrier until the waves fold their planes into
-// the workgroup's slab at the end, exactly as above. The regions are dealt to waves instead of workgroups, so the
-// partial sums are other (equally fixed) partial sums than the kernel above forms.
-template <int PT, int MT>
-__device__ __forceinline__ void scanpool_bprop_dense_act_wave_body(const wg_t wg, unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
-                                                                   const uint32_t* __restrict__ R, size_t P,
-                                                                   const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
-                                                                   const float* __restrict__ dpooled,
-                                                                   const unsigned long long* __restrict__ act,
-                                                                   float* __restrict__ slabs, size_t stride)
-{
-    extern __shared__ __align__(16) unsigned char smem[];
-    const unsigned nw = blockDim.x >> 6;
-    constexpr unsigned XB = (3 * PSUB + 4 * window<MT>::words + 15) & ~15u;   // letters behind the four windows of a round
-    static_assert(XB <= 128, "a lane stages at most two letters per round");
-    float* lut = reinterpret_cast<float*>(smem);                   // [MT*4][FT]: only the cross-wave fold at the end uses it
-    float* dbacc = lut + (size_t)MT * 4 * FT;                      // [nw][FT]
-    // the wave's index, region bounds and loop control are wave-uniform: kept in scalar registers
-    const unsigned lane = threadIdx.x & 63, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    uint8_t* xw = reinterpret_cast<uint8_t*>(dbacc + (size_t)nw * FT) + (size_t)wave * XB;
-    const unsigned f0 = wg.y * FT, f = f0 + lane;
-    const size_t n = N + 1 >= (size_t)m + 1 ? N - m + 1 : 0;
-    float db = 0.0f;
-    grad_planes<MT> planes;
-    planes.clear();
-
-    struct pooled_in { float davg, pmax, dmax; unsigned arg; };
-    auto load_pooled = [&](size_t r_) -> pooled_in {
-        pooled_in q = { 0.0f, 0.0f, 0.0f, 0u };
-        if (f < F) {
-            const size_t j0 = r_ * F + f;
-            q.davg = PT == DBK_PT_AVG ? dpooled[j0] : dpooled[2 * j0 + 1];
-            if (PT == DBK_PT_ALL) { q.pmax = pooled[2 * j0]; q.dmax = dpooled[2 * j0]; q.arg = argmax[j0]; }
-        }
-        return q;
-    };
-    const size_t step = (size_t)wg.gx * nw;
-    size_t r = (size_t)wg.x * nw + wave;
-    size_t a = 0, b = 0;
-    pooled_in q = { 0.0f, 0.0f, 0.0f, 0u };
-    auto bound = [&](size_t idx) -> size_t { return (unsigned)__builtin_amdgcn_readfirstlane((int)R[idx]); };
-    if (r < P) { a = bound(2 * r); b = bound(2 * r + 1); q = load_pooled(r); }
-    while (r < P) {                                                // uniform over the wave
-        const size_t rn = r + step;
-        size_t na = 0, nb = 0;
-        pooled_in nq = { 0.0f, 0.0f, 0.0f, 0u };
-        if (rn < P) { na = bound(2 * rn); nb = bound(2 * rn + 1); nq = load_pooled(rn); }
-        const float gavg = q.davg / (float)(b - a);
-        float gmax = 0.0f;                                         // max+avg pooling: the winning row also gets the max gradient
-        size_t imax = ~(size_t)0;
-        if (PT == DBK_PT_ALL && q.pmax > 0.0f) { gmax = q.dmax; imax = q.arg / F; }
-        for (size_t c0 = a; c0 < b; c0 += 4 * PSUB) {
-            const unsigned rows = (unsigned)((b - c0) < 4 * PSUB ? (b - c0) : 4 * PSUB);
-            // letters of positions c0 .. c0 + XB - 1 (two per lane) and the masks of the round's rows (lane t: row t)
-            const size_t g0 = c0 + lane, g1 = g0 + 64;
-            const unsigned v0 = g0 < N ? letter_of(X[g0]) : 5u;
-            const unsigned v1 = (lane + 64 < XB && g1 < N) ? letter_of(X[g1]) : 5u;
-            const unsigned long long mkall = lane < rows ? act[(c0 + lane) * wg.gy + wg.y] : 0ull;
-            __builtin_amdgcn_wave_barrier();                       // the previous round's window reads come first
-            xw[lane] = (uint8_t)v0;
-            if (lane + 64 < XB) xw[lane + 64] = (uint8_t)v1;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            const unsigned mlo = (unsigned)mkall, mhi = (unsigned)(mkall >> 32);
-#pragma unroll 1
-            for (unsigned p0 = 0; p0 < rows; p0 += PSUB) {
-                unsigned wq[window<MT>::words];
-                load_window<MT>(xw, p0, wq);
-                float g[PSUB];
-                const size_t w0 = c0 + p0;
-                const int relmax = (PT == DBK_PT_ALL && imax >= w0 && imax - w0 < (size_t)PSUB) ? (int)(imax - w0) : -1;
-                const int nrel = n > w0 ? (n - w0 < (size_t)PSUB ? (int)(n - w0) : PSUB) : 0;
-#pragma unroll
-                for (int p = 0; p < PSUB; ++p) {
-                    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)mlo, (int)p0 + p);
-                    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)mhi, (int)p0 + p);
-                    const bool open = __builtin_amdgcn_inverse_ballot_w64(((unsigned long long)hi << 32) | lo);
-                    float gg = open ? gavg : 0.0f;
-                    if (PT == DBK_PT_ALL) gg += p == relmax ? gmax : 0.0f;
-                    db += gg;
-                    g[p] = p < nrel ? gg : 0.0f;                   // rows past the scan's end carry bias only
-                }
-                grad_planes_window<MT>(planes, wq, g);
-            }
-        }
-        r = rn; a = na; b = nb; q = nq;
-    }
-    float aw[MT][4];
-    grad_planes_read<MT>(planes, aw);
-    dbacc[wave * FT + lane] = db;
-    float* fold = lut + lane;
-    for (unsigned w = 0; w < nw; ++w) {
-        __syncthreads();
-        if (wave == w) {
-#pragma unroll
-            for (int j = 0; j < MT; ++j)
-                if ((unsigned)j < m) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        float* cell = fold + (j * 4 + c) * FT;
-                        *cell = w == 0 ? aw[j][c] : *cell + aw[j][c];
-                    }
-                }
-        }
-    }
-    __syncthreads();
-    const unsigned f0w = f0;
-    float* out = slabs + (size_t)wg.x * stride;
-    for (unsigned e = threadIdx.x; e < m * 4 * FT; e += blockDim.x) {
-        const unsigned row = e / FT, fl = e % FT;
-        if (f0w + fl < F) out[(size_t)row * F + f0w + fl] = lut[e];
-    }
-    if (wave == 0 && f < F) {
-        float t = dbacc[lane];
-        for (unsigned w = 1; w < nw; ++w) t += dbacc[w * FT + lane];
-        out[(size_t)4 * m * F + f] = t;
-    }
-}
-
-template <int PT, int MT>
-__global__ __launch_bounds__(256) void scanpool_bprop_dense_act_wave_kernel(unsigned m, unsigned F, const uint8_t* __restrict__ X, size_t N,
-                                                                            const uint32_t* __restrict__ R, size_t P,
-                                                                            const float* __restrict__ pooled, const uint32_t* __restrict__ argmax,
-                                                                            const float* __restrict__ dpooled,
-                                                                            const unsigned long long* __restrict__ act,
-                                                                            float* __restrict__ slabs, size_t stride)
-{
-    scanpool_bprop_dense_act_wave_body<PT, MT>(this_wg(), m, F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
+    scanpool_bprop_bits_body<PT, MT>(this_wg(), m, F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
 }
 
 // Launch shapes, shared by the single-group launchers and the multi-group ones.
@@ -978,18 +867,22 @@ inline unsigned wide_grid_x(unsigned ftiles, size_t P)
     return gx;
 }
 inline size_t wide_smem(unsigned mt) { return (size_t)mt * NL * FT * sizeof(float) + 4 * (mt == 16 ? wide_shape<16>::xbytes : wide_shape<24>::xbytes); }
-// The wave-per-region dense backward: same threshold as the wide forward (enough regions to keep every wave busy
-// with whole regions); the smallest grid that gives every wave the same number of regions as the resident grid would.
-inline bool dense_wave_takes(unsigned ftiles, size_t P) { return P * (size_t)ftiles >= 512; }
-inline unsigned dense_wave_grid_x(unsigned mt, unsigned ftiles, size_t P)
+// The bit-count backward: a wave per region, two workgroups per CU resident (its 5 x MT sums take ~170 registers);
+// the smallest grid that gives every wave the same number of regions as the resident grid would.
+inline unsigned bits_grid_x(unsigned ftiles, size_t P)
 {
-    unsigned gx = (mt == 8 ? 768u : 512u) / ftiles;                // the resident grid ...
-    if (P < 32 * (size_t)gx) gx = 256u / ftiles;                   // ... or one workgroup per CU when that leaves a wave under 8 regions
+    unsigned gx = 512u / ftiles;
     if (gx < 1) gx = 1;
-    if (gx > (P + 3) / 4) gx = (unsigned)((P + 3) / 4);
+    // at least three regions per wave: the fold of a workgroup's sums and its slab cost about as much as two regions,
+    // and with several groups in one launch (a calibration batch) the grids then still fit the GPU in one round
+    if (gx > (P + 11) / 12) gx = (unsigned)((P + 11) / 12);
     const size_t per_wave = (P + (size_t)gx * 4 - 1) / ((size_t)gx * 4);
     return (unsigned)((P + 4 * per_wave - 1) / (4 * per_wave));
 }
+// Max pooling goes through it while the regions are short on average (it visits every 64-row chunk of a region to
+// find each filter's winning row; the sparse kernel goes straight to that row).
+inline bool bits_takes_max(size_t N, size_t P) { return N <= 128 * P; }
+inline size_t bits_smem(unsigned mt) { return ((size_t)mt * 4 * FT + 4 * FT) * sizeof(float); }
 inline size_t sparse_smem(size_t m) { return m * SPARSE_ROWS * FT * sizeof(float); }
 inline size_t dense_smem(unsigned mt) { return ((size_t)mt * NL * FT + 4 * FT) * sizeof(float) + ((4 * XCH_SUBS * PSUB + mt - 1 + 7) & ~(size_t)3); }
 
@@ -1054,14 +947,8 @@ int launch_dense(hipStream_t st, unsigned gx, unsigned ftiles, size_t smem, cons
                   const uint8_t* X, size_t N, const uint32_t* R, size_t P, const float* pooled, const uint32_t* argmax,
                   const float* dpooled, const unsigned long long* act, float* slabs, size_t stride)
 {
-    if (act && dense_wave_takes(ftiles, P)) {
-        auto kern = scanpool_bprop_dense_act_wave_kernel<PT, MT>;
-        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
-        return 0;
-    }
     if (act) {
-        auto kern = scanpool_bprop_dense_act_kernel<PT, MT>;
+        auto kern = scanpool_bprop_bits_kernel<PT, MT>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), smem, st, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled, act, slabs, stride);
         return 0;
@@ -1103,13 +990,20 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         DBK_LAUNCH_OK();
     }
     // with max+avg pooling the dense half carries the maxima along
-    const unsigned gxs = PT == DBK_PT_MAX ? sparse_grid_x(ftiles, P) : 0u;
-    const unsigned gxd = PT == DBK_PT_MAX ? 0u : (act && dense_wave_takes(ftiles, P)) ? dense_wave_grid_x(mt, ftiles, P) : dense_grid_x(mt, ftiles, P);
+    const bool max_bits = PT == DBK_PT_MAX && bits_takes_max(N, P);
+    const unsigned gxs = PT == DBK_PT_MAX ? (max_bits ? bits_grid_x(ftiles, P) : sparse_grid_x(ftiles, P)) : 0u;
+    const unsigned gxd = PT == DBK_PT_MAX ? 0u : act ? bits_grid_x(ftiles, P) : dense_grid_x(mt, ftiles, P);
     const size_t smem_s = sparse_smem(m), smem_d = dense_smem(mt);
     DBK_CHECK(smem_s <= lds_limit() && smem_d <= lds_limit(), "ValueError: filter length %zu does not fit in LDS", m);
     float* slabs = (float*)dbk::workspace(stride * (gxs + gxd) * sizeof(float), st);
     DBK_CHECK(slabs != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", stride * (gxs + gxd) * sizeof(float), dbk::workspace_error());
-    if (gxs) {
+    if (gxs && max_bits) {
+        auto kern = mt == 8 ? scanpool_bprop_bits_kernel<DBK_PT_MAX, 8> : mt == 16 ? scanpool_bprop_bits_kernel<DBK_PT_MAX, 16> : scanpool_bprop_bits_kernel<DBK_PT_MAX, 24>;
+        const size_t smem_b = bits_smem(mt);
+        DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_b));
+        hipLaunchKernelGGL(kern, dim3(gxs, ftiles), dim3(256), smem_b, st, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, dpooled,
+                           (const unsigned long long*)nullptr, slabs, stride);
+    } else if (gxs) {
         constexpr int PS = PT == DBK_PT_AVG ? DBK_PT_MAX : PT;
         auto kern = mt == 8 ? scanpool_bprop_sparse_kernel<PS, 8> : mt == 16 ? scanpool_bprop_sparse_kernel<PS, 16> : scanpool_bprop_sparse_kernel<PS, 24>;
         DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_s));
@@ -1200,8 +1094,8 @@ __global__ __launch_bounds__(256) void scanpool_fprop_multi_kernel(const multi_a
         scanpool_fprop_body<DBK_PT_AVG, false, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, nullptr, nullptr, j.act);
 }
 
-// Max pooling: the one-wave sparse kernel in the first wave of the workgroup (the other waves leave at once);
-// otherwise the mask-driven dense kernel.
+// The bit-count kernel; for max pooling over long regions the one-wave sparse kernel in the first wave of the
+// workgroup (the other waves leave at once).
 template <int MT>
 __global__ __launch_bounds__(256) void scanpool_bprop_multi_kernel(const multi_args a)
 {
@@ -1209,17 +1103,14 @@ __global__ __launch_bounds__(256) void scanpool_bprop_multi_kernel(const multi_a
     const unsigned gi = multi_locate(a, wg);
     const dbk::scan_group& j = a.g[gi];
     if (j.ptype == DBK_PT_MAX) {
-        if (threadIdx.x < 64)
+        if (a.wide[gi])
+            scanpool_bprop_bits_body<DBK_PT_MAX, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, nullptr, j.slabs, j.slab_stride);
+        else if (threadIdx.x < 64)
             scanpool_bprop_sparse_body<DBK_PT_MAX, MT>(wg, a.m, j.F, j.X, a.N, a.P, j.pooled, j.argmax, j.dpooled, j.slabs, j.slab_stride);
-    } else if (a.wide[gi]) {
-        if (j.ptype == DBK_PT_ALL)
-            scanpool_bprop_dense_act_wave_body<DBK_PT_ALL, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
-        else
-            scanpool_bprop_dense_act_wave_body<DBK_PT_AVG, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
     } else if (j.ptype == DBK_PT_ALL) {
-        scanpool_bprop_dense_act_body<DBK_PT_ALL, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
+        scanpool_bprop_bits_body<DBK_PT_ALL, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
     } else {
-        scanpool_bprop_dense_act_body<DBK_PT_AVG, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
+        scanpool_bprop_bits_body<DBK_PT_AVG, MT>(wg, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.dpooled, j.act, j.slabs, j.slab_stride);
     }
 }
 
@@ -1264,11 +1155,15 @@ int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
     a.n = n; a.m = (unsigned)m; a.N = N; a.P = P; a.R = R;
     a.first[0] = 0;
     bool any_wide = false;
+    unsigned tiles = 0;
+    for (unsigned i = 0; i < n; ++i) tiles += dbk::divup(g[i].F, FT);
     for (unsigned i = 0; i < n; ++i) {
         a.g[i] = g[i];
         a.ftiles[i] = dbk::divup(g[i].F, FT);
-        a.wide[i] = wide_takes(m, a.ftiles[i], P);                 // as the group's own launch would choose
-        a.gx[i] = a.wide[i] ? wide_grid_x(a.ftiles[i], P) : fprop_grid_x(mt, a.ftiles[i], P);
+        a.wide[i] = wide_takes(m, a.ftiles[i], P);                 // the kernel body the group's own launch would choose
+        // the groups share the GPU: the grids are sized so that all of them are resident together, and a workgroup
+        // amortises its filter tile's table over more regions (a region's results do not depend on the grid)
+        a.gx[i] = a.wide[i] ? wide_grid_x(tiles, P) : fprop_grid_x(mt, tiles, P);
         a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
         if (a.wide[i]) any_wide = true;
     }
@@ -1288,9 +1183,9 @@ int scan_bprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
     size_t total = 0;
     for (unsigned i = 0; i < n; ++i) {
         a.ftiles[i] = dbk::divup(g[i].F, FT);
-        a.wide[i] = g[i].ptype != DBK_PT_MAX && dense_wave_takes(a.ftiles[i], P);     // as the group's own launch would choose
-        a.gx[i] = g[i].ptype == DBK_PT_MAX ? sparse_grid_x(a.ftiles[i], P)
-                  : a.wide[i] ? dense_wave_grid_x(mt, a.ftiles[i], P) : dense_grid_x(mt, a.ftiles[i], P);
+        // as the group's own launch would choose: the bit-count kernel, or the sparse one for max pooling over long regions
+        a.wide[i] = g[i].ptype != DBK_PT_MAX || bits_takes_max(N, P);
+        a.gx[i] = a.wide[i] ? bits_grid_x(a.ftiles[i], P) : sparse_grid_x(a.ftiles[i], P);
         a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
         g[i].slab_stride = 4 * m * (size_t)g[i].F + g[i].F;
         g[i].nslab = a.gx[i];

@@ -305,7 +305,8 @@ def test_scanpool_bprop(ks, ptype, B, lo, hi, m, F):
                                           (25, 200, 300, 7, 64), (40, 20, 40, 24, 144), (12, 480, 520, 30, 40)])
 def test_scanpool_bprop_with_activity_masks_equals_recomputation(ks, ptype, B, lo, hi, m, F):
     """The forward pass can leave one bit per (row, filter) - rectifier open or not - and the backward pass
-    then skips recomputing the map: same gradient values added in the same order, so the same bits. Also
+    then skips recomputing the map: it counts the open rows per (tap, letter) and multiplies once where the
+    recomputing kernel adds the same gradient row by row, so the two agree to rounding. Also
     checks the masks themselves against the oracle's activation map, with letters that contribute nothing
     (code 254) and regions that end where the stream ends."""
     rng, W, b, X, R = _fused_case(3 * B + F, B, lo, hi, m, F, p254=0.02)
@@ -338,7 +339,11 @@ def test_scanpool_bprop_with_activity_masks_equals_recomputation(ks, ptype, B, l
     dW1 = dev(np.ones(W.shape, np.float32)); db1 = dev(np.ones((1, F), np.float32))
     ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P0, I0, dP, dW0, db0, overwrite=True)
     ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P0, I0, dP, dW1, db1, overwrite=True, act=act)
-    assert np.array_equal(host(dW0), host(dW1)) and np.array_equal(host(db0), host(db1))
+    assert_close(host(dW1), host(dW0), 1e-5, "dW from masks vs recomputed")
+    assert_close(host(db1), host(db0), 1e-5, "db from masks vs recomputed")
+    dW2 = dev(np.ones(W.shape, np.float32)); db2 = dev(np.ones((1, F), np.float32))
+    ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P0, I0, dP, dW2, db2, overwrite=True, act=act)
+    assert np.array_equal(host(dW1), host(dW2)) and np.array_equal(host(db1), host(db2))      # run to run: the same bits
     with pytest.raises(Exception):
         ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, path="kmer", act=act)
 
