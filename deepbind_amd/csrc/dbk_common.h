@@ -20,8 +20,9 @@ void clear_error();
 // passes to the new stream (after draining the device). Growing a buffer or recycling a slot synchronises
 // the device, which a stream under capture does not allow: null then, and when memory runs out, with the
 // reason in workspace_error().
-// `which` selects one of two independent buffers of the stream (a call that must keep one kernel's partial
-// results while another kernel fills its own uses the second).
+// `which` selects one of four independent buffers of the stream: 0 and 1 hold kernels' partial results (a call
+// that must keep one kernel's partial results while another kernel fills its own uses the second), 2 and 3 the
+// whole maps of the unfused scan + pool chain, whose kernels use buffer 0 themselves.
 void* workspace(size_t bytes, hipStream_t stream, int which = 0);
 const char* workspace_error();
 

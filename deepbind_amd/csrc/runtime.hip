@@ -17,7 +17,8 @@ void set_error(const char* fmt, ...)
 
 void clear_error() { g_err[0] = 0; }
 
-struct ws_t { hipStream_t stream = nullptr; void* ptr[2] = {nullptr, nullptr}; size_t bytes[2] = {0, 0}; bool used = false; uint64_t tick = 0; };
+constexpr int WS_BUFFERS = 4;   // 0, 1: partial sums of the kernels; 2, 3: whole maps of the unfused scan + pool chain
+struct ws_t { hipStream_t stream = nullptr; void* ptr[WS_BUFFERS] = {}; size_t bytes[WS_BUFFERS] = {}; bool used = false; uint64_t tick = 0; };
 constexpr int WS_DEVICES = 64, WS_STREAMS = 64;
 static ws_t g_ws[WS_DEVICES][WS_STREAMS];
 static uint64_t g_ws_tick = 0;
@@ -37,7 +38,7 @@ void* workspace(size_t bytes, hipStream_t stream, int which)
 {
     int dev = 0;
     g_ws_why[0] = 0;
-    if (which < 0 || which > 1) return nullptr;
+    if (which < 0 || which >= WS_BUFFERS) return nullptr;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= WS_DEVICES) {
         snprintf(g_ws_why, sizeof(g_ws_why), "no current device below %d", WS_DEVICES);
         return nullptr;

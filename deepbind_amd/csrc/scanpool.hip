@@ -1219,7 +1219,9 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream, const float* W, const float*
                                const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
                                float* pooled, uint32_t* argmax, uint64_t* act)
 {
-    DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
+    // sum pooling has no fused kernel: the operator chain computes it (no activity masks are written)
+    if (ptype == DBK_PT_SUM) return dbk_scanpool_fprop_unfused(stream, W, bias, m, nfilter, X, N, regions, nregion, 2, ptype, pooled, argmax);
+    DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: unknown pooling type %d", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
     // argmax entries are flat 32-bit indices row*nfilter + f into the (virtual) map, as in the reference (uindex_t)
@@ -1250,7 +1252,9 @@ int dbk_scanpool_fprop(dbk_stream_t stream, const float* W, const float* bias, s
                        const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
                        float* pooled, uint32_t* argmax, uint64_t* act)
 {
-    DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
+    // sum pooling has no fused kernel: the operator chain computes it (no activity masks are written)
+    if (ptype == DBK_PT_SUM) return dbk_scanpool_fprop_unfused(stream, W, bias, m, nfilter, X, N, regions, nregion, 2, ptype, pooled, argmax);
+    DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: unknown pooling type %d", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
     // argmax entries are flat 32-bit indices row*nfilter + f into the (virtual) map, as in the reference (uindex_t)
@@ -1274,6 +1278,8 @@ int dbk_scanpool_bprop(dbk_stream_t stream, const float* W, const float* bias, s
                        const uint64_t* act)
 {
     using namespace dbk_scanpool_general;
+    if (ptype == DBK_PT_SUM && !dbk::deferred())
+        return dbk_scanpool_bprop_unfused(stream, W, bias, m, nfilter, X, N, regions, nregion, 2, ptype, argmax, dpooled, dW, dbias, overwrite);
     DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (nfilter == 0) { dbk::clear_error(); return 0; }

@@ -165,10 +165,14 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=
     sequence bytes; calls that overlap on one GPU must not use it together).
     out (optional): (pooled, argmax|None) tensors to write into instead of new ones, so that the call allocates nothing.
     act (optional, from activity_words): receives 1 bit per row and filter - rectifier open or not - which
-    scanpool_bprop takes in place of recomputing the map (general kernel only)."""
+    scanpool_bprop takes in place of recomputing the map (general kernel only).
+    Sum pooling and 3-column regions (row step) run the operator kernels one after another inside the library, with
+    the map in its scratch: same results as the reference's chain; path must be "auto" and no masks are written."""
     _u8(X)
     _regions(regions)
-    require(regions.shape[1] == 2, "ValueError: the fused path takes 2-column regions")
+    unfused = regions.shape[1] == 3 or ptype == "sum"
+    require(not unfused or (path == "auto" and act is None),
+            "ValueError: sum pooling and stepped regions run the operator chain: no kernel choice, no activity masks")
     require(W.dtype == torch.float32 and b.dtype == torch.float32, "TypeError: the fused path is float32 only")
     require(W.shape[0] % 4 == 0 and b.numel() == W.shape[1], "ValueError: W must be (4m x P) and b must have P entries")
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
@@ -182,6 +186,10 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=
     else:
         pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
         argmax = torch.empty((P, F), dtype=uindex, device=W.device) if want_argmax else None
+    if unfused:
+        call("dbk_scanpool_fprop_unfused", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, regions.shape[1],
+             str2pooltype[ptype], ptr(pooled), ptr(argmax))
+        return pooled, argmax
     entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "wide": "dbk_scanpool_fprop_wide",
              "kmer": "dbk_scanpool_fprop_kmer", "kmer_static": "dbk_scanpool_fprop_kmer_static"}[path]
     args = [stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax)]
@@ -210,5 +218,10 @@ def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db, ove
     require(dW.shape == W.shape and db.numel() == W.shape[1], "ValueError: dW / db shapes must match W / b")
     require(dpooled.shape == pooled.shape, "ValueError: dpooled must have pooled's shape")
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
+    if regions.shape[1] == 3 or ptype == "sum":
+        require(act is None, "ValueError: sum pooling and stepped regions take no activity masks")
+        call("dbk_scanpool_bprop_unfused", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, regions.shape[1],
+             str2pooltype[ptype], ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)))
+        return
     call("dbk_scanpool_bprop", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype],
          ptr(pooled), ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)), _act(act, X, F))

@@ -109,7 +109,8 @@ int dbk_dropoutord_mirror(dbk_stream_t stream, const uint8_t* X, uint8_t* Z, uin
 /* ------------------------------------------------------------------ fused scan + bias + ReLU + pool */
 
 /* pooled[r, .] = pool_{i in region r} relu(scan(W,X)[i,f] + bias[f]) without materialising the
- * (N, F) map. Regions have 2 columns. ptype per call (max / avg / all); pooled layout and argmax
+ * (N, F) map. Regions have 2 columns. ptype per call (max / avg / all fused; sum goes through
+ * dbk_scanpool_fprop_unfused and writes no activity masks); pooled layout and argmax
  * (flat row*F+f into the virtual map, may be NULL) exactly as dbk_poolrgn. X has N bytes; windows
  * reaching past N contribute nothing (the unfused chain leaves those rows at relu(bias)).
  * float32 only. Replaces the chain corr1ord -> bias -> relu -> poolrgn
@@ -182,6 +183,28 @@ int dbk_scanpool_bprop(dbk_stream_t stream,
                        const uint32_t* regions, size_t nregion, int ptype,
                        const float* pooled, const uint32_t* argmax, const float* dpooled,
                        float* dW, float* dbias, int overwrite, const uint64_t* act);
+
+/* The same chain for what the fused kernels do not take: sum pooling and regions with a third column (row step).
+ * Runs the library's operator kernels one after another (dbk_corr1ord, bias + rectifier, dbk_poolrgn) with the
+ * (N x nfilter) map in the stream's scratch (N * nfilter * 4 bytes, grown on demand), so every value is the one the
+ * reference's chain produces: rows whose window passes the end of X hold relu(bias), as there. region_columns is 2 or 3;
+ * ptype any of the four. dbk_scanpool_fprop / dbk_scanpool_bprop call these for DBK_PT_SUM.
+ * reference: kangaroo/_ext/corr1ord.py:97-117, deepity/std/elemwise.py:71-82,162-180, kangaroo/_ext/poolrgn.py:56-76 */
+int dbk_scanpool_fprop_unfused(dbk_stream_t stream,
+                               const float* W, const float* bias, size_t m, size_t nfilter,
+                               const uint8_t* X, size_t N,
+                               const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                               float* pooled, uint32_t* argmax);
+/* Its backward: recomputes the rectified map, spreads dpooled over it (dbk_poolrgn_bprop), gates it by the rectifier,
+ * sums the columns into dbias (=) and accumulates dW (+=, or = with overwrite) with dbk_corr1ord_bprop_W. Two maps of
+ * scratch. argmax is read for max / all pooling only.
+ * reference: kangaroo/_ext/poolrgn.py:78-82, deepity/std/elemwise.py:78,172-180, kangaroo/_ext/corr1ord.py:120-138 */
+int dbk_scanpool_bprop_unfused(dbk_stream_t stream,
+                               const float* W, const float* bias, size_t m, size_t nfilter,
+                               const uint8_t* X, size_t N,
+                               const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                               const uint32_t* argmax, const float* dpooled,
+                               float* dW, float* dbias, int overwrite);
 
 /* ------------------------------------------------------------------ dense head (deepity_smat) */
 

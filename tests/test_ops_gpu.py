@@ -300,6 +300,60 @@ def test_scanpool_bprop(ks, ptype, B, lo, hi, m, F):
     assert np.array_equal(host(dW), host(dW2)) and np.array_equal(host(db), host(db2))
 
 
+@pytest.mark.parametrize("stepped", [False, True])
+@pytest.mark.parametrize("ptype", ["max", "avg", "sum", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (33, 1, 300, 11, 70), (17, 0, 9, 5, 33)])
+def test_scanpool_sum_pooling_and_stepped_regions(ks, ptype, stepped, B, lo, hi, m, F):
+    """What the fused kernels do not take - sum pooling, a third region column (row step) - goes through the same two
+    calls and comes out as the reference's operator chain gives it, forward and backward."""
+    if ptype != "sum" and not stepped:
+        pytest.skip("covered by the fused kernels' tests")
+    rng, W, b, X, R = _fused_case(B + F + 3, B, lo, hi, m, F, p254=0.01)
+    if stepped:
+        R = np.concatenate([R, rng.integers(1, 5, size=(len(R), 1)).astype(np.uint32)], axis=1)
+    A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True)
+    assert_close(host(P), Pr, ACT, "pooled")
+    assert (I is None) == (Ir is None)
+    if Ir is not None and not np.array_equal(host(I), Ir):
+        va, vb = A.ravel()[host(I)], A.ravel()[Ir]
+        assert np.all(np.abs(va - vb) <= ACT * np.abs(A).max()), "argmax differs off a tie"
+        pytest.skip("argmax moved on a round-off tie; gradient comparison needs identical argmax")
+    dP = rng.standard_normal(Pr.shape).astype(np.float32)
+    dA = np.zeros_like(A)
+    orc.poolrgn_bprop(dA, R, dP.astype(np.float64), Ir, ptype)
+    dZ = orc.relu_bprop(dA, A)
+    dbr = orc.bias_bprop(dZ)[1]
+    dWr = np.zeros(W.shape); orc.corr1ord_bprop_W(dWr, X, dZ)
+    for overwrite in (False, True):
+        dW = dev(np.ones(W.shape, np.float32)); db = dev(np.full((1, F), 7.0, np.float32))
+        ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P, I, dev(dP), dW, db, overwrite=overwrite)
+        assert_close(host(dW), dWr + (0.0 if overwrite else 1.0), GRAD, "dW")
+        assert_close(host(db), dbr, GRAD, "db")
+    with pytest.raises(Exception, match="operator chain"):
+        ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, path="general")
+
+
+def test_scanpool_unfused_chain_agrees_with_the_fused_kernels(ks):
+    """Step 1 in the third column is the 2-column case: the chain and the fused kernels then compute the same function."""
+    rng, W, b, X, R = _fused_case(77, 40, 20, 60, 16, 48)
+    R3 = np.concatenate([R, np.ones((len(R), 1), np.uint32)], axis=1)
+    Wd, bd, Xd = dev(W), dev(b), dev(X)
+    for ptype in ("max", "avg", "all"):
+        P, I = ks.scanpool_fprop(Wd, bd, Xd, dev(R), ptype, want_argmax=True)
+        Pc, Ic = ks.scanpool_fprop(Wd, bd, Xd, dev(R3), ptype, want_argmax=True)
+        assert_close(host(Pc), host(P), ACT, "pooled " + ptype)
+        if I is not None:
+            assert (host(I) == host(Ic)).mean() > 0.99
+        dP = dev(rng.standard_normal(tuple(P.shape)).astype(np.float32))
+        dW, db, dWc, dbc = (dev(np.zeros(s, np.float32)) for s in (W.shape, (1, 48), W.shape, (1, 48)))
+        ks.scanpool_bprop(Wd, bd, Xd, dev(R), ptype, P, I, dP, dW, db, overwrite=True)
+        ks.scanpool_bprop(Wd, bd, Xd, dev(R3), ptype, P, I, dP, dWc, dbc, overwrite=True)
+        assert_close(host(dWc), host(dW), GRAD, "dW " + ptype)
+        assert_close(host(dbc), host(db), GRAD, "db " + ptype)
+
+
 @pytest.mark.parametrize("ptype", ["avg", "all"])
 @pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (33, 1, 300, 11, 70), (17, 0, 9, 5, 33),
                                           (25, 200, 300, 7, 64), (40, 20, 40, 24, 144), (12, 480, 520, 30, 40)])
