@@ -41,6 +41,7 @@ _SIGNATURES = {
     "dbk_scanpool_fprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
     "dbk_scanpool_fprop_general": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
     "dbk_scanpool_fprop_wide": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
+    "dbk_scanpool_fprop_mfma": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P],
     "dbk_scanpool_fprop_kmer": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
     "dbk_scanpool_fprop_kmer_static": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P],
     "dbk_scanpool_bprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P, _P, _P, _I, _P],

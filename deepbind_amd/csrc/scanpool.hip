@@ -282,6 +282,12 @@ __global__ __launch_bounds__(256) void scanpool_fprop_wide_kernel(const float* _
     scanpool_fprop_wide_body<PT, WANT_ARGMAX, MT>(this_wg(), W, bias, m, F, X, N, R, P, pooled, argmax, act);
 }
 
+}  // namespace dbk_scanpool_general
+
+#include "scan_mfma.h"
+
+namespace dbk_scanpool_general {
+
 // ---------------------------------------------------------------------------------------------
 // backward
 // ---------------------------------------------------------------------------------------------
@@ -859,6 +865,8 @@ inline unsigned dense_grid_x(unsigned mt, unsigned ftiles, size_t P)
 // items to keep every CU's LDS busy; a small batch is latency-bound and better off with four waves per region.
 inline bool wide_takes(size_t m, unsigned ftiles, size_t P) { return m > 8 && m <= 24 && P * (size_t)ftiles >= 512; }
 inline unsigned wide_tier(size_t m) { return m <= 16 ? 16u : 24u; }
+// The matrix-core forward takes those batches (same break-even: it needs enough (region, tile) items to fill the GPU).
+inline bool mfma_pays(size_t m, unsigned ftiles, size_t P) { return m > 8 && m <= 32 && P * (size_t)ftiles >= 512; }
 inline unsigned wide_grid_x(unsigned ftiles, size_t P)
 {
     unsigned gx = 768u / ftiles;                                  // three workgroups per CU are resident (150-160 registers)
@@ -918,6 +926,38 @@ int launch_fprop_wide(hipStream_t st, unsigned ftiles, const float* W, const flo
     DBK_LAUNCH_OK();
 }
 
+// The matrix-core forward: a workgroup holds a 64-filter tile (two waves per half) and walks two regions at a time.
+inline unsigned mfma_grid_x(unsigned ftiles, size_t P)
+{
+    unsigned gx = 768u / ftiles;                                  // three workgroups per CU resident
+    if (gx < 1) gx = 1;
+    if (gx > (P + 1) / 2) gx = (unsigned)((P + 1) / 2);
+    return gx;
+}
+
+template <int PT, int KS>
+int launch_fprop_mfma_ks(hipStream_t st, unsigned ftiles, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+                         const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, unsigned long long* act)
+{
+    const unsigned gx = mfma_grid_x(ftiles, P);
+    auto kern = argmax ? (act ? scanpool_fprop_mfma_kernel<PT, true, true, KS> : scanpool_fprop_mfma_kernel<PT, true, false, KS>)
+                       : (act ? scanpool_fprop_mfma_kernel<PT, false, true, KS> : scanpool_fprop_mfma_kernel<PT, false, false, KS>);
+    hipLaunchKernelGGL(kern, dim3(gx, ftiles), dim3(256), MFMA_SMEM, st, W, bias, (unsigned)m, (unsigned)F, X, N, R, P, pooled, argmax, act);
+    DBK_LAUNCH_OK();
+}
+
+template <int PT>
+int launch_fprop_mfma(hipStream_t st, unsigned ftiles, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+                      const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, unsigned long long* act)
+{
+    switch ((mfma_ksteps(m) + 1) / 2) {
+    case 1:  return launch_fprop_mfma_ks<PT, 2>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    case 2:  return launch_fprop_mfma_ks<PT, 4>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    case 3:  return launch_fprop_mfma_ks<PT, 6>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    default: return launch_fprop_mfma_ks<PT, 8>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    }
+}
+
 template <int PT>
 int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                     const uint32_t* R, size_t P, float* pooled, uint32_t* argmax, const unsigned* run_if_flag, unsigned long long* act)
@@ -928,7 +968,7 @@ int launch_fprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     DBK_CHECK(smem <= lds_limit(), "ValueError: filter length %zu needs %zu bytes of LDS (limit %zu)", m, smem, lds_limit());
     unsigned ftiles = dbk::divup(F, FT);
     DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
-    if (!run_if_flag && wide_takes(m, ftiles, P)) return launch_fprop_wide<PT>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    if (!run_if_flag && mfma_pays(m, ftiles, P)) return launch_fprop_mfma<PT>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
     const unsigned gx = fprop_grid_x(mt, ftiles, P);
     int rc = 0;
     switch (mt) {
@@ -1023,6 +1063,18 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     DBK_LAUNCH_OK();
 }
 
+int fprop_mfma(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
+               const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, unsigned long long* act)
+{
+    const unsigned ftiles = dbk::divup(F, FT);
+    DBK_CHECK(ftiles <= 65535u, "ValueError: too many filters (%zu) for one launch", F);
+    switch (ptype) {
+    case DBK_PT_MAX: return launch_fprop_mfma<DBK_PT_MAX>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    case DBK_PT_AVG: return launch_fprop_mfma<DBK_PT_AVG>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, nullptr, act);
+    default:         return launch_fprop_mfma<DBK_PT_ALL>(st, ftiles, W, bias, m, F, X, N, R, P, pooled, argmax, act);
+    }
+}
+
 int fprop_wide(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N,
                const uint32_t* R, size_t P, int ptype, float* pooled, uint32_t* argmax, unsigned long long* act)
 {
@@ -1056,7 +1108,7 @@ struct multi_args {
     size_t N, P;
     const uint32_t* R;
     unsigned first[dbk::MULTI_MAX + 1], gx[dbk::MULTI_MAX], ftiles[dbk::MULTI_MAX];
-    unsigned wide[dbk::MULTI_MAX];                                 // the group goes through the many-regions kernel body (forward: four filters per lane; backward: a wave per region)
+    unsigned wide[dbk::MULTI_MAX];                                 // the group goes through the many-regions kernel body (forward: the matrix-core scan; backward: a wave per region)
     dbk::scan_group g[dbk::MULTI_MAX];
 };
 
@@ -1070,7 +1122,7 @@ __device__ __forceinline__ unsigned multi_locate(const multi_args& a, wg_t& wg)
 }
 
 template <int MT>
-__global__ __launch_bounds__(256) void scanpool_fprop_multi_kernel(const multi_args a)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MT == 24 ? 3 : 1))) void scanpool_fprop_multi_kernel(const multi_args a)
 {
     wg_t wg;
     const unsigned gi = multi_locate(a, wg);
@@ -1078,11 +1130,11 @@ __global__ __launch_bounds__(256) void scanpool_fprop_multi_kernel(const multi_a
     if constexpr (MT == 16 || MT == 24) {
         if (a.wide[gi]) {
             if (j.ptype == DBK_PT_MAX)
-                scanpool_fprop_wide_body<DBK_PT_MAX, true, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr);
+                scanpool_fprop_mfma_body<DBK_PT_MAX, true, false, MT / 4>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, nullptr);
             else if (j.ptype == DBK_PT_ALL)
-                scanpool_fprop_wide_body<DBK_PT_ALL, true, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.act);
+                scanpool_fprop_mfma_body<DBK_PT_ALL, true, true, MT / 4>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, j.argmax, j.act);
             else
-                scanpool_fprop_wide_body<DBK_PT_AVG, false, MT>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, nullptr, j.act);
+                scanpool_fprop_mfma_body<DBK_PT_AVG, false, true, MT / 4>(wg, j.W, j.bias, a.m, j.F, j.X, a.N, a.R, a.P, j.pooled, nullptr, j.act);
             return;
         }
     }
@@ -1160,15 +1212,15 @@ int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
     for (unsigned i = 0; i < n; ++i) {
         a.g[i] = g[i];
         a.ftiles[i] = dbk::divup(g[i].F, FT);
-        a.wide[i] = wide_takes(m, a.ftiles[i], P);                 // the kernel body the group's own launch would choose
+        a.wide[i] = mfma_pays(m, a.ftiles[i], P) && m <= 24;      // the kernel body the group's own launch would choose
         // the groups share the GPU: the grids are sized so that all of them are resident together, and a workgroup
         // amortises its filter tile's table over more regions (a region's results do not depend on the grid)
-        a.gx[i] = a.wide[i] ? wide_grid_x(tiles, P) : fprop_grid_x(mt, tiles, P);
+        a.gx[i] = a.wide[i] ? mfma_grid_x(tiles, P) : fprop_grid_x(mt, tiles, P);
         a.first[i + 1] = a.first[i] + a.gx[i] * a.ftiles[i];
         if (a.wide[i]) any_wide = true;
     }
     size_t smem = fprop_smem(mt, m);
-    if (any_wide && wide_smem(wide_tier(m)) > smem) smem = wide_smem(wide_tier(m));
+    if (any_wide && MFMA_SMEM > smem) smem = MFMA_SMEM;
     if (mt == 8) return launch_multi(scanpool_fprop_multi_kernel<8>, st, smem, a);
     if (mt == 16) return launch_multi(scanpool_fprop_multi_kernel<16>, st, smem, a);
     return launch_multi(scanpool_fprop_multi_kernel<24>, st, smem, a);
@@ -1245,6 +1297,21 @@ int dbk_scanpool_fprop_wide(dbk_stream_t stream, const float* W, const float* bi
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
     return dbk_scanpool_general::fprop_wide(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax,
+                                            reinterpret_cast<unsigned long long*>(act));
+}
+
+int dbk_scanpool_fprop_mfma(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
+                            const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int ptype,
+                            float* pooled, uint32_t* argmax, uint64_t* act)
+{
+    DBK_CHECK(ptype == DBK_PT_MAX || ptype == DBK_PT_AVG || ptype == DBK_PT_ALL, "ValueError: fused pooling type must be max, avg or all (got %d)", ptype);
+    DBK_CHECK(dbk_scanpool_general::mfma_takes(m), "NotImplementedError: the matrix-core forward kernel takes filters of 1 to 32 taps (got %zu)", m);
+    DBK_CHECK(!(argmax && ptype == DBK_PT_AVG), "ValueError: pooledmaps_argmax can only be used for max/all pooling.");
+    DBK_CHECK(!argmax || (double)N * (double)nfilter <= 4294967296.0,
+              "ValueError: %zu rows x %zu filters overflow the 32-bit argmax index; score in smaller batches or without argmax", N, nfilter);
+    if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
+    DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
+    return dbk_scanpool_general::fprop_mfma(dbk::as_stream(stream), W, bias, m, nfilter, X, N, regions, nregion, ptype, pooled, argmax,
                                             reinterpret_cast<unsigned long long*>(act));
 }
 

@@ -190,7 +190,7 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=
         call("dbk_scanpool_fprop_unfused", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, regions.shape[1],
              str2pooltype[ptype], ptr(pooled), ptr(argmax))
         return pooled, argmax
-    entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "wide": "dbk_scanpool_fprop_wide",
+    entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "wide": "dbk_scanpool_fprop_wide", "mfma": "dbk_scanpool_fprop_mfma",
              "kmer": "dbk_scanpool_fprop_kmer", "kmer_static": "dbk_scanpool_fprop_kmer_static"}[path]
     args = [stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype], ptr(pooled), ptr(argmax)]
     if path not in ("kmer", "kmer_static"):

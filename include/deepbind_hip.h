@@ -146,6 +146,17 @@ int dbk_scanpool_fprop_wide(dbk_stream_t stream,
                             const uint32_t* regions, size_t nregion, int ptype,
                             float* pooled, uint32_t* argmax, uint64_t* act);
 
+/* Same contract through the matrix-core kernel regardless of problem size, for filters of up to 32 taps
+ * (NotImplementedError otherwise): the scan as a product of the windows' one-hot letters with W, each float32
+ * weight entering as three bf16 pieces that add up to it exactly, accumulated in float32 by
+ * v_mfma_f32_32x32x16_bf16. The sums are those of the lookup kernels in another order: results agree with them
+ * to round-off, not bit for bit (an argmax can move between rows whose values tie to round-off). */
+int dbk_scanpool_fprop_mfma(dbk_stream_t stream,
+                            const float* W, const float* bias, size_t m, size_t nfilter,
+                            const uint8_t* X, size_t N,
+                            const uint32_t* regions, size_t nregion, int ptype,
+                            float* pooled, uint32_t* argmax, uint64_t* act);
+
 /* Same contract through the 3-mer lookup-table kernel regardless of problem size; fails with
  * NotImplementedError for shapes that kernel does not take (filter length > 24, avg/all pooling,
  * argmax requested). Inputs it cannot express (code 254, regions outside the sequence) are detected

@@ -244,19 +244,57 @@ def test_scanpool_fprop_wide_kernel(ks, ptype, B, lo, hi, m, F):
     assert np.array_equal(host(P2)[keep], got[keep])
 
 
-@pytest.mark.parametrize("m", [24, 16])
-def test_scanpool_general_path_picks_the_wide_kernel_for_many_regions(ks, m):
-    """From 512 (region, tile) items on, the general path runs the many-regions kernel: same results as forcing it."""
+@pytest.mark.parametrize("m", [24, 16, 30])
+def test_scanpool_general_path_picks_the_matrix_core_kernel_for_many_regions(ks, m):
+    """From 512 (region, tile) items on, the general path runs the matrix-core kernel: same bits as forcing it."""
     rng, W, b, X, R = _fused_case(5, 1100, 18, 40, m, 40, p254=0.01)
     Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
     for ptype in ("max", "avg", "all"):
         P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="general")
-        Pw, Iw = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="wide")
+        Pw, Iw = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="mfma")
         assert np.array_equal(host(P), host(Pw))
         if I is not None:
             assert np.array_equal(host(I), host(Iw))
         A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
         assert_close(host(P), Pr, ACT, "pooled " + ptype)
+
+
+@pytest.mark.parametrize("ptype", ["max", "avg", "all"])
+@pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (40, 20, 40, 24, 144), (9, 1, 300, 11, 70),
+                                          (17, 0, 9, 5, 33), (25, 60, 90, 32, 64), (30, 10, 50, 1, 40), (20, 30, 64, 20, 100)])
+def test_scanpool_fprop_matrix_core_kernel(ks, ptype, B, lo, hi, m, F):
+    """The scan as a product on the matrix cores (weights as three exact bf16 pieces): pooled values, argmax and the
+    activity masks against the operator chain; bits may differ from the lookup kernels' only where values tie to round-off."""
+    rng, W, b, X, R = _fused_case(B + m + F + 1, B, lo, hi, m, F, p254=0.01)
+    A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    act = ks.activity_words(Xd, Wd); act.fill_(-1)
+    P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True, path="mfma", act=act)
+    assert_close(host(P), Pr, ACT, "pooled")
+    scale = np.abs(A).max()
+    if Ir is not None:
+        got = host(I)
+        same = got == Ir
+        if not same.all():
+            va, vb = A.ravel()[got[~same]], A.ravel()[Ir[~same]]
+            assert np.all(np.abs(va - vb) <= ACT * scale), "argmax differs off a tie"
+            assert (~same).mean() < 0.01
+        rows, cols = got // F, got % F
+        assert np.array_equal(cols, np.tile(np.arange(F), (len(R), 1)))
+        assert np.all(rows >= R[:, :1]) and np.all((rows < R[:, 1:2]) | (R[:, 1:2] == R[:, :1]))
+    # masks: bit f of word (row, tile) <=> rectifier open, for rows inside a region; rows outside stay untouched
+    Z = np.zeros((X.size, F)); orc.corr1ord(W.astype(np.float64), X, Z)
+    pre = Z + b.astype(np.float64)
+    words = host(act).view(np.uint64).reshape(X.size, -1)
+    bits = ((words[:, :, None] >> np.arange(64, dtype=np.uint64)[None, None, :]) & np.uint64(1)).reshape(X.size, -1)[:, :F].astype(bool)
+    inside = np.zeros(X.size, bool)
+    for a_, b_ in R:
+        inside[a_:b_] = True
+    clear = np.abs(pre) > ACT * scale                                  # away from a round-off tie with zero
+    assert np.array_equal(bits[inside][clear[inside]], (pre > 0)[inside][clear[inside]])
+    assert np.all(words[~inside] == np.uint64(0xFFFFFFFFFFFFFFFF))
+    P2, _ = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=False, path="mfma")
+    assert np.array_equal(host(P), host(P2))
 
 
 def test_scanpool_regions_past_the_end_and_gaps(ks):
