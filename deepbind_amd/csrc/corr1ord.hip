@@ -10,6 +10,8 @@
 // order), corr1ord_bprop.cuh:91-137 (filter gradient), corr1ord_bprop.cu:191-201 (input gradient).
 #include "dbk_common.h"
 #include "scan_common.h"
+#include "mfma_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -530,6 +532,198 @@ int launch_fprop(hipStream_t st, const T* W, size_t m, size_t F, const uint8_t* 
     DBK_LAUNCH_OK();
 }
 
+// The same sum for many slabs: a workgroup takes 64 elements, each of its four waves a quarter of the slabs (pairwise
+// in eights, as above), and the four quarter sums are added as (q0 + q1) + (q2 + q3): four times as many loads in
+// flight per element, a shape that depends on nslab only.
+__global__ __launch_bounds__(256) void reduce_partials_quarters_kernel(float* __restrict__ dW, const float* __restrict__ partial, size_t nelem, unsigned nslab)
+{
+    __shared__ float part[4][64];
+    const unsigned el = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const size_t e = (size_t)blockIdx.x * 64 + el;
+    const unsigned per = (nslab + 3) / 4, first = q * per, last = first + per < nslab ? first + per : nslab;
+    float total = 0.0f;
+    if (e < nelem) {
+        for (unsigned base = first; base < last; base += 8) {
+            float buf[8];
+#pragma unroll
+            for (unsigned s = 0; s < 8; ++s) buf[s] = base + s < last ? partial[(size_t)(base + s) * nelem + e] : 0.0f;
+            total += ((buf[0] + buf[1]) + (buf[2] + buf[3])) + ((buf[4] + buf[5]) + (buf[6] + buf[7]));
+        }
+    }
+    part[q][el] = total;
+    __syncthreads();
+    if (q == 0 && e < nelem) dW[e] += (part[0][el] + part[1][el]) + (part[2][el] + part[3][el]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// filter gradient on the matrix cores (float32, filters of up to 32 taps, bulk sizes)
+// ---------------------------------------------------------------------------------------------
+// dW (4m x F) = H^T (4m x n) . dZ (n x F), H the one-hot windows: row 4j + k of H^T has a 1 at output row i where
+// X[i + j] is letter k (1/4 in all four rows for code 255 and other non-letters, nothing for 254). 0, 1 and 1/4 are
+// exact in bf16 and every dZ value enters as three bf16 pieces that add up to it exactly, so the products are exact
+// and v_mfma_f32_32x32x16_bf16 accumulates them in float32: the sums of the kernels above in another order.
+// A wave owns 32 filters and all 4m rows of dW (up to four 32 x 32 accumulators) over its workgroup's share of the
+// rows; the four waves of a workgroup take four neighbouring blocks of 32 filters. Per round of 64 rows the wave
+// turns the letters into one bit per (letter, position) with ballots; a lane (row 4j + k of a 32-row block, half
+// g) shifts its letter's bits by (j mod 8) + 8g once, after which the eight bits of a k-step are a whole byte of
+// the shifted word, and a 256-entry table in LDS turns the byte into the eight bf16 of the operand.
+// Deterministic: a fixed order per wave, one partial result per workgroup, the fixed-shape reduction above.
+constexpr unsigned GW_ROUND = 64;                                  // rows per round: four k-steps of 16
+
+template <int MB>
+__global__ __launch_bounds__(256) void corr1ord_bprop_W_mfma_kernel(float* __restrict__ partial, unsigned m, unsigned F,
+                                                                    const uint8_t* __restrict__ X, size_t n,
+                                                                    const float* __restrict__ dZ, unsigned rounds_per_wg)
+{
+    using namespace dbk_mfma;
+    __shared__ uint4 ones[256];                                    // byte -> eight bf16: 1.0 where the bit is set
+    const unsigned lane = threadIdx.x & 63, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const unsigned col = lane & 31, g = lane >> 5;
+    {
+        const unsigned v = threadIdx.x;
+        unsigned d[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) d[q] = ((v >> (2 * q)) & 1u ? 0x3f80u : 0u) | ((v >> (2 * q + 1)) & 1u ? 0x3f800000u : 0u);
+        ones[v] = make_uint4(d[0], d[1], d[2], d[3]);
+    }
+    const unsigned f = (blockIdx.x * 4 + wave) * 32 + col;
+    const bool fok = f < F;
+    const size_t nbytes = n + m - 1, nround = (n + GW_ROUND - 1) / GW_ROUND, nfull = n / GW_ROUND;
+    size_t rd = (size_t)blockIdx.y * rounds_per_wg;               // round in work
+    const size_t rd_end = rd + rounds_per_wg < nround ? rd + rounds_per_wg : nround;
+    const unsigned k = col & 3u, sh = (col >> 2) + 8u * g;         // this lane's letter; its bit offset within a byte step
+    f32x16_t acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[b][i] = 0.0f;
+    // a round's operands as loaded: dZ rows 16 ks + 8g + t of this lane's filter (a column past F reads the last one,
+    // and is not written), and two letters per lane (positions lane and 64 + lane of the round; past the end: "nothing")
+    const float* src = dZ + (rd * GW_ROUND + 8u * g) * F + (fok ? f : F - 1);
+    const size_t hop = (size_t)GW_ROUND * F;
+    struct round_in { float d[4][8]; unsigned x0, x1; };
+#define DBK_LOAD_ROUND(IN, RD)                                                                            \
+    {                                                                                                     \
+        const size_t g0 = (RD) * GW_ROUND + lane, g1 = g0 + 64;                                           \
+        IN.x0 = X[g0 < nbytes ? g0 : nbytes - 1];                                                         \
+        IN.x1 = X[g1 < nbytes ? g1 : nbytes - 1];                                                         \
+        IN.x0 = g0 < nbytes ? IN.x0 : 254u;                                                               \
+        IN.x1 = g1 < nbytes ? IN.x1 : 254u;                                                               \
+        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                  \
+            _Pragma("unroll") for (int t = 0; t < 8; ++t) IN.d[ks][t] = src[(size_t)(16 * ks + t) * F];   \
+        src += hop;                                                                                       \
+    }
+    // The products of a round. One bit per position: this lane's letter, and "any letter" (weight 1/4, the products add).
+#define DBK_ROUND(IN)                                                                                     \
+    {                                                                                                     \
+        const unsigned v0 = letter_of(IN.x0), v1 = letter_of(IN.x1);                                      \
+        unsigned long long L0[4], L1[4];                                                                  \
+        _Pragma("unroll") for (int l = 0; l < 4; ++l) { L0[l] = __ballot(v0 == (unsigned)l); L1[l] = __ballot(v1 == (unsigned)l); } \
+        const unsigned long long N0 = __ballot(v0 == 4u), N1 = __ballot(v1 == 4u);                        \
+        const unsigned long long m0 = k == 0u ? L0[0] : k == 1u ? L0[1] : k == 2u ? L0[2] : L0[3];        \
+        const unsigned long long m1 = k == 0u ? L1[0] : k == 1u ? L1[1] : k == 2u ? L1[2] : L1[3];        \
+        const unsigned w0 = (unsigned)m0, w1 = (unsigned)(m0 >> 32), w2 = (unsigned)m1, w3 = (unsigned)(m1 >> 32); \
+        const unsigned V[3] = { __builtin_amdgcn_alignbit(w1, w0, sh), __builtin_amdgcn_alignbit(w2, w1, sh), __builtin_amdgcn_alignbit(w3, w2, sh) }; \
+        const bool any_n = (N0 | N1) != 0ull;                                                             \
+        const unsigned q0 = (unsigned)N0, q1 = (unsigned)(N0 >> 32), q2 = (unsigned)N1, q3 = (unsigned)(N1 >> 32); \
+        const unsigned VN[3] = { __builtin_amdgcn_alignbit(q1, q0, sh), __builtin_amdgcn_alignbit(q2, q1, sh), __builtin_amdgcn_alignbit(q3, q2, sh) }; \
+        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks) {                                                \
+            unsigned pc[3][8];                                                                            \
+            _Pragma("unroll") for (int t = 0; t < 8; ++t) split3(IN.d[ks][t], pc[0][t], pc[1][t], pc[2][t]); \
+            uint4 B[3];                                                                                   \
+            _Pragma("unroll") for (int q = 0; q < 3; ++q)                                                 \
+                B[q] = make_uint4(pack_upper_halves(pc[q][0], pc[q][1]), pack_upper_halves(pc[q][2], pc[q][3]), \
+                                  pack_upper_halves(pc[q][4], pc[q][5]), pack_upper_halves(pc[q][6], pc[q][7])); \
+            /* taps 8b .. 8b + 7: byte 2 ks + b of the shifted bits holds rows 16 ks + 8g .. + 7 at this lane's tap */ \
+            _Pragma("unroll") for (int b = 0; b < MB; ++b) {                                              \
+                const uint4 A = ones[(V[(2 * ks + b) >> 2] >> (8 * ((2 * ks + b) & 3))) & 0xffu];         \
+                _Pragma("unroll") for (int q = 0; q < 3; ++q) acc[b] = mfma_bf16(A, B[q], acc[b]);        \
+            }                                                                                             \
+            if (any_n) {                                                                                  \
+                _Pragma("unroll") for (int b = 0; b < MB; ++b) {                                          \
+                    uint4 A = ones[(VN[(2 * ks + b) >> 2] >> (8 * ((2 * ks + b) & 3))) & 0xffu];          \
+                    A.x &= 0x3e803e80u; A.y &= 0x3e803e80u; A.z &= 0x3e803e80u; A.w &= 0x3e803e80u;       \
+                    _Pragma("unroll") for (int q = 0; q < 3; ++q) acc[b] = mfma_bf16(A, B[q], acc[b]);    \
+                }                                                                                         \
+            }                                                                                             \
+        }                                                                                                 \
+    }
+    // whole rounds, two per turn: the one being multiplied and the one on its way change places without copies
+    const bool owns_last = rd_end == nround && nfull < nround && rd <= nfull;   // the partial round at the end is this workgroup's
+    const size_t full_end = rd_end < nfull ? rd_end : nfull;
+    round_in ra, rb;
+    if (rd < full_end) DBK_LOAD_ROUND(ra, rd)
+    __syncthreads();
+    while (rd < full_end) {
+        if (rd + 1 < full_end) DBK_LOAD_ROUND(rb, rd + 1)
+        DBK_ROUND(ra)
+        if (++rd >= full_end) break;
+        if (rd + 1 < full_end) DBK_LOAD_ROUND(ra, rd + 1)
+        DBK_ROUND(rb)
+        ++rd;
+    }
+    if (owns_last) {
+        // the last, partial round: a row past the end reads the last row and counts as zero
+        const size_t base = nfull * GW_ROUND, left = n - base;
+        const size_t g0 = base + lane, g1 = g0 + 64;
+        ra.x0 = X[g0 < nbytes ? g0 : nbytes - 1];
+        ra.x1 = X[g1 < nbytes ? g1 : nbytes - 1];
+        ra.x0 = g0 < nbytes ? ra.x0 : 254u;
+        ra.x1 = g1 < nbytes ? ra.x1 : 254u;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const size_t rel = 16u * ks + 8u * g + t;
+                const float v = dZ[(base + (rel < left ? rel : left - 1)) * F + (fok ? f : F - 1)];
+                ra.d[ks][t] = rel < left ? v : 0.0f;
+            }
+        DBK_ROUND(ra)
+    }
+#undef DBK_LOAD_ROUND
+#undef DBK_ROUND
+    // ---- the workgroup's partial result: rows 32b + (i & 3) + 8 (i >> 2) + 4g of this lane's filter
+    float* out = partial + (size_t)blockIdx.y * 4 * m * F;
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const unsigned row = 32u * b + (i & 3) + 8 * (i >> 2) + 4u * g;
+            if (row < 4u * m && fok) out[(size_t)row * F + f] = acc[b][i];
+        }
+}
+
+template <int MB>
+void launch_bprop_W_mfma_mb(hipStream_t st, float* partial, unsigned gy, unsigned rounds, size_t m, size_t F, const uint8_t* X, size_t n, const float* dZ)
+{
+    hipLaunchKernelGGL(corr1ord_bprop_W_mfma_kernel<MB>, dim3(dbk::divup(F, 128), gy), dim3(256), 0, st, partial, (unsigned)m, (unsigned)F, X, n, dZ, rounds);
+}
+
+// Bulk sizes only: below, the partial results (one 4m x F block per workgroup) cost more than the rows.
+inline bool bprop_W_mfma_takes(size_t m, size_t F, size_t n) { return m <= 32 && F >= 32 && n * F >= ((size_t)1 << 22) && n >= 4096; }
+
+inline int launch_bprop_W_mfma(hipStream_t st, float* dW, size_t m, size_t F, const uint8_t* X, size_t n, const float* dZ)
+{
+    const unsigned fgroups = dbk::divup(F, 128);
+    const size_t nround = dbk::divup(n, GW_ROUND);
+    size_t gy = 512 / fgroups;                                     // two workgroups per CU's worth (more only adds partial results)
+    if (gy < 1) gy = 1;
+    if (gy > nround / 4) gy = nround / 4 ? nround / 4 : 1;         // at least four rounds per workgroup
+    const unsigned rounds = (unsigned)dbk::divup(nround, gy);
+    gy = dbk::divup(nround, rounds);
+    const size_t nelem = 4 * m * F;
+    float* partial = (float*)dbk::workspace(nelem * gy * sizeof(float), st);
+    DBK_CHECK(partial != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", nelem * gy * sizeof(float), dbk::workspace_error());
+    switch ((4 * m + 31) / 32) {
+    case 1:  launch_bprop_W_mfma_mb<1>(st, partial, (unsigned)gy, rounds, m, F, X, n, dZ); break;
+    case 2:  launch_bprop_W_mfma_mb<2>(st, partial, (unsigned)gy, rounds, m, F, X, n, dZ); break;
+    case 3:  launch_bprop_W_mfma_mb<3>(st, partial, (unsigned)gy, rounds, m, F, X, n, dZ); break;
+    default: launch_bprop_W_mfma_mb<4>(st, partial, (unsigned)gy, rounds, m, F, X, n, dZ); break;
+    }
+    hipLaunchKernelGGL(reduce_partials_quarters_kernel, dim3((unsigned)dbk::divup(nelem, 64)), dim3(256), 0, st, dW, (const float*)partial, nelem, (unsigned)gy);
+    DBK_LAUNCH_OK();
+}
+
 // float32 filters of at most 24 taps: register-resident gradient columns
 inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, const uint8_t* X, size_t n, const float* dZ)
 {
@@ -619,6 +813,7 @@ int dbk_corr1ord_bprop_W(dbk_stream_t stream, int dtype, void* dW, size_t m, siz
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(dW && X && dZ, "ValueError: null pointer argument");
+    if (dtype == DBK_F32 && bprop_W_mfma_takes(m, nfilter, n)) return launch_bprop_W_mfma(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     if (dtype == DBK_F32 && m <= 24) return launch_bprop_W_window(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     if (dtype == DBK_F32) return launch_bprop_W<float>(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     return launch_bprop_W<double>(dbk::as_stream(stream), (double*)dW, m, nfilter, X, n, (const double*)dZ);

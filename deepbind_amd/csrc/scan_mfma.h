@@ -14,11 +14,11 @@
 // accumulator layout (lane = filter, 16 registers = rows (i & 3) + 8 * (i >> 2) + 4 * (lane >> 5)).
 // reference chain: kangaroo/_ext/corr1ord.py:97-117, deepity/std/elemwise.py:71-82,162-180, kangaroo/_ext/poolrgn.py:56-76
 #pragma once
+#include "mfma_common.h"
 
 namespace dbk_scanpool_general {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
+using namespace dbk_mfma;
 
 constexpr unsigned MFMA_ROWS = 32;                                // positions per block
 constexpr unsigned MFMA_CHUNK = 192;                              // rows whose letters a wave stages at a time: six blocks
@@ -26,19 +26,6 @@ constexpr unsigned MFMA_XBYTES = 256;                             // a chunk's p
 constexpr size_t MFMA_SMEM = 256 * 8 + 32 * 16 + 4 * 2 * MFMA_XBYTES * 16;   // letter table + 32 empty entries + four waves' one-hot tables, two chunks each
 inline unsigned mfma_ksteps(size_t m) { return (unsigned)((4 * m + 15) / 16); }
 inline bool mfma_takes(size_t m) { return m >= 1 && m <= 32; }
-
-// two float32 bit patterns -> their upper halves as (bf16 e0, bf16 e1), e0 in the low half
-__device__ __forceinline__ unsigned pack_upper_halves(unsigned e0, unsigned e1) { return (e1 & 0xffff0000u) | (e0 >> 16); }
-
-// w = hi + mid + lo, each with at most 8 significant bits (truncations of the running remainder; the subtractions are exact)
-__device__ __forceinline__ void split3(float w, unsigned& lo, unsigned& mid, unsigned& hi)
-{
-    hi = __float_as_uint(w) & 0xffff0000u;
-    const float r1 = w - __uint_as_float(hi);
-    mid = __float_as_uint(r1) & 0xffff0000u;
-    const float r2 = r1 - __uint_as_float(mid);
-    lo = __float_as_uint(r2) & 0xffff0000u;
-}
 
 // The words of eight ballots into the lanes that carry their rows' numbers. Register I of the accumulator holds row
 // (I & 3) + 8 * (I >> 2) in lanes 0-31 and that row + 4 in lanes 32-63, so ballot I's low word belongs in lane

@@ -77,10 +77,13 @@ def test_corr1ord_rejects_bad_arguments(ks):
 @pytest.mark.parametrize("N,m,F,dense,dtype", [(400, 24, 16, True, np.float32), (3000, 16, 100, True, np.float32),
                                                (2000, 24, 64, False, np.float32), (50, 7, 5, True, np.float32),
                                                (70000, 24, 200, True, np.float32), (900, 30, 40, True, np.float32),
+                                               (60001, 11, 70, True, np.float32), (40000, 32, 160, True, np.float32),
+                                               (33000, 5, 130, False, np.float32),
                                                (600, 24, 33, True, np.float64), (20, 24, 8, True, np.float32)])
 def test_corr1ord_bprop_W(ks, N, m, F, dense, dtype):
-    """Several chunks per workgroup (N = 70000), the any-length kernel (m = 30), float64, and a stream shorter
-    than the filter (no row defined: the gradient is zero)."""
+    """Several chunks per workgroup (N = 70000), the any-length kernel (m = 30), float64, a stream shorter than the
+    filter (no row defined: the gradient is zero), and bulk sizes, which go through the matrix-core kernel (from
+    4 M gradient values on: tap counts that fill one to four 32-row blocks of dW, filters that do not fill a block)."""
     rng = np.random.default_rng(N + F)
     X = random_codes(rng, N, 0.05, 0.02)
     dZ = rng.standard_normal((N, F)).astype(dtype)
