@@ -556,6 +556,121 @@ __global__ __launch_bounds__(256) void reduce_partials_quarters_kernel(float* __
 }
 
 // ---------------------------------------------------------------------------------------------
+// forward on the matrix cores (float32, filters of up to 32 taps, bulk sizes)
+// ---------------------------------------------------------------------------------------------
+// Z (n x F) = H (n x 4m) . W (4m x F), H the one-hot windows (see the filter gradient below: the same exact
+// bf16 operands, here with W in three pieces). A wave owns 32 filters (its pieces of W stay in registers) and a
+// share of the rows, which it takes in chunks of 192: the chunk's letters become a table in LDS of one entry per
+// position (the one-hot rows of this letter and the next, 8 bf16), a lane's operand for a k-step is one 16-byte
+// read, and each block of 32 rows leaves the accumulator as 16 row segments of 128 bytes. The sums are those of the
+// lookup kernels above in another order: equal to round-off, not bit for bit (which is why only bulk sizes come here).
+constexpr unsigned GF_CHUNK = 192, GF_TABLE = 256;                 // rows per chunk; positions in its table (rows + window)
+
+template <int KS>
+__global__ __launch_bounds__(256) void corr1ord_mfma_kernel(const float* __restrict__ W, unsigned m, unsigned F,
+                                                            const uint8_t* __restrict__ X, size_t n, float* __restrict__ Z,
+                                                            unsigned chunks_per_wg)
+{
+    using namespace dbk_mfma;
+    extern __shared__ __align__(16) unsigned char smem[];
+    uint2* onehot = reinterpret_cast<uint2*>(smem);               // [256]: the four bf16 of a letter code's rows
+    const unsigned lane = threadIdx.x & 63, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const unsigned col = lane & 31, g = lane >> 5;
+    uint4* hotw = reinterpret_cast<uint4*>(smem + 256 * 8) + (size_t)wave * (2 * GF_TABLE);   // this wave's tables: the chunk in work, the next one
+    {
+        const unsigned c = threadIdx.x, one = 0x3f80u, quarter = 0x3e803e80u;
+        uint2 e;
+        if (c < 4u) { e.x = c == 0u ? one : (c == 1u ? one << 16 : 0u); e.y = c == 2u ? one : (c == 3u ? one << 16 : 0u); }
+        else if (c == 254u) { e.x = 0u; e.y = 0u; }
+        else { e.x = quarter; e.y = quarter; }
+        onehot[c] = e;
+    }
+    const size_t nbytes = n + m - 1;
+    size_t c = (size_t)blockIdx.y * chunks_per_wg * GF_CHUNK;     // first row of the chunk in work
+    const size_t end = c + (size_t)chunks_per_wg * GF_CHUNK < n ? c + (size_t)chunks_per_wg * GF_CHUNK : n;
+    unsigned letters = c < end ? load_letters4(X, nbytes, c + 4u * lane) : 0xfefefefeu;
+    // ---- this lane's column of W, rows 16s + 8g .. + 7 of every k-step, in three bf16 pieces
+    const unsigned f = (blockIdx.x * 4 + wave) * 32 + col;
+    uint4 B[KS][3];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        unsigned pc[3][8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const unsigned row = 16u * s + 8u * g + i;
+            const float w = (row < 4u * m && f < F) ? W[(size_t)row * F + f] : 0.0f;
+            split3(w, pc[0][i], pc[1][i], pc[2][i]);
+        }
+#pragma unroll
+        for (int q = 0; q < 3; ++q)
+            B[s][q] = make_uint4(pack_upper_halves(pc[q][0], pc[q][1]), pack_upper_halves(pc[q][2], pc[q][3]),
+                                 pack_upper_halves(pc[q][4], pc[q][5]), pack_upper_halves(pc[q][6], pc[q][7]));
+    }
+    __syncthreads();
+    unsigned buf = 0u;
+    for (; c < end; c += GF_CHUNK, buf ^= 1u) {
+        // ---- the chunk's table; the next chunk's letters start their way
+        uint4* hc = hotw + buf * GF_TABLE;
+        const unsigned after = (unsigned)__shfl_down((int)letters, 1, 64);   // the next lane's four letters
+        uint2 t[5];
+#pragma unroll
+        for (int k2 = 0; k2 < 4; ++k2) t[k2] = onehot[(letters >> (8 * k2)) & 0xffu];
+        t[4] = onehot[after & 0xffu];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int k2 = 0; k2 < 4; ++k2) hc[4u * lane + k2] = make_uint4(t[k2].x, t[k2].y, t[k2 + 1].x, t[k2 + 1].y);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (c + GF_CHUNK < end) letters = load_letters4(X, nbytes, c + GF_CHUNK + 4u * lane);
+        const size_t cend = c + GF_CHUNK < end ? c + GF_CHUNK : end;
+        for (size_t c0 = c; c0 < cend; c0 += 32) {
+            const uint4* hot = hc + (c0 - c) + col + 2u * g;
+            f32x16_t acc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const uint4 A = hot[4 * s];
+#pragma unroll
+                for (int q = 0; q < 3; ++q) acc = mfma_bf16(A, B[s][q], acc);
+            }
+            if (f < F) {
+                float* out = Z + (c0 + 4u * g) * F + f;
+                if (c0 + 32 <= cend) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) out[(size_t)((i & 3) + 8 * (i >> 2)) * F] = acc[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        if (c0 + 4u * g + (i & 3) + 8 * (i >> 2) < cend) out[(size_t)((i & 3) + 8 * (i >> 2)) * F] = acc[i];
+                }
+            }
+        }
+    }
+}
+
+// Bulk sizes only (the results differ from the lookup kernels' in the last bits).
+inline bool fprop_mfma_takes(size_t m, size_t F, size_t n) { return m <= 32 && F >= 32 && n * F >= ((size_t)1 << 25); }
+
+inline int launch_fprop_mfma(hipStream_t st, const float* W, size_t m, size_t F, const uint8_t* X, size_t n, float* Z)
+{
+    const unsigned fgroups = dbk::divup(F, 128);
+    const size_t nchunk = dbk::divup(n, GF_CHUNK);
+    size_t gy = 768 / fgroups;                                     // three workgroups per CU's worth
+    if (gy < 1) gy = 1;
+    if (gy > nchunk) gy = nchunk;
+    const unsigned per = (unsigned)dbk::divup(nchunk, gy);
+    gy = dbk::divup(nchunk, per);
+    const size_t smem = 256 * 8 + 4 * 2 * GF_TABLE * 16;
+    const unsigned ks = (unsigned)((4 * m + 15) / 16);
+    auto kern = ks <= 2 ? corr1ord_mfma_kernel<2> : ks <= 4 ? corr1ord_mfma_kernel<4> : ks <= 6 ? corr1ord_mfma_kernel<6> : corr1ord_mfma_kernel<8>;
+    DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3(fgroups, (unsigned)gy), dim3(256), smem, st, W, (unsigned)m, (unsigned)F, X, n, Z, per);
+    DBK_LAUNCH_OK();
+}
+
+// ---------------------------------------------------------------------------------------------
 // filter gradient on the matrix cores (float32, filters of up to 32 taps, bulk sizes)
 // ---------------------------------------------------------------------------------------------
 // dW (4m x F) = H^T (4m x n) . dZ (n x F), H the one-hot windows: row 4j + k of H^T has a 1 at output row i where
@@ -801,6 +916,7 @@ int dbk_corr1ord(dbk_stream_t stream, int dtype, const void* W, size_t m, size_t
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && X && Z, "ValueError: null pointer argument");
+    if (dtype == DBK_F32 && fprop_mfma_takes(m, nfilter, n)) return launch_fprop_mfma(dbk::as_stream(stream), (const float*)W, m, nfilter, X, n, (float*)Z);
     if (dtype == DBK_F32) return launch_fprop<float>(dbk::as_stream(stream), (const float*)W, m, nfilter, X, n, (float*)Z);
     return launch_fprop<double>(dbk::as_stream(stream), (const double*)W, m, nfilter, X, n, (double*)Z);
 }

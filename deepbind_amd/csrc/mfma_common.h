@@ -2,6 +2,8 @@
 // v_mfma_f32_32x32x16_bf16 and the exact split of a float32 number into three bf16 numbers.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstddef>
 
 namespace dbk_mfma {
 
@@ -27,6 +29,21 @@ __device__ __forceinline__ void split3(float w, unsigned& lo, unsigned& mid, uns
 __device__ __forceinline__ f32x16_t mfma_bf16(const uint4& a, const uint4& b, const f32x16_t& c)
 {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// Four bytes of X at offset o (any alignment); bytes past the end read as 254, "nothing".
+__device__ __forceinline__ unsigned load_letters4(const uint8_t* __restrict__ X, size_t N, size_t o)
+{
+    unsigned v;
+    if (o + 4 <= N) {
+        __builtin_memcpy(&v, X + o, 4);
+    } else {
+        v = 0xfefefefeu;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (o + t < N) v = (v & ~(0xffu << (8 * t))) | ((unsigned)X[o + t] << (8 * t));
+    }
+    return v;
 }
 
 }  // namespace dbk_mfma

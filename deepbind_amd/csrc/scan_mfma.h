@@ -56,21 +56,6 @@ __device__ __forceinline__ unsigned ballots_to_lanes(unsigned v, const unsigned 
     return v;
 }
 
-// Four bytes of X at offset o (any alignment); bytes past the end read as 254, "nothing".
-__device__ __forceinline__ unsigned load_letters4(const uint8_t* __restrict__ X, size_t N, size_t o)
-{
-    unsigned v;
-    if (o + 4 <= N) {
-        __builtin_memcpy(&v, X + o, 4);
-    } else {
-        v = 0xfefefefeu;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (o + t < N) v = (v & ~(0xffu << (8 * t))) | ((unsigned)X[o + t] << (8 * t));
-    }
-    return v;
-}
-
 // One block of 32 rows as the wave walks its regions: where its one-hot letters lie, and what the pooling needs to know.
 struct mfma_block {
     const uint4* hot;         // the block's first position in the chunk's one-hot table

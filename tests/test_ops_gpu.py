@@ -48,6 +48,25 @@ def test_corr1ord_bit_exact(ks, N, m, F):
     assert np.array_equal(host(Z), Zr)
 
 
+@pytest.mark.parametrize("N,m,F", [(300000, 24, 128), (600001, 11, 70), (1100000, 32, 32)])
+def test_corr1ord_bulk_sizes_on_the_matrix_cores(ks, N, m, F):
+    """From 2^25 map values on, float32 maps come from the matrix-core kernel: the same sums in another order, so the
+    comparison is to round-off; rows past N - m + 1 stay untouched, codes 254 / 255 are in the input."""
+    rng = np.random.default_rng(N + m + F)
+    X = random_codes(rng, N, 0.05, 0.03)
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
+    Zr = np.full((N, F), 5.0, np.float64)
+    orc.corr1ord(W.astype(np.float64), X, Zr)
+    Z = dev(np.full((N, F), 5.0, np.float32))
+    ks.corr1ord(dev(W), dev(X.reshape(-1, 1)), Z, 4)
+    got = host(Z)
+    assert np.all(got[N - m + 1:] == 5.0)
+    assert_close(got[: N - m + 1], Zr[: N - m + 1], ACT, "map")
+    Z2 = dev(np.full((N, F), 5.0, np.float32))
+    ks.corr1ord(dev(W), dev(X.reshape(-1, 1)), Z2, 4)
+    assert np.array_equal(host(Z2), got)
+
+
 def test_corr1ord_float64_and_short_input(ks):
     rng = np.random.default_rng(1)
     X = random_codes(rng, 400, 0.1)
