@@ -238,20 +238,11 @@ __device__ __forceinline__ void scanpool_fprop_mfma_body(const wg_t wg, const fl
         }
     };
 
-    // the next block's matrix instructions are issued before a block's pooling, so that the two overlap; the two
-    // accumulators change roles from block to block
-    mfma_block cur = next_block();
-    f32x16_t acc0 = scan_block(cur), acc1;
-    while (cur.valid) {
-        mfma_block nxt = next_block();
-        acc1 = scan_block(nxt);
-        pool_block(cur, acc0);
-        cur = nxt;
-        if (!cur.valid) break;
-        nxt = next_block();
-        acc0 = scan_block(nxt);
-        pool_block(cur, acc1);
-        cur = nxt;
+    // (Matrix and vector instructions do not overlap on a SIMD: issuing the next block's products before this block's
+    // pooling gains nothing, so the blocks are simply taken one after the other; other waves fill the LDS latency.)
+    for (mfma_block cur = next_block(); cur.valid; cur = next_block()) {
+        const f32x16_t acc = scan_block(cur);
+        pool_block(cur, acc);
     }
 }
 
