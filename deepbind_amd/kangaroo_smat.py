@@ -159,8 +159,10 @@ def activity_words(X, W):
 def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=None, out=None):
     """pool(relu(corr1ord(W, X) + b)) per region without storing the (N x P) map.
     Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only.
-    path: "auto" lets the library choose; "general" / "wide" / "kmer" force the general path (which picks its
-    kernel by size), its many-regions kernel (17-24 taps) or the table kernel; "kmer_static" is the table kernel
+    path: "auto" lets the library choose; "general" / "mfma" / "wide" / "kmer" force the general path (which picks its
+    kernel by size), its matrix-core kernel for many regions (filters of up to 32 taps; sums in another order than
+    the lookup kernels', equal to round-off), the four-filters-per-lane lookup kernel (9-24 taps; the bits of the
+    one-filter-per-lane kernel) or the table kernel; "kmer_static" is the table kernel
     with the scratch buffer that is built into the library (no allocation inside the call; at most 64 MiB of
     sequence bytes; calls that overlap on one GPU must not use it together).
     out (optional): (pooled, argmax|None) tensors to write into instead of new ones, so that the call allocates nothing.

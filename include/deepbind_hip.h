@@ -48,6 +48,8 @@ int dbk_sync(dbk_stream_t stream);
 /* Z[i,f] = sum_{j<m} w(j, X[i+j], f) for i < n, where w = W[(C*j+k)*F+f] for k<C, 0 for k==254,
  * and the channel mean for any other code (255 = N / padding). n = number of outputs written
  * (N-m+1); rows >= n of Z are left untouched. W is (C*m, F), X has n+m-1 bytes, Z is (>=n, F).
+ * The taps are added in ascending order (the reference's bits) except for float32 maps of 2^25 values or more, which
+ * the matrix cores compute (filters of up to 32 taps, at least 32 filters): the same sums in another order.
  * reference: launch_corr1ord, kangaroo/kangaroo_smat/kangaroo_smat.cpp:43-46, corr1ord.cu:136-148 */
 int dbk_corr1ord(dbk_stream_t stream, int dtype,
                  const void* W, size_t m, size_t nfilter,
@@ -55,7 +57,8 @@ int dbk_corr1ord(dbk_stream_t stream, int dtype,
                  void* Z);
 
 /* dW[(C*j+k),f] += sum_{i<n} dZ[i,f] * [X[i+j]==k]; N/pad codes add dZ/C to all C rows, 254 nothing.
- * Deterministic: per-workgroup private accumulators and a fixed-order reduction, no float atomics.
+ * Deterministic: per-workgroup private accumulators and a fixed-order reduction, no float atomics (from 4 M
+ * float32 gradient values on the matrix cores form the partial sums: another fixed order).
  * reference: launch_corr1ord_bprop_W, kangaroo_smat.cpp:48-51, corr1ord_bprop.cu:97-108 */
 int dbk_corr1ord_bprop_W(dbk_stream_t stream, int dtype,
                          void* dW, size_t m, size_t nfilter,
@@ -135,18 +138,18 @@ int dbk_scanpool_fprop_general(dbk_stream_t stream,
                                const uint32_t* regions, size_t nregion, int ptype,
                                float* pooled, uint32_t* argmax, uint64_t* act);
 
-/* Same contract through the general path's kernel for many regions regardless of problem size: four filters
- * per lane and one wave per region, for filters of 9 to 24 taps (NotImplementedError otherwise).
- * dbk_scanpool_fprop_general picks it once regions x filter tiles reach 512, where the one-filter-per-lane kernel
- * is bound by the rate of its 4-byte LDS reads. Per position the taps are added in the same order, so maxima,
- * argmax and activity masks are the same bits; averages add the same values in another order. */
+/* Same contract through the four-filters-per-lane lookup kernel regardless of problem size: one wave per region,
+ * filters of 9 to 24 taps (NotImplementedError otherwise). Per position the taps are added in the order of the
+ * one-filter-per-lane kernel, so maxima, argmax and activity masks are the same bits; averages add the same values in
+ * another order. (For many regions dbk_scanpool_fprop_general picks the matrix-core kernel below, which is faster.) */
 int dbk_scanpool_fprop_wide(dbk_stream_t stream,
                             const float* W, const float* bias, size_t m, size_t nfilter,
                             const uint8_t* X, size_t N,
                             const uint32_t* regions, size_t nregion, int ptype,
                             float* pooled, uint32_t* argmax, uint64_t* act);
 
-/* Same contract through the matrix-core kernel regardless of problem size, for filters of up to 32 taps
+/* Same contract through the matrix-core kernel regardless of problem size (dbk_scanpool_fprop_general picks it once
+ * regions x filter tiles reach 512, for filters of 9 to 32 taps), for filters of up to 32 taps
  * (NotImplementedError otherwise): the scan as a product of the windows' one-hot letters with W, each float32
  * weight entering as three bf16 pieces that add up to it exactly, accumulated in float32 by
  * v_mfma_f32_32x32x16_bf16. The sums are those of the lookup kernels in another order: results agree with them

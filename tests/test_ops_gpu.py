@@ -319,20 +319,24 @@ def test_scanpool_fprop_matrix_core_kernel(ks, ptype, B, lo, hi, m, F):
     assert np.array_equal(host(P), host(P2))
 
 
-def test_scanpool_regions_past_the_end_and_gaps(ks):
-    """Arbitrary (non-packed) regions, including rows the scan does not define (relu(bias) there)."""
+@pytest.mark.parametrize("path", ["auto", "mfma"])
+def test_scanpool_regions_past_the_end_and_gaps(ks, path):
+    """Arbitrary (non-packed) regions, including rows the scan does not define (relu(bias) there), regions that
+    overlap, a region longer than the matrix-core kernel's chunk of 192 rows and one of exactly 32 rows."""
     rng = np.random.default_rng(77)
-    m, F, N = 8, 20, 120
+    m, F, N = 8, 20, 520
     X = random_codes(rng, N, 0.1)
     W = rng.standard_normal((4 * m, F)).astype(np.float32)
     b = rng.standard_normal((1, F)).astype(np.float32)
-    R = np.array([[0, 10], [50, 51], [30, 90], [100, 120], [5, 6]], np.uint32)
+    R = np.array([[0, 10], [50, 51], [30, 90], [100, 120], [5, 6], [120, 520], [200, 232], [500, 520], [64, 257]], np.uint32)
     for ptype in ("max", "avg", "all"):
-        A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
-        P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=True)
+        A, Pr, Ir = _chain_oracle(W.astype(np.float64), b.astype(np.float64), X, R, ptype)
+        P, I = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), ptype, want_argmax=True, path=path)
         assert_close(host(P), Pr, ACT, ptype)
         if Ir is not None:
-            assert np.array_equal(host(I), Ir)
+            got = host(I)
+            same = got == Ir
+            assert np.all(np.abs(A.ravel()[got[~same]] - A.ravel()[Ir[~same]]) <= ACT * np.abs(A).max())
 
 
 @pytest.mark.parametrize("ptype", ["max", "avg", "all"])
