@@ -756,9 +756,12 @@ __global__ __launch_bounds__(256) void corr1ord_bprop_W_mfma_kernel(float* __res
             }                                                                                             \
             if (any_n) {                                                                                  \
                 _Pragma("unroll") for (int b = 0; b < MB; ++b) {                                          \
-                    uint4 A = ones[(VN[(2 * ks + b) >> 2] >> (8 * ((2 * ks + b) & 3))) & 0xffu];          \
-                    A.x &= 0x3e803e80u; A.y &= 0x3e803e80u; A.z &= 0x3e803e80u; A.w &= 0x3e803e80u;       \
-                    _Pragma("unroll") for (int q = 0; q < 3; ++q) acc[b] = mfma_bf16(A, B[q], acc[b]);    \
+                    const unsigned bits = (VN[(2 * ks + b) >> 2] >> (8 * ((2 * ks + b) & 3))) & 0xffu;    \
+                    if (__ballot(bits != 0u) != 0ull) {           /* some lane of the wave has one in these rows and taps */ \
+                        uint4 A = ones[bits];                                                             \
+                        A.x &= 0x3e803e80u; A.y &= 0x3e803e80u; A.z &= 0x3e803e80u; A.w &= 0x3e803e80u;   \
+                        _Pragma("unroll") for (int q = 0; q < 3; ++q) acc[b] = mfma_bf16(A, B[q], acc[b]); \
+                    }                                                                                     \
                 }                                                                                         \
             }                                                                                             \
         }                                                                                                 \
