@@ -862,6 +862,181 @@ inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, 
     DBK_LAUNCH_OK();
 }
 
+// ---------------------------------------------------------------------------------------------
+// input gradient on the matrix cores (float32, filters of up to 32 taps, bulk sizes)
+// ---------------------------------------------------------------------------------------------
+// Y (rows x 4m) = dZ (rows x F) . W^T (F x 4m), then dX[i, c] += sum_k Y[i - k, 4k + c]. Both operands are float32
+// data, so both enter as three bf16 pieces and six of the nine piece products are formed (hi.hi, hi.mid, mid.hi,
+// mid.mid, hi.lo, lo.hi; the three left out are below 2^-24 of the result), accumulated in float32.
+// A workgroup takes 512 output rows and 128 filters (the launcher issues one launch per 128 filters: dX accumulates),
+// wave b of it the taps 8b .. 8b + 7 (32 columns of Y; W's pieces for them stay in registers, 96 registers). A
+// block of 32 rows of dZ is read by the whole workgroup as whole 512-byte row segments and staged in LDS (the next
+// block's rows are on their way while this one is multiplied and go to LDS between the block's two barriers: a lane reading its own row from memory touches 32
+// cache lines per instruction, and the tag rate of the CU's cache then sets the pace); every wave reads the same
+// staged pieces (every value is split once, by the thread that loaded it: the planes hold bf16), the 32 x 4m tile of Y goes to LDS, and 128
+// threads add up the taps of their (row, letter) in ascending order, reaching into the previous block's tile for
+// rows before the block (the first block of a workgroup recomputes its predecessor's last rows instead of sharing
+// them). Deterministic: one writer per element, fixed orders.
+constexpr unsigned GX_ROWS = 512;                                  // output rows per workgroup
+constexpr unsigned GX_FILTERS = 128;                               // filters per launch: eight k-steps of 16
+constexpr unsigned GX_ZS = GX_FILTERS + 8;                         // row stride of a staged plane in bf16: 68 words = 4 mod 32, so that the 32 rows' 16-byte reads spread over the banks
+
+template <int MB, bool WHOLE>
+__global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* __restrict__ dX, size_t n, const float* __restrict__ W,
+                                                                        unsigned m, unsigned F, unsigned f0, const float* __restrict__ dZ)
+{
+    using namespace dbk_mfma;
+    constexpr int YS = 32 * MB + 4;                                // row stride of a tile of Y: 4 mod 32, so that the adders' reads spread over the banks
+    constexpr int NT = 64 * MB, PER = (32 * (GX_FILTERS / 4) + NT - 1) / NT;   // threads; 16-byte pieces of a dZ tile per thread
+    __shared__ float Y[2][32][YS];
+    __shared__ __align__(16) unsigned short Zt[3][32][GX_ZS];     // the block's rows of dZ (this launch's filters) as three planes of bf16 pieces (lo, mid, hi)
+    const unsigned lane = threadIdx.x & 63, nb = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const unsigned col = lane & 31, g = lane >> 5;
+    // ---- W's rows 32 nb + col (tap 8 nb + col / 4, letter col % 4), filters f0 + 16 ks + 8g .. + 7, in three pieces
+    uint4 B[8][3];
+    {
+        const unsigned wrow = 32u * nb + col;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            unsigned pc[3][8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const unsigned f = f0 + 16u * ks + 8u * g + t;
+                const float w = (wrow < 4u * m && f < F) ? W[(size_t)wrow * F + f] : 0.0f;
+                split3(w, pc[0][t], pc[1][t], pc[2][t]);
+            }
+#pragma unroll
+            for (int q = 0; q < 3; ++q)
+                B[ks][q] = make_uint4(pack_upper_halves(pc[q][0], pc[q][1]), pack_upper_halves(pc[q][2], pc[q][3]),
+                                      pack_upper_halves(pc[q][4], pc[q][5]), pack_upper_halves(pc[q][6], pc[q][7]));
+        }
+    }
+    const size_t o0 = (size_t)blockIdx.x * GX_ROWS, o1 = o0 + GX_ROWS < n ? o0 + GX_ROWS : n;
+    // A block's rows of dZ, requested by the whole workgroup as 16-byte pieces in row order (a wave reads whole
+    // 512-byte row segments); rows past the end and filters past F count as zero.
+    float4 piece[PER];
+    auto request = [&](size_t i0_) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const unsigned e = threadIdx.x + j * NT, r = e / (GX_FILTERS / 4), c4 = e % (GX_FILTERS / 4);
+            const size_t row = i0_ + r;
+            float4 p = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (e < 32 * (GX_FILTERS / 4) && row < n) {
+                const float* src = dZ + row * F + f0 + 4u * c4;
+                if (WHOLE) {
+                    p = *reinterpret_cast<const float4*>(src);
+                } else {
+                    const unsigned f = f0 + 4u * c4;
+                    p.x = f < F ? src[0] : 0.0f; p.y = f + 1 < F ? src[1] : 0.0f; p.z = f + 2 < F ? src[2] : 0.0f; p.w = f + 3 < F ? src[3] : 0.0f;
+                }
+            }
+            piece[j] = p;
+        }
+    };
+    // every value is split once, by the thread that loaded it: four values' pieces are 8 bytes per plane
+    auto deposit = [&]() {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const unsigned e = threadIdx.x + j * NT, r = e / (GX_FILTERS / 4), c4 = e % (GX_FILTERS / 4);
+            if (e < 32 * (GX_FILTERS / 4)) {
+                const float v[4] = { piece[j].x, piece[j].y, piece[j].z, piece[j].w };
+                unsigned pc[3][4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) split3(v[t], pc[0][t], pc[1][t], pc[2][t]);
+#pragma unroll
+                for (int q = 0; q < 3; ++q)
+                    *reinterpret_cast<uint2*>(&Zt[q][r][4 * c4]) = make_uint2(pack_upper_halves(pc[q][0], pc[q][1]), pack_upper_halves(pc[q][2], pc[q][3]));
+            }
+        }
+    };
+    unsigned slot = 0u;
+    size_t i0 = o0 >= 32 ? o0 - 32 : 0;
+    request(i0);
+    deposit();
+    __syncthreads();
+    for (; i0 < o1; i0 += 32, slot ^= 1u) {
+        // ---- the next block's rows and this block's rows of dX start their way; Y tile of rows i0 .. i0 + 31 from the staged pieces
+        const bool more = i0 + 32 < o1;
+        if (more) request(i0 + 32);
+        float old[2] = { 0.0f, 0.0f };
+        if (i0 >= o0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const unsigned t = threadIdx.x + h * NT;
+                if (t < 128 && (h == 0 || NT < 128) && i0 + (t >> 2) < o1) old[h] = dX[(i0 + (t >> 2)) * 4 + (t & 3u)];
+            }
+        }
+        f32x16_t acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+        // this lane supplies row i0 + col: its eight values of a k-step are 16 bytes of each plane
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            uint4 A[3];
+#pragma unroll
+            for (int q = 0; q < 3; ++q) A[q] = *reinterpret_cast<const uint4*>(&Zt[q][col][16 * ks + 8 * g]);
+            // pieces: 0 = lo, 1 = mid, 2 = hi; the small products first
+            acc = mfma_bf16(A[0], B[ks][2], acc);
+            acc = mfma_bf16(A[2], B[ks][0], acc);
+            acc = mfma_bf16(A[1], B[ks][1], acc);
+            acc = mfma_bf16(A[1], B[ks][2], acc);
+            acc = mfma_bf16(A[2], B[ks][1], acc);
+            acc = mfma_bf16(A[2], B[ks][2], acc);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) Y[slot][(i & 3) + 8 * (i >> 2) + 4 * g][32 * nb + col] = acc[i];
+        __syncthreads();                                           // the tile is complete; nobody reads the staged pieces any more
+        if (more) deposit();
+        if (i0 >= o0) {
+            // ---- dX rows i0 .. i0 + 31: taps in ascending order, rows before the block from the previous tile
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const unsigned t = threadIdx.x + h * NT;
+                if (!(t < 128 && (h == 0 || NT < 128))) continue;
+                const unsigned r = t >> 2, c = t & 3u;
+                const size_t i = i0 + r;
+                if (i < o1) {
+                    // all reads first (rows before the block come from the previous tile; rows before the first one count
+                    // as zero), then the sum in tap order
+                    float y[8 * MB];
+#pragma unroll
+                    for (int k = 0; k < 8 * MB; ++k) {
+                        const unsigned kk = (unsigned)k < m ? (unsigned)k : 0u;
+                        const float* tile = kk <= r ? &Y[slot][r - kk][0] : &Y[slot ^ 1u][32 + r - kk][0];
+                        y[k] = tile[4 * kk + c];
+                    }
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 8 * MB; ++k) sum += ((unsigned)k < m && i >= (size_t)k) ? y[k] : 0.0f;
+                    dX[i * 4 + c] = old[h] + sum;
+                }
+            }
+        }
+        __syncthreads();                                           // the next block's pieces are staged; this tile's readers are done
+    }
+}
+
+inline bool bprop_X_mfma_takes(size_t m, size_t F, size_t n) { return m <= 32 && F >= 64 && n * F >= ((size_t)1 << 22) && n >= 4096; }
+
+inline int launch_bprop_X_mfma(hipStream_t st, float* dX, size_t n, const float* W, size_t m, size_t F, const float* dZ)
+{
+    const unsigned gx = (unsigned)dbk::divup(n, GX_ROWS), mb = (unsigned)((4 * m + 31) / 32);
+    for (size_t f0 = 0; f0 < F; f0 += GX_FILTERS) {
+        const bool whole = F % 4 == 0 && f0 + GX_FILTERS <= F;
+#define DBK_GO(MB_)                                                                                                   \
+        if (whole) hipLaunchKernelGGL((corr1ord_bprop_X_mfma_kernel<MB_, true>), dim3(gx), dim3(64 * MB_), 0, st, dX, n, W, (unsigned)m, (unsigned)F, (unsigned)f0, dZ); \
+        else hipLaunchKernelGGL((corr1ord_bprop_X_mfma_kernel<MB_, false>), dim3(gx), dim3(64 * MB_), 0, st, dX, n, W, (unsigned)m, (unsigned)F, (unsigned)f0, dZ);
+        switch (mb) {
+        case 1:  DBK_GO(1) break;
+        case 2:  DBK_GO(2) break;
+        case 3:  DBK_GO(3) break;
+        default: DBK_GO(4) break;
+        }
+#undef DBK_GO
+    }
+    DBK_LAUNCH_OK();
+}
+
 inline int launch_bprop_X_ring(hipStream_t st, float* dX, size_t n, const float* W, size_t m, size_t F, const float* dZ)
 {
     if (m <= 8) {
@@ -946,6 +1121,7 @@ int dbk_corr1ord_bprop_X(dbk_stream_t stream, int dtype, void* dX, size_t n, siz
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(dX && W && dZ, "ValueError: null pointer argument");
+    if (dtype == DBK_F32 && bprop_X_mfma_takes(m, nfilter, n)) return launch_bprop_X_mfma(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     if (dtype == DBK_F32 && m <= 24) return launch_bprop_X_ring(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     if (dtype == DBK_F32) return launch_bprop_X<float>(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     return launch_bprop_X<double>(dbk::as_stream(stream), (double*)dX, n, (const double*)W, m, nfilter, (const double*)dZ);

@@ -66,7 +66,8 @@ int dbk_corr1ord_bprop_W(dbk_stream_t stream, int dtype,
                          const void* dZ);
 
 /* dX[i,c] += sum_f sum_{k<m, k<=i} dZ[i-k,f] * W[(C*k+c),f] for i < n; dX is (n, C), dZ is (n, F).
- * Computed on the device (the reference copies to the host and loops there).
+ * Computed on the device (the reference copies to the host and loops there); from 4 M float32 gradient values on as a
+ * product on the matrix cores (both operands in exact bf16 pieces): the same sums in another order.
  * reference: launch_corr1ord_bprop_X, kangaroo_smat.cpp:53-56, corr1ord_bprop.cu:167-224 */
 int dbk_corr1ord_bprop_X(dbk_stream_t stream, int dtype,
                          void* dX, size_t n, size_t nchannel,

@@ -121,10 +121,14 @@ def test_corr1ord_bprop_W(ks, N, m, F, dense, dtype):
 
 @pytest.mark.parametrize("n,m,F,dtype", [(300, 24, 48, np.float32), (1000, 11, 130, np.float32), (97, 5, 64, np.float32),
                                          (5000, 24, 256, np.float32), (3, 16, 7, np.float32), (50, 30, 20, np.float32),
-                                         (400, 24, 70, np.float64)])
+                                         (400, 24, 70, np.float64),
+                                         (40000, 24, 256, np.float32), (70001, 11, 130, np.float32), (66000, 32, 64, np.float32),
+                                         (33003, 5, 200, np.float32)])
 def test_corr1ord_bprop_X(ks, n, m, F, dtype):
     """Row counts around the per-wave block of 96 rows, several filter tiles, fewer rows than taps, the
-    any-length kernel (m = 30) and float64; accumulates into dX and is bit-stable."""
+    any-length kernel (m = 30) and float64; accumulates into dX and is bit-stable. From 4 M gradient values on
+    (float32, at least 64 filters) the matrix-core kernel: one to four blocks of taps, filter counts that are no
+    multiple of 128 or of 4, row counts that are no multiple of a workgroup's 1024 rows."""
     rng = np.random.default_rng(5 + n)
     W = (rng.standard_normal((4 * m, F)) * 0.1).astype(dtype)
     dZ = rng.standard_normal((n, F)).astype(dtype)
