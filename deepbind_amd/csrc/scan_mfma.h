@@ -56,6 +56,14 @@ __device__ __forceinline__ unsigned ballots_to_lanes(unsigned v, const unsigned 
     return v;
 }
 
+// max(a, b) as one instruction (the compiler's fmaxf first quiets a possible signalling NaN with an instruction of its own)
+__device__ __forceinline__ float plain_max(float a, float b)
+{
+    float r;
+    asm("v_max_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 // One block of 32 rows as the wave walks its regions: where its one-hot letters lie, and what the pooling needs to know.
 struct mfma_block {
     const uint4* hot;         // the block's first position in the chunk's one-hot table
@@ -217,7 +225,7 @@ __device__ __forceinline__ void scanpool_fprop_mfma_body(const wg_t wg, const fl
         if (PT != DBK_PT_MAX) {
             float part = 16.0f * bf;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) part += __builtin_fmaxf(z[i], nb);
+            for (int i = 0; i < 16; ++i) part += plain_max(z[i], nb);
             sum += part;
         }
         if (rows <= MFMA_ROWS) {
