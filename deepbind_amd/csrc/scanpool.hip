@@ -1030,6 +1030,18 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
         else hipLaunchKernelGGL(reduce_slabs_kernel, dim3(dbk::ew_grid(stride)), dim3(256), 0, st, dW, dbias, (const float*)slabs, nW, F, gx, overwrite);
         DBK_LAUNCH_OK();
     }
+    // Average pooling without the forward pass's activity masks: the matrix-core forward writes them again (into the
+    // stream's second scratch buffer, with its pooled values beside them), and the bit-count kernel takes them from
+    // there; less than half the time of recomputing the map through the letter table.
+    if (PT != DBK_PT_MAX && !act && !dbk::deferred() && mfma_pays(m, ftiles, P)) {
+        const size_t mask_bytes = N * ftiles * sizeof(unsigned long long), pooled_bytes = P * F * 2 * sizeof(float);
+        unsigned char* scratch = (unsigned char*)dbk::workspace(mask_bytes + pooled_bytes, st, 1);
+        DBK_CHECK(scratch != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", mask_bytes + pooled_bytes, dbk::workspace_error());
+        unsigned long long* masks = reinterpret_cast<unsigned long long*>(scratch);
+        const int rc = launch_fprop_mfma<PT>(st, ftiles, W, bias, m, F, X, N, R, P, reinterpret_cast<float*>(scratch + mask_bytes), nullptr, masks);
+        if (rc) return rc;
+        act = masks;
+    }
     // with max+avg pooling the dense half carries the maxima along
     const bool max_bits = PT == DBK_PT_MAX && bits_takes_max(N, P);
     const unsigned gxs = PT == DBK_PT_MAX ? (max_bits ? bits_grid_x(ftiles, P) : sparse_grid_x(ftiles, P)) : 0u;

@@ -474,8 +474,8 @@ def test_scanpool_bprop_with_activity_masks_equals_recomputation(ks, ptype, B, l
 @pytest.mark.parametrize("B,lo,hi,m,F", [(600, 0, 70, 24, 70), (520, 30, 45, 16, 16), (530, 1, 150, 7, 40), (130, 100, 260, 24, 300)])
 def test_scanpool_bprop_many_regions_kernel(ks, ptype, B, lo, hi, m, F):
     """From 512 (region, filter tile) items on, the mask-driven dense backward deals whole regions to waves (no
-    barrier per region chunk). Its partial sums are other partial sums than the recomputing kernel's, so the two
-    agree to round-off, not bit for bit; it is checked against the float64 chain too, must be deterministic, and
+    barrier per region chunk). A call without masks recomputes them (a second forward pass on the matrix cores from
+    9 taps on, the map through the letter table below) and agrees with the call given masks to round-off; it is checked against the float64 chain too, must be deterministic, and
     must leave alone what lies outside its output. Regions of 0 to 260 rows (several 64-row rounds per region), all
     three tap tiers, code 254 and N present."""
     rng, W, b, X, R = _fused_case(7 * B + F, B, lo, hi, m, F, p254=0.02)
