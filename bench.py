@@ -162,7 +162,7 @@ def profiled_kernels(tag):
     return None
 
 
-def train_throughput(steps=300, warmup=30, cpu=True):
+def train_throughput(steps=3000, warmup=300, cpu=True):
     """Whole train steps (forward + backward + Nesterov update) per second on the three training configurations,
     fused mode: each step issued natively by one library call (the top-level figures; the calibration batch's
     architecture groups share every launch) and as one captured HIP graph per step ("graphed").

@@ -156,7 +156,8 @@ __device__ __forceinline__ void scan_block(const float* __restrict__ wt, const u
 
 // All workgroups of the grid meet here once. Accesses of many workgroups to ONE address at device scope are served
 // one after the other (measured: ~50 ns per read-modify-write, 6.5 us for a counter that 128 workgroups increment;
-// ~3 us when every workgroup reads every other's flag), so no word is shared more than it must be: each workgroup
+// 2-4 us per poll when every workgroup reads every other's flag, in lines of their own or side by side), so no word is
+// shared more than it must be: each workgroup
 // raises a flag in a 64-byte line of its own - the number of this launch, one more than the number the workspace
 // held when the kernel started; workgroup 0 alone reads all the flags (two per lane of its first wave) and, when
 // they all show the number, writes it to the "go" word; every other workgroup polls that one word with one lane.
@@ -170,7 +171,7 @@ __device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, uns
     if (threadIdx.x < 64) {
         const unsigned lane = threadIdx.x;
         if (lane == 0) {
-            __threadfence();                                       // this workgroup's shares are visible device-wide
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");     // this workgroup's shares are visible device-wide
             if (dbg) dbg[0] = (float)(wall_clock64() & 0xffffff);
             __hip_atomic_store(&flags[blockIdx.x * FLAG_STRIDE], launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -198,13 +199,56 @@ __device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, uns
             unsigned status = __hip_atomic_load(&sync[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (!done) { atomicExch(&sync[1], 1u); status = 1u; }
             if (dbg) { dbg[2] = (float)(wall_clock64() & 0xffffff); dbg[3] = (float)tries; }
-            __threadfence();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");     // the other workgroups' shares are read from memory, not from stale lines
             verdict = status;
         }
     }
     __syncthreads();
     return verdict;
 }
+
+// Quotient of small numbers without the integer division sequence: for e < 2^20 and any divisor, (e + 0.5) / d is at
+// least 0.5 / d away from a whole number while the reciprocal's and the product's rounding move it by less than
+// e / d * 2^-21, so truncating gives floor(e / d) exactly.
+struct small_div {
+    float inv; unsigned d;
+    __device__ __forceinline__ explicit small_div(unsigned d_) : inv(__builtin_amdgcn_rcpf((float)d_)), d(d_) {}
+    __device__ __forceinline__ unsigned quot(unsigned e) const
+    {
+        if (__builtin_constant_p(d) && d == 1u) return e;
+        return (unsigned)(((float)e + 0.5f) * inv);
+    }
+    __device__ __forceinline__ unsigned rem(unsigned e, unsigned q) const { return e - q * d; }
+};
+
+// Orders a wave's own LDS traffic: what its lanes stored before is what its lanes read after (the LDS serves a wave's
+// instructions in order; the fences keep the compiler from moving them and wait for the counter).
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// Sum over the wave's 64 lanes, the same bits in every lane: within a row of 16 lanes by data-parallel moves (lane ^ 1,
+// lane ^ 2, then the mirrored lane of the eight and of the row: it lies in the other half, and all lanes of a half
+// hold the same sum by then), across the rows by two exchanges through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float lane_move(float v) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true)); }
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v += lane_move<0xB1>(v);                                       // quad_perm [1, 0, 3, 2]
+    v += lane_move<0x4E>(v);                                       // quad_perm [2, 3, 0, 1]
+    v += lane_move<0x141>(v);                                      // row_half_mirror
+    v += lane_move<0x140>(v);                                      // row_mirror
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// A share is stored through the cache levels that other workgroups do not see (a relaxed store at device scope), on its
+// way while the workgroup computes the rest: the barrier's release fence then finds little left to write back.
+__device__ __forceinline__ void put_share(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 #ifdef DBK_STEP_PROF
 #define STAMP(i) do { if (threadIdx.x == 0) { const long long now_ = wall_clock64(); if (blockIdx.x == 0) reinterpret_cast<long long*>(a.sync + 3072)[i] = now_; \
@@ -213,12 +257,16 @@ __device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, uns
 #define STAMP(i) do {} while (0)
 #endif
 
-template <int MT>
+// ONE: the shape of a single 16-filter model on a batch of at most MAXG regions (one region per workgroup of 512
+// threads), known when the kernel is compiled: the index arithmetic of the general shape folds away, and with a step
+// this short the instructions a wave issues one after the other are what the step costs.
+template <int MT, bool ONE>
 __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
 {
     extern __shared__ __align__(16) unsigned smem[];
     const bool dense = a.ptype != DBK_PT_MAX, sparse = a.ptype != DBK_PT_AVG;
-    const lds_map L = make_map(MT, a.Fp, a.nmodel, a.kt, a.k, a.h1, (unsigned)a.nparam, a.RC, dense);
+    const unsigned nm = ONE ? 1u : a.nmodel, RC = ONE ? 1u : a.RC, Fp = ONE ? 16u : a.Fp, lgFp = ONE ? 4u : a.lgFp;
+    const lds_map L = make_map(MT, Fp, nm, a.kt, a.k, a.h1, (unsigned)a.nparam, RC, dense);
     float* wt = reinterpret_cast<float*>(smem + L.wt);
     float* Lk = reinterpret_cast<float*>(smem + L.look);
     const float* W1s = Lk + a.off_W1;
@@ -246,40 +294,34 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     float* zs = reinterpret_cast<float*>(smem + L.zs);
     uint8_t* kept = reinterpret_cast<uint8_t*>(smem + L.kept);
 
-    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, NT = blockDim.x, NW = NT >> 6;
-    const unsigned F = a.F, Fp = a.Fp, nm = a.nmodel, k = a.k, kt = a.kt, h1 = a.h1, hidden = a.hidden, m = a.m, RC = a.RC;
+    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, NT = ONE ? (unsigned)NTMAX : blockDim.x, NW = NT >> 6;
+    const unsigned F = a.F, k = a.k, kt = a.kt, h1 = a.h1, hidden = a.hidden, m = a.m;
     const unsigned r0 = blockIdx.x * RC;                           // first region of this workgroup
     const unsigned nreg = r0 < a.nregion ? (a.nregion - r0 < RC ? a.nregion - r0 : RC) : 0u;
     const unsigned kpf = a.ptype == DBK_PT_ALL ? 2u : 1u;          // pooled features per filter
+    const small_div by_nm(nm), by_k(k), by_nmk(nm * k), by_h1(h1), by_kt(kt), by_kf(a.kf), by_nmkf(nm * a.kf);
 
     STAMP(0);
-    // ---------------- everything this workgroup reads from global memory before the barrier, requested in ONE round:
-    // the look-ahead vector P + mrate * mP (gradstep.cu:41-51), its regions' bounds, targets, masks, dropout rates and
-    // the generator position. (Dependent round trips, not arithmetic, are what a step of this size costs.)
-    {
-        constexpr unsigned UN = 4;
-        for (size_t e0 = tid; e0 < a.nparam; e0 += UN * NT) {
-            float vp[UN], vr[UN], vm[UN];
-#pragma unroll
-            for (unsigned u = 0; u < UN; ++u) {
-                const size_t e = e0 + u * NT;
-                const bool in = e < a.nparam;
-                vp[u] = in ? a.P[e] : 0.0f;
-                vr[u] = in ? a.mrate[e] : 0.0f;
-                vm[u] = in ? a.mP[e] : 0.0f;
-            }
-#pragma unroll
-            for (unsigned u = 0; u < UN; ++u)
-                if (e0 + u * NT < a.nparam) Lk[e0 + u * NT] = vp[u] + vr[u] * vm[u];
-        }
-    }
+    // ---------------- everything this workgroup reads from global memory before the barrier, requested in one round:
+    // its regions' bounds, targets, masks, dropout rates, the generator position and the look-ahead vector
+    // P + mrate * mP (gradstep.cu:41-51). (Dependent round trips, not arithmetic, are what a step of this size costs.)
     {
         unsigned ra = 0, rb = 0;
         float y = 0.0f, dr = 0.0f;
         unsigned ym = 1u, c_lo = 0u, c_hi = 0u, tickets = 0u;
+        constexpr unsigned UN = 6;
+        float vp[UN], vr[UN], vm[UN];
+#pragma unroll
+        for (unsigned u = 0; u < UN; ++u) {
+            const size_t e = tid + u * NT;
+            const bool in = e < a.nparam;
+            vp[u] = in ? a.P[e] : 0.0f;
+            vr[u] = in ? a.mrate[e] : 0.0f;
+            vm[u] = in ? a.mP[e] : 0.0f;
+        }
         if (tid < RC && r0 + tid < a.nregion) { ra = a.R[2 * (r0 + tid)]; rb = a.R[2 * (r0 + tid) + 1]; }
-        if (tid < RC * nm && r0 + tid / nm < a.nregion) {
-            const size_t i = (size_t)(r0 + tid / nm) * nm + tid % nm;
+        if (tid < RC * nm && r0 + by_nm.quot(tid) < a.nregion) {
+            const size_t i = (size_t)r0 * nm + tid;
             y = a.Y[i];
             if (a.Ymask) ym = a.Ymask[i];
         }
@@ -288,6 +330,10 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             if (a.counter) { const unsigned long long c = a.counter[0]; c_lo = (unsigned)c; c_hi = (unsigned)(c >> 32); }
             tickets = __hip_atomic_load(&a.sync[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+#pragma unroll
+        for (unsigned u = 0; u < UN; ++u)
+            if (tid + u * NT < a.nparam) Lk[tid + u * NT] = vp[u] + vr[u] * vm[u];
+        for (size_t e = tid + (size_t)UN * NT; e < a.nparam; e += NT) Lk[e] = a.P[e] + a.mrate[e] * a.mP[e];      // a long parameter vector: the rest
         if (tid < RC) {
             unsigned rows = rb > ra ? rb - ra : 0u;
             if (rows > MAXROWS) {                                  // not a shape this kernel takes: flag it, touch nothing of the region
@@ -303,6 +349,10 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             misc[0] = c_lo; misc[1] = c_hi;
             misc[2] = tickets + 1u;                                // this launch's number (see grid_barrier)
         }
+    }
+    for (unsigned e = tid; e < RC * nm * a.kf; e += NT) {          // the shared feature columns follow each model's own inputs
+        const unsigned rl = by_nmkf.quot(e), rest = by_nmkf.rem(e, rl), b = by_kf.quot(rest), j = by_kf.rem(rest, b);
+        H0[(rl * nm + b) * kt + k + j] = (a.feats && rl < nreg) ? a.feats[((size_t)r0 + rl) * a.kf + j] : 0.0f;
     }
     for (unsigned e = tid; e < RC * 5 * LW; e += NT) lmask[e] = 0u;
     if (dense)
@@ -331,7 +381,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         for (unsigned i = 0; i < TXN; ++i) lt[i] = tid + i * NT < RC * TXTB ? letter_at(tid + i * NT) : 254u;
     }
     for (unsigned e = tid; e < MT * Fp; e += NT) {
-        const unsigned t = e / Fp, f = e % Fp;
+        const unsigned t = e >> lgFp, f = e & (Fp - 1u);
         float w0 = 0.0f, w1 = 0.0f, w2 = 0.0f, w3 = 0.0f;
         if (t < m && f < F) {
             const float* w = Lk + a.off_Wc + (size_t)(4 * t) * F + f;
@@ -350,8 +400,8 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     {
         const size_t ncol = (size_t)k * nm;
         const unsigned long long off = (unsigned long long)misc[1] << 32 | misc[0];
-        for (unsigned e = tid; e < RC * nm * k; e += NT) {
-            const unsigned rl = e / (nm * k), col = e % (nm * k), b = col / k;
+        for (unsigned e = NT - 1u - tid; e < RC * nm * k; e += NT) {      // (the last threads first: the first ones build the table)
+            const unsigned rl = by_nmk.quot(e), col = by_nmk.rem(e, rl), b = by_k.quot(col);
             const size_t rr = (size_t)r0 + rl;
             bool kp = true;
             if (rl < nreg && a.rate) kp = dbk_rng::uniform_at(a.seed, off, (a.revcomp ? (rr >> 1) : rr) * ncol + col) >= rates[b];
@@ -369,18 +419,19 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
 
     STAMP(2);
     // ---------------- forward: scan + bias + ReLU + pooling, region by region, all four waves on one region
-    const unsigned PG = 64u >> a.lgFp, NG = NW * PG;               // position groups per wave / per workgroup
-    const unsigned f = lane & (Fp - 1), gidx = wave * PG + (lane >> a.lgFp);
+    const unsigned PG = 64u >> lgFp, NG = NW * PG;               // position groups per wave / per workgroup
+    const unsigned lgNG4 = (NT == NTMAX ? 3u : 2u) + 6u - lgFp + 2u;                            // log2(4 * NG): NT is 256 or 512
+    const unsigned f = lane & (Fp - 1), gidx = wave * PG + (lane >> lgFp);
     const float bf = f < F ? Lk[a.off_bc + f] : 0.0f;
     const size_t nscan = a.N + 1 >= (size_t)m + 1 ? a.N - m + 1 : 0;
     for (unsigned rl = 0; rl < nreg; ++rl) {
         const unsigned rows = rinfo[2 * rl];
-        const unsigned Bq = 4u * ((rows + 4u * NG - 1u) / (4u * NG));
+        const unsigned Bq = 4u * ((rows + 4u * NG - 1u) >> lgNG4);
         const unsigned start = gidx * Bq;
         float mx = -1.0f, sum = 0.0f;
         unsigned xi = 0xffffffffu;
         if (start < rows)
-            scan_block<MT>(wt, reinterpret_cast<const unsigned*>(text + rl * TXTB), start, Bq, rows, rinfo[2 * rl + 1], nscan, f, a.lgFp, bf,
+            scan_block<MT>(wt, reinterpret_cast<const unsigned*>(text + rl * TXTB), start, Bq, rows, rinfo[2 * rl + 1], nscan, f, lgFp, bf,
                            dense, amask + (rl * Fp + f) * AW, mx, xi, sum);
         // fold the position groups of the wave (lanes f, f + Fp, ...): larger value wins, equal values keep the earlier row
         for (unsigned d = Fp; d < 64u; d <<= 1) {
@@ -396,13 +447,21 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         }
         __syncthreads();
         if (tid < Fp) {
-            float bm = red[tid], bs = red[2 * Fp + tid];
-            unsigned bi = __float_as_uint(red[Fp + tid]);
-            for (unsigned w = 1; w < NW; ++w) {
-                const float vm = red[(w * 3 + 0) * Fp + tid];
-                const unsigned vi = __float_as_uint(red[(w * 3 + 1) * Fp + tid]);
-                if (vm > bm || (vm == bm && vi < bi)) { bm = vm; bi = vi; }
-                bs += red[(w * 3 + 2) * Fp + tid];
+            float vm[NWMAX], vs[NWMAX];
+            unsigned vi[NWMAX];
+#pragma unroll
+            for (unsigned w = 0; w < NWMAX; ++w) {                 // all waves' values requested at once; a wave that is not there never wins and adds 0
+                const bool in = w < NW;
+                vm[w] = in ? red[(w * 3 + 0) * Fp + tid] : -2.0f;
+                vi[w] = in ? __float_as_uint(red[(w * 3 + 1) * Fp + tid]) : 0xffffffffu;
+                vs[w] = in ? red[(w * 3 + 2) * Fp + tid] : 0.0f;
+            }
+            float bm = vm[0], bs = vs[0];
+            unsigned bi = vi[0];
+#pragma unroll
+            for (unsigned w = 1; w < NWMAX; ++w) {
+                if (vm[w] > bm || (vm[w] == bm && vi[w] < bi)) { bm = vm[w]; bi = vi[w]; }
+                bs += vs[w];
             }
             bm = bm > 0.0f ? bm : 0.0f;
             if (bi == 0xffffffffu) bi = 0u;
@@ -415,125 +474,210 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
                 else { out[0] = bm; out[1] = mean; }
             }
         }
-        __syncthreads();
+        if constexpr (!ONE) __syncthreads();                       // (ONE: the wave that wrote the pooled features is the one that goes on with them)
     }
 
     STAMP(3);
     // ---------------- dense head, forward and backward, for this workgroup's rows
     const float inv_n = 1.0f / (float)a.nregion;
-    for (unsigned e = tid; e < RC * nm * k; e += NT) {             // inputs after dropout
-        const unsigned rl = e / (nm * k), col = e % (nm * k), b = col / k, kk = col % k;
-        H0[((size_t)rl * nm + b) * kt + kk] = (rl < nreg && kept[e]) ? PL[e] : 0.0f;
-    }
-    for (unsigned e = tid; e < RC * nm * a.kf; e += NT) {          // the shared feature columns follow each model's own inputs
-        const unsigned rl = e / (nm * a.kf), rest = e % (nm * a.kf), b = rest / a.kf, j = rest % a.kf;
-        H0[((size_t)rl * nm + b) * kt + k + j] = (a.feats && rl < nreg) ? a.feats[((size_t)r0 + rl) * a.kf + j] : 0.0f;
-    }
-    __syncthreads();
-    STAMP(8);
-    if (hidden) {
-        for (unsigned e = tid; e < RC * nm * hidden; e += NT) {
-            const unsigned rb = e / hidden, h = e % hidden, b = rb % nm;
-            const float* x = H0 + (size_t)rb * kt;
-            const float* wcol = W1s + (size_t)b * kt * hidden + h;
-            float s = 0.0f;
+    if (RC == 1u) {
+        // A single region: wave b takes model b through the whole head on its own - inputs, hidden layer, prediction,
+        // loss gradient, gradients of the hidden units and of the pooled features - and waits for nothing but its own
+        // LDS traffic (no workgroup barrier between the steps).
+        if (wave < nm) {
+            const unsigned b = ONE ? 0u : wave;
+            const bool live = nreg != 0u;
+            if constexpr (ONE) wave_lds_sync();
+            for (unsigned kk = lane; kk < k; kk += 64) H0[b * kt + kk] = (live && kept[b * k + kk]) ? PL[b * k + kk] : 0.0f;
+            wave_lds_sync();
+            const float* x = H0 + b * kt;
+            float hv = 0.0f, w2 = 0.0f, part = 0.0f;               // lane h: hidden unit h and its output weight
+            if (hidden) {
+                if (lane < hidden) {
+                    const float* wcol = W1s + (size_t)b * kt * hidden + lane;
+                    float sacc = 0.0f;
 #pragma unroll 8
-            for (unsigned kk = 0; kk < kt; ++kk) s += x[kk] * wcol[kk * hidden];
-            s += b1s[b * hidden + h];
-            H1[e] = s > 0.0f ? s : 0.0f;
+                    for (unsigned kk = 0; kk < kt; ++kk) sacc += x[kk] * wcol[kk * hidden];
+                    sacc += b1s[b * hidden + lane];
+                    hv = sacc > 0.0f ? sacc : 0.0f;
+                    w2 = W2s[b * hidden + lane];
+                    H1[b * hidden + lane] = hv;
+                    part += hv * w2;
+                }
+            } else {
+                for (unsigned kk = lane; kk < kt; kk += 64) part += x[kk] * W1s[(size_t)b * kt + kk];
+            }
+            part = wave_sum(part);
+            const float out = part + (hidden ? b2s[b] : b1s[b]);
+            // (the logistic through the hardware's exponential and reciprocal, as the reference's kernels are built: -use_fast_math)
+            const float z = a.loss_kind == 0 ? __builtin_amdgcn_rcpf(1.0f + __expf(-out)) : out;
+            float dA = 0.0f;
+            if (live && Yms[b] != 0u) dA = (z - Ys[b]) * inv_n;
+            if (lane == 0) { zs[b] = z; dAs[b] = dA; }             // (the loss term is formed later, off this wave's path)
+            if (hidden && lane < hidden) D1[b * hidden + lane] = hv > 0.0f ? dA * w2 : 0.0f;
+            wave_lds_sync();
+            // gradient at the pooled features -> what the scan's backward pass needs
+            auto put_pool_grad = [&](unsigned kk, float g) {
+                if (!kept[b * k + kk]) g = 0.0f;
+                const unsigned fl = b * a.nfilter + (kk >> (kpf - 1u));
+                const bool is_avg = a.ptype == DBK_PT_AVG || (a.ptype == DBK_PT_ALL && (kk & 1u));
+                if (is_avg) cavg[fl] = (live && rinfo[0]) ? g / (float)rinfo[0] : 0.0f;
+                else gmax[fl] = (live && PL[b * k + kk] > 0.0f) ? g : 0.0f;
+            };
+            // Up to 32 features: the wave's lanes are (64 / 16 or 64 / 32 groups of hidden units) x features, a lane adds
+            // its group's products (starting at a unit that depends on the feature: neighbouring lanes then read
+            // different LDS banks of the weight rows) and the groups' sums meet in a fixed butterfly.
+            const unsigned lgkP = k <= 16 ? 4u : 5u, hs = hidden >> (6u - lgkP);
+            if (hidden && k <= 32 && (hs << (6u - lgkP)) == hidden && hs >= 2 && (hs & (hs - 1u)) == 0) {
+                const unsigned kk = lane & ((1u << lgkP) - 1u), hq = lane >> lgkP;
+                float g = 0.0f;
+                if (kk < k) {
+                    const float* wrow = W1s + ((size_t)b * kt + kk) * hidden + hq * hs;
+                    const float* drow = D1 + b * hidden + hq * hs;
+#pragma unroll 8
+                    for (unsigned j = 0; j < hs; ++j) {
+                        const unsigned h = (j + kk) & (hs - 1u);
+                        g += drow[h] * wrow[h];
+                    }
+                }
+                for (unsigned d = 1u << lgkP; d < 64u; d <<= 1) g += __shfl_xor(g, (int)d, 64);
+                if (lane < k) put_pool_grad(lane, g);
+            } else {
+                for (unsigned kk = lane; kk < k; kk += 64) {
+                    float g;
+                    if (hidden) {
+                        g = 0.0f;
+                        const float* wrow = W1s + ((size_t)b * kt + kk) * hidden;
+#pragma unroll 8
+                        for (unsigned h = 0; h < hidden; ++h) g += D1[b * hidden + h] * wrow[h];
+                    } else {
+                        g = dA * W1s[(size_t)b * kt + kk];
+                    }
+                    put_pool_grad(kk, g);
+                }
+            }
+        }
+    } else {
+        for (unsigned e = tid; e < RC * nm * k; e += NT) {             // inputs after dropout
+            const unsigned rl = by_nmk.quot(e), col = by_nmk.rem(e, rl), b = by_k.quot(col), kk = by_k.rem(col, b);
+            H0[(rl * nm + b) * kt + kk] = (rl < nreg && kept[e]) ? PL[e] : 0.0f;
         }
         __syncthreads();
-    }
-    STAMP(9);
-    // output pre-activation and prediction of (row, model): one wave per output, a lane per input, summed by a fixed butterfly
-    for (unsigned e = wave; e < RC * nm; e += NW) {
-        const unsigned b = e % nm;
-        float part = 0.0f;
+        STAMP(8);
         if (hidden) {
-            for (unsigned h = lane; h < hidden; h += 64) part += H1[(size_t)e * hidden + h] * W2s[b * hidden + h];
-        } else {
-            for (unsigned kk = lane; kk < kt; kk += 64) part += H0[(size_t)e * kt + kk] * W1s[(size_t)b * kt + kk];
-        }
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
-        if (lane == 0) {
-            const float out = part + (hidden ? b2s[b] : b1s[b]);
-            zs[e] = a.loss_kind == 0 ? 1.0f / (1.0f + expf(-out)) : out;
-        }
-    }
-    __syncthreads();
-    STAMP(10);
-    // loss gradient of (row, model), formed by every thread that needs it; the hidden units' gradients with it
-    for (unsigned e = tid; e < RC * nm * h1; e += NT) {
-        const unsigned rb = e / h1, h = e % h1, rl = rb / nm, b = rb % nm;
-        const size_t rr = (size_t)r0 + rl;
-        float dA = 0.0f, lterm = 0.0f;
-        if (rl < nreg) {
-            const float z = zs[rb], y = Ys[rb];
-            bool use = Yms[rb] != 0u;
-            if (a.revcomp) {                                       // of a (fwd, rev) pair only the larger prediction trains; ties keep the first
-                const float zo = zs[(rl ^ 1u) * nm + b];
-                use = use && ((rr & 1) ? !(zo >= z) : (z >= zo));
-            }
-            if (use) {
-                dA = (z - y) * inv_n;
-                if (h == 0)
-                    lterm = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
-            }
-            if (h == 0) a.Z[rr * nm + b] = z;
-        }
-        if (h == 0) { dAs[rb] = dA; lss[rb] = lterm; }
-        if (hidden) D1[e] = H1[e] > 0.0f ? dA * W2s[b * hidden + h] : 0.0f;
-    }
-    __syncthreads();
-    STAMP(12);
-    for (unsigned e = tid; e < RC * nm * k; e += NT) {             // gradient at the pooled features -> what the scan's backward pass needs
-        const unsigned rl = e / (nm * k), col = e % (nm * k), b = col / k, kk = col % k, rb = rl * nm + b;
-        float g;
-        if (hidden) {
-            g = 0.0f;
-            const float* wrow = W1s + ((size_t)b * kt + kk) * hidden;
+            for (unsigned e = tid; e < RC * nm * hidden; e += NT) {
+                const unsigned rb = by_h1.quot(e), h = by_h1.rem(e, rb), b = by_nm.rem(rb, by_nm.quot(rb));
+                const float* x = H0 + rb * kt;
+                const float* wcol = W1s + (size_t)b * kt * hidden + h;
+                float s = 0.0f;
 #pragma unroll 8
-            for (unsigned h = 0; h < hidden; ++h) g += D1[(size_t)rb * hidden + h] * wrow[h];
-        } else {
-            g = dAs[rb] * W1s[(size_t)b * kt + kk];
+                for (unsigned kk = 0; kk < kt; ++kk) s += x[kk] * wcol[kk * hidden];
+                s += b1s[b * hidden + h];
+                H1[e] = s > 0.0f ? s : 0.0f;
+            }
+            __syncthreads();
         }
-        if (!kept[e]) g = 0.0f;
-        const unsigned fl = b * a.nfilter + kk / kpf;             // filter of the group
-        const bool is_avg = a.ptype == DBK_PT_AVG || (a.ptype == DBK_PT_ALL && (kk & 1u));
-        if (is_avg) cavg[rl * Fp + fl] = (rl < nreg && rinfo[2 * rl]) ? g / (float)rinfo[2 * rl] : 0.0f;
-        else gmax[rl * Fp + fl] = (rl < nreg && PL[e] > 0.0f) ? g : 0.0f;
+        STAMP(9);
+        // output pre-activation and prediction of (row, model): one wave per output, a lane per input, summed by a fixed butterfly
+        for (unsigned e = wave; e < RC * nm; e += NW) {
+            const unsigned b = by_nm.rem(e, by_nm.quot(e));
+            float part = 0.0f;
+            if (hidden) {
+                for (unsigned h = lane; h < hidden; h += 64) part += H1[(size_t)e * hidden + h] * W2s[b * hidden + h];
+            } else {
+                for (unsigned kk = lane; kk < kt; kk += 64) part += H0[(size_t)e * kt + kk] * W1s[(size_t)b * kt + kk];
+            }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
+            if (lane == 0) {
+                const float out = part + (hidden ? b2s[b] : b1s[b]);
+                zs[e] = a.loss_kind == 0 ? 1.0f / (1.0f + expf(-out)) : out;
+            }
+        }
+        __syncthreads();
+        STAMP(10);
+        // loss gradient of (row, model), formed by every thread that needs it; the hidden units' gradients with it
+        for (unsigned e = tid; e < RC * nm * h1; e += NT) {
+            const unsigned rb = by_h1.quot(e), h = by_h1.rem(e, rb), rl = by_nm.quot(rb), b = by_nm.rem(rb, rl);
+            const size_t rr = (size_t)r0 + rl;
+            float dA = 0.0f, lterm = 0.0f;
+            if (rl < nreg) {
+                const float z = zs[rb], y = Ys[rb];
+                bool use = Yms[rb] != 0u;
+                if (a.revcomp) {                                       // of a (fwd, rev) pair only the larger prediction trains; ties keep the first
+                    const float zo = zs[(rl ^ 1u) * nm + b];
+                    use = use && ((rr & 1) ? !(zo >= z) : (z >= zo));
+                }
+                if (use) {
+                    dA = (z - y) * inv_n;
+                    if (h == 0)
+                        lterm = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
+                }
+            }
+            if (h == 0) { dAs[rb] = dA; lss[rb] = lterm; }
+            if (hidden) D1[e] = H1[e] > 0.0f ? dA * W2s[b * hidden + h] : 0.0f;
+        }
+        __syncthreads();
+        STAMP(12);
+        for (unsigned e = tid; e < RC * nm * k; e += NT) {             // gradient at the pooled features -> what the scan's backward pass needs
+            const unsigned rl = by_nmk.quot(e), col = by_nmk.rem(e, rl), b = by_k.quot(col), kk = by_k.rem(col, b), rb = rl * nm + b;
+            float g;
+            if (hidden) {
+                g = 0.0f;
+                const float* wrow = W1s + ((size_t)b * kt + kk) * hidden;
+#pragma unroll 8
+                for (unsigned h = 0; h < hidden; ++h) g += D1[(size_t)rb * hidden + h] * wrow[h];
+            } else {
+                g = dAs[rb] * W1s[(size_t)b * kt + kk];
+            }
+            if (!kept[e]) g = 0.0f;
+            const unsigned fl = b * a.nfilter + (kk >> (kpf - 1u));   // filter of the group
+            const bool is_avg = a.ptype == DBK_PT_AVG || (a.ptype == DBK_PT_ALL && (kk & 1u));
+            if (is_avg) cavg[rl * Fp + fl] = (rl < nreg && rinfo[2 * rl]) ? g / (float)rinfo[2 * rl] : 0.0f;
+            else gmax[rl * Fp + fl] = (rl < nreg && PL[e] > 0.0f) ? g : 0.0f;
+        }
     }
+    __syncthreads();
     STAMP(13);
+    // (from here to the grid barrier nothing waits for a store to global memory: the shares travel while the filter
+    // gradients are counted)
     // this workgroup's share of the dense layers' gradients and of the loss, rows ascending
     float* share = a.partial + (size_t)blockIdx.x * a.pstride;
     for (unsigned e = tid; e < nm * kt * h1; e += NT) {
-        const unsigned b = e / (kt * h1), kk = (e / h1) % kt, h = e % h1;
+        const unsigned q1 = by_h1.quot(e), h = by_h1.rem(e, q1), b = by_kt.quot(q1), kk = by_kt.rem(q1, b);
         float s = 0.0f;
         for (unsigned rl = 0; rl < RC; ++rl) {
             const unsigned rb = rl * nm + b;
             s += H0[(size_t)rb * kt + kk] * (hidden ? D1[(size_t)rb * hidden + h] : dAs[rb]);
         }
-        share[a.off_W1 + e] = s;
+        put_share(&share[a.off_W1 + e], s);
     }
     for (unsigned e = tid; e < nm * h1; e += NT) {
-        const unsigned b = e / h1, h = e % h1;
+        const unsigned b = by_h1.quot(e), h = by_h1.rem(e, b);
         float gb1 = 0.0f, gW2 = 0.0f;
         for (unsigned rl = 0; rl < RC; ++rl) {
             const unsigned rb = rl * nm + b;
             if (hidden) { gb1 += D1[(size_t)rb * hidden + h]; gW2 += H1[(size_t)rb * hidden + h] * dAs[rb]; }
             else gb1 += dAs[rb];
         }
-        share[a.off_b1 + e] = gb1;
-        if (hidden) share[a.off_W2 + e] = gW2;
+        put_share(&share[a.off_b1 + e], gb1);
+        if (hidden) put_share(&share[a.off_W2 + e], gW2);
     }
-    for (unsigned b = tid; b < nm; b += NT) {
+    for (unsigned b = NT - 1u - tid; b < nm; b += NT) {
         float gb2 = 0.0f, ls = 0.0f;
-        for (unsigned rl = 0; rl < RC; ++rl) { gb2 += dAs[rl * nm + b]; ls += lss[rl * nm + b]; }
-        if (hidden) share[a.off_b2 + b] = gb2;
-        share[a.nparam + b] = ls;
+        if (RC == 1u) {
+            gb2 = dAs[b];
+            if (nreg && Yms[b] != 0u) {
+                const float z = zs[b], y = Ys[b];
+                ls = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
+            }
+        } else {
+            for (unsigned rl = 0; rl < RC; ++rl) { gb2 += dAs[rl * nm + b]; ls += lss[rl * nm + b]; }
+        }
+        if (hidden) put_share(&share[a.off_b2 + b], gb2);
+        put_share(&share[a.nparam + b], ls);
     }
-    __syncthreads();
+    for (unsigned e = tid; e < nreg * nm; e += NT) put_share(&a.Z[(size_t)r0 * nm + e], zs[e]);      // the predictions of this workgroup's rows
 
     STAMP(4);
     // ---------------- scan filters: a thread's (tap, filter) pairs, five letter accumulators each, regions ascending
@@ -542,7 +686,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     for (unsigned i = 0; i < MAXPAIR; ++i) {
         const unsigned e = tid + i * NT;
         if (e >= MT * Fp) break;
-        const unsigned t = e >> a.lgFp, fl = e & (Fp - 1);
+        const unsigned t = e >> lgFp, fl = e & (Fp - 1);
         float acc[5] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f}, accb = 0.0f;
         for (unsigned rl = 0; rl < nreg; ++rl) {
             const unsigned rows = rinfo[2 * rl];
@@ -575,9 +719,9 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         }
         if (t < m && fl < F) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) share[a.off_Wc + (size_t)(4 * t + c) * F + fl] = acc[c] + 0.25f * acc[4];
+            for (int c = 0; c < 4; ++c) put_share(&share[a.off_Wc + (size_t)(4 * t + c) * F + fl], acc[c] + 0.25f * acc[4]);
         }
-        if (t == 0 && fl < F) share[a.off_bc + fl] = accb;
+        if (t == 0 && fl < F) put_share(&share[a.off_bc + fl], accb);
     }
 
     STAMP(5);
@@ -602,12 +746,12 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     const unsigned g0 = sub * per, g1 = g0 + per < a.G ? g0 + per : a.G;
     for (size_t e = efirst; e < total; e += estep) {
         float s = 0.0f;
-        for (unsigned c0 = g0; c0 < g1; c0 += 8) {
-            float v[8];
+        for (unsigned c0 = g0; c0 < g1; c0 += 16) {               // all of a lane's workgroups requested at once (a full grid: 16)
+            float v[16];
 #pragma unroll
-            for (unsigned u = 0; u < 8; ++u) v[u] = c0 + u < g1 ? a.partial[(size_t)(c0 + u) * a.pstride + e] : 0.0f;
+            for (unsigned u = 0; u < 16; ++u) v[u] = c0 + u < g1 ? a.partial[(size_t)(c0 + u) * a.pstride + e] : 0.0f;
 #pragma unroll
-            for (unsigned u = 0; u < 8; ++u)
+            for (unsigned u = 0; u < 16; ++u)
                 if (c0 + u < g1) s += v[u];
         }
         s += __shfl_xor(s, 1, 64);                                 // fixed butterfly: every lane of the eight ends with the same bits
@@ -711,7 +855,9 @@ extern "C" int dbk_train_step_single(dbk_stream_t stream, const dbk_train_step_a
     s.freeze_scan = a->freeze_scan; s.Z = a->Z; s.loss = a->loss;
     s.sync = (unsigned*)work;
     s.partial = (float*)((char*)work + WORK_HEADER);
-    auto kern = MT == 16 ? k_step_single<16> : (MT == 24 ? k_step_single<24> : k_step_single<32>);
+    const bool one = s.nmodel == 1 && s.RC == 1 && s.Fp == 16;
+    auto kern = one ? (MT == 16 ? k_step_single<16, true> : (MT == 24 ? k_step_single<24, true> : k_step_single<32, true>))
+                    : (MT == 16 ? k_step_single<16, false> : (MT == 24 ? k_step_single<24, false> : k_step_single<32, false>));
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(kern, dim3(s.G), dim3(s.RC == 1 ? NTMAX : NTMIN), lds, dbk::as_stream(stream), s);
     DBK_LAUNCH_OK();
