@@ -27,8 +27,9 @@
 //                (letter) >> tap) with one bit per position (the rectifier bits are left by the forward pass,
 //                the letter bits by the staging). The max-pooling part adds the pooled gradient at the argmax
 //                row's letters (corr1ord_bprop.cuh:91-137, poolrgn_bprop.cuh:45-127)
-//   update       g = sum of the workgroups' shares, eight lanes per parameter (each adds a contiguous run of
-//                workgroups in ascending order, then a fixed butterfly), + L1 term, frozen filters zeroed,
+//   update       g = sum of the workgroups' shares: a workgroup takes 64 consecutive parameters, each of its waves
+//                adds a run of workgroups in ascending order (one contiguous load per wave and workgroup), a fixed
+//                tree adds the waves' sums; + L1 term, frozen filters zeroed,
 //                Nesterov step from the look-ahead P + mrate * mP (gradstep.cu:41-72, full.py:111-119,
 //                corr1ord.py:120-138)
 //
@@ -51,11 +52,10 @@ constexpr unsigned MAXROWS = 256;                 // rows of one region
 constexpr unsigned AW = MAXROWS / 32;             // words of rectifier bits per (region, filter)
 constexpr unsigned LW = AW + 2;                   // words of letter bits per (region, letter): rows + taps - 1 positions
 constexpr unsigned TXTB = 384;                    // staged letters per region (a dword-aligned copy, padded with "nothing")
-constexpr unsigned LPE = 8;                       // lanes that share one parameter in the update
 constexpr unsigned MAXG = 128;                    // workgroups of a launch
 constexpr size_t WORK_HEADER = 16384;              // bytes of the workspace before the shares: launch number, status, "go", flags
 constexpr unsigned GO_AT = 32, FLAGS_AT = 64;     // words of the workspace: the "go" word; the first workgroup flag
-constexpr unsigned FLAG_STRIDE = 16;              // words from one workgroup's flag to the next (a 64-byte line each)
+constexpr unsigned FLAG_STRIDE = 4;               // words from one workgroup's flag to the next (measured: 4 beats 1 and 16 by ~0.1 us per step)
 constexpr unsigned SPIN_LIMIT = 400000;           // polls of the barrier before a workgroup gives up (~0.2 s)
 
 struct single_args {
@@ -158,7 +158,7 @@ __device__ __forceinline__ void scan_block(const float* __restrict__ wt, const u
 // one after the other (measured: ~50 ns per read-modify-write, 6.5 us for a counter that 128 workgroups increment;
 // 2-4 us per poll when every workgroup reads every other's flag, in lines of their own or side by side), so no word is
 // shared more than it must be: each workgroup
-// raises a flag in a 64-byte line of its own - the number of this launch, one more than the number the workspace
+// raises a flag of its own - the number of this launch, one more than the number the workspace
 // held when the kernel started; workgroup 0 alone reads all the flags (two per lane of its first wave) and, when
 // they all show the number, writes it to the "go" word; every other workgroup polls that one word with one lane.
 // Returns 0 when the step may go on, else the status to leave with (1: this workgroup gave up waiting; otherwise
@@ -727,10 +727,13 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     STAMP(5);
     // ---------------- every workgroup's share is written: meet, then add them up and step the parameters.
     // What the update reads of the parameter vectors is requested before the wait (nothing changes it until then).
-    const size_t total = a.nparam + nm, estep = (size_t)a.G * NT / LPE, efirst = ((size_t)blockIdx.x * NT + tid) / LPE;
-    const unsigned sub = tid & (LPE - 1);
+    // A workgroup steps 64 consecutive parameters: wave w adds the shares of its run of workgroups for them (a lane per
+    // parameter: every load of a wave is one contiguous 256 bytes), the waves' sums meet in LDS and wave 0 adds them in a
+    // fixed tree and applies the step.
+    const size_t total = a.nparam + nm, estep = (size_t)a.G * 64;
+    const size_t efirst = (size_t)blockIdx.x * 64 + lane;
     float q_p = 0.0f, q_rm = 0.0f, q_mp = 0.0f, q_dr = 0.0f, q_dec = 0.0f;
-    if (sub == 0 && efirst < a.nparam) {
+    if (wave == 0 && efirst < a.nparam) {
         q_p = a.P[efirst]; q_rm = a.mrate[efirst]; q_mp = a.mP[efirst]; q_dr = a.drate[efirst];
         if (a.decay) q_dec = a.decay[efirst];
     }
@@ -742,22 +745,30 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     // (every workgroup read the launch number before it raised its flag, so it can move on now)
     if (blockIdx.x == 0 && tid == 0) __hip_atomic_store(&a.sync[0], misc[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);              // flagged (by any workgroup, before the barrier) or gave up: no update
     STAMP(6);
-    const unsigned per = (a.G + LPE - 1) / LPE;                    // workgroups each of the eight lanes adds, ascending
-    const unsigned g0 = sub * per, g1 = g0 + per < a.G ? g0 + per : a.G;
-    for (size_t e = efirst; e < total; e += estep) {
+    float* sums = wt;                                              // (the letter table is no longer needed)
+    const unsigned per = (a.G + NW - 1) / NW;                      // workgroups each wave adds, ascending
+    const unsigned g0 = wave * per, g1 = g0 + per < a.G ? g0 + per : a.G;
+    for (size_t base = (size_t)blockIdx.x * 64; base < total; base += estep) {
+        const size_t e = base + lane;
         float s = 0.0f;
-        for (unsigned c0 = g0; c0 < g1; c0 += 16) {               // all of a lane's workgroups requested at once (a full grid: 16)
-            float v[16];
+        if (e < total) {
+            for (unsigned c0 = g0; c0 < g1; c0 += 16) {           // all of a wave's workgroups requested at once (a full grid: 16)
+                float v[16];
 #pragma unroll
-            for (unsigned u = 0; u < 16; ++u) v[u] = c0 + u < g1 ? a.partial[(size_t)(c0 + u) * a.pstride + e] : 0.0f;
+                for (unsigned u = 0; u < 16; ++u) v[u] = c0 + u < g1 ? a.partial[(size_t)(c0 + u) * a.pstride + e] : 0.0f;
 #pragma unroll
-            for (unsigned u = 0; u < 16; ++u)
-                if (c0 + u < g1) s += v[u];
+                for (unsigned u = 0; u < 16; ++u)
+                    if (c0 + u < g1) s += v[u];
+            }
         }
-        s += __shfl_xor(s, 1, 64);                                 // fixed butterfly: every lane of the eight ends with the same bits
-        s += __shfl_xor(s, 2, 64);
-        s += __shfl_xor(s, 4, 64);
-        if (sub) continue;
+        if (base != (size_t)blockIdx.x * 64) __syncthreads();      // (a further round: the sums of the last one have been read)
+        sums[wave * 64 + lane] = s;
+        __syncthreads();
+        if (wave != 0 || e >= total) continue;
+        float pw[NWMAX];
+#pragma unroll
+        for (unsigned w = 0; w < NWMAX; ++w) pw[w] = w < NW ? sums[w * 64 + lane] : 0.0f;
+        s = ((pw[0] + pw[1]) + (pw[2] + pw[3])) + ((pw[4] + pw[5]) + (pw[6] + pw[7]));
         if (e >= a.nparam) {
             if (a.loss) a.loss[e - a.nparam] = a.loss_kind == 0 ? -s / (float)a.nregion : 0.5f * s / (float)a.nregion;
             continue;
