@@ -82,6 +82,21 @@ inline unsigned ew_grid(size_t n, unsigned block = 256)
     return (unsigned)g;
 }
 
+
+// Quotient of small numbers without the integer division sequence: for e < 2^20 and any divisor, (e + 0.5) / d is at
+// least 0.5 / d away from a whole number while the reciprocal's and the product's rounding move it by less than
+// e / d * 2^-21, so truncating gives floor(e / d) exactly.
+struct small_div {
+    float inv; unsigned d;
+    __device__ __forceinline__ explicit small_div(unsigned d_) : inv(__builtin_amdgcn_rcpf((float)d_)), d(d_) {}
+    __device__ __forceinline__ unsigned quot(unsigned e) const
+    {
+        if (__builtin_constant_p(d) && d == 1u) return e;
+        return (unsigned)(((float)e + 0.5f) * inv);
+    }
+    __device__ __forceinline__ unsigned rem(unsigned e, unsigned q) const { return e - q * d; }
+};
+
 }  // namespace dbk
 
 #define DBK_CHECK(cond, ...)                                  \

@@ -60,6 +60,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
     float* dAs = D1s + RB * hst;            // [RB]      gradient at the output pre-activation
     float* lss = dAs + RB;                  // [RB]      loss terms
     unsigned char* kept = reinterpret_cast<unsigned char*>(lss + RB);   // [RB][k] dropout keep flags
+    const dbk::small_div by_h1((unsigned)h1), by_k((unsigned)k), by_kf((unsigned)a.kf);      // (all dividends below are < 2^20)
 
     // four loads in flight per thread and round (a plain strided loop waits for each load before the next)
     for (int e0 = tid; e0 < kt * h1; e0 += 4 * NT) {
@@ -69,7 +70,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int e = e0 + j * NT;
-            if (e < kt * h1) w1s[(e / h1) * wst + e % h1] = v[j];
+            if (e < kt * h1) { const unsigned kk = by_h1.quot(e); w1s[kk * wst + by_h1.rem(e, kk)] = v[j]; }
         }
     }
     for (int e = tid; e < h1; e += NT) {                          // both vectors' loads are issued before either is stored
@@ -88,33 +89,58 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
     const float inv_n = 1.0f / (float)a.n;
 
     // ---------------- inputs of the chunk, dropout applied (same element numbering as the stand-alone dropout kernels)
-    for (int e0 = tid; e0 < RB * k; e0 += 4 * NT) {
-        float xv[4], uv[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {                              // the loads of a round first
-            const int e = e0 + j * NT, er = e / k, kk = e % k;
+    if (!a.U && (k & 3) == 0 && (ncol & 3) == 0 && ((uintptr_t)a.pooled & 15) == 0) {
+        // four consecutive features of a row per thread: one 16-byte load and ONE call of the generator for their four
+        // uniforms (flat elements 4q .. 4q+3 share a counter value)
+        const unsigned kq = (unsigned)k >> 2;
+        const dbk::small_div by_kq(kq);
+        for (unsigned e = tid; e < RB * kq; e += NT) {
+            const unsigned er = by_kq.quot(e), kk = 4u * by_kq.rem(e, er);
             const size_t rr = r0 + er, col = (size_t)b * k + kk;
-            const bool in = e < RB * k && rr < a.n;
-            xv[j] = in ? a.pooled[rr * ncol + col] : 0.0f;
-            uv[j] = (in && a.rate && a.U) ? a.U[(a.revcomp ? (rr & ~(size_t)1) : rr) * ncol + col] : 1.0f;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int e = e0 + j * NT, er = e / k, kk = e % k;
-            if (e >= RB * k) break;
-            const size_t rr = r0 + er, col = (size_t)b * k + kk;
-            bool kp = true;
-            if (rr < a.n && a.rate) {
-                const float u = a.U ? uv[j] : dbk_rng::uniform_at(a.seed, off, a.revcomp ? (rr >> 1) * ncol + col : rr * ncol + col);
-                kp = u >= p_drop;
+            float4 xv = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            float u[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            const bool in = rr < a.n;
+            if (in) {
+                xv = *reinterpret_cast<const float4*>(a.pooled + rr * ncol + col);
+                if (a.rate) dbk_rng::uniform4_at(a.seed, off, ((a.revcomp ? (rr >> 1) : rr) * ncol + col) >> 2, u);
             }
-            H0s[er * ks + kk] = kp ? xv[j] : 0.0f;
-            kept[e] = kp;
+            const float x4[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool kp = !(in && a.rate) || u[j] >= p_drop;
+                H0s[er * ks + kk + j] = kp ? x4[j] : 0.0f;
+                kept[er * k + kk + j] = kp;
+            }
+        }
+    } else {
+        for (int e0 = tid; e0 < RB * k; e0 += 4 * NT) {
+            float xv[4], uv[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {                              // the loads of a round first
+                const int e = e0 + j * NT, er = (int)by_k.quot((unsigned)e), kk = e - er * k;
+                const size_t rr = r0 + er, col = (size_t)b * k + kk;
+                const bool in = e < RB * k && rr < a.n;
+                xv[j] = in ? a.pooled[rr * ncol + col] : 0.0f;
+                uv[j] = (in && a.rate && a.U) ? a.U[(a.revcomp ? (rr & ~(size_t)1) : rr) * ncol + col] : 1.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int e = e0 + j * NT, er = (int)by_k.quot((unsigned)e), kk = e - er * k;
+                if (e >= RB * k) break;
+                const size_t rr = r0 + er, col = (size_t)b * k + kk;
+                bool kp = true;
+                if (rr < a.n && a.rate) {
+                    const float u = a.U ? uv[j] : dbk_rng::uniform_at(a.seed, off, a.revcomp ? (rr >> 1) * ncol + col : rr * ncol + col);
+                    kp = u >= p_drop;
+                }
+                H0s[er * ks + kk] = kp ? xv[j] : 0.0f;
+                kept[e] = kp;
+            }
         }
     }
     // the shared feature columns follow the model's own inputs in the row (a null pointer stands for all zeros)
     for (int e = tid; e < RB * a.kf; e += NT) {
-        const int er = e / a.kf, kk = e % a.kf;
+        const int er = (int)by_kf.quot((unsigned)e), kk = e - er * a.kf;
         const size_t rr = r0 + er;
         H0s[er * ks + k + kk] = (a.feats && rr < a.n) ? a.feats[rr * a.kf + kk] : 0.0f;
     }
@@ -185,7 +211,7 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
     // ---------------- this chunk's share of the parameter gradients, rows ascending
     float* part_out = a.partial + ((size_t)chunk * a.nblock + b) * a.pstride;
     for (int pidx = tid; pidx < kt * h1; pidx += NT) {
-        const int kk = pidx / h1, h = pidx % h1;
+        const int kk = (int)by_h1.quot((unsigned)pidx), h = pidx - kk * h1;
         float s = 0.0f;
         if (hidden > 0) {
 #pragma unroll 8

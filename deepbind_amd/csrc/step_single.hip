@@ -33,8 +33,8 @@
 //                Nesterov step from the look-ahead P + mrate * mP (gradstep.cu:41-72, full.py:111-119,
 //                corr1ord.py:120-138)
 //
-// The barrier is a ticket counter in the caller's workspace; every workgroup of the grid must be resident, so
-// the grid never exceeds 128 workgroups of 256 threads (a CU holds at least one), and the wait is bounded:
+// The barrier is a set of flags in the caller's workspace; every workgroup of the grid must be resident, so
+// the grid never exceeds 128 workgroups of at most 512 threads (a CU holds at least one), and the wait is bounded:
 // a workgroup that gives up sets the workspace's status word and leaves without touching the parameters.
 // Results are deterministic (no float atomics; LDS atomics only OR bits), within the tolerances of the
 // multi-launch step but not its bits (other summation orders).
@@ -46,6 +46,7 @@ namespace {
 
 using dbk_scan::NL;
 using dbk_scan::letter_of;
+using dbk::small_div;
 
 constexpr int NTMIN = 256, NTMAX = 512, NWMAX = NTMAX / 64;    // threads of a workgroup: 256, or 512 when it has a single region
 constexpr unsigned MAXROWS = 256;                 // rows of one region
@@ -206,20 +207,6 @@ __device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, uns
     __syncthreads();
     return verdict;
 }
-
-// Quotient of small numbers without the integer division sequence: for e < 2^20 and any divisor, (e + 0.5) / d is at
-// least 0.5 / d away from a whole number while the reciprocal's and the product's rounding move it by less than
-// e / d * 2^-21, so truncating gives floor(e / d) exactly.
-struct small_div {
-    float inv; unsigned d;
-    __device__ __forceinline__ explicit small_div(unsigned d_) : inv(__builtin_amdgcn_rcpf((float)d_)), d(d_) {}
-    __device__ __forceinline__ unsigned quot(unsigned e) const
-    {
-        if (__builtin_constant_p(d) && d == 1u) return e;
-        return (unsigned)(((float)e + 0.5f) * inv);
-    }
-    __device__ __forceinline__ unsigned rem(unsigned e, unsigned q) const { return e - q * d; }
-};
 
 // Orders a wave's own LDS traffic: what its lanes stored before is what its lanes read after (the LDS serves a wave's
 // instructions in order; the fences keep the compiler from moving them and wait for the counter).
