@@ -1,13 +1,15 @@
 // Per-model ("blockwise") small dense products on the model axis, and the fused scoring head.
 //
-// The products are tiny (k, m <= a few dozen) and there are many of them (one per model), so they
-// are not GEMM-shaped work for the matrix cores: one thread owns one output element, the 64 lanes
-// of a wave own 64 consecutive output columns of one row, and the inner product runs in a fixed
-// order in registers. HBM traffic is one coalesced pass over the operands.
+// The products are tiny (k, m <= a few dozen) and there are many of them (one per model). The vector kernels: one
+// thread owns one output element (or four), the lanes of a wave own consecutive output columns of one row, the
+// inner product runs in a fixed order in registers. At bulk row counts, float32 products whose widths are multiples
+// of 16 run on the matrix cores instead (k_bdot_mfma): the vector kernels spend their time on LDS reads of the
+// weights (one per multiply-add), the matrix-core kernel moves at the rate of its one pass over the operands.
 //
 // Reference semantics: deepity_smat/blockwise_dot.cu:77-260 (pointer arithmetic per block) and
 // deepity/_ext/deepity_smat.py:169-251 (shapes).
 #include "dbk_common.h"
+#include "mfma_common.h"
 
 namespace {
 
@@ -587,10 +589,129 @@ int launch_rowtile(hipStream_t st, int nblock, int n, int ni, int no, bool bcast
     return 0;
 }
 
+// The per-model products at bulk row counts on the matrix cores: out[r, b*no + o] = sum_i in[r, b*ni + i] * w_b[i][o]
+// for ni = 16 * KS inputs and no <= 32 * NT outputs per model, both operands split into three bf16 pieces that add up
+// to the float32 value exactly (six piece products, the small ones first, float32 accumulation: float32 results, the
+// sums in another order than the vector kernels'). A wave owns one model and walks blocks of 32 rows; the model's
+// weight pieces stay in its registers; a lane reads 8 consecutive inputs of its row (the matrix instruction's operand
+// layout), the next block's while this block is multiplied (two blocks ahead: no faster). The four waves of a workgroup take four adjacent models,
+// so the rows' segments they read and write lie side by side. `transpose`: w_b[i][o] = W_b[o][i] (the dot_nt case).
+template <int KS, int NT>
+__global__ __launch_bounds__(256) void k_bdot_mfma(int nblock, size_t n, int ni, int no, bool transpose, int m, int p, int off,
+                                                   const float* __restrict__ in, const float* __restrict__ W, float* __restrict__ out)
+{
+    using namespace dbk_mfma;
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, col = lane & 31u, half = lane >> 5;
+    const unsigned b = blockIdx.x * 4u + wave;
+    if (b >= (unsigned)nblock) return;
+    // weight pieces: lane = output column `col` of tile nt, inputs 16 ks + 8 half .. + 7
+    uint4 B[KS][NT][3];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const unsigned o = nt * 32 + col, i0 = ks * 16 + 8 * half;
+            unsigned lo[8], mid[8], hi[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float w = 0.0f;
+                if (o < (unsigned)no)
+                    w = transpose ? W[((size_t)b * p + off + o) * m + i0 + j] : W[((size_t)b * p + off + i0 + j) * m + o];
+                split3(w, lo[j], mid[j], hi[j]);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                (&B[ks][nt][0].x)[q] = pack_upper_halves(lo[2 * q], lo[2 * q + 1]);
+                (&B[ks][nt][1].x)[q] = pack_upper_halves(mid[2 * q], mid[2 * q + 1]);
+                (&B[ks][nt][2].x)[q] = pack_upper_halves(hi[2 * q], hi[2 * q + 1]);
+            }
+        }
+    const size_t ldin = (size_t)ni * nblock, ldout = (size_t)no * nblock;
+    const float* src = in + (size_t)b * ni + 8 * half;
+    float* dst = out + (size_t)b * no + col;
+    const size_t nblk = (n + 31) / 32;
+    auto request = [&](size_t blk, float4 (&x)[KS][2]) {
+        size_t r = blk * 32 + col;
+        if (r >= n) r = n - 1;                                     // (a row past the end: a valid address, its results are not stored)
+        const float4* q = reinterpret_cast<const float4*>(src + r * ldin);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) { x[ks][0] = q[4 * ks]; x[ks][1] = q[4 * ks + 1]; }
+    };
+    float4 xn[KS][2];
+    size_t blk = blockIdx.y;
+    if (blk < nblk) request(blk, xn);
+    for (; blk < nblk; blk += gridDim.y) {
+        uint4 A[KS][3];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const float v[8] = {xn[ks][0].x, xn[ks][0].y, xn[ks][0].z, xn[ks][0].w, xn[ks][1].x, xn[ks][1].y, xn[ks][1].z, xn[ks][1].w};
+            unsigned lo[8], mid[8], hi[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) split3(v[j], lo[j], mid[j], hi[j]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                (&A[ks][0].x)[q] = pack_upper_halves(lo[2 * q], lo[2 * q + 1]);
+                (&A[ks][1].x)[q] = pack_upper_halves(mid[2 * q], mid[2 * q + 1]);
+                (&A[ks][2].x)[q] = pack_upper_halves(hi[2 * q], hi[2 * q + 1]);
+            }
+        }
+        if (blk + gridDim.y < nblk) request(blk + gridDim.y, xn);
+        const size_t r0 = blk * 32 + 4 * half;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            f32x16_t acc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                acc = mfma_bf16(A[ks][0], B[ks][nt][2], acc);     // lo . hi
+                acc = mfma_bf16(A[ks][2], B[ks][nt][0], acc);     // hi . lo
+                acc = mfma_bf16(A[ks][1], B[ks][nt][1], acc);     // mid . mid
+                acc = mfma_bf16(A[ks][1], B[ks][nt][2], acc);     // mid . hi
+                acc = mfma_bf16(A[ks][2], B[ks][nt][1], acc);     // hi . mid
+                acc = mfma_bf16(A[ks][2], B[ks][nt][2], acc);     // hi . hi
+            }
+            if (nt * 32 + col < (unsigned)no) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const size_t r = r0 + (i & 3) + 8 * (i >> 2);
+                    if (r < n) dst[r * ldout + nt * 32] = acc[i];
+                }
+            }
+        }
+    }
+}
+
+// returns -1 when the shape is not the matrix-core kernel's (the caller goes on to the vector kernels)
+inline int launch_bdot_mfma(hipStream_t st, int nblock, int n, int ni, int no, bool transpose, int m, int p, int off,
+                            const float* in, const float* W, float* out)
+{
+    if (n < 2048 || ni % 16 != 0 || ni > 64 || no % 16 != 0 || no > 64 || ((uintptr_t)in & 15) != 0) return -1;
+    const int ks = ni / 16, nt = (no + 31) / 32;
+    if (ks * nt > 4) return -1;
+    const unsigned groups = dbk::divup(nblock, 4);
+    unsigned gy = 2048u / groups;                                  // ~2 workgroups per SIMD in all
+    const unsigned nblk = dbk::divup((size_t)n, 32);
+    if (gy < 1) gy = 1;
+    if (gy > nblk) gy = nblk;
+    if (gy > 65535u) gy = 65535u;
+    const dim3 grid(groups, gy);
+#define DBK_BDOT_MFMA(KSV, NTV)                                                                                       \
+    if (ks == KSV && nt == NTV) {                                                                                     \
+        hipLaunchKernelGGL((k_bdot_mfma<KSV, NTV>), grid, dim3(256), 0, st, nblock, (size_t)n, ni, no, transpose, m, p, off, in, W, out); \
+        return 0;                                                                                                     \
+    }
+    DBK_BDOT_MFMA(1, 1) DBK_BDOT_MFMA(2, 1) DBK_BDOT_MFMA(3, 1) DBK_BDOT_MFMA(4, 1) DBK_BDOT_MFMA(1, 2) DBK_BDOT_MFMA(2, 2)
+#undef DBK_BDOT_MFMA
+    return -1;
+}
+
 template <typename T>
 int launch_bdot_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int off, bool bcast, bool accumulate,
                      const T* X, const T* W, T* Z)
 {
+    if constexpr (sizeof(T) == 4)
+        if (!bcast && !accumulate && launch_bdot_mfma(st, nblock, n, k, m, false, m, p, off, X, W, Z) == 0) return 0;
     if (launch_rowtile<T>(st, nblock, n, k, m, bcast, accumulate, false, m, p, off, X, W, Z) == 0) return 0;
     const size_t smem = (size_t)k * m * TG * sizeof(T);
     if (smem > 65536) return -1;
@@ -611,6 +732,8 @@ int launch_bdot_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int
 template <typename T>
 int launch_bdot_nt_tile(hipStream_t st, int nblock, int n, int m, int k, int p, int off, const T* dZ, const T* W, T* dX)
 {
+    if constexpr (sizeof(T) == 4)
+        if (launch_bdot_mfma(st, nblock, n, m, k, true, m, p, off, dZ, W, dX) == 0) return 0;
     if (launch_rowtile<T>(st, nblock, n, m, k, false, false, true, m, p, off, dZ, W, dX) == 0) return 0;
     const size_t smem = (size_t)k * m * TG * sizeof(T);
     if (smem > 65536) return -1;

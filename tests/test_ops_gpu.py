@@ -615,10 +615,13 @@ def test_head_fprop_bulk_rows(ds, k, h, nb):
 
 
 @pytest.mark.parametrize("n,k,m,nb,dtype", [(2048, 16, 32, 7, np.float32), (5003, 32, 4, 33, np.float32), (3000, 16, 1, 5, np.float32),
-                                            (2500, 64, 64, 3, np.float32), (2100, 16, 32, 18, np.float64), (2049, 5, 12, 16, np.float32)])
+                                            (2500, 64, 64, 3, np.float32), (2100, 16, 32, 18, np.float64), (2049, 5, 12, 16, np.float32),
+                                            (8200, 32, 64, 6, np.float32), (4100, 48, 16, 5, np.float32), (33000, 16, 32, 64, np.float32)])
 def test_blockwise_dot_family_bulk_rows(ds, n, k, m, nb, dtype):
-    """Row counts that take the bulk kernels (16 models per workgroup; chunked weight gradient), model counts
-    off the group size, output widths that are / are not multiples of four (the latter fall back), float64."""
+    """Row counts that take the bulk kernels (16 models per workgroup; chunked weight gradient; float32 products with
+    multiples of 16 inputs and outputs on the matrix cores, tiles half used and model counts off the group of four
+    included), model counts off the group size, output widths that are / are not multiples of four (the latter fall
+    back), float64."""
     rng = np.random.default_rng(n + k + m)
     tol = ACT if dtype == np.float32 else 1e-12
     X = rng.standard_normal((n, k * nb)).astype(dtype)
