@@ -868,7 +868,7 @@ inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, 
 // Y (rows x 4m) = dZ (rows x F) . W^T (F x 4m), then dX[i, c] += sum_k Y[i - k, 4k + c]. Both operands are float32
 // data, so both enter as three bf16 pieces and six of the nine piece products are formed (hi.hi, hi.mid, mid.hi,
 // mid.mid, hi.lo, lo.hi; the three left out are below 2^-24 of the result), accumulated in float32.
-// A workgroup takes 512 output rows and 128 filters (the launcher issues one launch per 128 filters: dX accumulates),
+// A workgroup takes 512 or more output rows (1/512 of all) and 128 filters (the launcher issues one launch per 128 filters: dX accumulates),
 // wave b of it the taps 8b .. 8b + 7 (32 columns of Y; W's pieces for them stay in registers, 96 registers). A
 // block of 32 rows of dZ is read by the whole workgroup as whole 512-byte row segments and staged in LDS (the next
 // block's rows are on their way while this one is multiplied and go to LDS between the block's two barriers: a lane reading its own row from memory touches 32
@@ -877,13 +877,13 @@ inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, 
 // threads add up the taps of their (row, letter) in ascending order, reaching into the previous block's tile for
 // rows before the block (the first block of a workgroup recomputes its predecessor's last rows instead of sharing
 // them). Deterministic: one writer per element, fixed orders.
-constexpr unsigned GX_ROWS = 512;                                  // output rows per workgroup
+constexpr unsigned GX_ROWS = 512;                                  // output rows per workgroup, at least (a multiple of 32)
 constexpr unsigned GX_FILTERS = 128;                               // filters per launch: eight k-steps of 16
 constexpr unsigned GX_ZS = GX_FILTERS + 8;                         // row stride of a staged plane in bf16: 68 words = 4 mod 32, so that the 32 rows' 16-byte reads spread over the banks
 
 template <int MB, bool WHOLE>
 __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* __restrict__ dX, size_t n, const float* __restrict__ W,
-                                                                        unsigned m, unsigned F, unsigned f0, const float* __restrict__ dZ)
+                                                                        unsigned m, unsigned F, unsigned f0, const float* __restrict__ dZ, unsigned rows_per_wg)
 {
     using namespace dbk_mfma;
     constexpr int YS = 32 * MB + 4;                                // row stride of a tile of Y: 4 mod 32, so that the adders' reads spread over the banks
@@ -911,7 +911,7 @@ __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* _
                                       pack_upper_halves(pc[q][4], pc[q][5]), pack_upper_halves(pc[q][6], pc[q][7]));
         }
     }
-    const size_t o0 = (size_t)blockIdx.x * GX_ROWS, o1 = o0 + GX_ROWS < n ? o0 + GX_ROWS : n;
+    const size_t o0 = (size_t)blockIdx.x * rows_per_wg, o1 = o0 + rows_per_wg < n ? o0 + rows_per_wg : n;
     // A block's rows of dZ, requested by the whole workgroup as 16-byte pieces in row order (a wave reads whole
     // 512-byte row segments); rows past the end and filters past F count as zero.
     float4 piece[PER];
@@ -1020,12 +1020,16 @@ inline bool bprop_X_mfma_takes(size_t m, size_t F, size_t n) { return m <= 32 &&
 
 inline int launch_bprop_X_mfma(hipStream_t st, float* dX, size_t n, const float* W, size_t m, size_t F, const float* dZ)
 {
-    const unsigned gx = (unsigned)dbk::divup(n, GX_ROWS), mb = (unsigned)((4 * m + 31) / 32);
+    // two workgroups fit a CU: about 512 of them in all, so that the weights' pieces are formed once per many rows
+    // (512 rows per workgroup: 0.61 ms at 1.0 M rows x 256 filters; 1/512 of the rows: 0.54 ms)
+    unsigned rows = (unsigned)(((n + 511) / 512 + 31) / 32 * 32);
+    if (rows < GX_ROWS) rows = GX_ROWS;
+    const unsigned gx = (unsigned)dbk::divup(n, rows), mb = (unsigned)((4 * m + 31) / 32);
     for (size_t f0 = 0; f0 < F; f0 += GX_FILTERS) {
         const bool whole = F % 4 == 0 && f0 + GX_FILTERS <= F;
 #define DBK_GO(MB_)                                                                                                   \
-        if (whole) hipLaunchKernelGGL((corr1ord_bprop_X_mfma_kernel<MB_, true>), dim3(gx), dim3(64 * MB_), 0, st, dX, n, W, (unsigned)m, (unsigned)F, (unsigned)f0, dZ); \
-        else hipLaunchKernelGGL((corr1ord_bprop_X_mfma_kernel<MB_, false>), dim3(gx), dim3(64 * MB_), 0, st, dX, n, W, (unsigned)m, (unsigned)F, (unsigned)f0, dZ);
+        if (whole) hipLaunchKernelGGL((corr1ord_bprop_X_mfma_kernel<MB_, true>), dim3(gx), dim3(64 * MB_), 0, st, dX, n, W, (unsigned)m, (unsigned)F, (unsigned)f0, dZ, rows); \
+        else hipLaunchKernelGGL((corr1ord_bprop_X_mfma_kernel<MB_, false>), dim3(gx), dim3(64 * MB_), 0, st, dX, n, W, (unsigned)m, (unsigned)F, (unsigned)f0, dZ, rows);
         switch (mb) {
         case 1:  DBK_GO(1) break;
         case 2:  DBK_GO(2) break;
