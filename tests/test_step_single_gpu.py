@@ -46,6 +46,10 @@ CASES = [
     ("max", 0, "mse", 3, 12, 9, 33, (5, 30), False, 0),            # 36 filters: padded to 64 lanes
     ("all", 16, "nll", 2, 16, 20, 64, (30, 200), True, 0),         # reverse-complement pairs, regions up to 219 rows
     ("max", 32, "nll", 1, 16, 32, 300, (20, 60), False, 16),       # four regions per workgroup
+    # one 16-filter model, one region per workgroup (the instance with that shape compiled in), its other branches:
+    ("all", 32, "nll", 1, 16, 24, 100, (20, 90), False, 0),        # 32 pooled features into a hidden layer (two lane groups per feature)
+    ("avg", 20, "mse", 1, 12, 32, 77, (8, 50), False, 16),         # 12 filters in 16 lanes, 32 taps, shared feature columns, a hidden width the lane groups do not divide
+    ("max", 64, "nll", 1, 16, 8, 128, (30, 60), False, 0),         # 64 hidden units
 ]
 
 
