@@ -1033,8 +1033,8 @@ int launch_bprop_pt(hipStream_t st, const float* W, const float* bias, size_t m,
     // Average pooling without the forward pass's activity masks: the matrix-core forward writes them again (into the
     // stream's second scratch buffer, with its pooled values beside them), and the bit-count kernel takes them from
     // there; less than half the time of recomputing the map through the letter table.
-    if (PT != DBK_PT_MAX && !act && !dbk::deferred() && mfma_pays(m, ftiles, P)) {
-        const size_t mask_bytes = N * ftiles * sizeof(unsigned long long), pooled_bytes = P * F * 2 * sizeof(float);
+    const size_t mask_bytes = N * ftiles * sizeof(unsigned long long), pooled_bytes = P * F * 2 * sizeof(float);
+    if (PT != DBK_PT_MAX && !act && !dbk::deferred() && mfma_pays(m, ftiles, P) && mask_bytes + pooled_bytes <= ((size_t)1 << 30)) {   // (at most 1 GiB of scratch for it)
         unsigned char* scratch = (unsigned char*)dbk::workspace(mask_bytes + pooled_bytes, st, 1);
         DBK_CHECK(scratch != nullptr, "MemoryError: could not allocate %zu bytes of scratch (%s)", mask_bytes + pooled_bytes, dbk::workspace_error());
         unsigned long long* masks = reinterpret_cast<unsigned long long*>(scratch);

@@ -190,7 +190,7 @@ int dbk_scanpool_fprop_kmer_static(dbk_stream_t stream,
  * instead, which saves the caller a fill) and writes dbias (1, F) =. Deterministic (no float atomics).
  * act (may be NULL): the activity masks dbk_scanpool_fprop wrote for the same W, bias, X and regions;
  * without them the avg / all gradient recomputes them first (a second forward pass into the stream's scratch
- * at bulk sizes, the map through the letter table otherwise).
+ * at bulk sizes while that takes at most 1 GiB, the map through the letter table otherwise).
  * reference chain: poolrgn_bprop -> relu bprop -> bias bprop -> corr1ord_bprop_W
  * (kangaroo/_ext/poolrgn.py:78-82, deepity/std/elemwise.py:78,172-180, kangaroo/_ext/corr1ord.py:120-138) */
 int dbk_scanpool_bprop(dbk_stream_t stream,
