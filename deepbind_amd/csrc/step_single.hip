@@ -38,6 +38,7 @@
 // a workgroup that gives up sets the workspace's status word and leaves without touching the parameters.
 // Results are deterministic (no float atomics; LDS atomics only OR bits), within the tolerances of the
 // multi-launch step but not its bits (other summation orders).
+#include <type_traits>
 #include "dbk_common.h"
 #include "rng.h"
 #include "scan_common.h"
@@ -59,6 +60,10 @@ constexpr unsigned GO_AT = 32, FLAGS_AT = 64;     // words of the workspace: the
 constexpr unsigned FLAG_STRIDE = 4;               // words from one workgroup's flag to the next (measured: 4 beats 1 and 16 by ~0.1 us per step)
 constexpr unsigned SPIN_LIMIT = 400000;           // polls of the barrier before a workgroup gives up (~0.2 s)
 
+// LDS carve-up (all offsets in 4-byte words), computed on the host for the launch size and handed to the kernel.
+struct lds_map {
+    unsigned wt, look, Y, Ym, misc, text, lmask, amask, PL, arg, gmax, cavg, rows, red, H0, H1, D1, dA, ls, zs, kept, total;
+};
 struct single_args {
     unsigned nmodel, nfilter, F, Fp, lgFp, m, hidden, h1, k, kt, kf, ptype, loss_kind, revcomp;
     unsigned RC, G;                               // regions per workgroup, workgroups
@@ -74,13 +79,10 @@ struct single_args {
     float *Z, *loss;
     unsigned* sync;                               // [0] number of the last launch, [1] status (non-zero: see grid_barrier), [64..] flags
     float* partial;                               // [G][pstride]
+    lds_map L;
 };
 
-// LDS carve-up (all offsets in 4-byte words), computed identically on the host for the launch size.
-struct lds_map {
-    unsigned wt, look, Y, Ym, misc, text, lmask, amask, PL, arg, gmax, cavg, rows, red, H0, H1, D1, dA, ls, zs, kept, total;
-};
-__host__ __device__ inline lds_map make_map(unsigned MT, unsigned Fp, unsigned nm, unsigned kt, unsigned k, unsigned h1, unsigned nparam,
+inline lds_map make_map(unsigned MT, unsigned Fp, unsigned nm, unsigned kt, unsigned k, unsigned h1, unsigned nparam,
                                             unsigned RC, bool dense)
 {
     lds_map o;
@@ -244,16 +246,20 @@ __device__ __forceinline__ void put_share(float* p, float v) { __hip_atomic_stor
 #define STAMP(i) do {} while (0)
 #endif
 
-// ONE: the shape of a single 16-filter model on a batch of at most MAXG regions (one region per workgroup of 512
-// threads), known when the kernel is compiled: the index arithmetic of the general shape folds away, and with a step
-// this short the instructions a wave issues one after the other are what the step costs.
-template <int MT, bool ONE>
+// SHAPE: what of the launch shape is known when the kernel is compiled. 1: one region per workgroup of 512 threads
+// (batches of at most MAXG regions). 2: that, and a single model of at most 16 filters. 3 / 4: one region per workgroup
+// and 17-32 / 33-64 filters in all. 0: nothing. Whatever is known
+// folds out of the index arithmetic and takes whole branches with it (the instance for shape 2 is a third as long as
+// the general one), and with a step this short the instructions a wave issues one after the other are what it costs.
+template <int MT, int SHAPE>
 __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
 {
     extern __shared__ __align__(16) unsigned smem[];
     const bool dense = a.ptype != DBK_PT_MAX, sparse = a.ptype != DBK_PT_AVG;
-    const unsigned nm = ONE ? 1u : a.nmodel, RC = ONE ? 1u : a.RC, Fp = ONE ? 16u : a.Fp, lgFp = ONE ? 4u : a.lgFp;
-    const lds_map L = make_map(MT, Fp, nm, a.kt, a.k, a.h1, (unsigned)a.nparam, RC, dense);
+    constexpr bool ONE = SHAPE == 2;
+    const unsigned nm = ONE ? 1u : a.nmodel, RC = SHAPE ? 1u : a.RC;
+    const unsigned Fp = ONE ? 16u : SHAPE == 3 ? 32u : SHAPE == 4 ? 64u : a.Fp, lgFp = ONE ? 4u : SHAPE == 3 ? 5u : SHAPE == 4 ? 6u : a.lgFp;
+    const lds_map& L = a.L;
     float* wt = reinterpret_cast<float*>(smem + L.wt);
     float* Lk = reinterpret_cast<float*>(smem + L.look);
     const float* W1s = Lk + a.off_W1;
@@ -281,7 +287,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     float* zs = reinterpret_cast<float*>(smem + L.zs);
     uint8_t* kept = reinterpret_cast<uint8_t*>(smem + L.kept);
 
-    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, NT = ONE ? (unsigned)NTMAX : blockDim.x, NW = NT >> 6;
+    const unsigned tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, NT = SHAPE ? (unsigned)NTMAX : blockDim.x, NW = NT >> 6;
     const unsigned F = a.F, k = a.k, kt = a.kt, h1 = a.h1, hidden = a.hidden, m = a.m;
     const unsigned r0 = blockIdx.x * RC;                           // first region of this workgroup
     const unsigned nreg = r0 < a.nregion ? (a.nregion - r0 < RC ? a.nregion - r0 : RC) : 0u;
@@ -807,8 +813,8 @@ bool plan(const dbk_train_step_args* a, single_args& s, unsigned& MT, size_t& ld
     s.nparam = a->nparam;
     s.pstride = (a->nparam + a->nmodel + 63) & ~(size_t)63;
     if (a->nparam > 24576) return false;
-    const lds_map L = make_map(MT, s.Fp, s.nmodel, s.kt, s.k, s.h1, (unsigned)a->nparam, s.RC, a->ptype != DBK_PT_MAX);
-    lds_bytes = (size_t)L.total * 4;
+    s.L = make_map(MT, s.Fp, s.nmodel, s.kt, s.k, s.h1, (unsigned)a->nparam, s.RC, a->ptype != DBK_PT_MAX);
+    lds_bytes = (size_t)s.L.total * 4;
     return lds_bytes <= dbk_scan::lds_limit();
 }
 
@@ -853,9 +859,13 @@ extern "C" int dbk_train_step_single(dbk_stream_t stream, const dbk_train_step_a
     s.freeze_scan = a->freeze_scan; s.Z = a->Z; s.loss = a->loss;
     s.sync = (unsigned*)work;
     s.partial = (float*)((char*)work + WORK_HEADER);
-    const bool one = s.nmodel == 1 && s.RC == 1 && s.Fp == 16;
-    auto kern = one ? (MT == 16 ? k_step_single<16, true> : (MT == 24 ? k_step_single<24, true> : k_step_single<32, true>))
-                    : (MT == 16 ? k_step_single<16, false> : (MT == 24 ? k_step_single<24, false> : k_step_single<32, false>));
+    const int shape = s.RC != 1 ? 0 : (s.Fp == 32 ? 3 : s.Fp == 64 ? 4 : s.nmodel == 1 ? 2 : 1);
+    auto pick = [&](auto mt) {
+        constexpr int M = decltype(mt)::value;
+        return shape == 4 ? k_step_single<M, 4> : shape == 3 ? k_step_single<M, 3> : shape == 2 ? k_step_single<M, 2>
+             : shape == 1 ? k_step_single<M, 1> : k_step_single<M, 0>;
+    };
+    auto kern = MT == 16 ? pick(std::integral_constant<int, 16>{}) : (MT == 24 ? pick(std::integral_constant<int, 24>{}) : pick(std::integral_constant<int, 32>{}));
     DBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(kern, dim3(s.G), dim3(s.RC == 1 ? NTMAX : NTMIN), lds, dbk::as_stream(stream), s);
     DBK_LAUNCH_OK();
