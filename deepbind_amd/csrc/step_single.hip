@@ -34,7 +34,7 @@
 //                corr1ord.py:120-138)
 //
 // The barrier is a set of flags in the caller's workspace; every workgroup of the grid must be resident, so
-// the grid never exceeds 128 workgroups of at most 512 threads (a CU holds at least one), and the wait is bounded:
+// the grid never exceeds 256 workgroups of at most 512 threads (a CU holds at least one), and the wait is bounded:
 // a workgroup that gives up sets the workspace's status word and leaves without touching the parameters.
 // Results are deterministic (no float atomics; LDS atomics only OR bits), within the tolerances of the
 // multi-launch step but not its bits (other summation orders).
@@ -54,9 +54,11 @@ constexpr unsigned MAXROWS = 256;                 // rows of one region
 constexpr unsigned AW = MAXROWS / 32;             // words of rectifier bits per (region, filter)
 constexpr unsigned LW = AW + 2;                   // words of letter bits per (region, letter): rows + taps - 1 positions
 constexpr unsigned TXTB = 384;                    // staged letters per region (a dword-aligned copy, padded with "nothing")
-constexpr unsigned MAXG = 128;                    // workgroups of a launch
-constexpr size_t WORK_HEADER = 16384;              // bytes of the workspace before the shares: launch number, status, "go", flags
+constexpr unsigned MAXG = 256;                    // workgroups of a launch (all resident at once: a CU holds at least one)
+constexpr size_t WORK_HEADER = 32768;              // bytes of the workspace before the shares: launch number, status, "go", flags, pair words
 constexpr unsigned GO_AT = 32, FLAGS_AT = 64;     // words of the workspace: the "go" word; the first workgroup flag
+constexpr unsigned PAIR_AT = 2048;                // ... the predictions that the two workgroups of a (forward, reverse) pair show each other: [workgroup][model] 8 bytes
+constexpr unsigned STAMP_AT = 4096 + 2048;        // ... time stamps of a profiling build
 constexpr unsigned FLAG_STRIDE = 4;               // words from one workgroup's flag to the next (measured: 4 beats 1 and 16 by ~0.1 us per step)
 constexpr unsigned SPIN_LIMIT = 400000;           // polls of the barrier before a workgroup gives up (~0.2 s)
 
@@ -67,11 +69,11 @@ struct lds_map {
 struct single_args {
     unsigned nmodel, nfilter, F, Fp, lgFp, m, hidden, h1, k, kt, kf, ptype, loss_kind, revcomp;
     unsigned RC, G;                               // regions per workgroup, workgroups
-    size_t nparam, pstride;                       // parameters; floats of one workgroup's share (nparam + nmodel, padded)
+    unsigned nparam, pstride;                     // parameters; floats of one workgroup's share (nparam + nmodel, padded)
     float *P, *dP, *mP;
     const float *drate, *mrate, *decay;
-    size_t off_Wc, off_bc, off_W1, off_b1, off_W2, off_b2;
-    const uint8_t* X; size_t N;
+    unsigned off_Wc, off_bc, off_W1, off_b1, off_W2, off_b2;
+    const uint8_t* X; unsigned N;                 // (fewer than 2^32 - 256 rows: checked on the host)
     const uint32_t* R; unsigned nregion;
     const float* Y; const uint8_t* Ymask; const float* feats;
     const float* rate; unsigned long long seed; unsigned long long* counter; unsigned long long draws;
@@ -118,7 +120,7 @@ inline lds_map make_map(unsigned MT, unsigned Fp, unsigned nm, unsigned kt, unsi
 // first row in X; nscan: rows of X the scan defines (later rows read as bias only).
 template <int MT>
 __device__ __forceinline__ void scan_block(const float* __restrict__ wt, const unsigned* __restrict__ tw, unsigned start, unsigned Bq,
-                                           unsigned rows, size_t row0, size_t nscan, unsigned f, unsigned lgFp, float bf, bool want_bits,
+                                           unsigned rows, unsigned row0, unsigned nscan, unsigned f, unsigned lgFp, float bf, bool want_bits,
                                            unsigned* __restrict__ abits, float& mx, unsigned& xi, float& sum)
 {
     constexpr int WN = (MT + 6) / 4;                              // dwords covering the letters of four positions
@@ -162,7 +164,7 @@ __device__ __forceinline__ void scan_block(const float* __restrict__ wt, const u
 // 2-4 us per poll when every workgroup reads every other's flag, in lines of their own or side by side), so no word is
 // shared more than it must be: each workgroup
 // raises a flag of its own - the number of this launch, one more than the number the workspace
-// held when the kernel started; workgroup 0 alone reads all the flags (two per lane of its first wave) and, when
+// held when the kernel started; workgroup 0 alone reads all the flags (up to four per lane of its first wave) and, when
 // they all show the number, writes it to the "go" word; every other workgroup polls that one word with one lane.
 // Returns 0 when the step may go on, else the status to leave with (1: this workgroup gave up waiting; otherwise
 // what another workgroup flagged before it arrived).
@@ -182,9 +184,14 @@ __device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, uns
         bool done = false;
         if (blockIdx.x == 0) {
             for (;;) {
-                const unsigned v0 = lane < G ? __hip_atomic_load(&flags[lane * FLAG_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : launch;
-                const unsigned v1 = lane + 64 < G ? __hip_atomic_load(&flags[(lane + 64) * FLAG_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : launch;
-                done = __all(v0 == launch && v1 == launch);
+                unsigned v[MAXG / 64];
+#pragma unroll
+                for (unsigned u = 0; u < MAXG / 64; ++u)
+                    v[u] = lane + 64u * u < G ? __hip_atomic_load(&flags[(lane + 64u * u) * FLAG_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : launch;
+                bool mine = true;
+#pragma unroll
+                for (unsigned u = 0; u < MAXG / 64; ++u) mine = mine && v[u] == launch;
+                done = __all(mine);
                 if (dbg && tries == 0 && lane == 0) dbg[1] = (float)(wall_clock64() & 0xffffff);
                 if (done || ++tries >= SPIN_LIMIT) break;
                 __builtin_amdgcn_s_sleep(1);
@@ -240,8 +247,8 @@ __device__ __forceinline__ float wave_sum(float v)
 __device__ __forceinline__ void put_share(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 #ifdef DBK_STEP_PROF
-#define STAMP(i) do { if (threadIdx.x == 0) { const long long now_ = wall_clock64(); if (blockIdx.x == 0) reinterpret_cast<long long*>(a.sync + 3072)[i] = now_; \
-    if ((i) == 0 || (i) == 5 || (i) == 6) a.partial[(size_t)blockIdx.x * a.pstride + a.nparam + a.nmodel + ((i) == 0 ? 0 : (i) - 4)] = (float)(now_ & 0xffffff); } } while (0)
+#define STAMP(i) do { if (threadIdx.x == 0) { const long long now_ = wall_clock64(); if (blockIdx.x == 0) reinterpret_cast<long long*>(a.sync + STAMP_AT)[i] = now_; \
+    if ((i) == 0 || (i) == 5 || (i) == 6) a.partial[(unsigned)blockIdx.x * a.pstride + a.nparam + a.nmodel + ((i) == 0 ? 0 : (i) - 4)] = (float)(now_ & 0xffffff); } } while (0)
 #else
 #define STAMP(i) do {} while (0)
 #endif
@@ -306,7 +313,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         float vp[UN], vr[UN], vm[UN];
 #pragma unroll
         for (unsigned u = 0; u < UN; ++u) {
-            const size_t e = tid + u * NT;
+            const unsigned e = tid + u * NT;
             const bool in = e < a.nparam;
             vp[u] = in ? a.P[e] : 0.0f;
             vr[u] = in ? a.mrate[e] : 0.0f;
@@ -314,7 +321,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         }
         if (tid < RC && r0 + tid < a.nregion) { ra = a.R[2 * (r0 + tid)]; rb = a.R[2 * (r0 + tid) + 1]; }
         if (tid < RC * nm && r0 + by_nm.quot(tid) < a.nregion) {
-            const size_t i = (size_t)r0 * nm + tid;
+            const unsigned i = (unsigned)r0 * nm + tid;
             y = a.Y[i];
             if (a.Ymask) ym = a.Ymask[i];
         }
@@ -326,7 +333,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
 #pragma unroll
         for (unsigned u = 0; u < UN; ++u)
             if (tid + u * NT < a.nparam) Lk[tid + u * NT] = vp[u] + vr[u] * vm[u];
-        for (size_t e = tid + (size_t)UN * NT; e < a.nparam; e += NT) Lk[e] = a.P[e] + a.mrate[e] * a.mP[e];      // a long parameter vector: the rest
+        for (unsigned e = tid + (unsigned)UN * NT; e < a.nparam; e += NT) Lk[e] = a.P[e] + a.mrate[e] * a.mP[e];      // a long parameter vector: the rest
         if (tid < RC) {
             unsigned rows = rb > ra ? rb - ra : 0u;
             if (rows > MAXROWS) {                                  // not a shape this kernel takes: flag it, touch nothing of the region
@@ -345,7 +352,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     }
     for (unsigned e = tid; e < RC * nm * a.kf; e += NT) {          // the shared feature columns follow each model's own inputs
         const unsigned rl = by_nmkf.quot(e), rest = by_nmkf.rem(e, rl), b = by_kf.quot(rest), j = by_kf.rem(rest, b);
-        H0[(rl * nm + b) * kt + k + j] = (a.feats && rl < nreg) ? a.feats[((size_t)r0 + rl) * a.kf + j] : 0.0f;
+        H0[(rl * nm + b) * kt + k + j] = (a.feats && rl < nreg) ? a.feats[((unsigned)r0 + rl) * a.kf + j] : 0.0f;
     }
     for (unsigned e = tid; e < RC * 5 * LW; e += NT) lmask[e] = 0u;
     if (dense)
@@ -360,7 +367,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     auto letter_at = [&](unsigned e) -> unsigned {
         const unsigned rl = e / TXTB, q = e % TXTB;
         const unsigned rows = rinfo[2 * rl];
-        const size_t g = (size_t)rinfo[2 * rl + 1] + q;
+        const unsigned g = (unsigned)rinfo[2 * rl + 1] + q;
         return (rows && q < rows + MT - 1 && g < a.N) ? (unsigned)a.X[g] : 254u;
     };
     auto put_letter = [&](unsigned e, unsigned code) {
@@ -377,25 +384,25 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         const unsigned t = e >> lgFp, f = e & (Fp - 1u);
         float w0 = 0.0f, w1 = 0.0f, w2 = 0.0f, w3 = 0.0f;
         if (t < m && f < F) {
-            const float* w = Lk + a.off_Wc + (size_t)(4 * t) * F + f;
+            const float* w = Lk + a.off_Wc + (unsigned)(4 * t) * F + f;
             w0 = w[0]; w1 = w[F]; w2 = w[2 * F]; w3 = w[3 * F];
         }
         float z = w0;
         z += w1;
         z += w2;
         z += w3;
-        float* row = wt + (size_t)t * NL * Fp + f;
+        float* row = wt + (unsigned)t * NL * Fp + f;
         row[0 * Fp] = w0; row[1 * Fp] = w1; row[2 * Fp] = w2; row[3 * Fp] = w3;
         row[4 * Fp] = z * 0.25f;
         row[5 * Fp] = 0.0f;
     }
     // which pooled features the dropout keeps (element numbering of the stand-alone kernels): drawn now, while the letters travel
     {
-        const size_t ncol = (size_t)k * nm;
+        const unsigned ncol = (unsigned)k * nm;
         const unsigned long long off = (unsigned long long)misc[1] << 32 | misc[0];
         for (unsigned e = NT - 1u - tid; e < RC * nm * k; e += NT) {      // (the last threads first: the first ones build the table)
             const unsigned rl = by_nmk.quot(e), col = by_nmk.rem(e, rl), b = by_k.quot(col);
-            const size_t rr = (size_t)r0 + rl;
+            const unsigned rr = (unsigned)r0 + rl;
             bool kp = true;
             if (rl < nreg && a.rate) kp = dbk_rng::uniform_at(a.seed, off, (a.revcomp ? (rr >> 1) : rr) * ncol + col) >= rates[b];
             kept[e] = kp;
@@ -416,7 +423,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     const unsigned lgNG4 = (NT == NTMAX ? 3u : 2u) + 6u - lgFp + 2u;                            // log2(4 * NG): NT is 256 or 512
     const unsigned f = lane & (Fp - 1), gidx = wave * PG + (lane >> lgFp);
     const float bf = f < F ? Lk[a.off_bc + f] : 0.0f;
-    const size_t nscan = a.N + 1 >= (size_t)m + 1 ? a.N - m + 1 : 0;
+    const unsigned nscan = a.N + 1 >= (unsigned)m + 1 ? a.N - m + 1 : 0;
     for (unsigned rl = 0; rl < nreg; ++rl) {
         const unsigned rows = rinfo[2 * rl];
         const unsigned Bq = 4u * ((rows + 4u * NG - 1u) >> lgNG4);
@@ -460,7 +467,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             if (bi == 0xffffffffu) bi = 0u;
             argp[rl * Fp + tid] = bi;
             if (tid < F) {
-                float* out = PL + (size_t)rl * nm * k + (size_t)tid * kpf;
+                float* out = PL + (unsigned)rl * nm * k + (unsigned)tid * kpf;
                 const float mean = rows ? bs / (float)rows : 0.0f;
                 if (a.ptype == DBK_PT_MAX) out[0] = bm;
                 else if (a.ptype == DBK_PT_AVG) out[0] = mean;
@@ -487,7 +494,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             float hv = 0.0f, w2 = 0.0f, part = 0.0f;               // lane h: hidden unit h and its output weight
             if (hidden) {
                 if (lane < hidden) {
-                    const float* wcol = W1s + (size_t)b * kt * hidden + lane;
+                    const float* wcol = W1s + (unsigned)b * kt * hidden + lane;
                     float sacc = 0.0f;
 #pragma unroll 8
                     for (unsigned kk = 0; kk < kt; ++kk) sacc += x[kk] * wcol[kk * hidden];
@@ -498,15 +505,39 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
                     part += hv * w2;
                 }
             } else {
-                for (unsigned kk = lane; kk < kt; kk += 64) part += x[kk] * W1s[(size_t)b * kt + kk];
+                for (unsigned kk = lane; kk < kt; kk += 64) part += x[kk] * W1s[(unsigned)b * kt + kk];
             }
             part = wave_sum(part);
             const float out = part + (hidden ? b2s[b] : b1s[b]);
             // (the logistic through the hardware's exponential and reciprocal, as the reference's kernels are built: -use_fast_math)
             const float z = a.loss_kind == 0 ? __builtin_amdgcn_rcpf(1.0f + __expf(-out)) : out;
+            bool use = live && Yms[b] != 0u;
+            if (a.revcomp) {
+                // Of a (forward, reverse) pair of rows only the larger prediction trains; ties keep the first row. The
+                // partner row is the neighbouring workgroup's: the two show each other their predictions through one
+                // 8-byte word each (the number of this launch beside the value, so that a word left by the launch before
+                // is not taken for it), one trip through memory. The wait is bounded like the barrier's.
+                unsigned long long* words = reinterpret_cast<unsigned long long*>(a.sync + PAIR_AT);
+                const unsigned launch = misc[2];
+                unsigned long long seen = 0ull;
+                if (lane == 0) {
+                    __hip_atomic_store(&words[(unsigned)blockIdx.x * 4u + b], ((unsigned long long)launch << 32) | __float_as_uint(z),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const unsigned long long* theirs = &words[(unsigned)(blockIdx.x ^ 1u) * 4u + b];
+                    for (unsigned tries = 0; tries < SPIN_LIMIT; ++tries) {
+                        seen = __hip_atomic_load(theirs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if ((unsigned)(seen >> 32) == launch) break;
+                        __builtin_amdgcn_s_sleep(1);
+                    }
+                    if ((unsigned)(seen >> 32) != launch) atomicExch(&a.sync[1], 1u);      // gave up: the grid barrier ends the step without an update
+                }
+                const unsigned tag = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(seen >> 32));
+                const float zo = __uint_as_float((unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)seen));
+                use = use && tag == launch && ((r0 & 1u) ? !(zo >= z) : (z >= zo));
+            }
             float dA = 0.0f;
-            if (live && Yms[b] != 0u) dA = (z - Ys[b]) * inv_n;
-            if (lane == 0) { zs[b] = z; dAs[b] = dA; }             // (the loss term is formed later, off this wave's path)
+            if (use) dA = (z - Ys[b]) * inv_n;
+            if (lane == 0) { zs[b] = z; dAs[b] = dA; lss[b] = use ? 1.0f : 0.0f; }      // (the loss term is formed later, off this wave's path, where lss says so)
             if (hidden && lane < hidden) D1[b * hidden + lane] = hv > 0.0f ? dA * w2 : 0.0f;
             wave_lds_sync();
             // gradient at the pooled features -> what the scan's backward pass needs
@@ -525,7 +556,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
                 const unsigned kk = lane & ((1u << lgkP) - 1u), hq = lane >> lgkP;
                 float g = 0.0f;
                 if (kk < k) {
-                    const float* wrow = W1s + ((size_t)b * kt + kk) * hidden + hq * hs;
+                    const float* wrow = W1s + ((unsigned)b * kt + kk) * hidden + hq * hs;
                     const float* drow = D1 + b * hidden + hq * hs;
 #pragma unroll 8
                     for (unsigned j = 0; j < hs; ++j) {
@@ -540,11 +571,11 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
                     float g;
                     if (hidden) {
                         g = 0.0f;
-                        const float* wrow = W1s + ((size_t)b * kt + kk) * hidden;
+                        const float* wrow = W1s + ((unsigned)b * kt + kk) * hidden;
 #pragma unroll 8
                         for (unsigned h = 0; h < hidden; ++h) g += D1[b * hidden + h] * wrow[h];
                     } else {
-                        g = dA * W1s[(size_t)b * kt + kk];
+                        g = dA * W1s[(unsigned)b * kt + kk];
                     }
                     put_pool_grad(kk, g);
                 }
@@ -561,7 +592,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             for (unsigned e = tid; e < RC * nm * hidden; e += NT) {
                 const unsigned rb = by_h1.quot(e), h = by_h1.rem(e, rb), b = by_nm.rem(rb, by_nm.quot(rb));
                 const float* x = H0 + rb * kt;
-                const float* wcol = W1s + (size_t)b * kt * hidden + h;
+                const float* wcol = W1s + (unsigned)b * kt * hidden + h;
                 float s = 0.0f;
 #pragma unroll 8
                 for (unsigned kk = 0; kk < kt; ++kk) s += x[kk] * wcol[kk * hidden];
@@ -576,9 +607,9 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             const unsigned b = by_nm.rem(e, by_nm.quot(e));
             float part = 0.0f;
             if (hidden) {
-                for (unsigned h = lane; h < hidden; h += 64) part += H1[(size_t)e * hidden + h] * W2s[b * hidden + h];
+                for (unsigned h = lane; h < hidden; h += 64) part += H1[(unsigned)e * hidden + h] * W2s[b * hidden + h];
             } else {
-                for (unsigned kk = lane; kk < kt; kk += 64) part += H0[(size_t)e * kt + kk] * W1s[(size_t)b * kt + kk];
+                for (unsigned kk = lane; kk < kt; kk += 64) part += H0[(unsigned)e * kt + kk] * W1s[(unsigned)b * kt + kk];
             }
 #pragma unroll
             for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
@@ -592,7 +623,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         // loss gradient of (row, model), formed by every thread that needs it; the hidden units' gradients with it
         for (unsigned e = tid; e < RC * nm * h1; e += NT) {
             const unsigned rb = by_h1.quot(e), h = by_h1.rem(e, rb), rl = by_nm.quot(rb), b = by_nm.rem(rb, rl);
-            const size_t rr = (size_t)r0 + rl;
+            const unsigned rr = (unsigned)r0 + rl;
             float dA = 0.0f, lterm = 0.0f;
             if (rl < nreg) {
                 const float z = zs[rb], y = Ys[rb];
@@ -617,11 +648,11 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             float g;
             if (hidden) {
                 g = 0.0f;
-                const float* wrow = W1s + ((size_t)b * kt + kk) * hidden;
+                const float* wrow = W1s + ((unsigned)b * kt + kk) * hidden;
 #pragma unroll 8
-                for (unsigned h = 0; h < hidden; ++h) g += D1[(size_t)rb * hidden + h] * wrow[h];
+                for (unsigned h = 0; h < hidden; ++h) g += D1[(unsigned)rb * hidden + h] * wrow[h];
             } else {
-                g = dAs[rb] * W1s[(size_t)b * kt + kk];
+                g = dAs[rb] * W1s[(unsigned)b * kt + kk];
             }
             if (!kept[e]) g = 0.0f;
             const unsigned fl = b * a.nfilter + (kk >> (kpf - 1u));   // filter of the group
@@ -635,13 +666,13 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     // (from here to the grid barrier nothing waits for a store to global memory: the shares travel while the filter
     // gradients are counted)
     // this workgroup's share of the dense layers' gradients and of the loss, rows ascending
-    float* share = a.partial + (size_t)blockIdx.x * a.pstride;
+    float* share = a.partial + (unsigned)blockIdx.x * a.pstride;
     for (unsigned e = tid; e < nm * kt * h1; e += NT) {
         const unsigned q1 = by_h1.quot(e), h = by_h1.rem(e, q1), b = by_kt.quot(q1), kk = by_kt.rem(q1, b);
         float s = 0.0f;
         for (unsigned rl = 0; rl < RC; ++rl) {
             const unsigned rb = rl * nm + b;
-            s += H0[(size_t)rb * kt + kk] * (hidden ? D1[(size_t)rb * hidden + h] : dAs[rb]);
+            s += H0[(unsigned)rb * kt + kk] * (hidden ? D1[(unsigned)rb * hidden + h] : dAs[rb]);
         }
         put_share(&share[a.off_W1 + e], s);
     }
@@ -650,7 +681,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         float gb1 = 0.0f, gW2 = 0.0f;
         for (unsigned rl = 0; rl < RC; ++rl) {
             const unsigned rb = rl * nm + b;
-            if (hidden) { gb1 += D1[(size_t)rb * hidden + h]; gW2 += H1[(size_t)rb * hidden + h] * dAs[rb]; }
+            if (hidden) { gb1 += D1[(unsigned)rb * hidden + h]; gW2 += H1[(unsigned)rb * hidden + h] * dAs[rb]; }
             else gb1 += dAs[rb];
         }
         put_share(&share[a.off_b1 + e], gb1);
@@ -660,7 +691,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         float gb2 = 0.0f, ls = 0.0f;
         if (RC == 1u) {
             gb2 = dAs[b];
-            if (nreg && Yms[b] != 0u) {
+            if (lss[b] != 0.0f) {
                 const float z = zs[b], y = Ys[b];
                 ls = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
             }
@@ -670,7 +701,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         if (hidden) put_share(&share[a.off_b2 + b], gb2);
         put_share(&share[a.nparam + b], ls);
     }
-    for (unsigned e = tid; e < nreg * nm; e += NT) put_share(&a.Z[(size_t)r0 * nm + e], zs[e]);      // the predictions of this workgroup's rows
+    for (unsigned e = tid; e < nreg * nm; e += NT) put_share(&a.Z[(unsigned)r0 * nm + e], zs[e]);      // the predictions of this workgroup's rows
 
     STAMP(4);
     // ---------------- scan filters: a thread's (tap, filter) pairs, five letter accumulators each, regions ascending
@@ -712,7 +743,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         }
         if (t < m && fl < F) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) put_share(&share[a.off_Wc + (size_t)(4 * t + c) * F + fl], acc[c] + 0.25f * acc[4]);
+            for (int c = 0; c < 4; ++c) put_share(&share[a.off_Wc + (unsigned)(4 * t + c) * F + fl], acc[c] + 0.25f * acc[4]);
         }
         if (t == 0 && fl < F) put_share(&share[a.off_bc + fl], accb);
     }
@@ -723,15 +754,15 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     // A workgroup steps 64 consecutive parameters: wave w adds the shares of its run of workgroups for them (a lane per
     // parameter: every load of a wave is one contiguous 256 bytes), the waves' sums meet in LDS and wave 0 adds them in a
     // fixed tree and applies the step.
-    const size_t total = a.nparam + nm, estep = (size_t)a.G * 64;
-    const size_t efirst = (size_t)blockIdx.x * 64 + lane;
+    const unsigned total = a.nparam + nm, estep = (unsigned)a.G * 64;
+    const unsigned efirst = (unsigned)blockIdx.x * 64 + lane;
     float q_p = 0.0f, q_rm = 0.0f, q_mp = 0.0f, q_dr = 0.0f, q_dec = 0.0f;
     if (wave == 0 && efirst < a.nparam) {
         q_p = a.P[efirst]; q_rm = a.mrate[efirst]; q_mp = a.mP[efirst]; q_dr = a.drate[efirst];
         if (a.decay) q_dec = a.decay[efirst];
     }
 #ifdef DBK_STEP_PROF
-    if (grid_barrier(a.sync, a.G, misc[2], a.partial + (size_t)blockIdx.x * a.pstride + a.nparam + a.nmodel + 3) != 0u) return;
+    if (grid_barrier(a.sync, a.G, misc[2], a.partial + (unsigned)blockIdx.x * a.pstride + a.nparam + a.nmodel + 3) != 0u) return;
 #else
     if (grid_barrier(a.sync, a.G, misc[2]) != 0u) return;
 #endif
@@ -741,20 +772,20 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     float* sums = wt;                                              // (the letter table is no longer needed)
     const unsigned per = (a.G + NW - 1) / NW;                      // workgroups each wave adds, ascending
     const unsigned g0 = wave * per, g1 = g0 + per < a.G ? g0 + per : a.G;
-    for (size_t base = (size_t)blockIdx.x * 64; base < total; base += estep) {
-        const size_t e = base + lane;
+    for (unsigned base = (unsigned)blockIdx.x * 64; base < total; base += estep) {
+        const unsigned e = base + lane;
         float s = 0.0f;
         if (e < total) {
             for (unsigned c0 = g0; c0 < g1; c0 += 16) {           // all of a wave's workgroups requested at once (a full grid: 16)
                 float v[16];
 #pragma unroll
-                for (unsigned u = 0; u < 16; ++u) v[u] = c0 + u < g1 ? a.partial[(size_t)(c0 + u) * a.pstride + e] : 0.0f;
+                for (unsigned u = 0; u < 16; ++u) v[u] = c0 + u < g1 ? a.partial[(unsigned)(c0 + u) * a.pstride + e] : 0.0f;
 #pragma unroll
                 for (unsigned u = 0; u < 16; ++u)
                     if (c0 + u < g1) s += v[u];
             }
         }
-        if (base != (size_t)blockIdx.x * 64) __syncthreads();      // (a further round: the sums of the last one have been read)
+        if (base != (unsigned)blockIdx.x * 64) __syncthreads();      // (a further round: the sums of the last one have been read)
         sums[wave * 64 + lane] = s;
         __syncthreads();
         if (wave != 0 || e >= total) continue;
@@ -773,7 +804,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         float g = s;
         const float lk = q_p + q_rm * q_mp;
         if (a.decay) g += (float)((lk > 0.0f) - (lk < 0.0f)) * q_dec;
-        if (a.freeze_scan && e - a.off_Wc < (size_t)4 * m * F) g = 0.0f;
+        if (a.freeze_scan && e - a.off_Wc < (unsigned)4 * m * F) g = 0.0f;
         a.dP[e] = g;
         const float delta = g * q_dr;
         a.mP[e] = q_mp * q_rm - delta;
@@ -805,13 +836,13 @@ bool plan(const dbk_train_step_args* a, single_args& s, unsigned& MT, size_t& ld
     // regions per workgroup: as few as keep the grid within MAXG workgroups (one region: eight waves share it),
     // an even number with reverse-complement pairs (a pair's two rows meet in one workgroup)
     unsigned RC = (unsigned)((a->nregion + MAXG - 1) / MAXG);
-    if (a->reverse_complement) RC += RC & 1u;
+    if (a->reverse_complement && RC > 1) RC += RC & 1u;        // (one region per workgroup: the pair's workgroups are neighbours)
     if (RC > 16) return false;
     s.RC = RC;
     s.G = (unsigned)((a->nregion + RC - 1) / RC);
     if (s.G > MAXG) return false;
-    s.nparam = a->nparam;
-    s.pstride = (a->nparam + a->nmodel + 63) & ~(size_t)63;
+    s.nparam = (unsigned)a->nparam;               // (at most 24576: checked below)
+    s.pstride = (unsigned)((a->nparam + a->nmodel + 63) & ~(size_t)63);
     if (a->nparam > 24576) return false;
     s.L = make_map(MT, s.Fp, s.nmodel, s.kt, s.k, s.h1, (unsigned)a->nparam, s.RC, a->ptype != DBK_PT_MAX);
     lds_bytes = (size_t)s.L.total * 4;
@@ -851,8 +882,9 @@ extern "C" int dbk_train_step_single(dbk_stream_t stream, const dbk_train_step_a
     const size_t need[6] = { a->off_Wc + nWc, a->off_bc + F, a->off_W1 + nW1, a->off_b1 + nb1, a->off_W2 + nW2, a->off_b2 + nb2 };
     for (size_t v : need) DBK_CHECK(v <= a->nparam, "ValueError: a parameter block reaches past the flat vector (%zu > %zu)", v, a->nparam);
     s.P = a->P; s.dP = a->dP; s.mP = a->mP; s.drate = a->drate; s.mrate = a->mrate; s.decay = a->decay;
-    s.off_Wc = a->off_Wc; s.off_bc = a->off_bc; s.off_W1 = a->off_W1; s.off_b1 = a->off_b1; s.off_W2 = a->off_W2; s.off_b2 = a->off_b2;
-    s.X = a->X; s.N = a->N; s.R = a->regions; s.nregion = (unsigned)a->nregion;
+    s.off_Wc = (unsigned)a->off_Wc; s.off_bc = (unsigned)a->off_bc; s.off_W1 = (unsigned)a->off_W1;       // (all below nparam: checked above)
+    s.off_b1 = (unsigned)a->off_b1; s.off_W2 = (unsigned)a->off_W2; s.off_b2 = (unsigned)a->off_b2;
+    s.X = a->X; s.N = (unsigned)a->N; s.R = a->regions; s.nregion = (unsigned)a->nregion;
     s.Y = a->Y; s.Ymask = a->Ymask; s.feats = a->feats;
     s.rate = a->rate; s.seed = a->seed; s.counter = (unsigned long long*)a->counter;
     s.draws = a->rate ? (a->nregion * s.k * a->nmodel + 3) / 4 : 0;

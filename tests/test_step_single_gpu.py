@@ -44,8 +44,11 @@ CASES = [
     ("avg", 8, "nll", 2, 16, 11, 60, (12, 70), False, 0),
     ("all", 32, "nll", 4, 16, 24, 50, (20, 40), False, 16),
     ("max", 0, "mse", 3, 12, 9, 33, (5, 30), False, 0),            # 36 filters: padded to 64 lanes
-    ("all", 16, "nll", 2, 16, 20, 64, (30, 200), True, 0),         # reverse-complement pairs, regions up to 219 rows
-    ("max", 32, "nll", 1, 16, 32, 300, (20, 60), False, 16),       # four regions per workgroup
+    ("all", 16, "nll", 2, 16, 20, 64, (30, 200), True, 0),         # reverse-complement pairs (a pair's rows in neighbouring workgroups), regions up to 219 rows
+    ("all", 16, "nll", 2, 16, 20, 150, (30, 120), True, 0),        # reverse-complement pairs, two regions (one pair) per workgroup
+    ("max", 32, "nll", 1, 16, 24, 64, (30, 101), True, 0),         # one model, reverse-complement pairs, one region per workgroup
+    ("max", 32, "nll", 1, 16, 24, 200, (20, 60), False, 0),        # 200 workgroups
+    ("max", 32, "nll", 1, 16, 32, 600, (20, 60), False, 16),       # three regions per workgroup
     # one 16-filter model, one region per workgroup (the instance with that shape compiled in), its other branches:
     ("all", 32, "nll", 1, 16, 24, 100, (20, 90), False, 0),        # 32 pooled features into a hidden layer (two lane groups per feature)
     ("avg", 20, "mse", 1, 12, 32, 77, (8, 50), False, 16),         # 12 filters in 16 lanes, 32 taps, shared feature columns, a hidden width the lane groups do not divide
