@@ -30,17 +30,19 @@ namespace {
 //   * adds the L1 term, zeroes the scan filters' gradient while they are frozen, stores the gradient,
 //   * applies the Nesterov update and forms the next step's look-ahead,
 //   * writes the per-model loss when asked and moves the dropout generator on.
+// (Sizes and offsets are 32-bit: the host checks that the flat vector and a slab have fewer than 2^31 elements. With
+// 64-bit fields the kernel spilled a hundred scalar registers and divided 64-bit numbers per element.)
 struct reduce_update_args {
-    size_t nparam;
+    unsigned nparam;
     float *P, *L, *dP, *mP;
     const float *drate, *mrate, *decay;
-    size_t off_Wc, off_bc, off_W1, off_b1, off_W2, off_b2;
-    size_t nWc, nbc, nW1, nb1, nW2, nb2;
-    const float* slabs; size_t slab_stride; unsigned nslab;
+    unsigned off_Wc, off_bc, off_W1, off_b1, off_W2, off_b2;
+    unsigned nWc, nbc, nW1, nb1, nW2, nb2;
+    const float* slabs; unsigned slab_stride; unsigned nslab;
     const float* head_partial; unsigned nchunk, pstride;
     unsigned nblock, k, h1, hidden;                                // k: rows of a model's block of W1
     int freeze_scan, loss_kind;
-    float* loss; size_t nrow;
+    float* loss; unsigned nrow;
     unsigned long long* counter; unsigned long long counter_advance;
 };
 
@@ -62,8 +64,8 @@ __device__ __forceinline__ float chunk_sum(const reduce_update_args& a, unsigned
 __device__ __forceinline__ void reduce_update_body(const reduce_update_args& a, const unsigned bx, const unsigned gx)
 {
     const unsigned nW1m = a.k * a.h1;                              // dense weights per model
-    const size_t total = a.nparam + (a.loss ? a.nblock : 0);
-    for (size_t e = (size_t)bx * blockDim.x + threadIdx.x; e < total; e += (size_t)gx * blockDim.x) {
+    const unsigned total = a.nparam + (a.loss ? a.nblock : 0u);
+    for (unsigned e = bx * blockDim.x + threadIdx.x; e < total; e += gx * blockDim.x) {
         if (e >= a.nparam) {                                       // per-model loss
             const unsigned b = (unsigned)(e - a.nparam);
             const float s = chunk_sum(a, b, nW1m + 2 * a.h1 + 1);
@@ -74,10 +76,10 @@ __device__ __forceinline__ void reduce_update_body(const reduce_update_args& a, 
         bool scan_weight = false;
         if (e - a.off_Wc < a.nWc) { g = dbk_scan::slab_sum(a.slabs, a.slab_stride, e - a.off_Wc, a.nslab); scan_weight = true; }
         else if (e - a.off_bc < a.nbc) g = dbk_scan::slab_sum(a.slabs, a.slab_stride, a.nWc + (e - a.off_bc), a.nslab);
-        else if (e - a.off_W1 < a.nW1) { const size_t q = e - a.off_W1; g = chunk_sum(a, (unsigned)(q / nW1m), (unsigned)(q % nW1m)); }
-        else if (e - a.off_b1 < a.nb1) { const size_t q = e - a.off_b1; g = chunk_sum(a, (unsigned)(q / a.h1), nW1m + (unsigned)(q % a.h1)); }
-        else if (e - a.off_W2 < a.nW2) { const size_t q = e - a.off_W2; g = chunk_sum(a, (unsigned)(q / a.hidden), nW1m + a.h1 + (unsigned)(q % a.hidden)); }
-        else { const size_t q = e - a.off_b2; g = chunk_sum(a, (unsigned)q, nW1m + 2 * a.h1); }
+        else if (e - a.off_W1 < a.nW1) { const unsigned q = e - a.off_W1, b = q / nW1m; g = chunk_sum(a, b, q - b * nW1m); }
+        else if (e - a.off_b1 < a.nb1) { const unsigned q = e - a.off_b1, b = q / a.h1; g = chunk_sum(a, b, nW1m + (q - b * a.h1)); }
+        else if (e - a.off_W2 < a.nW2) { const unsigned q = e - a.off_W2, b = q / a.hidden; g = chunk_sum(a, b, nW1m + a.h1 + (q - b * a.hidden)); }
+        else { const unsigned q = e - a.off_b2; g = chunk_sum(a, q, nW1m + 2 * a.h1); }
         const float look = a.L[e];
         if (a.decay) {
             const float sg = (float)((look > 0.0f) - (look < 0.0f));
@@ -187,15 +189,17 @@ int drop_inputs(dbk_stream_t stream, const dbk_train_step_args* a)
 int fill_update(reduce_update_args& u, const dbk_train_step_args* a, const block_sizes& z, const float* slabs, size_t slab_stride,
                 unsigned nslab, const float* head_partial, unsigned nchunk, unsigned pstride, uint64_t draws)
 {
-    u.nparam = a->nparam;
+    DBK_CHECK(a->nparam < ((size_t)1 << 31) && slab_stride < ((size_t)1 << 31) && a->nregion < ((size_t)1 << 31),
+              "ValueError: a group's flat parameter vector is limited to 2^31 elements");
+    u.nparam = (unsigned)a->nparam;
     u.P = a->P; u.L = a->L; u.dP = a->dP; u.mP = a->mP; u.drate = a->drate; u.mrate = a->mrate; u.decay = a->decay;
-    u.off_Wc = a->off_Wc; u.off_bc = a->off_bc; u.off_W1 = a->off_W1; u.off_b1 = a->off_b1;
-    u.off_W2 = a->hidden ? a->off_W2 : a->nparam; u.off_b2 = a->hidden ? a->off_b2 : a->nparam;
-    u.nWc = z.nWc; u.nbc = z.F; u.nW1 = z.nW1; u.nb1 = z.nb1; u.nW2 = z.nW2; u.nb2 = z.nb2;
-    u.slabs = slabs; u.slab_stride = slab_stride; u.nslab = nslab;
+    u.off_Wc = (unsigned)a->off_Wc; u.off_bc = (unsigned)a->off_bc; u.off_W1 = (unsigned)a->off_W1; u.off_b1 = (unsigned)a->off_b1;
+    u.off_W2 = (unsigned)(a->hidden ? a->off_W2 : a->nparam); u.off_b2 = (unsigned)(a->hidden ? a->off_b2 : a->nparam);
+    u.nWc = (unsigned)z.nWc; u.nbc = (unsigned)z.F; u.nW1 = (unsigned)z.nW1; u.nb1 = (unsigned)z.nb1; u.nW2 = (unsigned)z.nW2; u.nb2 = (unsigned)z.nb2;
+    u.slabs = slabs; u.slab_stride = (unsigned)slab_stride; u.nslab = nslab;
     u.head_partial = head_partial; u.nchunk = nchunk; u.pstride = pstride;
     u.nblock = (unsigned)a->nmodel; u.k = (unsigned)z.kt; u.h1 = (unsigned)(a->hidden ? a->hidden : 1); u.hidden = (unsigned)a->hidden;
-    u.freeze_scan = a->freeze_scan; u.loss_kind = a->loss_kind; u.loss = a->loss; u.nrow = a->nregion;
+    u.freeze_scan = a->freeze_scan; u.loss_kind = a->loss_kind; u.loss = a->loss; u.nrow = (unsigned)a->nregion;
     u.counter = (unsigned long long*)a->counter; u.counter_advance = draws;
     DBK_CHECK(z.nWc + z.F + z.nW1 + z.nb1 + z.nW2 + z.nb2 == a->nparam, "ValueError: the parameter blocks do not tile the flat vector (%zu of %zu elements)",
               z.nWc + z.F + z.nW1 + z.nb1 + z.nW2 + z.nb2, a->nparam);
