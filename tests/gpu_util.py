@@ -42,7 +42,7 @@ def assert_close_per_model(got, ref, rel, nmodel, axis, what=""):
 
 
 # Worst elementwise relative errors seen by the parity tests, printed in the run's summary
-# (tests/conftest.py) and written to gpurun_out/parity_elementwise.json when that folder exists.
+# (tests/conftest.py) and written as parity_elementwise.json to the run's output folder when there is one.
 # err_rel = |got - ref| / max(|ref|, FLOOR_FRAC * max|ref| of the compared block): a pure elementwise ratio
 # is meaningless where a sum of signed terms cancels to ~0, so magnitudes below a thousandth of the block's
 # largest are measured against that floor; `share_within` is the share of elements inside the stated
