@@ -444,15 +444,17 @@ int dbk_train_step(dbk_stream_t stream, const dbk_train_step_args* args);
  * all sampled models on the same batches (deepity/deepity/hpsearch.py:314-330, sgd.py:98-135). */
 int dbk_train_steps(dbk_stream_t stream, size_t ngroup, const dbk_train_step_args* const* args);
 /* The same step for a SMALL group in ONE launch: 1-4 models with at most 64 filters (of at most 32 taps) between
- * them, Nesterov momentum, no input dropout, at most 2048 regions of at most 256 rows each. A workgroup takes a few
- * regions through forward, dense head and backward without leaving the CU, and after one grid-wide barrier
- * (bounded wait) all workgroups add up their shares of the gradient in a fixed order and apply the update.
+ * them, Nesterov momentum, no input dropout, at most 4096 regions of at most 256 rows each. A workgroup takes one
+ * region (up to 256 regions; a few beyond) through forward, dense head and backward without leaving the CU, and after
+ * one grid-wide barrier (bounded wait) all workgroups add up their shares of the gradient in a fixed order and apply
+ * the update. With reverse-complement pairs and one region per workgroup, the two workgroups of a pair show each other
+ * their predictions through the workspace (bounded wait, status 1 if it runs out).
  * Reads pooled / argmax / dpooled / act / L of the block not at all (weights come from P + mrate * mP); writes Z,
  * dP, mP, P, loss and advances the generator position. Deterministic; within the tolerances of dbk_train_step,
  * not its bits (other summation orders).
  * work: caller-owned device memory of dbk_train_step_single_workspace() bytes, 16-byte aligned, ZERO before its
- * first use and from then on passed unchanged to every call with the same nregion (word 0 is the barrier's ticket
- * counter; word 1 a status the kernel sets: 1 = a workgroup gave up waiting at the barrier, 2 = a region had more
+ * first use and from then on passed unchanged to every call with the same nregion (word 0 is the number of the last
+ * launch; word 1 a status the kernel sets: 1 = a workgroup gave up waiting at the barrier, 2 = a region had more
  * than 256 rows; with a non-zero status the parameters are left untouched). Calls that share a workspace must not
  * overlap. *work_bytes = 0 from the query means the shape is not taken (use dbk_train_step).
  * reference: the body of the trainer's loop, deepity/deepity/sgd.py:98-135, as dbk_train_step. */
