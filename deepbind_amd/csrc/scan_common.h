@@ -387,5 +387,19 @@ inline size_t lds_limit()
     return cached[dev];
 }
 
+inline unsigned cu_count()
+{
+    // compute units of the current device (asked once per device); 1 when the question fails
+    static unsigned cached[64] = {0};
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 1u;
+    if (!cached[dev]) {
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            cached[dev] = (unsigned)v;
+        else
+            cached[dev] = 1u;
+    }
+    return cached[dev];
+}
 
 }  // namespace dbk_scan

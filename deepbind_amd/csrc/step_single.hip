@@ -34,7 +34,8 @@
 //                corr1ord.py:120-138)
 //
 // The barrier is a set of flags in the caller's workspace; every workgroup of the grid must be resident, so
-// the grid never exceeds 256 workgroups of at most 512 threads (a CU holds at least one), and the wait is bounded:
+// the grid never exceeds 256 workgroups of at most 512 threads, nor the device's number of CUs (a CU holds at least
+// one), and the wait is bounded:
 // a workgroup that gives up sets the workspace's status word and leaves without touching the parameters.
 // Results are deterministic (no float atomics; LDS atomics only OR bits), within the tolerances of the
 // multi-launch step but not its bits (other summation orders).
@@ -835,12 +836,14 @@ bool plan(const dbk_train_step_args* a, single_args& s, unsigned& MT, size_t& ld
     MT = a->m <= 16 ? 16u : (a->m <= 24 ? 24u : 32u);
     // regions per workgroup: as few as keep the grid within MAXG workgroups (one region: eight waves share it),
     // an even number with reverse-complement pairs (a pair's two rows meet in one workgroup)
-    unsigned RC = (unsigned)((a->nregion + MAXG - 1) / MAXG);
+    // (every workgroup must be resident while the grid waits at the barrier: no more of them than the device has CUs)
+    const unsigned cus = dbk_scan::cu_count(), maxg = cus < MAXG ? cus : MAXG;
+    unsigned RC = (unsigned)((a->nregion + maxg - 1) / maxg);
     if (a->reverse_complement && RC > 1) RC += RC & 1u;        // (one region per workgroup: the pair's workgroups are neighbours)
     if (RC > 16) return false;
     s.RC = RC;
     s.G = (unsigned)((a->nregion + RC - 1) / RC);
-    if (s.G > MAXG) return false;
+    if (s.G > maxg) return false;
     s.nparam = (unsigned)a->nparam;               // (at most 24576: checked below)
     s.pstride = (unsigned)((a->nparam + a->nmodel + 63) & ~(size_t)63);
     if (a->nparam > 24576) return false;
