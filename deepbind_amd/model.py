@@ -60,6 +60,7 @@ class SequenceNet(object):
         # (dbk_train_step_single) unless this is switched off; same numbers within tolerance, other summation orders
         self.single_launch = bool(single_launch)
         self._single_rows = {}               # longest region of the region tables seen, by (pointer, version, regions)
+        self._single_calls = 0               # single-launch steps issued (their status word is looked at now and then)
         self.step_count = 0
         self._step_args = None               # argument block and work buffers of the natively issued step
         self._step_bufs = {}
@@ -584,6 +585,9 @@ class SequenceNet(object):
         if work is not None:
             _lib.call("dbk_train_step_single", _lib.stream(), ctypes.addressof(self._step_args), _lib.ptr(work), work.numel())
             self._L_versions = None          # (this kernel forms the look-ahead itself and leaves none behind)
+            self._single_calls += 1
+            if self._single_calls % 4096 == 0 and not torch.cuda.is_current_stream_capturing():
+                self._check_single_status()  # a step that gave up leaves the parameters alone: do not train on in silence
         else:
             _lib.call("dbk_train_step", _lib.stream(), ctypes.addressof(self._step_args))
         self._finish_step(X, R)
