@@ -868,16 +868,20 @@ inline int launch_bprop_W_window(hipStream_t st, float* dW, size_t m, size_t F, 
 // Y (rows x 4m) = dZ (rows x F) . W^T (F x 4m), then dX[i, c] += sum_k Y[i - k, 4k + c]. Both operands are float32
 // data, so both enter as three bf16 pieces and six of the nine piece products are formed (hi.hi, hi.mid, mid.hi,
 // mid.mid, hi.lo, lo.hi; the three left out are below 2^-24 of the result), accumulated in float32.
-// A workgroup takes 512 or more output rows (1/512 of all) and 128 filters (the launcher issues one launch per 128 filters: dX accumulates),
+// A workgroup takes 512 to 1024 output rows and 128 filters (the launcher issues one launch per 128 filters: dX accumulates),
 // wave b of it the taps 8b .. 8b + 7 (32 columns of Y; W's pieces for them stay in registers, 96 registers). A
-// block of 32 rows of dZ is read by the whole workgroup as whole 512-byte row segments and staged in LDS (the next
-// block's rows are on their way while this one is multiplied and go to LDS between the block's two barriers: a lane reading its own row from memory touches 32
-// cache lines per instruction, and the tag rate of the CU's cache then sets the pace); every wave reads the same
-// staged pieces (every value is split once, by the thread that loaded it: the planes hold bf16), the 32 x 4m tile of Y goes to LDS, and 128
-// threads add up the taps of their (row, letter) in ascending order, reaching into the previous block's tile for
-// rows before the block (the first block of a workgroup recomputes its predecessor's last rows instead of sharing
-// them). Deterministic: one writer per element, fixed orders.
+// block of 32 rows of dZ is read by the whole workgroup as whole 512-byte row segments and staged in LDS (a lane
+// reading its own row from memory touches 32 cache lines per instruction, and the tag rate of the CU's cache then sets
+// the pace). The rows are requested a whole block ahead - right after the registers that carry them have been emptied
+// into LDS, between the two barriers of the block before - and nothing else goes to or comes from global memory inside
+// the loop (the workgroup's rows of the result collect in LDS and join dX in one pass at the end), so the wait for them
+// waits for nothing else. Every wave reads the same staged pieces (every value is split once, by the thread that loaded
+// it: the planes hold bf16), the 32 x 4m tile of Y goes to LDS, and 128 threads add up the taps of their (row, letter)
+// in ascending order, reaching into the previous block's tile for rows before the block (the first block of a
+// workgroup recomputes its predecessor's last rows instead of sharing them). Deterministic: one writer per element,
+// fixed orders.
 constexpr unsigned GX_ROWS = 512;                                  // output rows per workgroup, at least (a multiple of 32)
+constexpr unsigned GX_WGROWS = 1024;                               // ... and at most: they are held in LDS until the workgroup ends
 constexpr unsigned GX_FILTERS = 128;                               // filters per launch: eight k-steps of 16
 constexpr unsigned GX_ZS = GX_FILTERS + 8;                         // row stride of a staged plane in bf16: 68 words = 4 mod 32, so that the 32 rows' 16-byte reads spread over the banks
 
@@ -890,6 +894,7 @@ __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* _
     constexpr int NT = 64 * MB, PER = (32 * (GX_FILTERS / 4) + NT - 1) / NT;   // threads; 16-byte pieces of a dZ tile per thread
     __shared__ float Y[2][32][YS];
     __shared__ __align__(16) unsigned short Zt[3][32][GX_ZS];     // the block's rows of dZ (this launch's filters) as three planes of bf16 pieces (lo, mid, hi)
+    __shared__ float out[GX_WGROWS * 4];                          // the workgroup's rows of the result
     const unsigned lane = threadIdx.x & 63, nb = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const unsigned col = lane & 31, g = lane >> 5;
     // ---- W's rows 32 nb + col (tap 8 nb + col / 4, letter col % 4), filters f0 + 16 ks + 8g .. + 7, in three pieces
@@ -913,33 +918,41 @@ __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* _
     }
     const size_t o0 = (size_t)blockIdx.x * rows_per_wg, o1 = o0 + rows_per_wg < n ? o0 + rows_per_wg : n;
     // A block's rows of dZ, requested by the whole workgroup as 16-byte pieces in row order (a wave reads whole
-    // 512-byte row segments); rows past the end and filters past F count as zero.
-    float4 piece[PER];
-    auto request = [&](size_t i0_) {
+    // 512-byte row segments). Every thread loads every time (a row past the end reads the last row, a piece past the
+    // block the block's last piece; what must count as zero is zeroed when it is used): nothing but these loads is
+    // on its way to or from global memory inside the loop, the same number on every path, so that waiting for the
+    // older of two blocks' rows does not wait for the newer.
+    auto request = [&](size_t i0_, float4 (&piece)[PER]) {
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
-            const unsigned e = threadIdx.x + j * NT, r = e / (GX_FILTERS / 4), c4 = e % (GX_FILTERS / 4);
-            const size_t row = i0_ + r;
-            float4 p = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            if (e < 32 * (GX_FILTERS / 4) && row < n) {
-                const float* src = dZ + row * F + f0 + 4u * c4;
-                if (WHOLE) {
-                    p = *reinterpret_cast<const float4*>(src);
-                } else {
-                    const unsigned f = f0 + 4u * c4;
-                    p.x = f < F ? src[0] : 0.0f; p.y = f + 1 < F ? src[1] : 0.0f; p.z = f + 2 < F ? src[2] : 0.0f; p.w = f + 3 < F ? src[3] : 0.0f;
-                }
+            unsigned e = threadIdx.x + j * NT;
+            if (e >= 32u * (GX_FILTERS / 4)) e = 32u * (GX_FILTERS / 4) - 1u;
+            const unsigned r = e / (GX_FILTERS / 4), c4 = e % (GX_FILTERS / 4);
+            size_t row = i0_ + r;
+            if (row >= n) row = n - 1;
+            const float* src = dZ + row * F + f0 + 4u * c4;
+            float4 p;
+            if (WHOLE) {
+                p = *reinterpret_cast<const float4*>(src);
+            } else {
+                const unsigned f = f0 + 4u * c4;
+                p.x = src[f < F ? 0 : -(int)(f - (F - 1))]; p.y = src[f + 1 < F ? 1 : -(int)(f - (F - 1))];
+                p.z = src[f + 2 < F ? 2 : -(int)(f - (F - 1))]; p.w = src[f + 3 < F ? 3 : -(int)(f - (F - 1))];
             }
             piece[j] = p;
         }
     };
     // every value is split once, by the thread that loaded it: four values' pieces are 8 bytes per plane
-    auto deposit = [&]() {
+    auto deposit = [&](size_t i0_, const float4 (&piece)[PER]) {
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             const unsigned e = threadIdx.x + j * NT, r = e / (GX_FILTERS / 4), c4 = e % (GX_FILTERS / 4);
             if (e < 32 * (GX_FILTERS / 4)) {
-                const float v[4] = { piece[j].x, piece[j].y, piece[j].z, piece[j].w };
+                const bool row_in = i0_ + r < n;
+                float v[4] = { piece[j].x, piece[j].y, piece[j].z, piece[j].w };
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (!row_in || (!WHOLE && f0 + 4u * c4 + t >= F)) v[t] = 0.0f;
                 unsigned pc[3][4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) split3(v[t], pc[0][t], pc[1][t], pc[2][t]);
@@ -949,23 +962,12 @@ __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* _
             }
         }
     };
+    // One block: this block's tile of Y from the staged pieces; between the two barriers the next block's rows (on
+    // their way since the middle of the block before) go to LDS, the rows of the block after it are requested into the
+    // same registers, and this block's taps are added up into the workgroup's rows of the result in LDS.
     unsigned slot = 0u;
-    size_t i0 = o0 >= 32 ? o0 - 32 : 0;
-    request(i0);
-    deposit();
-    __syncthreads();
-    for (; i0 < o1; i0 += 32, slot ^= 1u) {
-        // ---- the next block's rows and this block's rows of dX start their way; Y tile of rows i0 .. i0 + 31 from the staged pieces
-        const bool more = i0 + 32 < o1;
-        if (more) request(i0 + 32);
-        float old[2] = { 0.0f, 0.0f };
-        if (i0 >= o0) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const unsigned t = threadIdx.x + h * NT;
-                if (t < 128 && (h == 0 || NT < 128) && i0 + (t >> 2) < o1) old[h] = dX[(i0 + (t >> 2)) * 4 + (t & 3u)];
-            }
-        }
+    float4 piece[PER];
+    auto block = [&](size_t i0) {
         f32x16_t acc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
@@ -986,9 +988,10 @@ __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* _
 #pragma unroll
         for (int i = 0; i < 16; ++i) Y[slot][(i & 3) + 8 * (i >> 2) + 4 * g][32 * nb + col] = acc[i];
         __syncthreads();                                           // the tile is complete; nobody reads the staged pieces any more
-        if (more) deposit();
+        if (i0 + 32 < o1) deposit(i0 + 32, piece);
+        request(i0 + 64, piece);
         if (i0 >= o0) {
-            // ---- dX rows i0 .. i0 + 31: taps in ascending order, rows before the block from the previous tile
+            // ---- rows i0 .. i0 + 31 of the result: taps in ascending order, rows before the block from the previous tile
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const unsigned t = threadIdx.x + h * NT;
@@ -996,8 +999,6 @@ __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* _
                 const unsigned r = t >> 2, c = t & 3u;
                 const size_t i = i0 + r;
                 if (i < o1) {
-                    // all reads first (rows before the block come from the previous tile; rows before the first one count
-                    // as zero), then the sum in tap order
                     float y[8 * MB];
 #pragma unroll
                     for (int k = 0; k < 8 * MB; ++k) {
@@ -1008,12 +1009,22 @@ __global__ __launch_bounds__(64 * MB) void corr1ord_bprop_X_mfma_kernel(float* _
                     float sum = 0.0f;
 #pragma unroll
                     for (int k = 0; k < 8 * MB; ++k) sum += ((unsigned)k < m && i >= (size_t)k) ? y[k] : 0.0f;
-                    dX[i * 4 + c] = old[h] + sum;
+                    out[(i - o0) * 4 + c] = sum;
                 }
             }
         }
         __syncthreads();                                           // the next block's pieces are staged; this tile's readers are done
-    }
+        slot ^= 1u;
+    };
+    size_t i0 = o0 >= 32 ? o0 - 32 : 0;
+    request(i0, piece);
+    deposit(i0, piece);
+    request(i0 + 32, piece);
+    __syncthreads();
+    for (; i0 < o1; i0 += 32) block(i0);
+    // ---- the workgroup's rows of the result join what is there (the launches of other filters): one coalesced pass
+    const size_t nout = (o1 - o0) * 4;
+    for (size_t e = threadIdx.x; e < nout; e += NT) dX[o0 * 4 + e] += out[e];
 }
 
 inline bool bprop_X_mfma_takes(size_t m, size_t F, size_t n) { return m <= 32 && F >= 64 && n * F >= ((size_t)1 << 22) && n >= 4096; }
@@ -1021,9 +1032,11 @@ inline bool bprop_X_mfma_takes(size_t m, size_t F, size_t n) { return m <= 32 &&
 inline int launch_bprop_X_mfma(hipStream_t st, float* dX, size_t n, const float* W, size_t m, size_t F, const float* dZ)
 {
     // two workgroups fit a CU: about 512 of them in all, so that the weights' pieces are formed once per many rows
-    // (512 rows per workgroup: 0.61 ms at 1.0 M rows x 256 filters; 1/512 of the rows: 0.54 ms)
+    // (512 rows per workgroup: 0.61 ms at 1.0 M rows x 256 filters; 1/512 of the rows: 0.54 ms; at most 1024, the result
+    // rows in LDS and the rows of dZ requested a block ahead: 0.51 ms)
     unsigned rows = (unsigned)(((n + 511) / 512 + 31) / 32 * 32);
     if (rows < GX_ROWS) rows = GX_ROWS;
+    if (rows > GX_WGROWS) rows = GX_WGROWS;
     const unsigned gx = (unsigned)dbk::divup(n, rows), mb = (unsigned)((4 * m + 31) / 32);
     for (size_t f0 = 0; f0 < F; f0 += GX_FILTERS) {
         const bool whole = F % 4 == 0 && f0 + GX_FILTERS <= F;
