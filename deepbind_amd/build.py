@@ -27,8 +27,6 @@ FLAGS = [
 # The running max of the k-mer kernel must compile to bare v_max / v_max3 instructions; with NaNs
 # honoured every fmaxf gets two extra canonicalising ops. Infinities stay honoured (-inf seeds the max).
 EXTRA = {"scanpool_kmer.hip": ["-fno-honor-nans"]}
-if os.environ.get("DBK_STEP_PROF"):
-    EXTRA["step_single.hip"] = ["-DDBK_STEP_PROF"]
 
 
 def _compile(src):

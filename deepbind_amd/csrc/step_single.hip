@@ -35,8 +35,10 @@
 //
 // The barrier is a set of flags in the caller's workspace; every workgroup of the grid must be resident, so
 // the grid never exceeds 256 workgroups of at most 512 threads, nor the device's number of CUs (a CU holds at least
-// one), and the wait is bounded:
-// a workgroup that gives up sets the workspace's status word and leaves without touching the parameters.
+// one), and the wait is bounded. Whether a launch steps or is abandoned (a workgroup waited too long, a region has too
+// many rows) is settled once for the whole grid by a compare-and-swap on one word (see grid_barrier): an abandoned
+// launch changes no parameter, sets the workspace's status word, and every later launch on that workspace does
+// nothing until the host has zeroed the workspace's header again.
 // Results are deterministic (no float atomics; LDS atomics only OR bits), within the tolerances of the
 // multi-launch step but not its bits (other summation orders).
 #include <type_traits>
@@ -59,7 +61,6 @@ constexpr unsigned MAXG = 256;                    // workgroups of a launch (all
 constexpr size_t WORK_HEADER = 32768;              // bytes of the workspace before the shares: launch number, status, "go", flags, pair words
 constexpr unsigned GO_AT = 32, FLAGS_AT = 64;     // words of the workspace: the "go" word; the first workgroup flag
 constexpr unsigned PAIR_AT = 2048;                // ... the predictions that the two workgroups of a (forward, reverse) pair show each other: [workgroup][model] 8 bytes
-constexpr unsigned STAMP_AT = 4096 + 2048;        // ... time stamps of a profiling build
 constexpr unsigned FLAG_STRIDE = 4;               // words from one workgroup's flag to the next (measured: 4 beats 1 and 16 by ~0.1 us per step)
 constexpr unsigned SPIN_LIMIT = 400000;           // polls of the barrier before a workgroup gives up (~0.2 s)
 
@@ -163,55 +164,73 @@ __device__ __forceinline__ void scan_block(const float* __restrict__ wt, const u
 // All workgroups of the grid meet here once. Accesses of many workgroups to ONE address at device scope are served
 // one after the other (measured: ~50 ns per read-modify-write, 6.5 us for a counter that 128 workgroups increment;
 // 2-4 us per poll when every workgroup reads every other's flag, in lines of their own or side by side), so no word is
-// shared more than it must be: each workgroup
-// raises a flag of its own - the number of this launch, one more than the number the workspace
-// held when the kernel started; workgroup 0 alone reads all the flags (up to four per lane of its first wave) and, when
-// they all show the number, writes it to the "go" word; every other workgroup polls that one word with one lane.
-// Returns 0 when the step may go on, else the status to leave with (1: this workgroup gave up waiting; otherwise
-// what another workgroup flagged before it arrived).
-__device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, unsigned launch, float* dbg = nullptr)
+// shared more than it must be: each workgroup raises a flag of its own; workgroup 0 alone reads all the flags (up to
+// four per lane of its first wave) and, when they are all up, publishes its decision in the "go" word, which every
+// other workgroup polls with one lane.
+//
+// Words carry the number of the launch (one more than the number the workspace held when the kernel started, 31 bits)
+// so that what an earlier launch left is never taken for this one's: flag = 2 * number + (1: this workgroup must not
+// update - a region too long, a partner that never answered); go = 2 * number + (1: the step is abandoned).
+// Whether the grid steps or abandons is decided ONCE, by whoever first moves the "go" word from a value of an earlier
+// launch to a value of this one with a compare-and-swap: workgroup 0 when it has seen all flags (go, or abandon if a
+// flag says so) or has waited SPIN_LIMIT polls for them (abandon); any other workgroup that has polled the word twice
+// as long (abandon: workgroup 0 is not running). Whoever loses the exchange takes the winner's value. So either every
+// workgroup of the launch applies its part of the update or none does.
+// Returns 0 when the step goes on, 1 when it is abandoned (the workspace's status word is then non-zero).
+__device__ __forceinline__ unsigned decide(unsigned* go, unsigned seen, unsigned want, unsigned number)
+{
+    for (;;) {
+        const unsigned old = atomicCAS(go, seen, want);
+        if (old == seen) return want;
+        if ((old >> 1) == number) return old;                      // decided by another workgroup
+        seen = old;
+    }
+}
+
+__device__ __forceinline__ unsigned grid_barrier(unsigned* sync, unsigned G, unsigned launch, bool bad)
 {
     __shared__ unsigned verdict;
     unsigned* flags = sync + FLAGS_AT;
+    unsigned* go = sync + GO_AT;
+    const unsigned number = launch & 0x7fffffffu;
     __syncthreads();
     if (threadIdx.x < 64) {
         const unsigned lane = threadIdx.x;
         if (lane == 0) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");     // this workgroup's shares are visible device-wide
-            if (dbg) dbg[0] = (float)(wall_clock64() & 0xffffff);
-            __hip_atomic_store(&flags[blockIdx.x * FLAG_STRIDE], launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&flags[blockIdx.x * FLAG_STRIDE], 2u * number + (bad ? 1u : 0u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        unsigned tries = 0;
-        bool done = false;
+        unsigned tries = 0, word = 0;
         if (blockIdx.x == 0) {
+            bool all_up = false, any_bad = false, decided = false;
             for (;;) {
                 unsigned v[MAXG / 64];
 #pragma unroll
                 for (unsigned u = 0; u < MAXG / 64; ++u)
-                    v[u] = lane + 64u * u < G ? __hip_atomic_load(&flags[(lane + 64u * u) * FLAG_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : launch;
-                bool mine = true;
+                    v[u] = lane + 64u * u < G ? __hip_atomic_load(&flags[(lane + 64u * u) * FLAG_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 2u * number;
+                if (lane == 0) word = __hip_atomic_load(go, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                bool mine = true, mine_bad = false;
 #pragma unroll
-                for (unsigned u = 0; u < MAXG / 64; ++u) mine = mine && v[u] == launch;
-                done = __all(mine);
-                if (dbg && tries == 0 && lane == 0) dbg[1] = (float)(wall_clock64() & 0xffffff);
-                if (done || ++tries >= SPIN_LIMIT) break;
+                for (unsigned u = 0; u < MAXG / 64; ++u) { mine = mine && (v[u] >> 1) == number; mine_bad = mine_bad || (v[u] & 1u); }
+                all_up = __all(mine);
+                any_bad = __any(mine && mine_bad);
+                decided = ((unsigned)__builtin_amdgcn_readfirstlane((int)word) >> 1) == number;      // (a workgroup that gave up was faster)
+                if (all_up || decided || ++tries >= SPIN_LIMIT) break;
                 __builtin_amdgcn_s_sleep(1);
             }
-            if (lane == 0 && done) __hip_atomic_store(&sync[GO_AT], launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0 && !decided) word = decide(go, word, 2u * number + ((all_up && !any_bad) ? 0u : 1u), number);
         } else if (lane == 0) {
             for (;;) {
-                done = __hip_atomic_load(&sync[GO_AT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == launch;
-                if (dbg && tries == 0) dbg[1] = (float)(wall_clock64() & 0xffffff);
-                if (done || ++tries >= SPIN_LIMIT) break;
+                word = __hip_atomic_load(go, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((word >> 1) == number) break;
+                if (++tries >= 2u * SPIN_LIMIT) { word = decide(go, word, 2u * number + 1u, number); break; }
                 __builtin_amdgcn_s_sleep(1);
             }
         }
         if (lane == 0) {
-            unsigned status = __hip_atomic_load(&sync[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (!done) { atomicExch(&sync[1], 1u); status = 1u; }
-            if (dbg) { dbg[2] = (float)(wall_clock64() & 0xffffff); dbg[3] = (float)tries; }
+            if (word & 1u) atomicCAS(&sync[1], 0u, 1u);            // (a more specific status set before the barrier stays)
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");     // the other workgroups' shares are read from memory, not from stale lines
-            verdict = status;
+            verdict = word & 1u;
         }
     }
     __syncthreads();
@@ -246,13 +265,6 @@ __device__ __forceinline__ float wave_sum(float v)
 // A share is stored through the cache levels that other workgroups do not see (a relaxed store at device scope), on its
 // way while the workgroup computes the rest: the barrier's release fence then finds little left to write back.
 __device__ __forceinline__ void put_share(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-
-#ifdef DBK_STEP_PROF
-#define STAMP(i) do { if (threadIdx.x == 0) { const long long now_ = wall_clock64(); if (blockIdx.x == 0) reinterpret_cast<long long*>(a.sync + STAMP_AT)[i] = now_; \
-    if ((i) == 0 || (i) == 5 || (i) == 6) a.partial[(unsigned)blockIdx.x * a.pstride + a.nparam + a.nmodel + ((i) == 0 ? 0 : (i) - 4)] = (float)(now_ & 0xffffff); } } while (0)
-#else
-#define STAMP(i) do {} while (0)
-#endif
 
 // SHAPE: what of the launch shape is known when the kernel is compiled. 1: one region per workgroup of 512 threads
 // (batches of at most MAXG regions). 2: that, and a single model of at most 16 filters. 3 / 4: one region per workgroup
@@ -302,14 +314,13 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     const unsigned kpf = a.ptype == DBK_PT_ALL ? 2u : 1u;          // pooled features per filter
     const small_div by_nm(nm), by_k(k), by_nmk(nm * k), by_h1(h1), by_kt(kt), by_kf(a.kf), by_nmkf(nm * a.kf);
 
-    STAMP(0);
     // ---------------- everything this workgroup reads from global memory before the barrier, requested in one round:
     // its regions' bounds, targets, masks, dropout rates, the generator position and the look-ahead vector
     // P + mrate * mP (gradstep.cu:41-51). (Dependent round trips, not arithmetic, are what a step of this size costs.)
     {
         unsigned ra = 0, rb = 0;
         float y = 0.0f, dr = 0.0f;
-        unsigned ym = 1u, c_lo = 0u, c_hi = 0u, tickets = 0u;
+        unsigned ym = 1u, c_lo = 0u, c_hi = 0u, tickets = 0u, stale = 0u;
         constexpr unsigned UN = 6;
         float vp[UN], vr[UN], vm[UN];
 #pragma unroll
@@ -330,25 +341,31 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         if (tid == 0) {
             if (a.counter) { const unsigned long long c = a.counter[0]; c_lo = (unsigned)c; c_hi = (unsigned)(c >> 32); }
             tickets = __hip_atomic_load(&a.sync[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            stale = __hip_atomic_load(&a.sync[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
 #pragma unroll
         for (unsigned u = 0; u < UN; ++u)
             if (tid + u * NT < a.nparam) Lk[tid + u * NT] = vp[u] + vr[u] * vm[u];
         for (unsigned e = tid + (unsigned)UN * NT; e < a.nparam; e += NT) Lk[e] = a.P[e] + a.mrate[e] * a.mP[e];      // a long parameter vector: the rest
+        bool too_long = false;
         if (tid < RC) {
             unsigned rows = rb > ra ? rb - ra : 0u;
             if (rows > MAXROWS) {                                  // not a shape this kernel takes: flag it, touch nothing of the region
                 atomicExch(&a.sync[1], 2u);
                 rows = 0u;
+                too_long = true;
             }
             rinfo[2 * tid] = rows;
             rinfo[2 * tid + 1] = ra;
         }
+        if (wave == 0) too_long = __any(too_long);                 // (RC <= 16: all in the first wave)
         if (tid < RC * nm) { Ys[tid] = y; Yms[tid] = ym; }
         if (tid < nm) rates[tid] = dr;
         if (tid == 0) {
             misc[0] = c_lo; misc[1] = c_hi;
             misc[2] = tickets + 1u;                                // this launch's number (see grid_barrier)
+            misc[3] = stale;                                       // the status the workspace held when this workgroup started
+            misc[4] = too_long ? 1u : 0u;                          // non-zero: this workgroup's flag will ask for the step to be abandoned
         }
     }
     for (unsigned e = tid; e < RC * nm * a.kf; e += NT) {          // the shared feature columns follow each model's own inputs
@@ -359,7 +376,18 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     if (dense)
         for (unsigned e = tid; e < RC * Fp * AW; e += NT) amask[e] = 0u;
     __syncthreads();
-    STAMP(1);
+    if (misc[3] != 0u) {
+        // A workspace that an earlier launch (or a faster workgroup of this one) flagged: nothing is stepped until the host
+        // has looked at the status and zeroed the workspace's header. The flag still goes up so that nobody waits for it,
+        // and workgroup 0 settles the launch as abandoned.
+        if (tid == 0) {
+            const unsigned number = misc[2] & 0x7fffffffu;
+            __hip_atomic_store(&a.sync[FLAGS_AT + blockIdx.x * FLAG_STRIDE], 2u * number + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (blockIdx.x == 0)
+                decide(a.sync + GO_AT, __hip_atomic_load(&a.sync[GO_AT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), 2u * number + 1u, number);
+        }
+        return;
+    }
     // ---------------- the regions' letters are requested; the letter table [tap][letter][filter] (zero rows past m) is
     // built from the look-ahead meanwhile; then the letters land dword-aligned per region, with one bit per (letter, position)
     constexpr unsigned TXN = (4 * TXTB + NTMIN - 1) / NTMIN;       // letters per thread when the workgroup has up to four regions
@@ -418,7 +446,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     }
     __syncthreads();
 
-    STAMP(2);
     // ---------------- forward: scan + bias + ReLU + pooling, region by region, all four waves on one region
     const unsigned PG = 64u >> lgFp, NG = NW * PG;               // position groups per wave / per workgroup
     const unsigned lgNG4 = (NT == NTMAX ? 3u : 2u) + 6u - lgFp + 2u;                            // log2(4 * NG): NT is 256 or 512
@@ -478,7 +505,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         if constexpr (!ONE) __syncthreads();                       // (ONE: the wave that wrote the pooled features is the one that goes on with them)
     }
 
-    STAMP(3);
     // ---------------- dense head, forward and backward, for this workgroup's rows
     const float inv_n = 1.0f / (float)a.nregion;
     if (RC == 1u) {
@@ -530,7 +556,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
                         if ((unsigned)(seen >> 32) == launch) break;
                         __builtin_amdgcn_s_sleep(1);
                     }
-                    if ((unsigned)(seen >> 32) != launch) atomicExch(&a.sync[1], 1u);      // gave up: the grid barrier ends the step without an update
+                    if ((unsigned)(seen >> 32) != launch) { atomicCAS(&a.sync[1], 0u, 1u); atomicOr(&misc[4], 1u); }      // gave up: this workgroup's flag asks for the step to be abandoned
                 }
                 const unsigned tag = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(seen >> 32));
                 const float zo = __uint_as_float((unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)seen));
@@ -588,7 +614,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             H0[(rl * nm + b) * kt + kk] = (rl < nreg && kept[e]) ? PL[e] : 0.0f;
         }
         __syncthreads();
-        STAMP(8);
         if (hidden) {
             for (unsigned e = tid; e < RC * nm * hidden; e += NT) {
                 const unsigned rb = by_h1.quot(e), h = by_h1.rem(e, rb), b = by_nm.rem(rb, by_nm.quot(rb));
@@ -602,7 +627,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             }
             __syncthreads();
         }
-        STAMP(9);
         // output pre-activation and prediction of (row, model): one wave per output, a lane per input, summed by a fixed butterfly
         for (unsigned e = wave; e < RC * nm; e += NW) {
             const unsigned b = by_nm.rem(e, by_nm.quot(e));
@@ -620,7 +644,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             }
         }
         __syncthreads();
-        STAMP(10);
         // loss gradient of (row, model), formed by every thread that needs it; the hidden units' gradients with it
         for (unsigned e = tid; e < RC * nm * h1; e += NT) {
             const unsigned rb = by_h1.quot(e), h = by_h1.rem(e, rb), rl = by_nm.quot(rb), b = by_nm.rem(rb, rl);
@@ -643,7 +666,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             if (hidden) D1[e] = H1[e] > 0.0f ? dA * W2s[b * hidden + h] : 0.0f;
         }
         __syncthreads();
-        STAMP(12);
         for (unsigned e = tid; e < RC * nm * k; e += NT) {             // gradient at the pooled features -> what the scan's backward pass needs
             const unsigned rl = by_nmk.quot(e), col = by_nmk.rem(e, rl), b = by_k.quot(col), kk = by_k.rem(col, b), rb = rl * nm + b;
             float g;
@@ -663,7 +685,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         }
     }
     __syncthreads();
-    STAMP(13);
     // (from here to the grid barrier nothing waits for a store to global memory: the shares travel while the filter
     // gradients are counted)
     // this workgroup's share of the dense layers' gradients and of the loss, rows ascending
@@ -704,7 +725,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
     }
     for (unsigned e = tid; e < nreg * nm; e += NT) put_share(&a.Z[(unsigned)r0 * nm + e], zs[e]);      // the predictions of this workgroup's rows
 
-    STAMP(4);
     // ---------------- scan filters: a thread's (tap, filter) pairs, five letter accumulators each, regions ascending
     constexpr unsigned MAXPAIR = (MT * 64 + NTMIN - 1) / NTMIN;
 #pragma unroll
@@ -749,7 +769,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         if (t == 0 && fl < F) put_share(&share[a.off_bc + fl], accb);
     }
 
-    STAMP(5);
     // ---------------- every workgroup's share is written: meet, then add them up and step the parameters.
     // What the update reads of the parameter vectors is requested before the wait (nothing changes it until then).
     // A workgroup steps 64 consecutive parameters: wave w adds the shares of its run of workgroups for them (a lane per
@@ -762,14 +781,9 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         q_p = a.P[efirst]; q_rm = a.mrate[efirst]; q_mp = a.mP[efirst]; q_dr = a.drate[efirst];
         if (a.decay) q_dec = a.decay[efirst];
     }
-#ifdef DBK_STEP_PROF
-    if (grid_barrier(a.sync, a.G, misc[2], a.partial + (unsigned)blockIdx.x * a.pstride + a.nparam + a.nmodel + 3) != 0u) return;
-#else
-    if (grid_barrier(a.sync, a.G, misc[2]) != 0u) return;
-#endif
+    if (grid_barrier(a.sync, a.G, misc[2], misc[4] != 0u) != 0u) return;
     // (every workgroup read the launch number before it raised its flag, so it can move on now)
-    if (blockIdx.x == 0 && tid == 0) __hip_atomic_store(&a.sync[0], misc[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);              // flagged (by any workgroup, before the barrier) or gave up: no update
-    STAMP(6);
+    if (blockIdx.x == 0 && tid == 0) __hip_atomic_store(&a.sync[0], misc[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // word 0 counts the launches that stepped
     float* sums = wt;                                              // (the letter table is no longer needed)
     const unsigned per = (a.G + NW - 1) / NW;                      // workgroups each wave adds, ascending
     const unsigned g0 = wave * per, g1 = g0 + per < a.G ? g0 + per : a.G;
@@ -811,7 +825,6 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         a.mP[e] = q_mp * q_rm - delta;
         a.P[e] = lk - delta;
     }
-    STAMP(7);
     if (a.counter && a.draws && blockIdx.x == 0 && tid == 0) a.counter[0] += a.draws;
 }
 

@@ -23,6 +23,7 @@ All models of one SequenceNet share pool type and hidden size; a calibration bat
 architectures is run as one SequenceNet per architecture (see ModelGroup).
 """
 import ctypes
+import weakref
 
 import numpy as np
 import torch
@@ -59,8 +60,9 @@ class SequenceNet(object):
         # small groups (1-4 models, at most 64 filters, regions of at most 256 rows) step in ONE launch
         # (dbk_train_step_single) unless this is switched off; same numbers within tolerance, other summation orders
         self.single_launch = bool(single_launch)
-        self._single_rows = {}               # longest region of the region tables seen, by (pointer, version, regions)
+        self._single_rows = {}               # longest region of the region tables seen, by tensor identity and version
         self._single_calls = 0               # single-launch steps issued (their status word is looked at now and then)
+        self._last_single = False            # the last natively issued step went through the single-launch kernel
         self.step_count = 0
         self._step_args = None               # argument block and work buffers of the natively issued step
         self._step_bufs = {}
@@ -161,6 +163,7 @@ class SequenceNet(object):
         if self.weight_decay_start > self.step_count:
             return np.zeros((1, ni))
         p = self.p
+        self._check_single_status()
         conv = sm.sum_axis0(sm.mul_sign(p["Wc"], p["Wc"]))                     # |W| summed over taps and channels
         torch.cuda.synchronize()
         cost = conv.cpu().numpy().astype(np.float64).reshape(ni, -1).sum(axis=1) * self.decay_conv.cpu().numpy().ravel()
@@ -189,25 +192,47 @@ class SequenceNet(object):
             buf["work"] = torch.zeros(need.value, dtype=torch.uint8, device=self.P.device) if need.value else None
         if buf["work"] is None:
             return None
-        key = (R.data_ptr(), R._version, R.shape[0])
-        rows = self._single_rows.get(key)
-        if rows is None:                     # one read-back per region table: the kernel keeps whole regions in LDS
+        # the longest region of this very tensor object in its present state: an address alone says nothing (a new
+        # tensor of a later batch can get the address of a freed one), so the entry holds a weak reference to the tensor
+        ent = self._single_rows.get(id(R))
+        if ent is None or ent[0]() is not R or ent[1] != R._version:
             if len(self._single_rows) >= 256:
                 self._single_rows.clear()
-            Rl = R.to(torch.int64)
-            rows = self._single_rows[key] = int((Rl[:, 1] - Rl[:, 0]).max().item()) if R.shape[0] else 0
-        return buf["work"] if rows <= 256 else None
+            Rl = R.to(torch.int64)           # one read-back per region table: the kernel keeps whole regions in LDS
+            rows = int((Rl[:, 1] - Rl[:, 0]).max().item()) if R.shape[0] else 0
+            ent = self._single_rows[id(R)] = (weakref.ref(R), R._version, rows)
+        return buf["work"] if ent[2] <= 256 else None
+
+    SINGLE_HEADER = 32768                    # bytes of a single-launch workspace before the gradient shares
 
     def _check_single_status(self):
-        """Raises when a single-launch step flagged its workspace (the step then left the parameters untouched)."""
+        """Raises when a single-launch step flagged its workspace. Such a launch, and every launch after it on that
+        workspace, changed nothing (parameters, momentum, generator position), so the host's step counter and
+        generator mirror are set back to what the device actually did, and the workspace's header is zeroed so that
+        the next step runs again."""
         for buf in self._step_bufs.values():
             work = buf.get("work")
-            if work is not None:
-                status = int(work[4:8].view(torch.int32).item())
-                if status:
-                    work[4:8].zero_()
-                    raise _lib.DeepbindError("RuntimeError: a single-launch training step was abandoned (%s)" %
-                                             ("a workgroup waited too long at the barrier" if status == 1 else "a region has more than 256 rows"))
+            if work is None:
+                continue
+            torch.cuda.synchronize()
+            stepped, status = (int(v) for v in work[0:8].view(torch.int32).tolist())
+            if status:
+                dropped = max(buf.get("issued", 0) - stepped, 0)
+                work[:self.SINGLE_HEADER].zero_()
+                buf["issued"] = 0
+                self.step_count -= dropped
+                self._rng_offset = int(self.rng_counter.item())
+                self._L_versions = None
+                raise _lib.DeepbindError("RuntimeError: a single-launch training step was abandoned (%s); %d step(s) were not applied" %
+                                         ("a workgroup waited too long" if status == 1 else "a region has more than 256 rows", dropped))
+
+    def _count_single_launch(self, buf):
+        """Book-keeping after a single-launch step was issued on the workspace in `buf` (or a graph holding one
+        replayed): the status word is looked at every 256 launches, so that an abandoned step does not go unnoticed."""
+        buf["issued"] = buf.get("issued", 0) + 1
+        self._single_calls += 1
+        if self._single_calls % 256 == 0:
+            self._check_single_status()
 
     def get_params(self):
         self._check_single_status()
@@ -215,6 +240,7 @@ class SequenceNet(object):
         return {name: self.p[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
     def get_grads(self):
+        self._check_single_status()
         torch.cuda.synchronize()
         return {name: self.g[name].cpu().numpy().copy() for name, _, _ in self.layout}
 
@@ -557,7 +583,7 @@ class SequenceNet(object):
         a.nfeat, a.feats = self.nfeat, pv(F)
         a.input_rate = self.input_dropout
         for name, t in buf.items():
-            if name != "work":
+            if name not in ("work", "issued"):
                 setattr(a, name, None if t is None else t.data_ptr())
         a.decay = self.decay_vec.data_ptr() if self.weight_decay_start <= self.step_count else None
         a.freeze_scan = int(self.step_count < self.start_training)
@@ -585,22 +611,29 @@ class SequenceNet(object):
         if work is not None:
             _lib.call("dbk_train_step_single", _lib.stream(), ctypes.addressof(self._step_args), _lib.ptr(work), work.numel())
             self._L_versions = None          # (this kernel forms the look-ahead itself and leaves none behind)
-            self._single_calls += 1
-            if self._single_calls % 4096 == 0 and not torch.cuda.is_current_stream_capturing():
-                self._check_single_status()  # a step that gave up leaves the parameters alone: do not train on in silence
         else:
             _lib.call("dbk_train_step", _lib.stream(), ctypes.addressof(self._step_args))
+        self._last_single = work is not None
         self._finish_step(X, R)
+        if work is not None and not torch.cuda.is_current_stream_capturing():
+            self._count_single_launch(buf)   # (may raise: a step that was abandoned must not be trained over in silence)
         self.enforce_constraints()
         return buf["Z"]
 
-    def make_graphed_step(self, X, R, Y, Ymask=None, F=None):
+    def make_graphed_step(self, X, R, Y, Ymask=None, F=None, force_graph=False):
         """Captures one fused training step on the given (static) batch tensors into a HIP graph and
         returns a function that replays it: for launch-bound batch sizes the step then costs one
         graph launch instead of ~10 kernel launches. Dropout masks stay fresh on every replay because
         the generator position lives in device memory. The graph bakes in whether L1 decay is
         active and whether the scan filters are still frozen, so it is re-captured when the step
-        counter crosses weight_decay_start or start_training."""
+        counter crosses weight_decay_start or start_training.
+        A step that the single-launch kernel takes is ONE launch already, and replaying a graph of one
+        node costs more than issuing that launch (measured 22 against 12 us per step), so for such a
+        net the function returned issues the step natively unless force_graph is set."""
+        fused = self.mode == "fused" and self.dtype == torch.float32 and self.loss is not None
+        if fused and self.single_launch and not force_graph:
+            if self._single_work(self._prepare_step(X, R, Y, Ymask, F), R) is not None:
+                return lambda: self._native_step(X, R, Y, Ymask, F)
         return _graphed_step([(self, X, R, Y, Ymask, F)])
 
     def train_step(self, X, R, Y, Ymask=None, U=None, U_input=None, F=None):
@@ -642,6 +675,7 @@ def _native_steps(jobs):
             blocks[j] = ctypes.addressof(net._step_args)
         _lib.call("dbk_train_steps", _lib.stream(), len(chunk), blocks)
         for net, X, R, *_ in chunk:
+            net._last_single = False
             net._finish_step(X, R)
             net.enforce_constraints()
 
@@ -700,6 +734,7 @@ def _graphed_step(jobs):
         for (net, *_), (off, count) in zip(jobs, host_off):
             net._rng_offset, net.step_count = off, count
         state["graph"], state["decay"] = g, decay_flags()
+        state["single"] = [(net, net._step_buf) for net, *_ in jobs if net._last_single]      # workspaces of single-launch steps in the graph
 
     def step():
         if state["graph"] is None or state["decay"] != decay_flags():
@@ -712,6 +747,8 @@ def _graphed_step(jobs):
             if net.use_dropout:
                 net._rng_offset += (R.shape[0] * net.k * net.ninst + 3) // 4
             net.step_count += 1
+        for net, buf in state["single"]:
+            net._count_single_launch(buf)
 
     return step
 

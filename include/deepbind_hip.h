@@ -453,10 +453,15 @@ int dbk_train_steps(dbk_stream_t stream, size_t ngroup, const dbk_train_step_arg
  * dP, mP, P, loss and advances the generator position. Deterministic; within the tolerances of dbk_train_step,
  * not its bits (other summation orders).
  * work: caller-owned device memory of dbk_train_step_single_workspace() bytes, 16-byte aligned, ZERO before its
- * first use and from then on passed unchanged to every call with the same nregion (word 0 is the number of the last
- * launch; word 1 a status the kernel sets: 1 = a workgroup gave up waiting at the barrier, 2 = a region had more
- * than 256 rows; with a non-zero status the parameters are left untouched). Calls that share a workspace must not
- * overlap. *work_bytes = 0 from the query means the shape is not taken (use dbk_train_step).
+ * first use and from then on passed unchanged to every call with the same nregion. Word 0 (uint32) counts the
+ * launches that stepped; word 1 is a status: 1 = a workgroup waited too long (at the barrier or for its
+ * reverse-complement partner), 2 = a region had more than 256 rows. Whether a launch steps is decided once for the
+ * whole grid (a compare-and-swap on one word of the workspace): an abandoned launch changes no parameter, neither
+ * momentum nor generator position, and sets the status; while the status is non-zero every further launch on that
+ * workspace returns without doing anything. To go on, wait for the stream, read words 0 and 1, and zero the first
+ * 32768 bytes of the workspace (status alone is not enough: the barrier's words hold the abandoned launch's number).
+ * Calls that share a workspace must not overlap. *work_bytes = 0 from the query means the shape is not taken
+ * (use dbk_train_step).
  * reference: the body of the trainer's loop, deepity/deepity/sgd.py:98-135, as dbk_train_step. */
 int dbk_train_step_single_workspace(const dbk_train_step_args* args, size_t* work_bytes);
 int dbk_train_step_single(dbk_stream_t stream, const dbk_train_step_args* args, void* work, size_t work_bytes);

@@ -246,7 +246,12 @@ def bias_fprop(X, b):
 
 
 def bias_bprop(dZ):
-    return dZ, dZ.sum(axis=0, dtype=dZ.dtype).reshape(1, -1)
+    """db = column sums, rows added one after the other in dZ's dtype: the order of the reference's column reduction,
+    one thread walking down a column (smat/src/smat_cuda/reduce_y.cuh:57-78). (ndarray.sum would add a single column
+    pairwise, which rounds less than the reference does.)"""
+    if dZ.shape[0] == 0:
+        return dZ, np.zeros((1, dZ.shape[1]), dZ.dtype)
+    return dZ, np.cumsum(dZ, axis=0, dtype=dZ.dtype)[-1].reshape(1, -1)
 
 
 def relu_fprop(X):

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import deepbind_oracle as orc
-from tests.gpu_util import assert_close_per_model, dev, host, record_error
+from tests.gpu_util import assert_close_per_model, assert_no_further_than_f32_reference as assert_vs_f32, dev, host, model_blocks, record_error
 
 pytestmark = pytest.mark.gpu
 
@@ -72,7 +72,10 @@ def test_single_launch_step_matches_the_oracle(pool, hidden, loss, nm, nf, m, B,
     F = rng.standard_normal((rows, nfeat)).astype(np.float32) if nfeat else None
     Xd, Rd, Yd, Md, Fd = dev(X), dev(R), dev(Y), dev(Ymask), (dev(F) if nfeat else None)
     ref_p, ref_m = _f64(params), {n: np.zeros(v.shape) for n, v in params.items()}
+    f32_p, f32_m = {n: v.copy() for n, v in params.items()}, {n: np.zeros(v.shape, np.float32) for n, v in params.items()}
     name = "single launch (%s/%d, %d x %d filters x %d taps)" % (pool, hidden, nm, nf, m)
+    f32 = lambda v: np.asarray(v, dtype=np.float32)
+    blocks = lambda a, axis: model_blocks(a, nm, axis)
     for step in range(3):
         U = host(ds.uniform_like(torch.empty((rows // (2 if rc else 1), net.k * nm), device="cuda"), net.rng_seed, net._rng_offset))
         if rc:
@@ -81,18 +84,27 @@ def test_single_launch_step_matches_the_oracle(pool, hidden, loss, nm, nf, m, B,
         st, g = orc.train_step(ref_p, ref_m, X, R, Y.astype(np.float64), nm, pool, hidden, loss, rate, mu, Ymask=Ymask, dropout=(drop, U),
                                decay_conv=dconv, decay_full=dfull, step=step, weight_decay_start=1, reverse_complement=rc, start_training=1,
                                features=None if F is None else F.astype(np.float64))
+        st32, g32 = orc.train_step(f32_p, f32_m, X, R, Y, nm, pool, hidden, loss, f32(rate), f32(mu), Ymask=Ymask, dropout=(f32(drop), U),
+                                   decay_conv=dconv, decay_full=f32(dfull), step=step, weight_decay_start=1, reverse_complement=rc,
+                                   start_training=1, features=F)
         got = net.get_grads()
         for pname, _, axis in net.layout:
             assert_close_per_model(got[pname], g[pname], GRAD, nm, axis, "step %d gradient %s" % (step, pname))
             record_error(name, "gradients", got[pname], g[pname], GRAD)
+            for b, (a64, a32, ag) in enumerate(zip(blocks(g[pname], axis), blocks(g32[pname], axis), blocks(got[pname], axis))):
+                assert_vs_f32(name, "gradients", ag, a64, a32, "step %d gradient %s [model %d]" % (step, pname, b))
         Z = host(net._step_bufs[(Xd.numel(), rows)]["Z"])
         assert_close_per_model(Z, st["Zout"], ACT, nm, 1, "step %d predictions" % step)
         record_error(name, "activations", Z, st["Zout"], ACT)
+        for b in range(nm):
+            assert_vs_f32(name, "activations", Z[:, b], st["Zout"][:, b], st32["Zout"][:, b], "step %d predictions [model %d]" % (step, b))
     assert _used_single(net), "the step did not go through the single-launch kernel"
     got = net.get_params()
     for pname, _, axis in net.layout:
         assert_close_per_model(got[pname], ref_p[pname], GRAD, nm, axis, "parameters %s" % pname)
         record_error(name, "parameters", got[pname], ref_p[pname], GRAD)
+        for b, (a64, a32, ag) in enumerate(zip(blocks(ref_p[pname], axis), blocks(f32_p[pname], axis), blocks(got[pname], axis))):
+            assert_vs_f32(name, "parameters", ag, a64, a32, "parameters %s [model %d]" % (pname, b))
 
 
 @pytest.mark.parametrize("pool,hidden,loss", [("max", 32, "nll"), ("all", 0, "mse")])
@@ -128,7 +140,7 @@ def test_single_launch_step_in_a_graph_and_loss_output():
         r2 = np.random.default_rng(9)
         nets.append(_net(r2, 1, 16, m, "all", 0, "mse", rate=0.02, momentum=0.9, dropout=0.25)[0])
     eager, graphed = nets
-    step = graphed.make_graphed_step(Xd, Rd, Yd)
+    step = graphed.make_graphed_step(Xd, Rd, Yd, force_graph=True)
     for i in range(4):
         eager.train_step(Xd, Rd, Yd)
         step()
@@ -138,6 +150,14 @@ def test_single_launch_step_in_a_graph_and_loss_output():
             assert np.array_equal(a[pname], b[pname]), "replay %d differs from the eager step in %s" % (i, pname)
     assert _used_single(eager) and _used_single(graphed)
     assert eager.step_count == graphed.step_count == 4 and eager._rng_offset == graphed._rng_offset
+    # without force_graph such a net gets its one launch issued directly (a graph of one node replays slower)
+    direct = graphed.make_graphed_step(Xd, Rd, Yd)
+    eager.train_step(Xd, Rd, Yd)
+    direct()
+    a, b = eager.get_params(), graphed.get_params()
+    for pname in a:
+        assert np.array_equal(a[pname], b[pname])
+    assert graphed.step_count == 5
 
 
 def test_shapes_the_single_launch_step_does_not_take_fall_back():
@@ -187,3 +207,78 @@ def test_region_longer_than_the_kernel_takes_is_flagged_and_leaves_the_parameter
     after = net.get_params()
     for pname in before:
         assert np.array_equal(before[pname], after[pname])
+
+
+def test_abandoned_steps_change_nothing_and_training_resumes_after_the_reset():
+    """A launch that the kernel's own guard abandons (a region of more than 256 rows, let through by switching the host's
+    check off), and the launch after it on the flagged workspace, leave parameters, momentum and generator position
+    alone; the host notices, sets its step counter and generator mirror back, re-arms the workspace, and the next step
+    gives the bits of a net that only ever saw the valid steps."""
+    from deepbind_amd import _lib, data
+    rng = np.random.default_rng(21)
+    m, nreg = 12, 16
+    letters = lambda n: "".join("ACGT"[c] for c in rng.integers(0, 4, size=n))
+    good = [letters(102 + (i & 1)) for i in range(nreg)]                       # 16 regions, 1640 letters
+    bad = [letters(290)] + [letters(90) for _ in range(nreg - 1)]              # the same number of regions and letters, one region too long
+    Xg, Rg = data.pack_sequences(good, m - 1)
+    Xb, Rb = data.pack_sequences(bad, m - 1)
+    assert Xg.size == Xb.size and len(Rg) == len(Rb)
+    Y = (rng.random((nreg, 1)) < 0.5).astype(np.float32)
+    Xgd, Rgd, Xbd, Rbd, Yd = dev(Xg), dev(Rg), dev(Xb), dev(Rb), dev(Y)
+    nets = [_net(np.random.default_rng(22), 1, 16, m, "all", 8, "nll", rate=0.05, momentum=0.9, dropout=0.5)[0] for _ in range(2)]
+    net, fresh = nets
+    for _ in range(2):
+        net.train_step(Xgd, Rgd, Yd)
+        fresh.train_step(Xgd, Rgd, Yd)
+    assert _used_single(net)
+    before, count, offset = net.get_params(), net.step_count, net._rng_offset
+    momentum = host(net.mP).copy()
+    host_check = net._single_work
+    net._single_work = lambda buf, R: buf["work"]                               # (the host's look at the region lengths, switched off)
+    net.train_step(Xbd, Rbd, Yd)                                                # abandoned by the kernel: status 2
+    net.train_step(Xgd, Rgd, Yd)                                                # a valid batch on the flagged workspace: nothing happens
+    net._single_work = host_check
+    with pytest.raises(_lib.DeepbindError, match="256 rows.*2 step"):
+        net.get_params()
+    assert net.step_count == count and net._rng_offset == offset == int(net.rng_counter.item())
+    after = net.get_params()                                                    # (the status is cleared: no second raise)
+    for pname in before:
+        assert np.array_equal(before[pname], after[pname]), pname
+    assert np.array_equal(momentum, host(net.mP))
+    net.train_step(Xgd, Rgd, Yd)
+    fresh.train_step(Xgd, Rgd, Yd)
+    a, b = net.get_params(), fresh.get_params()
+    for pname in a:
+        assert np.array_equal(a[pname], b[pname]), "after the reset %s differs from a net that never saw the abandoned steps" % pname
+    assert net.step_count == fresh.step_count == 3
+
+
+def test_region_table_cache_follows_the_tensor_not_its_address():
+    """A new region table at the address of an earlier one, with the same version count and row count (what a training
+    loop sees when the caching allocator hands a freed block to the next batch's table) is looked at again: its long
+    region sends the step to the multi-launch kernels instead of being dropped by the single-launch kernel's guard."""
+    from deepbind_amd import data
+    rng = np.random.default_rng(23)
+    m, nreg = 12, 16
+    letters = lambda n: "".join("ACGT"[c] for c in rng.integers(0, 4, size=n))
+    Xs, Rs = data.pack_sequences([letters(60) for _ in range(nreg)], m - 1)
+    Xl, Rl = data.pack_sequences([letters(300)] + [letters(44) for _ in range(nreg - 1)], m - 1)
+    assert Xs.size == Xl.size
+    Y = dev((rng.random((nreg, 1)) < 0.5).astype(np.float32))
+    net, _ = _net(np.random.default_rng(24), 1, 16, m, "max", 8, "nll", rate=0.05)
+    ref, _ = _net(np.random.default_rng(24), 1, 16, m, "max", 8, "nll", rate=0.05, single_launch=False)
+    Xd, R1 = dev(Xs), dev(Rs)
+    net.train_step(Xd, R1, Y)
+    ref.train_step(Xd, dev(Rs), Y)
+    assert _used_single(net)
+    torch.cuda.synchronize()
+    R1.data.copy_(dev(Rl))                   # the next batch's table lands in the same memory ...
+    R2 = R1.data                             # ... as a tensor object of its own, version count 0 like the first
+    assert R2 is not R1 and R2.data_ptr() == R1.data_ptr() and R2._version == R1._version and R2.shape == R1.shape
+    Xd2 = dev(Xl)
+    net.train_step(Xd2, R2, Y)
+    ref.train_step(Xd2, dev(Rl), Y)
+    a, b = net.get_params(), ref.get_params()                                   # (raises if the kernel had to abandon the step)
+    assert net.step_count == 2
+    for pname in a:
+        assert np.abs(a[pname] - b[pname]).max() <= GRAD * np.abs(b[pname]).max(), pname

@@ -5,7 +5,8 @@ import pytest
 import torch
 
 from oracle import deepbind_oracle as orc
-from tests.gpu_util import assert_close, assert_close_per_model, dev, host, model_blocks, record_error
+from tests.gpu_util import (assert_close, assert_close_per_model, assert_no_further_than_f32_reference as assert_vs_f32, dev, host,
+                            model_blocks, record_argmax, record_error)
 
 pytestmark = pytest.mark.gpu
 
@@ -32,28 +33,42 @@ def _run_config(cfg, mode, nsteps, dropout_rate=0.0, decay=(0.0, 0.0), weight_de
     U = cfg.get("U")
     Ud = dev(U) if (U is not None and dropout_rate > 0) else None
     ref_p, ref_m = _f64(params), {k: np.zeros(v.shape) for k, v in params.items()}
+    # the same trajectory once more with every array in float32: the reference's own arithmetic, in its own order
+    f32_p, f32_m = {k: v.copy() for k, v in params.items()}, {k: np.zeros(v.shape, np.float32) for k, v in params.items()}
     drop = (np.full(spec.nmodel, dropout_rate), U) if dropout_rate > 0 else None
+    drop32 = (np.full(spec.nmodel, dropout_rate, np.float32), U) if dropout_rate > 0 else None
+    kw = dict(decay_conv=decay[0], decay_full=decay[1], weight_decay_start=weight_decay_start)
     for step in range(nsteps):
         net.train_step(X, R, Y, U=Ud)
         st, g = orc.train_step(ref_p, ref_m, cfg["X"], cfg["R"], cfg["Y"].astype(np.float64), spec.nmodel, spec.pool[0],
-                               spec.hidden[0], spec.loss, cfg.get("rate", 0.01), cfg.get("momentum", 0.9), dropout=drop,
-                               decay_conv=decay[0], decay_full=decay[1], step=step, weight_decay_start=weight_decay_start)
+                               spec.hidden[0], spec.loss, cfg.get("rate", 0.01), cfg.get("momentum", 0.9), dropout=drop, step=step, **kw)
+        _, g32 = orc.train_step(f32_p, f32_m, cfg["X"], cfg["R"], cfg["Y"].astype(np.float32), spec.nmodel, spec.pool[0],
+                                spec.hidden[0], spec.loss, cfg.get("rate", 0.01), cfg.get("momentum", 0.9), dropout=drop32, step=step, **kw)
         got_g = net.get_grads()
         for k in g:
             assert_close(got_g[k], g[k], GRAD, "step %d grad %s (%s)" % (step, k, mode))
             if name:
                 record_error(name, "gradients", got_g[k], g[k], GRAD)
+                assert_vs_f32(name, "gradients", got_g[k], g[k], g32[k], "step %d grad %s (%s)" % (step, k, mode))
     got = net.get_params()
     for k in ref_p:
         assert_close(got[k], ref_p[k], GRAD, "params %s after %d steps (%s)" % (k, nsteps, mode))
         if name:
             record_error(name, "parameters", got[k], ref_p[k], GRAD)
+            assert_vs_f32(name, "parameters", got[k], ref_p[k], f32_p[k], "params %s after %d steps (%s)" % (k, nsteps, mode))
     if name:
-        st = orc.model_forward(ref_p, cfg["X"], cfg["R"], spec.nmodel, spec.pool[0], spec.hidden[0],
-                               out="logistic" if spec.loss == "nll" else "linear")
+        # forward pass at the parameters the DEVICE ended with, so that nothing but the forward arithmetic differs
+        out = "logistic" if spec.loss == "nll" else "linear"
+        st = orc.model_forward(_f64(got), cfg["X"], cfg["R"], spec.nmodel, spec.pool[0], spec.hidden[0], out=out)
+        st32 = orc.model_forward(got, cfg["X"], cfg["R"], spec.nmodel, spec.pool[0], spec.hidden[0], out=out)
         net.use_dropout, keep = False, net.use_dropout
-        record_error(name, "activations", host(net.predict(X, R)), st["Zout"], ACT)
-        record_error(name, "activations", host(net.forward(X, R)["pooled"]), st["Pl"], ACT)
+        Zd, fw = host(net.predict(X, R)), net.forward(X, R, want_argmax=True)
+        for what, a, b, b32 in (("predictions", Zd, st["Zout"], st32["Zout"]), ("pooled", host(fw["pooled"]), st["Pl"], st32["Pl"])):
+            assert_close(a, b, ACT, "%s at the final parameters (%s)" % (what, mode))
+            record_error(name, "activations", a, b, ACT)
+            assert_vs_f32(name, "activations", a, b, b32, "%s at the final parameters (%s)" % (what, mode))
+        if fw["argmax"] is not None:
+            record_argmax(name, host(fw["argmax"]), st32["I"])
         net.use_dropout = keep
     return net, got
 
@@ -91,10 +106,15 @@ def test_config1_forward_scores():
     net = SequenceNet(1, spec.nfilter, spec.m, pool="max", hidden=32, loss=None)
     net.set_params(cfg["params"])
     st = orc.model_forward(_f64(cfg["params"]), cfg["X"], cfg["R"], 1, "max", 32)
+    st32 = orc.model_forward(cfg["params"], cfg["X"], cfg["R"], 1, "max", 32)
     got = host(net.predict(dev(cfg["X"]), dev(cfg["R"])))
     assert got.shape == (64, 1)
     assert_close(got, st["A"], ACT, "config 1 scores")
     record_error("config1", "activations", got, st["A"], ACT)
+    assert_vs_f32("config1", "activations", got, st["A"], st32["A"], "config 1 scores")
+    fw = net.forward(dev(cfg["X"]), dev(cfg["R"]), want_argmax=True)
+    assert_vs_f32("config1", "activations", host(fw["pooled"]), st["Pl"], st32["Pl"], "config 1 pooled features")
+    assert record_argmax("config1", host(fw["argmax"]), st32["I"]) == 0        # taps added in the reference's order: its bits
     assert_close(host(net.forward(dev(cfg["X"]), dev(cfg["R"]))["Z"]), st["A"], ACT, "config 1 scores (layer by layer)")
 
 
@@ -113,7 +133,7 @@ def test_config4_calibration_batch_mixed_architectures():
     grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
                      decay_conv=hp["decay_conv"], decay_full=hp["decay_full"], dropout=hp["dropout"], weight_decay_start=1)
     assert len(grp.groups) <= 4 and sum(len(i) for i, _ in grp.groups) == 90
-    init, ref, mom = [], [], []
+    init, ref, mom, ref32, mom32 = [], [], [], [], []
     for gi, (idx, net) in enumerate(grp.groups):
         net.rng_seed = 40 + gi
         stacked = {name: np.concatenate([cfg["models"][j][name] for j in idx], axis=axis) for name, _, axis in net.layout}
@@ -121,6 +141,9 @@ def test_config4_calibration_batch_mixed_architectures():
         init.append(stacked)
         ref.append(_f64(stacked))
         mom.append({k: np.zeros(v.shape) for k, v in stacked.items()})
+        ref32.append({k: v.copy() for k, v in stacked.items()})                 # the same trajectory in float32, reference order
+        mom32.append({k: np.zeros(v.shape, np.float32) for k, v in stacked.items()})
+    CFG = "config4 (shared launches)"
     X, R, Y, M = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"]), dev(cfg["Ymask"])
     nsteps = 3
     for step in range(nsteps):
@@ -132,22 +155,33 @@ def test_config4_calibration_batch_mixed_architectures():
         # decay indexing depends on the number of models sharing a graph, so the grouping is part of the semantics)
         for gi, (idx, net) in enumerate(grp.groups):
             drop = (hp["dropout"][idx].astype(np.float64), Us[gi]) if net.use_dropout else None
+            drop32 = (hp["dropout"][idx], Us[gi]) if net.use_dropout else None
+            kw = dict(Ymask=cfg["Ymask"][:, idx], decay_conv=hp["decay_conv"][idx], decay_full=hp["decay_full"][idx], step=step,
+                      weight_decay_start=1)
             _, g = orc.train_step(ref[gi], mom[gi], cfg["X"], cfg["R"], cfg["Y"][:, idx].astype(np.float64), len(idx), net.pool,
-                                  net.hidden, "nll", hp["rate"][idx], hp["momentum"][idx], Ymask=cfg["Ymask"][:, idx], dropout=drop,
-                                  decay_conv=hp["decay_conv"][idx], decay_full=hp["decay_full"][idx], step=step, weight_decay_start=1)
+                                  net.hidden, "nll", hp["rate"][idx], hp["momentum"][idx], dropout=drop, **kw)
+            st32, g32 = orc.train_step(ref32[gi], mom32[gi], cfg["X"], cfg["R"], cfg["Y"][:, idx], len(idx), net.pool,
+                                       net.hidden, "nll", hp["rate"][idx], hp["momentum"][idx], dropout=drop32, **kw)
+            if step == 0:
+                # the pooling winners of the step's own forward launch (at the initial parameters: no momentum yet)
+                record_argmax(CFG, host(net._step_buf["argmax"]), st32["I"])
             got_g = net.get_grads()
             for name, _, axis in net.layout:
                 what = "step %d %s/%d gradient %s" % (step, net.pool, net.hidden, name)
                 assert_close_per_model(got_g[name], g[name], GRAD, len(idx), axis, what)
-                for a, b in zip(model_blocks(got_g[name], len(idx), axis), model_blocks(g[name], len(idx), axis)):
-                    record_error("config4 (shared launches)", "gradients", a, b, GRAD)
+                for b_, (a, b, b32) in enumerate(zip(model_blocks(got_g[name], len(idx), axis), model_blocks(g[name], len(idx), axis),
+                                                     model_blocks(g32[name], len(idx), axis))):
+                    record_error(CFG, "gradients", a, b, GRAD)
+                    assert_vs_f32(CFG, "gradients", a, b, b32, "%s [model %d]" % (what, b_))
     nmoved = 0
     for gi, (idx, net) in enumerate(grp.groups):
         got = net.get_params()
         for name, _, axis in net.layout:
             assert_close_per_model(got[name], ref[gi][name], GRAD, len(idx), axis, "%s/%d parameters %s" % (net.pool, net.hidden, name))
-            for a, b in zip(model_blocks(got[name], len(idx), axis), model_blocks(ref[gi][name], len(idx), axis)):
-                record_error("config4 (shared launches)", "parameters", a, b, GRAD)
+            for b_, (a, b, b32) in enumerate(zip(model_blocks(got[name], len(idx), axis), model_blocks(ref[gi][name], len(idx), axis),
+                                                 model_blocks(ref32[gi][name], len(idx), axis))):
+                record_error(CFG, "parameters", a, b, GRAD)
+                assert_vs_f32(CFG, "parameters", a, b, b32, "%s/%d parameters %s [model %d]" % (net.pool, net.hidden, name, b_))
         # every model trained: its filters changed by what the reference's update changes them by (compared as
         # CHANGES, so a model whose filters were left alone, or stepped with a neighbour's rate, fails even
         # when the change is far below the weights' own size); float32 storage rounds each of the steps
@@ -168,7 +202,14 @@ def test_config4_calibration_batch_mixed_architectures():
         st = orc.model_forward(ref[gi], cfg["X"], cfg["R"], len(idx), net.pool, net.hidden, out="logistic",
                                dropout=(hp["dropout"][idx].astype(np.float64), None) if net.use_dropout else None, train=False)
         assert_close(scores[:, idx], st["Zout"], 1e-4, "scores of group %d" % gi)
-        record_error("config4 (shared launches)", "activations", scores[:, idx], st["Zout"], ACT)
+        record_error(CFG, "activations", scores[:, idx], st["Zout"], ACT)
+        # the forward arithmetic alone: float64 and float32 evaluations at the parameters the device ended with
+        got = net.get_params()
+        dr = lambda t: (hp["dropout"][idx].astype(t), None) if net.use_dropout else None
+        s64 = orc.model_forward(_f64(got), cfg["X"], cfg["R"], len(idx), net.pool, net.hidden, out="logistic", dropout=dr(np.float64), train=False)
+        s32 = orc.model_forward(got, cfg["X"], cfg["R"], len(idx), net.pool, net.hidden, out="logistic", dropout=dr(np.float32), train=False)
+        for b_ in range(len(idx)):
+            assert_vs_f32(CFG, "activations", scores[:, idx[b_]], s64["Zout"][:, b_], s32["Zout"][:, b_], "scores of model %d of group %d" % (b_, gi))
 
 
 def test_reverse_complement_mode_train_and_predict():
@@ -277,7 +318,7 @@ def test_graphed_step_replays_match_eager_steps():
 
     eager, graphed = make(), make()
     X, R, Y = dev(cfg["X"]), dev(cfg["R"]), dev(cfg["Y"])
-    step = graphed.make_graphed_step(X, R, Y)
+    step = graphed.make_graphed_step(X, R, Y, force_graph=True)
     for i in range(6):
         eager.train_step(X, R, Y)
         step()
