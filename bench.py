@@ -419,6 +419,8 @@ def main():
             "frac": adds_per_s / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
             "frac_vs_add_issue_peak": adds_per_s / 1e12 / FP32_ADD_ISSUE_PEAK_TADDS,
             "traffic": measured_traffic(args.workload),
+            "traffic_source": "read from the committed counter profile profiles/scanpool_kmer_config5_counters.md (rocprofv3 --pmc FETCH_SIZE / "
+                              "WRITE_SIZE runs of this workload, scaled by a copy kernel of known size); not measured in this run",
             "kernel": "fused scan+bias+relu+maxpool (dbk_scanpool_fprop launches)", "kernel_ms": scan_ms,
             "algorithmic_adds_per_launch": adds,
             "hbm": {"algorithmic_bytes_per_launch": hbm_bytes, "achieved_GBs": hbm_bytes / (scan_ms * 1e-3) / 1e9,

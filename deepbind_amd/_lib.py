@@ -21,6 +21,8 @@ class DeepbindError(RuntimeError):
 DBK_F32, DBK_F64 = 0, 1
 PT_MAX, PT_AVG, PT_SUM, PT_ALL = 0, 1, 2, 3
 str2pooltype = {"max": PT_MAX, "avg": PT_AVG, "sum": PT_SUM, "all": PT_ALL}
+# loss_kind of dbk_head_train / dbk_train_step*: output non-linearity + loss (reference: deepity/std/loss.py:131-174)
+LOSS_KIND = {"nll": 0, "mse": 1, "hinge": 2}
 
 _P, _Z, _I, _U64, _F, _D = c_void_p, c_size_t, c_int, c_uint64, c_float, c_double
 
@@ -28,6 +30,7 @@ _P, _Z, _I, _U64, _F, _D = c_void_p, c_size_t, c_int, c_uint64, c_float, c_doubl
 _SIGNATURES = {
     "dbk_version": [],
     "dbk_device_count": [],
+    "dbk_set_exact_scan": [_I],
     "dbk_sync": [_P],
     "dbk_corr1ord": [_P, _I, _P, _Z, _Z, _P, _Z, _Z, _P],
     "dbk_corr1ord_bprop_W": [_P, _I, _P, _Z, _Z, _P, _Z, _Z, _P],
@@ -78,6 +81,7 @@ _SIGNATURES = {
     "dbk_logistic": [_P, _I, _P, _P, _Z],
     "dbk_loss_terms": [_P, _I, _I, _P, _P, _P, _Z],
     "dbk_sub_scale": [_P, _I, _P, _P, _D, _P, _Z],
+    "dbk_hinge_grad": [_P, _I, _P, _P, _D, _P, _Z],
     "dbk_head_train": [_P, _Z, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _U64, _U64, _P, _U64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "dbk_softmax": [_P, _I, _P, _P, _Z, _Z],
     "dbk_counter_add": [_P, _P, _U64],

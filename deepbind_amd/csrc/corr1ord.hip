@@ -1111,7 +1111,7 @@ int dbk_corr1ord(dbk_stream_t stream, int dtype, const void* W, size_t m, size_t
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && X && Z, "ValueError: null pointer argument");
-    if (dtype == DBK_F32 && fprop_mfma_takes(m, nfilter, n)) return launch_fprop_mfma(dbk::as_stream(stream), (const float*)W, m, nfilter, X, n, (float*)Z);
+    if (dtype == DBK_F32 && !dbk::exact_scan() && fprop_mfma_takes(m, nfilter, n)) return launch_fprop_mfma(dbk::as_stream(stream), (const float*)W, m, nfilter, X, n, (float*)Z);
     if (dtype == DBK_F32) return launch_fprop<float>(dbk::as_stream(stream), (const float*)W, m, nfilter, X, n, (float*)Z);
     return launch_fprop<double>(dbk::as_stream(stream), (const double*)W, m, nfilter, X, n, (double*)Z);
 }
@@ -1124,7 +1124,7 @@ int dbk_corr1ord_bprop_W(dbk_stream_t stream, int dtype, void* dW, size_t m, siz
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(dW && X && dZ, "ValueError: null pointer argument");
-    if (dtype == DBK_F32 && bprop_W_mfma_takes(m, nfilter, n)) return launch_bprop_W_mfma(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
+    if (dtype == DBK_F32 && !dbk::exact_scan() && bprop_W_mfma_takes(m, nfilter, n)) return launch_bprop_W_mfma(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     if (dtype == DBK_F32 && m <= 24) return launch_bprop_W_window(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     if (dtype == DBK_F32) return launch_bprop_W<float>(dbk::as_stream(stream), (float*)dW, m, nfilter, X, n, (const float*)dZ);
     return launch_bprop_W<double>(dbk::as_stream(stream), (double*)dW, m, nfilter, X, n, (const double*)dZ);
@@ -1138,7 +1138,7 @@ int dbk_corr1ord_bprop_X(dbk_stream_t stream, int dtype, void* dX, size_t n, siz
     DBK_CHECK(m >= 1, "ValueError: filter length must be >= 1");
     if (n == 0 || nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(dX && W && dZ, "ValueError: null pointer argument");
-    if (dtype == DBK_F32 && bprop_X_mfma_takes(m, nfilter, n)) return launch_bprop_X_mfma(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
+    if (dtype == DBK_F32 && !dbk::exact_scan() && bprop_X_mfma_takes(m, nfilter, n)) return launch_bprop_X_mfma(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     if (dtype == DBK_F32 && m <= 24) return launch_bprop_X_ring(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     if (dtype == DBK_F32) return launch_bprop_X<float>(dbk::as_stream(stream), (float*)dX, n, (const float*)W, m, nfilter, (const float*)dZ);
     return launch_bprop_X<double>(dbk::as_stream(stream), (double*)dX, n, (const double*)W, m, nfilter, (const double*)dZ);

@@ -19,7 +19,8 @@ void clear_error();
 // different streams never do. 64 stream slots per device; when all are taken the slot used longest ago
 // passes to the new stream (after draining the device). Growing a buffer or recycling a slot synchronises
 // the device, which a stream under capture does not allow: null then, and when memory runs out, with the
-// reason in workspace_error().
+// reason in workspace_error(). A buffer handed out DURING a capture is in a graph from then on: its slot is never
+// recycled and its buffers neither freed nor grown (a later, larger call on that stream fails and says so).
 // `which` selects one of four independent buffers of the stream: 0 and 1 hold kernels' partial results (a call
 // that must keep one kernel's partial results while another kernel fills its own uses the second), 2 and 3 the
 // whole maps of the unfused scan + pool chain, whose kernels use buffer 0 themselves.
@@ -69,6 +70,9 @@ int scan_fprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size
 int scan_bprop_multi(hipStream_t st, size_t m, size_t N, const uint32_t* R, size_t P, unsigned n, scan_group* g);
 int head_train_multi(hipStream_t st, size_t nrow, unsigned n, head_group* g);
 
+// dbk_set_exact_scan: the drop-in scan operators keep to the kernels that add in the reference's order at every size
+bool exact_scan();
+
 inline hipStream_t as_stream(dbk_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline unsigned divup(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
@@ -96,6 +100,27 @@ struct small_div {
     }
     __device__ __forceinline__ unsigned rem(unsigned e, unsigned q) const { return e - q * d; }
 };
+
+// The three losses of the path (deepity/deepity/std/loss.py:98-174): kind 0 = logistic output + negative log-likelihood,
+// 1 = linear output + squared error, 2 = linear output + bidirectional hinge. loss_grad is dLoss/d(output) before the
+// masks and the 1/rows factor (loss.py:98-112; hinge: 1 - 2Y where (1-Y)Z + Y(1-Z) > 0, loss.py:165-169), loss_term the
+// per-row term that is summed, loss_mean what the reported loss makes of the sum (-mean, mean/2, mean).
+constexpr int LOSS_NLL = 0, LOSS_MSE = 1, LOSS_HINGE = 2;
+__device__ __forceinline__ float loss_grad(int kind, float z, float y)
+{
+    if (kind == LOSS_HINGE) return ((1.0f - y) * z + y * (1.0f - z)) > 0.0f ? 1.0f - 2.0f * y : 0.0f;
+    return z - y;
+}
+__device__ __forceinline__ float loss_term(int kind, float z, float y)
+{
+    if (kind == LOSS_NLL) return logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y);
+    if (kind == LOSS_MSE) return (z - y) * (z - y);
+    return fmaxf(0.0f, (1.0f - y) * z + y * (1.0f - z));
+}
+__device__ __forceinline__ float loss_mean(int kind, float s, float n)
+{
+    return kind == LOSS_NLL ? -s / n : (kind == LOSS_MSE ? 0.5f * s / n : s / n);
+}
 
 }  // namespace dbk
 

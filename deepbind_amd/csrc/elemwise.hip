@@ -295,6 +295,9 @@ template <typename T> __global__ void k_loss_terms(int kind, const T* Z, const T
             T a = z > (T)1e-15 ? z : (T)1e-15;
             T b = ((T)1 - z) > (T)1e-15 ? ((T)1 - z) : (T)1e-15;
             L[i] = log(a) * y + log(b) * ((T)1 - y);
+        } else if (kind == 3) {                                    // bidirectional hinge (deepity/std/loss.py:162-163)
+            T l = ((T)1 - y) * z + y * ((T)1 - z);
+            L[i] = l > (T)0 ? l : (T)0;
         } else if (kind == 2) {                                    // several columns per output: multiclass term
             T a = z > (T)1e-15 ? z : (T)1e-15;
             L[i] = log(a) * y;
@@ -363,6 +366,14 @@ __global__ void k_counter_add(unsigned long long* ctr, unsigned long long delta)
 template <typename T> __global__ void k_sub_scale(const T* Z, const T* Y, T scale, T* dZ, size_t n)
 {
     GRID_STRIDE(i, n) dZ[i] = (Z[i] - Y[i]) * scale;
+}
+template <typename T> __global__ void k_hinge_grad(const T* Z, const T* Y, T scale, T* dZ, size_t n)
+{
+    GRID_STRIDE(i, n) {
+        const T z = Z[i], y = Y[i];
+        const T l = ((T)1 - y) * z + y * ((T)1 - z);
+        dZ[i] = l > (T)0 ? ((T)1 - (T)2 * y) * scale : (T)0;
+    }
 }
 
 }  // namespace
@@ -584,7 +595,7 @@ int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t 
 }
 int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, const void* Y, void* L, size_t n)
 {
-    DBK_CHECK(kind >= 0 && kind <= 2, "ValueError: loss kind must be 0 (nll), 1 (mse) or 2 (multiclass nll), got %d", kind);
+    DBK_CHECK(kind >= 0 && kind <= 3, "ValueError: loss kind must be 0 (nll), 1 (mse), 2 (multiclass nll) or 3 (hinge), got %d", kind);
     EW2(k_loss_terms, n, A(kind, CF32(Z), CF32(Y), F32(L), n), A(kind, CF64(Z), CF64(Y), F64(L), n));
 }
 int dbk_softmax(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n, size_t group)
@@ -596,6 +607,10 @@ int dbk_softmax(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n
 int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n)
 {
     EW2(k_sub_scale, n, A(CF32(Z), CF32(Y), (float)scale, F32(dZ), n), A(CF64(Z), CF64(Y), scale, F64(dZ), n));
+}
+int dbk_hinge_grad(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n)
+{
+    EW2(k_hinge_grad, n, A(CF32(Z), CF32(Y), (float)scale, F32(dZ), n), A(CF64(Z), CF64(Y), scale, F64(dZ), n));
 }
 
 int dbk_uniform_fill(dbk_stream_t stream, float* U, size_t n, uint64_t seed, uint64_t offset)

@@ -177,8 +177,8 @@ __device__ __forceinline__ void head_train_body(const head_args& a, const unsign
         bool use = use_row;
         if (a.revcomp) use = use && ((r & 1) ? !(zo >= z) : (z >= zo));
         if (use) {
-            dA = (z - y) * inv_n;
-            lterm = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
+            dA = dbk::loss_grad(a.loss_kind, z, y) * inv_n;
+            lterm = dbk::loss_term(a.loss_kind, z, y);
         }
         if (part == 0) a.Z[zi] = z;
     }
@@ -287,7 +287,7 @@ __global__ void k_head_reduce(head_args a)
         else if (idx < nW1 + h1) a.db1[(size_t)b * h1 + (idx - nW1)] = s;
         else if (idx < nW1 + 2 * h1) { if (hidden > 0) a.dW2[(size_t)b * hidden + (idx - nW1 - h1)] = s; }
         else if (idx == nW1 + 2 * h1) { if (hidden > 0) a.db2[b] = s; }
-        else if (a.loss) a.loss[b] = a.loss_kind == 0 ? -s / (float)a.n : 0.5f * s / (float)a.n;
+        else if (a.loss) a.loss[b] = dbk::loss_mean(a.loss_kind, s, (float)a.n);
     }
     // every workgroup of the forward/backward kernel has read the generator position by now: move it on
     if (a.counter && a.counter_advance && blockIdx.x == 0 && threadIdx.x == 0) a.counter[0] += a.counter_advance;
@@ -313,6 +313,7 @@ int dbk::head_train_multi(hipStream_t st, size_t nrow, unsigned n, dbk::head_gro
     for (unsigned i = 0; i < n; ++i) {
         const int h1 = g[i].hidden > 0 ? g[i].hidden : 1;
         DBK_CHECK(g[i].nblock >= 1 && g[i].k >= 1 && g[i].kf >= 0 && g[i].hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, nfeat=%d, hidden=%d)", g[i].nblock, g[i].k, g[i].kf, g[i].hidden);
+        DBK_CHECK(g[i].loss_kind >= 0 && g[i].loss_kind <= 2, "ValueError: loss kind must be 0 (logistic + nll), 1 (linear + mse) or 2 (linear + hinge), got %d", g[i].loss_kind);
         DBK_CHECK(!g[i].revcomp || nrow % 2 == 0, "ValueError: reverse-complement rows come in pairs, got %zu rows", nrow);
         const size_t need = head_smem(g[i].k, g[i].kf, h1);
         DBK_CHECK(need <= dbk_scan::lds_limit(), "ValueError: head of %d inputs x %d hidden units needs %zu bytes of LDS", g[i].k + g[i].kf, g[i].hidden, need);
@@ -348,7 +349,7 @@ extern "C" int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, 
                               float* Z, float* dpooled, float* dW1, float* db1, float* dW2, float* db2, float* loss)
 {
     DBK_CHECK(nblock >= 1 && k >= 1 && nfeat >= 0 && hidden >= 0, "ValueError: bad head shape (nblock=%d, k=%d, nfeat=%d, hidden=%d)", nblock, k, nfeat, hidden);
-    DBK_CHECK(loss_kind == 0 || loss_kind == 1, "ValueError: loss kind must be 0 (logistic + nll) or 1 (linear + mse), got %d", loss_kind);
+    DBK_CHECK(loss_kind >= 0 && loss_kind <= 2, "ValueError: loss kind must be 0 (logistic + nll), 1 (linear + mse) or 2 (linear + hinge), got %d", loss_kind);
     const int h1 = hidden > 0 ? hidden : 1;
     DBK_CHECK(!reverse_complement || n % 2 == 0, "ValueError: reverse-complement rows come in pairs, got %zu rows", n);
     if (n == 0) { dbk::clear_error(); return 0; }

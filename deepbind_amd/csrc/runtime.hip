@@ -1,4 +1,5 @@
 // Error state, version, device count, sync and the scratch workspace.
+#include <atomic>
 #include "dbk_common.h"
 #include <cstring>
 #include <mutex>
@@ -18,7 +19,9 @@ void set_error(const char* fmt, ...)
 void clear_error() { g_err[0] = 0; }
 
 constexpr int WS_BUFFERS = 4;   // 0, 1: partial sums of the kernels; 2, 3: whole maps of the unfused scan + pool chain
-struct ws_t { hipStream_t stream = nullptr; void* ptr[WS_BUFFERS] = {}; size_t bytes[WS_BUFFERS] = {}; bool used = false; uint64_t tick = 0; };
+// pinned: a capture has taken a buffer's address into a graph, which may be replayed for as long as the process lives,
+// so the slot never changes hands again and its buffers are never freed
+struct ws_t { hipStream_t stream = nullptr; void* ptr[WS_BUFFERS] = {}; size_t bytes[WS_BUFFERS] = {}; bool used = false, pinned = false; uint64_t tick = 0; };
 constexpr int WS_DEVICES = 64, WS_STREAMS = 64;
 static ws_t g_ws[WS_DEVICES][WS_STREAMS];
 static uint64_t g_ws_tick = 0;
@@ -49,7 +52,7 @@ void* workspace(size_t bytes, hipStream_t stream, int which)
         ws_t& c = g_ws[dev][i];
         if (c.used && c.stream == stream) w = &c;
         else if (!c.used) { if (!vacant) vacant = &c; }
-        else if (!oldest || c.tick < oldest->tick) oldest = &c;
+        else if (!c.pinned && (!oldest || c.tick < oldest->tick)) oldest = &c;
     }
     if (!w) w = vacant;
     if (!w) {
@@ -65,14 +68,27 @@ void* workspace(size_t bytes, hipStream_t stream, int which)
             snprintf(g_ws_why, sizeof(g_ws_why), "could not drain the device to recycle a stream slot");
             return nullptr;
         }
+        if (!oldest) {
+            snprintf(g_ws_why, sizeof(g_ws_why), "all %d stream slots hold scratch that captured graphs refer to", WS_STREAMS);
+            return nullptr;
+        }
         w = oldest;
     }
     w->used = true;
     w->stream = stream;
     w->tick = ++g_ws_tick;
-    if (w->bytes[which] >= bytes && w->ptr[which]) return w->ptr[which];
-    if (capturing(stream)) {
+    const bool under_capture = capturing(stream);
+    if (w->bytes[which] >= bytes && w->ptr[which]) {
+        if (under_capture) w->pinned = true;
+        return w->ptr[which];
+    }
+    if (under_capture) {
         snprintf(g_ws_why, sizeof(g_ws_why), "scratch cannot grow while the stream is capturing: run the call once eagerly on this stream first");
+        return nullptr;
+    }
+    if (w->ptr[which] && w->pinned) {
+        snprintf(g_ws_why, sizeof(g_ws_why), "a captured graph refers to this stream's scratch, which therefore cannot grow (%zu -> %zu bytes): issue the larger call on another stream",
+                 w->bytes[which], bytes);
         return nullptr;
     }
     if (w->ptr[which]) {
@@ -100,6 +116,9 @@ void* workspace(size_t bytes, hipStream_t stream, int which)
 static thread_local deferred_sums* g_deferred = nullptr;
 deferred_sums*& deferred() { return g_deferred; }
 
+static std::atomic<int> g_exact_scan{0};
+bool exact_scan() { return g_exact_scan.load(std::memory_order_relaxed) != 0; }
+
 }  // namespace dbk
 
 extern "C" {
@@ -113,6 +132,11 @@ int dbk_device_count(void)
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess) return -1;
     return n;
+}
+
+int dbk_set_exact_scan(int on)
+{
+    return dbk::g_exact_scan.exchange(on ? 1 : 0, std::memory_order_relaxed);
 }
 
 int dbk_sync(dbk_stream_t stream)

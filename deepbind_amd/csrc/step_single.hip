@@ -563,7 +563,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
                 use = use && tag == launch && ((r0 & 1u) ? !(zo >= z) : (z >= zo));
             }
             float dA = 0.0f;
-            if (use) dA = (z - Ys[b]) * inv_n;
+            if (use) dA = dbk::loss_grad((int)a.loss_kind, z, Ys[b]) * inv_n;
             if (lane == 0) { zs[b] = z; dAs[b] = dA; lss[b] = use ? 1.0f : 0.0f; }      // (the loss term is formed later, off this wave's path, where lss says so)
             if (hidden && lane < hidden) D1[b * hidden + lane] = hv > 0.0f ? dA * w2 : 0.0f;
             wave_lds_sync();
@@ -657,9 +657,8 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
                     use = use && ((rr & 1) ? !(zo >= z) : (z >= zo));
                 }
                 if (use) {
-                    dA = (z - y) * inv_n;
-                    if (h == 0)
-                        lterm = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
+                    dA = dbk::loss_grad((int)a.loss_kind, z, y) * inv_n;
+                    if (h == 0) lterm = dbk::loss_term((int)a.loss_kind, z, y);
                 }
             }
             if (h == 0) { dAs[rb] = dA; lss[rb] = lterm; }
@@ -715,7 +714,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
             gb2 = dAs[b];
             if (lss[b] != 0.0f) {
                 const float z = zs[b], y = Ys[b];
-                ls = a.loss_kind == 0 ? logf(fmaxf(1e-15f, z)) * y + logf(fmaxf(1e-15f, 1.0f - z)) * (1.0f - y) : (z - y) * (z - y);
+                ls = dbk::loss_term((int)a.loss_kind, z, y);
             }
         } else {
             for (unsigned rl = 0; rl < RC; ++rl) { gb2 += dAs[rl * nm + b]; ls += lss[rl * nm + b]; }
@@ -809,7 +808,7 @@ __global__ __launch_bounds__(NTMAX) void k_step_single(const single_args a)
         for (unsigned w = 0; w < NWMAX; ++w) pw[w] = w < NW ? sums[w * 64 + lane] : 0.0f;
         s = ((pw[0] + pw[1]) + (pw[2] + pw[3])) + ((pw[4] + pw[5]) + (pw[6] + pw[7]));
         if (e >= a.nparam) {
-            if (a.loss) a.loss[e - a.nparam] = a.loss_kind == 0 ? -s / (float)a.nregion : 0.5f * s / (float)a.nregion;
+            if (a.loss) a.loss[e - a.nparam] = dbk::loss_mean((int)a.loss_kind, s, (float)a.nregion);
             continue;
         }
         if (e != efirst) {
@@ -885,6 +884,7 @@ extern "C" int dbk_train_step_single(dbk_stream_t stream, const dbk_train_step_a
     size_t lds = 0;
     DBK_CHECK(plan(a, s, MT, lds), "NotImplementedError: the single-launch step takes 1-4 models with at most 64 filters of at most 32 taps, "
               "Nesterov momentum, no input dropout and at most %u x 16 regions of at most %u rows", MAXG, MAXROWS);
+    DBK_CHECK(a->loss_kind >= 0 && a->loss_kind <= 2, "ValueError: loss kind must be 0 (logistic + nll), 1 (linear + mse) or 2 (linear + hinge), got %d", a->loss_kind);
     DBK_CHECK(a->P && a->dP && a->mP && a->drate && a->mrate, "ValueError: null parameter vector");
     DBK_CHECK(a->X && a->regions && a->Y && a->Z, "ValueError: null batch or work buffer");
     DBK_CHECK(!a->rate || a->counter, "ValueError: dropout needs the device generator position");

@@ -69,7 +69,7 @@ __device__ __forceinline__ void reduce_update_body(const reduce_update_args& a, 
         if (e >= a.nparam) {                                       // per-model loss
             const unsigned b = (unsigned)(e - a.nparam);
             const float s = chunk_sum(a, b, nW1m + 2 * a.h1 + 1);
-            a.loss[b] = a.loss_kind == 0 ? -s / (float)a.nrow : 0.5f * s / (float)a.nrow;
+            a.loss[b] = dbk::loss_mean(a.loss_kind, s, (float)a.nrow);
             continue;
         }
         float g;

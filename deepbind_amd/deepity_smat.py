@@ -7,7 +7,7 @@ import numbers
 import numpy as np
 import torch
 
-from ._lib import call, dtype_code, ptr, require, stream
+from ._lib import LOSS_KIND, call, dtype_code, ptr, require, stream
 
 _rng_seed = 0
 _rng_offset = 0
@@ -259,7 +259,7 @@ def head_train(pooled, W1, b1, W2, b2, Y, nblock, loss, dW1, db1, dW2=None, db2=
     dpooled = torch.empty_like(pooled)
     L = torch.empty((1, nblock), dtype=torch.float32, device=pooled.device) if want_loss else None
     r = None if rate is None else _vec(rate, pooled)
-    call("dbk_head_train", stream(), n, nblock, k, hidden, {"nll": 0, "mse": 1}[loss], int(bool(reverse_complement)),
+    call("dbk_head_train", stream(), n, nblock, k, hidden, LOSS_KIND[loss], int(bool(reverse_complement)),
          ptr(pooled), int(nfeat), ptr(feats), ptr(r), ptr(U), int(seed), int(offset), ptr(counter), int(counter_advance), ptr(W1), ptr(b1), ptr(W2), ptr(b2), ptr(Y), ptr(Ymask),
          ptr(Z), ptr(dpooled), ptr(dW1), ptr(db1), ptr(dW2), ptr(db2), ptr(L))
     return Z, dpooled, L

@@ -31,6 +31,15 @@ def _regions(R):
     return R
 
 
+def set_exact_scan(on):
+    """on: corr1ord, corr1ord_bprop_W and corr1ord_bprop_X keep to the kernels that sum in one fixed order at every
+    size (corr1ord: the reference's own order, so its bits whatever the batch size). Off (the default) float32 calls
+    switch to the faster matrix-core kernels at bulk sizes, whose results equal these to round-off. Process-wide;
+    returns the previous setting."""
+    from ._lib import dll
+    return bool(dll().dbk_set_exact_scan(int(bool(on))))
+
+
 def corr1ord(W, X, Z, nchannel):
     """Cross-correlates the filter bank W ((M*nchannel) x P) with the ordinal vector X (N uint8,
     values 0..nchannel-1, 255 = all ordinals, 254 = none) into Z (N x P). The final M-1 rows of Z

@@ -39,7 +39,7 @@ class SequenceNet(object):
                  rate=0.01, momentum=0.9, decay_conv=0.0, decay_full=0.0, dropout=0.0,
                  weight_decay_start=100, nesterov=True, mode="fused", reverse_complement=False, input_dropout=0.0,
                  start_training=0, feature_columns=0, constraint=None, single_launch=True, device="cuda"):
-        assert pool in ("max", "avg", "all") and loss in ("nll", "mse", None)
+        assert pool in ("max", "avg", "all") and loss in ("nll", "mse", "hinge", None)
         self.ninst, self.nfilter, self.m = int(nmodel), int(nfilter), int(m)
         self.pool, self.hidden, self.loss = pool, int(hidden), loss
         self.dtype, self.device, self.mode, self.nesterov = dtype, device, mode, nesterov
@@ -437,13 +437,13 @@ class SequenceNet(object):
         L = sm.sum_axis0(L)
         torch.cuda.synchronize()
         L = L.cpu().numpy() / st["Z"].shape[0]
-        return -L if self.loss == "nll" else 0.5 * L
+        return -L if self.loss == "nll" else (L if self.loss == "hinge" else 0.5 * L)
 
     # ------------------------------------------------------------------ backward
     def backward(self, X, R, st, Y, Ymask=None):
         """Fills dP with the gradient of the summed per-model losses (plus L1 decay when active)."""
         p, g, ni = self.p, self.g, self.ninst
-        dA = sm.sub_scale(st["Z"], Y, 1.0 / st["Z"].shape[0])
+        dA = (sm.hinge_grad if self.loss == "hinge" else sm.sub_scale)(st["Z"], Y, 1.0 / st["Z"].shape[0])
         if Ymask is not None:
             ds.maskout(Ymask, dA)
         if "Zmask" in st:
@@ -541,7 +541,7 @@ class SequenceNet(object):
             a = self._step_args = _lib.TrainStepArgs()
             off = {name: int(o) for (name, _, _), o in zip(self.layout, self.offsets[:-1])}
             a.nmodel, a.nfilter, a.m, a.hidden = ni, self.nfilter, self.m, self.hidden
-            a.ptype, a.loss_kind = _lib.str2pooltype[self.pool], {"nll": 0, "mse": 1}[self.loss]
+            a.ptype, a.loss_kind = _lib.str2pooltype[self.pool], _lib.LOSS_KIND[self.loss]
             a.reverse_complement = int(self.reverse_complement)
             a.nparam = self.P.numel()
             a.P, a.dP, a.mP = self.P.data_ptr(), self.dP.data_ptr(), self.mP.data_ptr()

@@ -109,11 +109,20 @@ def softmax(X, nchunk=1):
 
 
 def loss_terms(Z, Y, kind):
-    """Elementwise loss terms before masking / averaging; kind is "nll", "mse" or "nll_multiclass"
-    (several columns per output: log(max(1e-15, Z)) * Y, reference: deepity/std/loss.py:147-151)."""
+    """Elementwise loss terms before masking / averaging; kind is "nll", "mse", "nll_multiclass"
+    (several columns per output: log(max(1e-15, Z)) * Y, reference: deepity/std/loss.py:147-151) or "hinge"
+    (max(0, (1-Y)Z + Y(1-Z)), loss.py:162-163)."""
     L = torch.empty_like(Z)
-    call("dbk_loss_terms", stream(), dtype_code(Z), {"nll": 0, "mse": 1, "nll_multiclass": 2}[kind], ptr(Z), ptr(Y), ptr(L), Z.numel())
+    call("dbk_loss_terms", stream(), dtype_code(Z), {"nll": 0, "mse": 1, "nll_multiclass": 2, "hinge": 3}[kind], ptr(Z), ptr(Y), ptr(L), Z.numel())
     return L
+
+
+def hinge_grad(Z, Y, scale=1.0):
+    """Gradient of the hinge loss at the outputs: (1 - 2Y) * scale where (1-Y)Z + Y(1-Z) > 0, else 0
+    (reference: hinge._calc_dZ, deepity/std/loss.py:165-169)."""
+    dZ = torch.empty_like(Z)
+    call("dbk_hinge_grad", stream(), dtype_code(Z), ptr(Z), ptr(Y), float(scale), ptr(dZ), Z.numel())
+    return dZ
 
 
 def sub_scale(Z, Y, scale):

@@ -40,6 +40,13 @@ const char* dbk_last_error(void);
 int dbk_version(void);
 /* Number of HIP devices visible; <0 on failure. Touches the runtime only to count devices. */
 int dbk_device_count(void);
+/* on != 0: from now on dbk_corr1ord, dbk_corr1ord_bprop_W and dbk_corr1ord_bprop_X keep to their lookup / vector
+ * kernels at EVERY size, so that a row's result does not depend on the size of the batch it arrives in: dbk_corr1ord
+ * then adds the taps in the reference's order (corr1ord.cuh:139-157: its bits) for any number of rows, and the two
+ * gradients keep one summation order. Off (the default) float32 calls switch to the matrix-core kernels at bulk sizes
+ * (2^25 map values for the forward, 2^22 for the gradients): the same sums in another order, 1.5-2x faster.
+ * Process-wide; returns the previous setting. No counterpart in the reference (it has one kernel per operator). */
+int dbk_set_exact_scan(int on);
 /* Blocks until `stream` has drained. reference: api_sync, smat_cuda/cuda_context.cpp:198-202 */
 int dbk_sync(dbk_stream_t stream);
 
@@ -335,10 +342,14 @@ int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t 
  * smat/py/smat/tests/unittest.py:601-603 */
 int dbk_softmax(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n, size_t group);
 /* Elementwise loss terms L (n rows, m cols): kind 0 = log(max(1e-15,Z))*Y + log(max(1e-15,1-Z))*(1-Y),
- * kind 1 = (Z-Y)^2, kind 2 = log(max(1e-15,Z))*Y (multiclass). reference: deepity/std/loss.py:131-151 */
+ * kind 1 = (Z-Y)^2, kind 2 = log(max(1e-15,Z))*Y (multiclass), kind 3 = max(0, (1-Y)*Z + Y*(1-Z)) (bidirectional
+ * hinge). reference: deepity/std/loss.py:131-151,162-163 */
 int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, const void* Y, void* L, size_t n);
 /* dZ = (Z - Y) * scale. reference: deepity/std/loss.py:98-112 */
 int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n);
+/* Gradient of the hinge loss: dZ = (1 - 2Y) * scale where (1-Y)*Z + Y*(1-Z) > 0, else 0.
+ * reference: hinge._calc_dZ, deepity/std/loss.py:165-169 (dZ = 1-2Y, then maskout(L > 0, dZ)) */
+int dbk_hinge_grad(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n);
 
 /* The scan filters' constraint, applied to W (4m, nfilter) in place after every parameter update:
  * kind 0 ("pfm"): the four letter weights of every (tap, filter) become log(exp(w) / sum of the four exp(w));
@@ -369,7 +380,8 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
  * dropout (rate per model, NULL = none; uniforms from U when given, else from the generator at
  * (seed, offset), or at (seed, *counter) when counter is a device pointer; after the masks are drawn
  * *counter is advanced by counter_advance) -> dense (+bias, ReLU, dense
- * when hidden > 0) -> bias -> logistic (loss_kind 0) or identity (loss_kind 1) -> dA = (Z-Y)/n masked by
+ * when hidden > 0) -> bias -> logistic (loss_kind 0) or identity (loss_kind 1, 2) -> dA = (Z-Y)/n (loss_kind 2,
+ * the hinge loss: (1-2Y)/n where (1-Y)Z + Y(1-Z) > 0, else 0) masked by
  * Ymask (may be NULL) and, with reverse_complement, by the pair rule of dbk_calc_zmask -> all gradients.
  * Writes Z (n, nblock), dpooled (n, k*nblock), dW1, db1, dW2, db2 (overwritten, not accumulated) and,
  * if loss is not NULL, the per-model mean loss (nblock). Masks drawn here equal those of
@@ -377,7 +389,7 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
  * nfeat, feats: shared feature columns as in dbk_head_fprop (no dropout on them, no gradient back to them;
  * W1 and dW1 then have k + nfeat rows per model).
  * Replaces the reference's layer-by-layer head in a training step (deepity/std/elemwise.py:71-180,
- * full.py:78-119, softmax.py:58-77, loss.py:98-119). */
+ * full.py:78-119, softmax.py:58-77, loss.py:98-119,157-174). */
 int dbk_head_train(dbk_stream_t stream, size_t n, int nblock, int k, int hidden, int loss_kind, int reverse_complement,
                    const float* pooled, int nfeat, const float* feats, const float* rate, const float* U, uint64_t seed, uint64_t offset,
                    uint64_t* counter, uint64_t counter_advance,
@@ -399,7 +411,7 @@ int dbk_counter_add(dbk_stream_t stream, uint64_t* counter, uint64_t delta);
  * nmodel*nfilter; unused for avg pooling), Z (nregion, nmodel), and with input dropout Xdrop, Mdrop (N). */
 typedef struct dbk_train_step_args {
     size_t nmodel, nfilter, m, hidden;      /* architecture: filters per model, filter length, hidden units (0 = none) */
-    int ptype, loss_kind;                   /* DBK_PT_MAX / AVG / ALL; 0 = logistic + nll, 1 = identity + mse */
+    int ptype, loss_kind;                   /* DBK_PT_MAX / AVG / ALL; 0 = logistic + nll, 1 = identity + mse, 2 = identity + hinge */
     int reverse_complement, nesterov;
     size_t nparam;
     float *P, *dP, *mP;

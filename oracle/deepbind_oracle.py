@@ -17,6 +17,8 @@ checks live in tests/test_oracle_pins.py):
   poolrgn / _bprop    - np.max / np.argmax / np.mean per slice; scatter / uniform-spread adjoints
   bias/relu/logistic/nll/mse/maskout/calc_zmask - NumPy closed forms the reference's own
                         unit tests compare against (smat/tests/unittest.py:425-471,531-623)
+  hinge loss          - hand-worked values on both sides of both kinks (Y = 0: cost Z above 0; Y = 1: cost 1 - Z
+                        below 1), gradient against central finite differences of the loss away from the kinks
   softmax             - scipy.special.softmax per chunk (the reference's own test compares with a NumPy softmax,
                         smat/py/smat/tests/unittest.py:601-603); rows sum to one per chunk
   blockwise_dot*      - np.dot per block; no reference test exists at that boundary
@@ -448,10 +450,13 @@ def calc_zmask(Z):
 
 
 def loss_fprop(Z, Y, kind, ninst, Ymask=None, Zmask=None):
-    """Per-model mean loss, shape (1, ninst). kind in {"nll", "mse"}; one output column per model."""
+    """Per-model mean loss, shape (1, ninst). kind in {"nll", "mse", "hinge"}; one output column per model.
+    hinge: max(0, (1-Y)Z + Y(1-Z)), the reference's bidirectional hinge (deepity/std/loss.py:157-174)."""
     if kind == "nll":
         eps = Z.dtype.type(1e-15)
         L = np.log(np.maximum(eps, Z)) * Y + np.log(np.maximum(eps, 1 - Z)) * (1 - Y)
+    elif kind == "hinge":
+        L = np.maximum(0, (1 - Y) * Z + Y * (1 - Z))
     else:
         L = (Z - Y) ** 2
     L = L.astype(Z.dtype)
@@ -461,11 +466,16 @@ def loss_fprop(Z, Y, kind, ninst, Ymask=None, Zmask=None):
         maskout(Zmask, L)
     L = L.mean(axis=0, dtype=Z.dtype)
     L = L.reshape(ninst, -1).sum(axis=1).reshape(1, -1)
-    return (-L if kind == "nll" else Z.dtype.type(0.5) * L)
+    return -L if kind == "nll" else (L if kind == "hinge" else Z.dtype.type(0.5) * L)
 
 
-def loss_bprop(Z, Y, Ymask=None, Zmask=None):
-    dZ = (Z - Y).astype(Z.dtype)
+def loss_bprop(Z, Y, Ymask=None, Zmask=None, kind="nll"):
+    """dLoss/d(output): Z - Y for nll (through the logistic) and mse (deepity/std/loss.py:98-112); for the hinge
+    1 - 2Y where its argument is positive, else 0 (loss.py:165-169); then the masks and the 1/rows factor."""
+    if kind == "hinge":
+        dZ = ((1 - 2 * Y) * (((1 - Y) * Z + Y * (1 - Z)) > 0)).astype(Z.dtype)
+    else:
+        dZ = (Z - Y).astype(Z.dtype)
     if Ymask is not None:
         maskout(Ymask, dZ)
     if Zmask is not None:
@@ -609,7 +619,7 @@ def train_step(params, mom, X, R, Y, nmodel, pool, hidden, loss, rate, momentum,
     st = model_forward(params, X, R, nmodel, pool, hidden, out=out, dropout=dropout, train=True, matchrows=reverse_complement,
                        features=features)
     Zmask = calc_zmask(st["Zout"]) if reverse_complement else None      # deepity/std/loss.py:114-119
-    dA = loss_bprop(st["Zout"], Y, Ymask=Ymask, Zmask=Zmask)
+    dA = loss_bprop(st["Zout"], Y, Ymask=Ymask, Zmask=Zmask, kind=loss)
     g = model_backward(params, X, R, st, dA, nmodel, pool, hidden, dropout=dropout, train=True)
     if weight_decay_start <= step:
         # scan filters: the reference indexes its per-model decay with block length rows/ninst over the

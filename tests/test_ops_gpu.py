@@ -49,6 +49,50 @@ def test_corr1ord_bit_exact(ks, N, m, F):
     assert np.array_equal(host(Z), Zr)
 
 
+def test_exact_scan_switch_keeps_the_reference_bits_at_bulk_sizes(ks):
+    """With the library's exact-scan switch on, a map of more than 2^25 values comes out with the bits of the
+    reference's tap order (what smaller maps always get), the two gradients come from the vector kernels, and the
+    same rows give the same bits whether they arrive in a small batch or a bulk one."""
+    N, m, F = 140000, 24, 256
+    rng = np.random.default_rng(5)
+    X = random_codes(rng, N, 0.05, 0.03)
+    W = (rng.standard_normal((4 * m, F)) * 0.1).astype(np.float32)
+    Zr = np.zeros((N, F), np.float32)
+    orc.corr1ord(W, X, Zr)
+    Wd, Xd = dev(W), dev(X.reshape(-1, 1))
+    Zfast = dev(np.zeros((N, F), np.float32))
+    ks.corr1ord(Wd, Xd, Zfast, 4)
+    assert not np.array_equal(host(Zfast), Zr)                      # bulk size: the matrix-core kernel, equal to round-off only
+    assert_close(host(Zfast), Zr.astype(np.float64), ACT, "bulk map, default path")
+    dZ = dev(rng.standard_normal((N, F)).astype(np.float32))
+    grads = {}
+    assert ks.set_exact_scan(True) is False
+    try:
+        Z = dev(np.zeros((N, F), np.float32))
+        ks.corr1ord(Wd, Xd, Z, 4)
+        assert np.array_equal(host(Z), Zr)
+        n_small = 3000                                              # the same leading rows as a small batch of their own
+        Zs = dev(np.zeros((n_small, F), np.float32))
+        ks.corr1ord(Wd, dev(X[:n_small].reshape(-1, 1)), Zs, 4)
+        assert np.array_equal(host(Zs)[: n_small - m + 1], Zr[: n_small - m + 1])
+        for name, fn, shape in (("dW", lambda out: ks.corr1ord_bprop_W(out, Xd, dZ, 4), W.shape),
+                                ("dX", lambda out: ks.corr1ord_bprop_X(out, Wd, dZ, 4), (N, 4))):
+            out = dev(np.zeros(shape, np.float32))
+            fn(out)
+            grads[name] = host(out)
+    finally:
+        assert ks.set_exact_scan(False) is True
+    for name, fn, shape in (("dW", lambda out: ks.corr1ord_bprop_W(out, Xd, dZ, 4), W.shape),
+                            ("dX", lambda out: ks.corr1ord_bprop_X(out, Wd, dZ, 4), (N, 4))):
+        out = dev(np.zeros(shape, np.float32))
+        fn(out)
+        fast = host(out)
+        assert not np.array_equal(fast, grads[name]), "%s: the switch did not change the kernel" % name
+        assert_close(fast, grads[name].astype(np.float64), GRAD, "%s, matrix-core vs vector kernel" % name)
+    dWr = np.zeros(W.shape); orc.corr1ord_bprop_W(dWr, X, host(dZ).astype(np.float64))
+    assert_close(grads["dW"], dWr, GRAD, "dW with the switch on vs the oracle")
+
+
 @pytest.mark.parametrize("N,m,F", [(300000, 24, 128), (600001, 11, 70), (1100000, 32, 32)])
 def test_corr1ord_bulk_sizes_on_the_matrix_cores(ks, N, m, F):
     """From 2^25 map values on, float32 maps come from the matrix-core kernel: the same sums in another order, so the
@@ -762,6 +806,13 @@ def test_masks_dropout_and_loss_ops(ds, sm, ks):
     assert_close(host(sm.loss_terms(dev(Zl), dev(Y), "nll")), ref, ACT, "nll terms")
     assert_close(host(sm.loss_terms(dev(A), dev(Y), "mse")), (A - Y) ** 2, ACT, "mse terms")
     assert_close(host(sm.sub_scale(dev(Zl), dev(Y), 1.0 / n)), orc.loss_bprop(Zl, Y), ACT, "dZ")
+    # bidirectional hinge (deepity/std/loss.py:157-174): terms and gradient, float32 and float64, kinks included
+    for dt in (np.float32, np.float64):
+        Ah = (rng.standard_normal((n, nb)) * 2).astype(dt)
+        Ah[0, 0], Ah[1, 0], Y[0, 0], Y[1, 0] = 0.0, 1.0, 0.0, 1.0                  # exactly on the kinks: no cost, no gradient
+        Yh = Y.astype(dt)
+        assert np.array_equal(host(sm.loss_terms(dev(Ah), dev(Yh), "hinge")), np.maximum(0, (1 - Yh) * Ah + Yh * (1 - Ah)).astype(dt))
+        assert np.array_equal(host(sm.hinge_grad(dev(Ah), dev(Yh), 1.0 / n)), orc.loss_bprop(Ah, Yh, kind="hinge"))
     assert_close(host(sm.dot(dev(X), dev(X.T.copy()))), X.astype(np.float64) @ X.T.astype(np.float64), ACT, "dot")
     assert_close(host(sm.dot_nt(dev(X), dev(X))), X.astype(np.float64) @ X.T.astype(np.float64), ACT, "dot_nt")
     assert_close(host(sm.dot_tn(dev(X), dev(X))), X.T.astype(np.float64) @ X.astype(np.float64), ACT, "dot_tn")

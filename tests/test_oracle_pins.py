@@ -243,6 +243,36 @@ def test_loss_closed_forms_and_gradient():
     np.testing.assert_allclose(orc.loss_bprop(A, Yr), (A - Yr) / n, rtol=1e-12)
 
 
+def test_hinge_loss_worked_values_and_gradient():
+    """The bidirectional hinge (deepity/std/loss.py:157-174): a label-0 row costs its output where that is positive, a
+    label-1 row costs 1 - output where that is positive. Hand-worked rows on both sides of both kinks, then the
+    gradient against central finite differences of the loss at points away from the kinks."""
+    Z = np.array([[-0.5], [0.25], [2.0], [0.75], [1.5], [-1.0]])
+    Y = np.array([[0.0], [0.0], [0.0], [1.0], [1.0], [1.0]])
+    terms = np.array([0.0, 0.25, 2.0, 0.25, 0.0, 2.0])                # by hand: max(0, Z) for Y = 0, max(0, 1 - Z) for Y = 1
+    np.testing.assert_allclose(orc.loss_fprop(Z, Y, "hinge", 1).ravel(), [terms.mean()], rtol=1e-15)
+    slopes = np.array([0.0, 1.0, 1.0, -1.0, 0.0, -1.0])               # d term / dZ, by hand
+    np.testing.assert_allclose(orc.loss_bprop(Z, Y, kind="hinge").ravel(), slopes / len(Z), rtol=1e-15)
+    # masks drop rows from loss and gradient alike
+    Ymask = np.array([[True], [False], [True], [True], [True], [False]])
+    np.testing.assert_allclose(orc.loss_fprop(Z, Y, "hinge", 1, Ymask=Ymask).ravel(), [(terms * Ymask.ravel()).sum() / len(Z)], rtol=1e-15)
+    np.testing.assert_allclose(orc.loss_bprop(Z, Y, Ymask=Ymask, kind="hinge").ravel(), slopes * Ymask.ravel() / len(Z), rtol=1e-15)
+    rng = np.random.default_rng(31)
+    n, ninst = 40, 3
+    A = rng.standard_normal((n, ninst)) * 2
+    Yb = (rng.random((n, ninst)) < 0.5).astype(np.float64)
+    A[np.abs(A) < 0.05] = 0.3                                         # keep clear of the kinks at 0 (Y = 0) and 1 (Y = 1)
+    A[np.abs(A - 1) < 0.05] = 1.4
+    dA = orc.loss_bprop(A, Yb, kind="hinge")
+    eps = 1e-4
+    for i in range(n):
+        for j in range(ninst):
+            Ap = A.copy(); Ap[i, j] += eps
+            Am = A.copy(); Am[i, j] -= eps
+            fd = (orc.loss_fprop(Ap, Yb, "hinge", ninst).sum() - orc.loss_fprop(Am, Yb, "hinge", ninst).sum()) / (2 * eps)
+            np.testing.assert_allclose(dA[i, j], fd, rtol=1e-9, atol=1e-12)
+
+
 def test_zmask_and_maskout():
     Z = np.array([[1.0, 5.0], [2.0, 5.0], [3.0, -1.0], [0.0, np.nan]])
     M = orc.calc_zmask(Z)

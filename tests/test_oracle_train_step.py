@@ -92,7 +92,8 @@ def _fd_gradient(cost, p, h=1e-6):
     return g
 
 
-@pytest.mark.parametrize("pool,hid,loss,revcomp", [("max", 3, "nll", False), ("all", 0, "mse", False), ("max", 2, "nll", True)])
+@pytest.mark.parametrize("pool,hid,loss,revcomp", [("max", 3, "nll", False), ("all", 0, "mse", False), ("max", 2, "nll", True),
+                                                   ("avg", 2, "hinge", False)])
 def test_two_nesterov_steps_follow_the_docstring_recurrence_with_finite_difference_gradients(pool, hid, loss, revcomp):
     """P <- P + mu*mP ; g = dCost/dP there ; mP <- mu*mP - eta*g ; P <- P - eta*g, twice from mP = 0,
     where Cost is what the reference reports: per-model loss summed over models + L1 weight cost."""

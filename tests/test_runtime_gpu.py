@@ -88,3 +88,64 @@ def test_scratch_allocation_under_capture_is_refused_with_a_clear_error():
     finally:
         torch.cuda.synchronize()
         hip.hipStreamDestroy(raw)
+
+
+def test_scratch_of_a_captured_graph_survives_slot_recycling():
+    """A graph captured on a stream keeps the addresses of that stream's scratch. 70 further streams then ask for
+    scratch of their own (more than there are slots): the captured stream's slot is not handed on, and a replay of the
+    graph afterwards still gives the right sums. A larger eager call on the captured stream is refused (its buffer
+    cannot be replaced while the graph refers to it)."""
+    from deepbind_amd import _lib, smat as sm
+    hip = _hip()
+    hip.hipStreamCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    hip.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+    raw = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(raw)) == 0
+    side = torch.cuda.ExternalStream(raw.value)
+    rng = np.random.default_rng(1)
+    A = rng.standard_normal((5000, 64)).astype(np.float32)
+    Ad = dev(A)
+    other = dev(rng.standard_normal((5000, 48)).astype(np.float32))
+    streams = []
+    try:
+        with torch.cuda.stream(side):
+            first = host(sm.sum_axis0(Ad))                                  # eager: the stream's scratch exists from here on
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side, capture_error_mode="thread_local"):
+            out = sm.sum_axis0(Ad)
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(out), first)
+        for i in range(70):
+            s_ = ctypes.c_void_p()
+            assert hip.hipStreamCreate(ctypes.byref(s_)) == 0
+            streams.append(s_)
+            junk = torch.empty((1, 48), dtype=torch.float32, device="cuda")
+            _lib.call("dbk_colsum", s_, _lib.DBK_F32, _lib.ptr(other), _lib.ptr(junk), 5000, 48)
+            assert hip.hipStreamSynchronize(s_) == 0
+        out.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(out), first)
+        # a call whose partial sums (5.8 MB) do not fit the stream's first buffer (1 MB): refused there, fine elsewhere
+        from deepbind_amd import deepity_smat as ds
+        n, nb, k, h = 20000, 4, 16, 32
+        t = lambda *shape: torch.randn(shape, dtype=torch.float32, device="cuda") * 0.1
+        pooled, W1, b1, W2, b2, Y = t(n, k * nb), t(k * nb, h), t(1, h * nb), t(h * nb, 1), t(1, nb), (t(n, nb) > 0).float()
+        grads = lambda: (torch.empty_like(W1), torch.empty_like(b1), torch.empty_like(W2), torch.empty_like(b2))
+        with torch.cuda.stream(side):
+            with pytest.raises(_lib.DeepbindError, match="captured graph"):
+                ds.head_train(pooled, W1, b1, W2, b2, Y, nb, "nll", *grads())
+        Z, _, _ = ds.head_train(pooled, W1, b1, W2, b2, Y, nb, "nll", *grads())
+        assert bool(torch.isfinite(Z).all())
+        out.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(out), first)
+        del g
+    finally:
+        torch.cuda.synchronize()
+        for s_ in streams:
+            hip.hipStreamDestroy(s_)
+        hip.hipStreamDestroy(raw)

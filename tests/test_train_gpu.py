@@ -299,6 +299,44 @@ def test_head_train_loss_output():
     assert_close(host(dP), orc.blockwise_dot_nt(dA1, W1.astype(np.float64), nb), GRAD, "dpooled")
 
 
+@pytest.mark.parametrize("mode,single", [("fused", True), ("fused", False), ("unfused", False)])
+@pytest.mark.parametrize("pool,hidden,nm", [("max", 32, 1), ("all", 0, 3)])
+def test_hinge_loss_train_steps(mode, single, pool, hidden, nm):
+    """The reference's third loss (linear output, bidirectional hinge: deepity/std/loss.py:157-174) through the
+    single-launch step, the multi-launch step and layer by layer, against the oracle's whole step."""
+    from deepbind_amd import data
+    from deepbind_amd.model import SequenceNet
+    rng = np.random.default_rng(41)
+    m, nf, B = 12, 16, 96
+    seqs = ["".join("ACGT"[c] for c in rng.integers(0, 4, size=int(rng.integers(25, 60)))) for _ in range(B)]
+    X, R = data.pack_sequences(seqs, m - 1)
+    net = SequenceNet(nm, nf, m, pool=pool, hidden=hidden, loss="hinge", rate=0.05, momentum=0.9, decay_full=1e-3, weight_decay_start=1,
+                      mode=mode, single_launch=single)
+    params = {name: (rng.standard_normal(shape) * (0.3 if name.startswith("W") else 0.05)).astype(np.float32) for name, shape, _ in net.layout}
+    net.set_params(params)
+    Y = (rng.random((B, nm)) < 0.5).astype(np.float32)
+    Ymask = rng.random((B, nm)) < 0.9
+    Xd, Rd, Yd, Md = dev(X), dev(R), dev(Y), dev(Ymask)
+    ref_p, ref_m = _f64(params), {k: np.zeros(v.shape) for k, v in params.items()}
+    for step in range(3):
+        net.train_step(Xd, Rd, Yd, Md)
+        st, g = orc.train_step(ref_p, ref_m, X, R, Y.astype(np.float64), nm, pool, hidden, "hinge", 0.05, 0.9, Ymask=Ymask,
+                               decay_full=1e-3, step=step, weight_decay_start=1)
+        # (a prediction within round-off of a kink would flip a whole row's gradient: none is that close here)
+        act = (1 - Y) * st["Zout"] + Y * (1 - st["Zout"])
+        assert np.abs(act).min() > 1e-4
+        got_g = net.get_grads()
+        for name, _, axis in net.layout:
+            assert_close_per_model(got_g[name], g[name], GRAD, nm, axis, "step %d gradient %s" % (step, name))
+    assert any(buf.get("work") is not None for buf in net._step_bufs.values()) == (single and mode == "fused")
+    got = net.get_params()
+    for name, _, axis in net.layout:
+        assert_close_per_model(got[name], ref_p[name], GRAD, nm, axis, "parameters %s" % name)
+    st = net.forward(Xd, Rd)
+    want = orc.loss_fprop(orc.model_forward(ref_p, X, R, nm, pool, hidden)["Zout"], Y.astype(np.float64), "hinge", nm, Ymask=Ymask)
+    assert_close(net.loss_value(st, Yd, Md), want, 1e-4, "reported hinge loss")
+
+
 def test_graphed_step_replays_match_eager_steps():
     """A captured step must give the eager result on EVERY replay (fresh dropout masks included), with
     other work and synchronisations between the replays, and across the L1-decay switch-on."""

@@ -31,10 +31,13 @@ def test_static_scratch_entry_point_matches_the_allocating_one_on_consecutive_ca
         out_p = torch.full_like(want_p, float("nan"))
         out_i = torch.zeros_like(want_i) if want_i is not None else None
         torch.cuda.synchronize()
-        before = torch.cuda.memory_stats().get("allocation.all.allocated", 0)        # count of allocations made so far
+        before = torch.cuda.memory_stats().get("allocation.all.allocated", 0)        # count of allocations torch has made so far
+        free_before = torch.cuda.mem_get_info()[0]                                   # free device memory as the driver counts it
         got_p, got_i = ks.scanpool_fprop(W, b, Xd, Rd, ptype, want_argmax=want_argmax, path="kmer_static", out=(out_p, out_i))
         torch.cuda.synchronize()
         assert torch.cuda.memory_stats().get("allocation.all.allocated", 0) == before, "the host wrapper allocated"
+        # an allocation made inside the library (hipMalloc, not torch's) shows up here and nowhere else
+        assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated or freed during the call"
         assert np.array_equal(host(got_p), host(want_p)), "pooled differs (%d x %d, %s)" % (nseq, L, ptype)
         if want_i is not None:
             assert np.array_equal(host(got_i), host(want_i)), "argmax differs (%d x %d, %s)" % (nseq, L, ptype)
