@@ -50,6 +50,8 @@ _SIGNATURES = {
     "dbk_scanpool_bprop": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _P, _P, _P, _P, _P, _I, _P],
     "dbk_scanpool_fprop_unfused": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _I, _P, _P],
     "dbk_scanpool_bprop_unfused": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _I, _P, _P, _P, _P, _I],
+    "dbk_scanpool_fprop_f64": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _I, _P, _P],
+    "dbk_scanpool_bprop_f64": [_P, _P, _P, _Z, _Z, _P, _Z, _P, _Z, _I, _I, _P, _P, _P, _P, _I],
     "dbk_blockwise_dot": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
     "dbk_blockwise_dot_nt": [_P, _I, _I, _I, _I, _I, _P, _P, _P],
     "dbk_blockwise_dot_tn": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P],

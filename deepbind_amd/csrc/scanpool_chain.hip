@@ -9,49 +9,53 @@ namespace {
 
 // Z[i, f] = max(0, Z[i, f] + b[f]) for rows the scan wrote (i < n), max(0, b[f]) for the rest: the scan leaves rows
 // whose window passes the end of the sequence untouched, the bias and the rectifier apply to every row.
-__global__ __launch_bounds__(256) void k_bias_relu_rows(float* Z, const float* __restrict__ b, size_t n, size_t N, size_t F)
+template <typename T>
+__global__ __launch_bounds__(256) void k_bias_relu_rows(T* Z, const T* __restrict__ b, size_t n, size_t N, size_t F)
 {
     const size_t total = N * F;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
         const size_t i = e / F, f = e - i * F;
-        const float z = (i < n ? Z[e] : 0.0f) + b[f];
-        Z[e] = z > 0.0f ? z : 0.0f;
+        const T z = (i < n ? Z[e] : (T)0) + b[f];
+        Z[e] = z > (T)0 ? z : (T)0;
     }
 }
 
-__global__ __launch_bounds__(256) void k_fill_zero(float* p, size_t n)
+template <typename T>
+__global__ __launch_bounds__(256) void k_fill_zero(T* p, size_t n)
 {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.0f;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = (T)0;
 }
 
-int fill_zero(hipStream_t st, float* p, size_t n)
+template <typename T>
+int fill_zero(hipStream_t st, T* p, size_t n)
 {
-    hipLaunchKernelGGL(k_fill_zero, dim3(dbk::ew_grid(n)), dim3(256), 0, st, p, n);
+    hipLaunchKernelGGL(k_fill_zero<T>, dim3(dbk::ew_grid(n)), dim3(256), 0, st, p, n);
     DBK_LAUNCH_OK();
 }
 
+template <typename T> constexpr int dtype_of() { return sizeof(T) == 4 ? DBK_F32 : DBK_F64; }
+
 // relu(scan(W, X) + bias) for all N rows into `map`.
-int rectified_map(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t F, const uint8_t* X, size_t N, float* map)
+template <typename T>
+int rectified_map(dbk_stream_t stream, const T* W, const T* bias, size_t m, size_t F, const uint8_t* X, size_t N, T* map)
 {
     const size_t n = N >= m ? N - m + 1 : 0;
-    if (n > 0 && dbk_corr1ord(stream, DBK_F32, W, m, F, X, n, 4, map) != 0) return 1;
-    hipLaunchKernelGGL(k_bias_relu_rows, dim3(dbk::ew_grid(N * F)), dim3(256), 0, dbk::as_stream(stream), map, bias, n, N, F);
+    if (n > 0 && dbk_corr1ord(stream, dtype_of<T>(), W, m, F, X, n, 4, map) != 0) return 1;
+    hipLaunchKernelGGL(k_bias_relu_rows<T>, dim3(dbk::ew_grid(N * F)), dim3(256), 0, dbk::as_stream(stream), map, bias, n, N, F);
     DBK_LAUNCH_OK();
     return 0;
 }
 
-float* map_scratch(size_t N, size_t F, dbk_stream_t stream, int which)
+template <typename T>
+T* map_scratch(size_t N, size_t F, dbk_stream_t stream, int which)
 {
-    return (float*)dbk::workspace(N * F * sizeof(float), dbk::as_stream(stream), which);
+    return (T*)dbk::workspace(N * F * sizeof(T), dbk::as_stream(stream), which);
 }
 
-}  // namespace
-
-extern "C" {
-
-int dbk_scanpool_fprop_unfused(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
-                               const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
-                               float* pooled, uint32_t* argmax)
+template <typename T>
+int chain_fprop(dbk_stream_t stream, const T* W, const T* bias, size_t m, size_t nfilter,
+                const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                T* pooled, uint32_t* argmax)
 {
     DBK_CHECK(ptype >= DBK_PT_MAX && ptype <= DBK_PT_ALL, "ValueError: unknown pooling type %d", ptype);
     DBK_CHECK(region_columns == 2 || region_columns == 3, "ValueError: regions have 2 columns, or 3 with a row step (got %d)", region_columns);
@@ -62,15 +66,16 @@ int dbk_scanpool_fprop_unfused(dbk_stream_t stream, const float* W, const float*
     if (nfilter == 0 || nregion == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && X && regions && pooled, "ValueError: null pointer argument");
     DBK_CHECK(N > 0, "ValueError: regions over an empty sequence");
-    float* map = map_scratch(N, nfilter, stream, 2);
+    T* map = map_scratch<T>(N, nfilter, stream, 2);
     DBK_CHECK(map, "MemoryError: no scratch for the %zu x %zu map: %s", N, nfilter, dbk::workspace_error());
-    if (rectified_map(stream, W, bias, m, nfilter, X, N, map) != 0) return 1;
-    return dbk_poolrgn(stream, DBK_F32, map, nfilter, regions, nregion, region_columns == 3, pooled, argmax, ptype);
+    if (rectified_map<T>(stream, W, bias, m, nfilter, X, N, map) != 0) return 1;
+    return dbk_poolrgn(stream, dtype_of<T>(), map, nfilter, regions, nregion, region_columns == 3, pooled, argmax, ptype);
 }
 
-int dbk_scanpool_bprop_unfused(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
-                               const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
-                               const uint32_t* argmax, const float* dpooled, float* dW, float* dbias, int overwrite)
+template <typename T>
+int chain_bprop(dbk_stream_t stream, const T* W, const T* bias, size_t m, size_t nfilter,
+                const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                const uint32_t* argmax, const T* dpooled, T* dW, T* dbias, int overwrite)
 {
     DBK_CHECK(ptype >= DBK_PT_MAX && ptype <= DBK_PT_ALL, "ValueError: unknown pooling type %d", ptype);
     DBK_CHECK(region_columns == 2 || region_columns == 3, "ValueError: regions have 2 columns, or 3 with a row step (got %d)", region_columns);
@@ -79,23 +84,56 @@ int dbk_scanpool_bprop_unfused(dbk_stream_t stream, const float* W, const float*
     if (nfilter == 0) { dbk::clear_error(); return 0; }
     DBK_CHECK(W && bias && dW && dbias, "ValueError: null pointer argument");
     hipStream_t st = dbk::as_stream(stream);
-    if (overwrite && fill_zero(st, dW, 4 * m * nfilter) != 0) return 2;
-    if (nregion == 0 || N == 0) return fill_zero(st, dbias, nfilter);
+    if (overwrite && fill_zero<T>(st, dW, 4 * m * nfilter) != 0) return 2;
+    if (nregion == 0 || N == 0) return fill_zero<T>(st, dbias, nfilter);
     DBK_CHECK(!peak || argmax != nullptr, "ValueError: pooledmaps_argmax must be specified for max pooling.");
     DBK_CHECK(X && regions && dpooled, "ValueError: null pointer argument");
-    float* map = map_scratch(N, nfilter, stream, 2);
+    T* map = map_scratch<T>(N, nfilter, stream, 2);
     DBK_CHECK(map, "MemoryError: no scratch for the %zu x %zu map: %s", N, nfilter, dbk::workspace_error());
-    float* dmap = map_scratch(N, nfilter, stream, 3);
+    T* dmap = map_scratch<T>(N, nfilter, stream, 3);
     DBK_CHECK(dmap, "MemoryError: no scratch for the %zu x %zu map gradient: %s", N, nfilter, dbk::workspace_error());
-    if (rectified_map(stream, W, bias, m, nfilter, X, N, map) != 0) return 1;
-    if (fill_zero(st, dmap, N * nfilter) != 0) return 2;
-    if (dbk_poolrgn_bprop(stream, DBK_F32, dmap, nfilter, regions, nregion, region_columns == 3, dpooled, peak ? argmax : nullptr, ptype) != 0) return 1;
-    if (dbk_mul_sign(stream, DBK_F32, dmap, map, dmap, N * nfilter) != 0) return 1;
-    if (dbk_colsum(stream, DBK_F32, dmap, dbias, N, nfilter) != 0) return 1;
+    const int dt = dtype_of<T>();
+    if (rectified_map<T>(stream, W, bias, m, nfilter, X, N, map) != 0) return 1;
+    if (fill_zero<T>(st, dmap, N * nfilter) != 0) return 2;
+    if (dbk_poolrgn_bprop(stream, dt, dmap, nfilter, regions, nregion, region_columns == 3, dpooled, peak ? argmax : nullptr, ptype) != 0) return 1;
+    if (dbk_mul_sign(stream, dt, dmap, map, dmap, N * nfilter) != 0) return 1;
+    if (dbk_colsum(stream, dt, dmap, dbias, N, nfilter) != 0) return 1;
     const size_t n = N >= m ? N - m + 1 : 0;
-    if (n > 0 && dbk_corr1ord_bprop_W(stream, DBK_F32, dW, m, nfilter, X, n, 4, dmap) != 0) return 1;
+    if (n > 0 && dbk_corr1ord_bprop_W(stream, dt, dW, m, nfilter, X, n, 4, dmap) != 0) return 1;
     dbk::clear_error();
     return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dbk_scanpool_fprop_unfused(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
+                               const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                               float* pooled, uint32_t* argmax)
+{
+    return chain_fprop<float>(stream, W, bias, m, nfilter, X, N, regions, nregion, region_columns, ptype, pooled, argmax);
+}
+
+int dbk_scanpool_bprop_unfused(dbk_stream_t stream, const float* W, const float* bias, size_t m, size_t nfilter,
+                               const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                               const uint32_t* argmax, const float* dpooled, float* dW, float* dbias, int overwrite)
+{
+    return chain_bprop<float>(stream, W, bias, m, nfilter, X, N, regions, nregion, region_columns, ptype, argmax, dpooled, dW, dbias, overwrite);
+}
+
+int dbk_scanpool_fprop_f64(dbk_stream_t stream, const double* W, const double* bias, size_t m, size_t nfilter,
+                           const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                           double* pooled, uint32_t* argmax)
+{
+    return chain_fprop<double>(stream, W, bias, m, nfilter, X, N, regions, nregion, region_columns, ptype, pooled, argmax);
+}
+
+int dbk_scanpool_bprop_f64(dbk_stream_t stream, const double* W, const double* bias, size_t m, size_t nfilter,
+                           const uint8_t* X, size_t N, const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                           const uint32_t* argmax, const double* dpooled, double* dW, double* dbias, int overwrite)
+{
+    return chain_bprop<double>(stream, W, bias, m, nfilter, X, N, regions, nregion, region_columns, ptype, argmax, dpooled, dW, dbias, overwrite);
 }
 
 }  // extern "C"

@@ -167,7 +167,8 @@ def activity_words(X, W):
 
 def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=None, out=None):
     """pool(relu(corr1ord(W, X) + b)) per region without storing the (N x P) map.
-    Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32 only.
+    Returns (pooled, argmax|None) laid out exactly as poolrgn's. float32; float64 tensors run the operator kernels in
+    double precision one after another inside the library (no fused float64 kernel).
     path: "auto" lets the library choose; "general" / "mfma" / "wide" / "kmer" force the general path (which picks its
     kernel by size), its matrix-core kernel for many regions (filters of up to 32 taps; sums in another order than
     the lookup kernels', equal to round-off), the four-filters-per-lane lookup kernel (9-24 taps; the bits of the
@@ -181,25 +182,27 @@ def scanpool_fprop(W, b, X, regions, ptype, want_argmax=False, path="auto", act=
     the map in its scratch: same results as the reference's chain; path must be "auto" and no masks are written."""
     _u8(X)
     _regions(regions)
-    unfused = regions.shape[1] == 3 or ptype == "sum"
+    f64 = W.dtype == torch.float64
+    unfused = regions.shape[1] == 3 or ptype == "sum" or f64
     require(not unfused or (path == "auto" and act is None),
-            "ValueError: sum pooling and stepped regions run the operator chain: no kernel choice, no activity masks")
-    require(W.dtype == torch.float32 and b.dtype == torch.float32, "TypeError: the fused path is float32 only")
+            "ValueError: sum pooling, stepped regions and float64 run the operator chain: no kernel choice, no activity masks")
+    require(W.dtype in (torch.float32, torch.float64) and b.dtype == W.dtype, "TypeError: W and b must both be float32 or both float64")
     require(W.shape[0] % 4 == 0 and b.numel() == W.shape[1], "ValueError: W must be (4m x P) and b must have P entries")
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
     want_argmax = want_argmax and ptype in ("max", "all")
     if out is not None:
         pooled, argmax = out
-        require(pooled.dtype == torch.float32 and tuple(pooled.shape) == (P, F * (2 if ptype == "all" else 1)),
-                "ValueError: out[0] must be float32 (regions x pooled features)")
+        require(pooled.dtype == W.dtype and tuple(pooled.shape) == (P, F * (2 if ptype == "all" else 1)),
+                "ValueError: out[0] must be (regions x pooled features) of W's dtype")
         require((argmax is not None) == bool(want_argmax), "ValueError: out[1] must be given exactly when argmax is wanted")
         require(argmax is None or (argmax.dtype == uindex and tuple(argmax.shape) == (P, F)), "ValueError: out[1] must be (regions x filters) indices")
     else:
-        pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=torch.float32, device=W.device)
+        pooled = torch.empty((P, F * (2 if ptype == "all" else 1)), dtype=W.dtype, device=W.device)
         argmax = torch.empty((P, F), dtype=uindex, device=W.device) if want_argmax else None
     if unfused:
-        call("dbk_scanpool_fprop_unfused", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, regions.shape[1],
-             str2pooltype[ptype], ptr(pooled), ptr(argmax))
+        # (float64: the operator kernels in double precision, as the reference compiles every operator for both types)
+        call("dbk_scanpool_fprop_f64" if f64 else "dbk_scanpool_fprop_unfused", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(),
+             ptr(regions), P, regions.shape[1], str2pooltype[ptype], ptr(pooled), ptr(argmax))
         return pooled, argmax
     entry = {"auto": "dbk_scanpool_fprop", "general": "dbk_scanpool_fprop_general", "wide": "dbk_scanpool_fprop_wide", "mfma": "dbk_scanpool_fprop_mfma",
              "kmer": "dbk_scanpool_fprop_kmer", "kmer_static": "dbk_scanpool_fprop_kmer_static"}[path]
@@ -225,14 +228,16 @@ def scanpool_bprop(W, b, X, regions, ptype, pooled, argmax, dpooled, dW, db, ove
     act: the activity masks the forward call filled (same W, b, X, regions), if it was given any."""
     _u8(X)
     _regions(regions)
-    require(W.dtype == torch.float32 and dpooled.dtype == torch.float32, "TypeError: the fused path is float32 only")
+    f64 = W.dtype == torch.float64
+    require(W.dtype in (torch.float32, torch.float64) and all(t.dtype == W.dtype for t in (b, dpooled, dW, db)),
+            "TypeError: W, b, dpooled, dW and db must all be float32 or all float64")
     require(dW.shape == W.shape and db.numel() == W.shape[1], "ValueError: dW / db shapes must match W / b")
     require(dpooled.shape == pooled.shape, "ValueError: dpooled must have pooled's shape")
     m, F, P = W.shape[0] // 4, W.shape[1], regions.shape[0]
-    if regions.shape[1] == 3 or ptype == "sum":
-        require(act is None, "ValueError: sum pooling and stepped regions take no activity masks")
-        call("dbk_scanpool_bprop_unfused", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, regions.shape[1],
-             str2pooltype[ptype], ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)))
+    if regions.shape[1] == 3 or ptype == "sum" or f64:
+        require(act is None, "ValueError: sum pooling, stepped regions and float64 take no activity masks")
+        call("dbk_scanpool_bprop_f64" if f64 else "dbk_scanpool_bprop_unfused", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(),
+             ptr(regions), P, regions.shape[1], str2pooltype[ptype], ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)))
         return
     call("dbk_scanpool_bprop", stream(), ptr(W), ptr(b), m, F, ptr(X), X.numel(), ptr(regions), P, str2pooltype[ptype],
          ptr(pooled), ptr(argmax), ptr(dpooled), ptr(dW), ptr(db), int(bool(overwrite)), _act(act, X, F))

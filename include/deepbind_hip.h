@@ -228,6 +228,21 @@ int dbk_scanpool_bprop_unfused(dbk_stream_t stream,
                                const uint32_t* regions, size_t nregion, int region_columns, int ptype,
                                const uint32_t* argmax, const float* dpooled,
                                float* dW, float* dbias, int overwrite);
+/* The two calls above in float64, for callers that run the whole path in double precision as the reference can
+ * (every operator there is compiled for both float types, corr1ord.cu:129-133): same arguments, same chain of
+ * operator kernels (there is no fused float64 kernel), any pooling type, 2 or 3 region columns.
+ * reference: as dbk_scanpool_fprop_unfused / dbk_scanpool_bprop_unfused */
+int dbk_scanpool_fprop_f64(dbk_stream_t stream,
+                           const double* W, const double* bias, size_t m, size_t nfilter,
+                           const uint8_t* X, size_t N,
+                           const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                           double* pooled, uint32_t* argmax);
+int dbk_scanpool_bprop_f64(dbk_stream_t stream,
+                           const double* W, const double* bias, size_t m, size_t nfilter,
+                           const uint8_t* X, size_t N,
+                           const uint32_t* regions, size_t nregion, int region_columns, int ptype,
+                           const uint32_t* argmax, const double* dpooled,
+                           double* dW, double* dbias, int overwrite);
 
 /* ------------------------------------------------------------------ dense head (deepity_smat) */
 

@@ -461,6 +461,35 @@ def test_scanpool_sum_pooling_and_stepped_regions(ks, ptype, stepped, B, lo, hi,
         ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, path="general")
 
 
+@pytest.mark.parametrize("ptype,stepped", [("max", False), ("avg", False), ("all", False), ("sum", True)])
+def test_scanpool_float64(ks, ptype, stepped):
+    """The two fused calls with float64 tensors (the reference compiles every operator for both float types): the
+    operator kernels in double precision inside the library, forward and backward against the float64 oracle chain
+    at float64 accuracy."""
+    rng, W, b, X, R = _fused_case(91, 40, 5, 120, 13, 37, p254=0.01)
+    if stepped:
+        R = np.concatenate([R, rng.integers(1, 4, size=(len(R), 1)).astype(np.uint32)], axis=1)
+    W, b = W.astype(np.float64), b.astype(np.float64)
+    A, Pr, Ir = _chain_oracle(W, b, X, R, ptype)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    P, I = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=True)
+    assert P.dtype == torch.float64
+    assert_close(host(P), Pr, 1e-13, "pooled")
+    if Ir is not None:
+        assert np.array_equal(host(I), Ir)
+    dP = rng.standard_normal(Pr.shape)
+    dA = np.zeros_like(A)
+    orc.poolrgn_bprop(dA, R, dP, Ir, ptype)
+    dZ = orc.relu_bprop(dA, A)
+    dWr = np.zeros(W.shape); orc.corr1ord_bprop_W(dWr, X, dZ)
+    dW, db = dev(np.ones(W.shape)), dev(np.full((1, W.shape[1]), 7.0))
+    ks.scanpool_bprop(Wd, bd, Xd, Rd, ptype, P, I, dev(dP), dW, db)
+    assert_close(host(dW), dWr + 1.0, 1e-12, "dW")
+    assert_close(host(db), orc.bias_bprop(dZ)[1], 1e-12, "db")
+    with pytest.raises(Exception, match="both be float32 or both float64"):
+        ks.scanpool_fprop(Wd, dev(b.astype(np.float32)), Xd, Rd, ptype)
+
+
 def test_scanpool_unfused_chain_agrees_with_the_fused_kernels(ks):
     """Step 1 in the third column is the 2-column case: the chain and the fused kernels then compute the same function."""
     rng, W, b, X, R = _fused_case(77, 40, 20, 60, 16, 48)

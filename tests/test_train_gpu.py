@@ -578,10 +578,12 @@ def test_init_params_penalty_and_frozen_filters():
     assert_close(net.penalty_value(), want, ACT, "L1 cost")
 
 
+@pytest.mark.parametrize("mode", ["unfused", "fused"])
 @pytest.mark.parametrize("pool,hidden,loss", [("max", 6, "nll"), ("all", 0, "mse"), ("avg", 4, "nll")])
-def test_gradcheck_float64_layer_by_layer(pool, hidden, loss):
+def test_gradcheck_float64_layer_by_layer(pool, hidden, loss, mode):
     """The trainer's own finite-difference check, on the device in float64: HIP forward against HIP backward,
-    no oracle involved; and the checker must notice a wrong gradient."""
+    no oracle involved; and the checker must notice a wrong gradient. Mode "fused" takes the scan + pool chain through
+    the two fused calls, which run the operator kernels in double precision inside the library."""
     from deepbind_amd import data
     from deepbind_amd.gradcheck import gradcheck
     from deepbind_amd.model import SequenceNet
@@ -590,7 +592,7 @@ def test_gradcheck_float64_layer_by_layer(pool, hidden, loss):
     seqs = ["".join("ACGTN"[v] for v in rng.choice(5, int(rng.integers(8, 16)), p=[.24, .24, .24, .24, .04])) for _ in range(12)]
     X, R = data.pack_sequences(seqs, m - 1)
     net = SequenceNet(ni, nf, m, pool=pool, hidden=hidden, loss=loss, dtype=torch.float64, dropout=[0.0, 0.3],
-                      decay_conv=[1e-3, 1e-3], decay_full=[3e-3, 1e-3], weight_decay_start=0, mode="unfused")
+                      decay_conv=[1e-3, 1e-3], decay_full=[3e-3, 1e-3], weight_decay_start=0, mode=mode)
     # (equal scan-filter decays: with different ones the reference's gradient uses its rows/ninst block length,
     # kangaroo/_ext/corr1ord.py:126, and is not the derivative of its own cost; that quirk is kept and tested elsewhere)
     net.init_params(init_conv=0.5, init_full=0.5, init_mu=0.1, seed=5)
