@@ -176,9 +176,13 @@ def train_throughput(steps=3000, warmup=300, cpu=True):
     out = {}
 
     def timed(fn, nseq, nmodel):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
+        # Two warm-up bursts: the first pays for scratch buffers and first launches, the second lets the host run as far
+        # ahead of the GPU as it does in the timed loop - the first time the launch queue fills up, the HIP runtime
+        # stalls one call for tens of milliseconds (measured: 52 ms, once per process), which belongs to neither step.
+        for _ in range(2):
+            for _ in range(warmup):
+                fn()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()

@@ -36,9 +36,224 @@ struct head_args {
     unsigned nchunk, pstride;
 };
 
+// Orders a wave's own LDS traffic: what its lanes stored before is what its lanes read after (the LDS serves a wave's
+// instructions in order; the fences keep the compiler from moving them and wait for the counter).
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+template <int CTRL>
+__device__ __forceinline__ float lane_move(float v) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true)); }
+
+// The head of a model with 32 hidden units and 16 or 32 inputs (the shapes of the reference's models: 16 filters, max or
+// max + average pooling, cfg/classification/M1.cfg) for a chunk of 32 rows, with the weights in REGISTERS while they
+// are used: the workgroup stages the model's W1 in LDS with one 16-byte load per thread, then each of the four waves
+// takes eight rows through forward and backward on its own, two rows at a time (a row per half wave), with no
+// workgroup barrier until the chunk's gradient sums. A lane holds column j of W1 for the forward pass (lane = hidden
+// unit: 32 multiply-adds per row, the row's inputs read from LDS as broadcasts) and row j for the way back (lane =
+// input). The eight rows' output non-linearity, loss gradient and loss term are computed ONCE, eight lanes side by side
+// (the general body below computes them in every lane of a row, and reads a weight from LDS per multiply-add).
+// Every sum is formed in the order of the general body (inputs ascending, hidden units ascending, rows ascending; the
+// output sum as eight partial sums of every eighth unit folded by a butterfly), so the two bodies give the same bits.
+template <int KT>
+__device__ __forceinline__ void head_train_h32(const head_args& a, const unsigned b, const unsigned chunk)
+{
+    extern __shared__ float hs[];
+    constexpr int H = 32, WS = 36;          // hidden units; floats from one row of W1 to the next in LDS (16-byte reads of
+                                            // neighbouring rows then start four banks apart)
+    float* w1s = hs;                        // [KT][WS]
+    float* xs = w1s + KT * WS;              // [RB][KT] inputs after dropout
+    float* H1s = xs + RB * KT;              // [RB][H]  hidden activations
+    float* D1s = H1s + RB * H;              // [RB][H]  gradient at the hidden pre-activations
+    float* dAs = D1s + RB * H;              // [RB]
+    float* lss = dAs + RB;                  // [RB]
+    unsigned char* kept = reinterpret_cast<unsigned char*>(lss + RB);   // [RB][KT] dropout keep flags
+    const unsigned tid = threadIdx.x, lane = tid & 63u, j = lane & 31u, half = lane >> 5;
+    const unsigned wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const int k = a.k;
+    const size_t r0 = (size_t)chunk * RB, ncol = (size_t)k * a.nblock;
+
+    // ---------------- everything the workgroup reads from global memory, requested in one round
+    const float p_drop = a.rate ? a.rate[b] : 0.0f;
+    const unsigned long long off = a.counter ? a.counter[0] : a.offset;
+    float4 wv = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (tid < (unsigned)(KT * H / 4)) wv = reinterpret_cast<const float4*>(a.W1 + (size_t)b * KT * H)[tid];
+    // lane L < 8 of a wave holds the target and mask of the wave's row L
+    const size_t r_mine = r0 + 8u * wave + (lane & 7u);
+    const bool live_mine = lane < 8u && r_mine < a.n;
+    const size_t zi_mine = live_mine ? r_mine * a.nblock + b : 0;
+    const float y_mine = live_mine ? a.Y[zi_mine] : 0.0f;
+    const bool use_mine = (live_mine && a.Ymask) ? a.Ymask[zi_mine] != 0 : true;
+    const float b1v = a.b1[(size_t)b * H + j], w2v = a.W2[(size_t)b * H + j], bias2 = a.b2[b];
+    const float inv_n = 1.0f / (float)a.n;
+    {   // the chunk's inputs, dropout applied (element numbering of the stand-alone dropout kernels): four consecutive
+        // features per thread - one 16-byte load and ONE call of the generator for their four uniforms
+        const unsigned kq = (unsigned)k >> 2;
+        const dbk::small_div by_kq(kq), by_kf((unsigned)(a.kf > 0 ? a.kf : 1));
+        for (unsigned e = tid; e < RB * kq; e += NT) {
+            const unsigned row = by_kq.quot(e), kk = 4u * by_kq.rem(e, row);
+            const size_t rr = r0 + row, col = (size_t)b * k + kk;
+            float4 xv = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            float u[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            const bool in = rr < a.n;
+            if (in) {
+                xv = *reinterpret_cast<const float4*>(a.pooled + rr * ncol + col);
+                if (a.rate) dbk_rng::uniform4_at(a.seed, off, ((a.revcomp ? (rr >> 1) : rr) * ncol + col) >> 2, u);
+            }
+            const float x4[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const bool kp = !(in && a.rate) || u[c] >= p_drop;
+                xs[row * KT + kk + c] = kp ? x4[c] : 0.0f;
+                kept[row * KT + kk + c] = kp;
+            }
+        }
+        for (unsigned e = tid; e < RB * (unsigned)a.kf; e += NT) {      // the shared feature columns follow the model's own inputs
+            const unsigned row = by_kf.quot(e), jj = by_kf.rem(e, row);
+            const size_t rr = r0 + row;
+            xs[row * KT + k + jj] = (a.feats && rr < a.n) ? a.feats[rr * a.kf + jj] : 0.0f;
+        }
+    }
+    if (tid < (unsigned)(KT * H / 4)) *reinterpret_cast<float4*>(w1s + (tid >> 3) * WS + 4u * (tid & 7u)) = wv;
+    __syncthreads();
+    float wc[KT], wr[H];
+#pragma unroll
+    for (int kk = 0; kk < KT; ++kk) wc[kk] = w1s[kk * WS + j];
+#pragma unroll
+    for (int q = 0; q < H / 4; ++q) {
+        const float4 v = reinterpret_cast<const float4*>(w1s + (j < (unsigned)KT ? j : 0u) * WS)[q];
+        wr[4 * q] = v.x; wr[4 * q + 1] = v.y; wr[4 * q + 2] = v.z; wr[4 * q + 3] = v.w;
+    }
+
+    // ---------------- forward, two rows per round: lane = hidden unit j of the half wave's row
+    // (the four rows' sums advance side by side: each is a chain of dependent additions, inputs ascending)
+    float sv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int q = 0; q < KT / 4; ++q) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 x4 = reinterpret_cast<const float4*>(xs + (8u * wave + 2u * i + half) * KT)[q];
+            sv[i] += x4.x * wc[4 * q];
+            sv[i] += x4.y * wc[4 * q + 1];
+            sv[i] += x4.z * wc[4 * q + 2];
+            sv[i] += x4.w * wc[4 * q + 3];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float s = sv[i] + b1v;
+        s = s > 0.0f ? s : 0.0f;
+        sv[i] = s;
+        H1s[(8u * wave + 2u * i + half) * H + j] = s;
+    }
+    // the rows' output sums: units p, p + 8, p + 16, p + 24 added in that order (p < 8), then a butterfly over the eight;
+    // row L of the wave's eight ends up in lane L
+    float o_mine = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float v = 0.0f + sv[i] * w2v;
+        const float u16 = __shfl_down(v, 16, 64), u24 = __shfl_down(v, 24, 64);
+        float t = v + lane_move<0x128>(v);                            // row_ror:8 - unit p + 8 of the same sixteen lanes
+        t += u16;
+        t += u24;
+        t += lane_move<0xB1>(t);                                      // quad_perm [1, 0, 3, 2]
+        t += lane_move<0x4E>(t);                                      // quad_perm [2, 3, 0, 1]
+        t += lane_move<0x141>(t);                                     // row_half_mirror: the other four of the eight
+        const float ta = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t), 0));
+        const float tb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t), 32));
+        if ((lane >> 1) == (unsigned)i) o_mine = (lane & 1u) ? tb : ta;
+    }
+    {   // output non-linearity, loss gradient and loss term of the eight rows, in lanes 0..7
+        const float out = o_mine + bias2;
+        const float z = a.loss_kind == 0 ? 1.0f / (1.0f + expf(-out)) : out;
+        // of each (fwd, rev) row pair only the larger prediction trains; ties keep the first row
+        const float zo = lane_move<0xB1>(z);
+        float dA = 0.0f, lterm = 0.0f;
+        if (live_mine) {
+            bool use = use_mine;
+            if (a.revcomp) use = use && ((r_mine & 1) ? !(zo >= z) : (z >= zo));
+            if (use) {
+                dA = dbk::loss_grad(a.loss_kind, z, y_mine) * inv_n;
+                lterm = dbk::loss_term(a.loss_kind, z, y_mine);
+            }
+            a.Z[zi_mine] = z;
+        }
+        if (lane < 8u) { dAs[8u * wave + lane] = dA; lss[8u * wave + lane] = lterm; }
+    }
+    wave_lds_sync();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const unsigned row = 8u * wave + 2u * i + half;
+        D1s[row * H + j] = sv[i] > 0.0f ? dAs[row] * w2v : 0.0f;
+    }
+    wave_lds_sync();
+
+    // ---------------- gradient back to the pooled features: lane = input j of the half wave's row
+    float gv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int q = 0; q < H / 4; ++q) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 d4 = reinterpret_cast<const float4*>(D1s + (8u * wave + 2u * i + half) * H)[q];
+            gv[i] += d4.x * wr[4 * q];
+            gv[i] += d4.y * wr[4 * q + 1];
+            gv[i] += d4.z * wr[4 * q + 2];
+            gv[i] += d4.w * wr[4 * q + 3];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const unsigned row = 8u * wave + 2u * i + half;
+        const size_t r = r0 + row;
+        if (r < a.n && j < (unsigned)k) a.dpooled[r * ncol + (size_t)b * k + j] = kept[row * KT + j] ? gv[i] : 0.0f;
+    }
+    __syncthreads();
+
+    // ---------------- this chunk's share of the parameter gradients, rows ascending
+    float* part_out = a.partial + ((size_t)chunk * a.nblock + b) * a.pstride;
+    constexpr int PER = KT / 8;                                       // consecutive inputs per thread
+    const unsigned kk0 = (unsigned)PER * (2u * wave + half);
+    float acc[PER], gb1 = 0.0f;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) acc[c] = 0.0f;
+#pragma unroll 16
+    for (int rr = 0; rr < RB; ++rr) {
+        const float d = D1s[rr * H + j];
+#pragma unroll
+        for (int c = 0; c < PER; ++c) acc[c] += xs[rr * KT + kk0 + c] * d;
+        gb1 += d;
+    }
+#pragma unroll
+    for (int c = 0; c < PER; ++c) part_out[(kk0 + c) * H + j] = acc[c];
+    // the small sums, one per wave (the wave's number is a scalar: no lane masks, the reads of a loop in flight together)
+    if (wave == 0) {
+        if (half == 0) part_out[KT * H + j] = gb1;
+    } else if (wave == 1) {
+        float gW2 = 0.0f;
+#pragma unroll 16
+        for (int rr = 0; rr < RB; ++rr) gW2 += H1s[rr * H + j] * dAs[rr];
+        if (half == 0) part_out[KT * H + H + j] = gW2;
+    } else {
+        const float* src = wave == 2 ? dAs : lss;
+        float sum = 0.0f;
+#pragma unroll 16
+        for (int rr = 0; rr < RB; ++rr) sum += src[rr];
+        if (lane == 0) part_out[KT * H + 2 * H + (wave == 2 ? 0 : 1)] = sum;
+    }
+}
+
 // b: model of the group, chunk: which RB rows
 __device__ __forceinline__ void head_train_body(const head_args& a, const unsigned b, const unsigned chunk)
 {
+    if (a.hidden == 32 && !a.U && (a.k & 3) == 0 && (((size_t)a.k * a.nblock) & 3) == 0 && ((uintptr_t)a.pooled & 15) == 0 &&
+        (a.k + a.kf == 16 || a.k + a.kf == 32)) {
+        if (a.k + a.kf == 32) head_train_h32<32>(a, b, chunk);
+        else head_train_h32<16>(a, b, chunk);
+        return;
+    }
     extern __shared__ float hs[];
     // kt inputs per model: its k pooled features, then the kf shared feature columns (no dropout, no gradient back)
     const int k = a.k, kt = a.k + a.kf, hidden = a.hidden, h1 = hidden > 0 ? hidden : 1;
@@ -296,7 +511,9 @@ __global__ void k_head_reduce(head_args a)
 inline size_t head_smem(int k, int kf, int h1)
 {
     const int kt = k + kf;
-    return ((size_t)kt * (h1 | 1) + 2 * h1 + (size_t)RB * (kt | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
+    const size_t general = ((size_t)kt * (h1 | 1) + 2 * h1 + (size_t)RB * (kt | 1) + 2 * (size_t)RB * (h1 | 1) + 2 * RB) * sizeof(float) + (size_t)RB * k;
+    const size_t h32 = ((size_t)kt * 36 + (size_t)RB * kt + 2 * (size_t)RB * 32 + 2 * RB) * sizeof(float) + (size_t)RB * kt;      // head_train_h32's carve-up
+    return general > h32 ? general : h32;
 }
 
 }  // namespace

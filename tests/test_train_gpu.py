@@ -299,6 +299,38 @@ def test_head_train_loss_output():
     assert_close(host(dP), orc.blockwise_dot_nt(dA1, W1.astype(np.float64), nb), GRAD, "dpooled")
 
 
+@pytest.mark.parametrize("k,nfeat,loss,rc", [(16, 0, "nll", False), (32, 0, "nll", True), (16, 16, "mse", False), (32, 0, "hinge", False),
+                                             (12, 4, "nll", True)])
+def test_head_train_register_body_gives_the_bits_of_the_general_body(k, nfeat, loss, rc):
+    """Heads of 32 hidden units on 16 or 32 inputs run with the weights in registers (head_train.hip, head_train_h32);
+    with uniforms supplied the call takes the general body. Same uniforms -> every output bit for bit the same:
+    the register body forms each sum in the general body's order. 333 rows: the last chunk is ragged."""
+    from deepbind_amd import deepity_smat as ds
+    rng = np.random.default_rng(k + nfeat)
+    n, nb, h = 334 if rc else 333, 6, 32
+    kt = k + nfeat
+    t = lambda *shape, s=0.3: dev((rng.standard_normal(shape) * s).astype(np.float32))
+    Pl = dev(np.abs(rng.standard_normal((n, k * nb))).astype(np.float32))
+    W1, b1, W2, b2 = t(kt * nb, h), t(1, h * nb, s=0.1), t(h * nb, 1), t(1, nb, s=0.1)
+    F = t(n, nfeat, s=1.0) if nfeat else None
+    Y = dev((rng.random((n, nb)) < 0.5).astype(np.float32))
+    M = dev(rng.random((n, nb)) < 0.8)
+    rate = dev(np.array([0.0, 0.5, 0.25, 0.5, 0.0, 0.9], np.float32))
+    seed, offset = 11, 1234
+    U = ds.uniform_like(torch.empty((n // 2 if rc else n, k * nb), device="cuda"), seed, offset)
+    if rc:
+        U = U.repeat_interleave(2, dim=0).contiguous()                # a (fwd, rev) pair shares its draw
+    outs = []
+    for uniforms in (None, U):
+        g = [torch.full_like(w, float("nan")) for w in (W1, b1, W2, b2)]
+        Z, dP, L = ds.head_train(Pl, W1, b1, W2, b2, Y, nb, loss, g[0], g[1], g[2], g[3], Ymask=M, rate=rate, U=uniforms, seed=seed,
+                                 offset=offset, reverse_complement=rc, want_loss=True, nfeat=nfeat, feats=F)
+        outs.append([host(x) for x in (Z, dP, L, *g)])
+    for name, a, b in zip(("Z", "dpooled", "loss", "dW1", "db1", "dW2", "db2"), *outs):
+        assert np.isfinite(a).all() and np.array_equal(a, b), name
+    assert (outs[0][1] == 0).mean() > 0.2                               # dropout did drop inputs
+
+
 @pytest.mark.parametrize("mode,single", [("fused", True), ("fused", False), ("unfused", False)])
 @pytest.mark.parametrize("pool,hidden,nm", [("max", 32, 1), ("all", 0, 3)])
 def test_hinge_loss_train_steps(mode, single, pool, hidden, nm):
