@@ -179,10 +179,14 @@ def train_throughput(steps=3000, warmup=300, cpu=True):
         # Two warm-up bursts: the first pays for scratch buffers and first launches, the second lets the host run as far
         # ahead of the GPU as it does in the timed loop - the first time the launch queue fills up, the HIP runtime
         # stalls one call for tens of milliseconds (measured: 52 ms, once per process), which belongs to neither step.
-        for _ in range(2):
+        # ... and the bursts go on until a quarter of a second of GPU work has passed: after seconds of host-only work
+        # (the CPU baselines) the GPU takes a while to return to the clock it holds under load.
+        t_warm, bursts = time.perf_counter(), 0
+        while bursts < 2 or time.perf_counter() - t_warm < 0.25:
             for _ in range(warmup):
                 fn()
             torch.cuda.synchronize()
+            bursts += 1
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()
@@ -206,6 +210,7 @@ def train_throughput(steps=3000, warmup=300, cpu=True):
             r["dominant_kernel"] = dom
         return r
 
+    cpu_jobs = []                        # the CPU baselines run after every GPU timing: seconds of host-only work in between let the GPU clock down
     for tag, name, cfg, drop in (("config2", "config2_rna_regression", synth.config2(), 0.0),
                                  ("config3", "config3_classification", synth.config3(), 0.5)):
         spec = cfg["spec"]
@@ -218,7 +223,7 @@ def train_throughput(steps=3000, warmup=300, cpu=True):
         out[name]["roofline"] = roofline(tag, cfg, out[name])
         if cpu:
             cfg["dropout_rate"] = drop
-            out[name]["cpu_baseline"] = train_cpu_baseline(cfg, [([0], spec.pool[0], spec.hidden[0], cfg["params"])], nsteps=5)
+            cpu_jobs.append((name, cfg, [([0], spec.pool[0], spec.hidden[0], cfg["params"])], 5))
     cfg = synth.config4()
     spec, hp = cfg["spec"], cfg["hp"]
     grp = ModelGroup(spec.pool, spec.hidden, spec.nfilter, spec.m, loss="nll", rate=hp["rate"], momentum=hp["momentum"],
@@ -235,7 +240,9 @@ def train_throughput(steps=3000, warmup=300, cpu=True):
     out[name]["graphed"] = timed(grp.make_graphed_step(X, R, Y, M), len(cfg["R"]), spec.nmodel)
     out[name]["roofline"] = roofline("config4", cfg, out[name])
     if cpu:
-        out[name]["cpu_baseline"] = train_cpu_baseline(cfg, stacked, nsteps=2)
+        cpu_jobs.append((name, cfg, stacked, 2))
+    for name, cfg, groups, nsteps in cpu_jobs:
+        out[name]["cpu_baseline"] = train_cpu_baseline(cfg, groups, nsteps=nsteps)
     return out
 
 
