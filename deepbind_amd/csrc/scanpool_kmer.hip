@@ -113,45 +113,50 @@ __device__ __forceinline__ unsigned row_share(unsigned v)
     return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + SRC, 0xf, 0xf, false);
 }
 
-// One unrolled block of 3G text positions for one lane.
-//   k0, k1    table byte offsets (triple index * bytes per triple) of this block's positions, spread
-//             over the stream's 16 lanes: lane i holds position i in k0 and position 16+i in k1
-//   acc       ring of partial sums (2 filters per lane), mx the running max
 // MODE bits: what a finished position is folded into
 constexpr int M_MAX = 1, M_ARG = 2, M_SUM = 4;
 
-template <int G, int MODE>
-__device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigned k0, unsigned k1,
-                                           float2 (&acc)[3][G], float2& mx, uint2& best, float2& sum, unsigned lanebase, unsigned triple0)
+// The table byte offset of block position T, taken from the lane of the stream that fetched it.
+template <int T>
+__device__ __forceinline__ unsigned block_offset(unsigned k0, unsigned k1)
 {
-    constexpr int H = G / 2;
+    if constexpr (T < 16) return row_share<T>(k0);
+    else return row_share<T - 16>(k1);
+}
+
+// A step's G/2 table lines for this lane: 16 bytes of each.
+template <int G, int T>
+__device__ __forceinline__ void read_step(const char* __restrict__ lds, unsigned k0, unsigned k1, unsigned lanebase, float4 (&v)[G / 2])
+{
+    const unsigned addr = block_offset<T>(k0, k1) + lanebase;
 #pragma unroll
-    for (int q = 0; q < G; ++q) {
+    for (int i = 0; i < G / 2; ++i) v[i] = *reinterpret_cast<const float4*>(lds + addr + i * 256);
+}
+
+template <int G, int MODE, int T>
+__device__ __forceinline__ void scan_steps(const char* __restrict__ lds, unsigned k0, unsigned k1, unsigned n0, unsigned n1,
+                                           float2 (&acc)[3][G], float2& mx, uint2& best, float2& sum, unsigned lanebase, unsigned triple0,
+                                           float4 (&cur)[G / 2])
+{
+    constexpr int H = G / 2, q = T / 3, c = T % 3;
+    // the next step's lines (the next block's first step after the last one) are asked for before this step's are added:
+    // a wave keeps G/2 to G reads in flight and waits once per step
+    float4 nxt[H];
+    if constexpr (T + 1 < 3 * G) read_step<G, T + 1>(lds, k0, k1, lanebase, nxt);
+    else read_step<G, 0>(lds, n0, n1, lanebase, nxt);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 3; ++c) {
-            const int t = 3 * q + c;
-            unsigned koff;
-            switch (t) {
-#define DBK_CASE(T) case T: koff = (T < 16) ? row_share<(T < 16 ? T : 0)>(k0) : row_share<(T < 16 ? 0 : T - 16)>(k1); break;
-                DBK_CASE(0) DBK_CASE(1) DBK_CASE(2) DBK_CASE(3) DBK_CASE(4) DBK_CASE(5) DBK_CASE(6) DBK_CASE(7)
-                DBK_CASE(8) DBK_CASE(9) DBK_CASE(10) DBK_CASE(11) DBK_CASE(12) DBK_CASE(13) DBK_CASE(14) DBK_CASE(15)
-                DBK_CASE(16) DBK_CASE(17) DBK_CASE(18) DBK_CASE(19) DBK_CASE(20) DBK_CASE(21) DBK_CASE(22) DBK_CASE(23)
-#undef DBK_CASE
-                default: koff = 0; break;
-            }
-            const unsigned addr = koff + lanebase;
-#pragma unroll
-            for (int i = 0; i < H; ++i) {
-                const float4 v = *reinterpret_cast<const float4*>(lds + addr + i * 256);
-                const int s0 = (((q - 2 * i) % G) + G) % G;          // position t - 6i   takes group 2i
-                const int s1 = (((q - 2 * i - 1) % G) + G) % G;      // position t - 6i-3 takes group 2i+1
-                if (i == 0) { acc[c][s0].x = v.x; acc[c][s0].y = v.y; }     // group 0 starts a position
-                else { acc[c][s0].x += v.x; acc[c][s0].y += v.y; }
-                acc[c][s1].x += v.z; acc[c][s1].y += v.w;
-            }
-        }
+    for (int i = 0; i < H; ++i) {
+        const float4 v = cur[i];
+        const int s0 = (((q - 2 * i) % G) + G) % G;          // position t - 6i   takes group 2i
+        const int s1 = (((q - 2 * i - 1) % G) + G) % G;      // position t - 6i-3 takes group 2i+1
+        if (i == 0) { acc[c][s0].x = v.x; acc[c][s0].y = v.y; }     // group 0 starts a position
+        else { acc[c][s0].x += v.x; acc[c][s0].y += v.y; }
+        acc[c][s1].x += v.z; acc[c][s1].y += v.w;
+    }
+    if constexpr (c == 2) {
         // group G-1 just landed in slot (q+1) mod G of each class: three finished positions, in text order
-        const int cs = (q + 1) % G;
+        constexpr int cs = (q + 1) % G;
         if (MODE & M_ARG) {
             // remember which triple of positions holds the running maximum (strictly greater: the earliest
             // triple wins ties); the position inside the triple is settled when the region ends
@@ -169,12 +174,30 @@ __device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigne
         if (MODE & M_SUM) {
             // positions outside the region carry a poison term: their rectified value is exactly 0
 #pragma unroll
-            for (int c = 0; c < 3; ++c) {
-                sum.x += fmaxf(acc[c][cs].x, 0.f);
-                sum.y += fmaxf(acc[c][cs].y, 0.f);
+            for (int cc = 0; cc < 3; ++cc) {
+                sum.x += fmaxf(acc[cc][cs].x, 0.f);
+                sum.y += fmaxf(acc[cc][cs].y, 0.f);
             }
         }
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < H; ++i) cur[i] = nxt[i];
+    if constexpr (T + 1 < 3 * G) scan_steps<G, MODE, T + 1>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, triple0, cur);
+}
+
+// One unrolled block of 3G text positions for one lane.
+//   k0, k1    table byte offsets (triple index * bytes per triple) of this block's positions, spread
+//             over the stream's 16 lanes: lane i holds position i in k0 and position 16+i in k1
+//   n0, n1    the same for the block after it
+//   acc       ring of partial sums (2 filters per lane), mx the running max
+//   cur       the lines of this block's first step (read by the block before); on return, those of the next block's
+template <int G, int MODE>
+__device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigned k0, unsigned k1, unsigned n0, unsigned n1,
+                                           float2 (&acc)[3][G], float2& mx, uint2& best, float2& sum, unsigned lanebase, unsigned triple0,
+                                           float4 (&cur)[G / 2])
+{
+    scan_steps<G, MODE, 0>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, triple0, cur);
 }
 
 // The sum of one position's G table entries for this lane's two filters, groups in ascending order:
@@ -195,24 +218,14 @@ __device__ __forceinline__ float2 rescan_position(const char* __restrict__ lds, 
     return z;
 }
 
-template <int G, int MAXT, int MODE>
-__global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __restrict__ W, const float* __restrict__ bias,
-                                                            unsigned m, unsigned F, const uint8_t* __restrict__ K, size_t N,
-                                                            const uint32_t* __restrict__ R, unsigned P, unsigned nsplit,
-                                                            const unsigned* __restrict__ flag, float* __restrict__ pooled,
-                                                            uint32_t* __restrict__ argmax)
+// The workgroup's table for the 32 filters from f0 on: per-tap, per-letter weights first (taps >= m are zero), then
+// the 3-mer sums, taps in ascending order, bias first for group 0; entry 125 is all poison. All threads take part;
+// ends with a barrier.
+template <int G>
+__device__ __forceinline__ void build_table(float* __restrict__ lut, float* __restrict__ w5, const float* __restrict__ W,
+                                            const float* __restrict__ bias, unsigned m, unsigned F, unsigned f0)
 {
     constexpr int STEPS = 3 * G;
-    constexpr unsigned KSTRIDE = G * ROWB;                     // bytes per triple: G/2 lines of 256 B
-    extern __shared__ __align__(16) unsigned char smem[];
-    if (flag[0] != 0) return;                                   // the general kernel takes this call
-    float* lut = reinterpret_cast<float*>(smem);
-    float* w5 = lut + (size_t)(NKMER + 1) * G * FTILE;         // [3G taps][5 letters][32 filters]
-
-    const unsigned split = blockIdx.x % nsplit, tile = blockIdx.x / nsplit;
-    const unsigned f0 = tile * FTILE;
-
-    // ---- per-tap, per-letter weights for this filter tile (taps >= m are zero)
     for (unsigned e = threadIdx.x; e < (unsigned)STEPS * FTILE; e += blockDim.x) {
         const unsigned j = e / FTILE, fl = e % FTILE, f = f0 + fl;
         float w0 = 0.f, w1 = 0.f, w2 = 0.f, w3 = 0.f;
@@ -227,7 +240,6 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
         row[0 * FTILE] = w0; row[1 * FTILE] = w1; row[2 * FTILE] = w2; row[3 * FTILE] = w3; row[4 * FTILE] = z * 0.25f;
     }
     __syncthreads();
-    // ---- the 3-mer table: taps in ascending order, bias first for group 0; entry 125 is all poison.
     //      element e -> (triple, line i, lane l, j): group 2i + j/2, filter 2l + j%2
     for (unsigned e = threadIdx.x; e < (unsigned)(NKMER + 1) * G * FTILE; e += blockDim.x) {
         const unsigned j = e & 3u, l = (e >> 2) & 15u, i = (e >> 6) % (unsigned)(G / 2), km = e / (unsigned)(G * FTILE);
@@ -243,17 +255,33 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
         lut[e] = s;
     }
     __syncthreads();
+}
 
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = blockDim.x >> 6;
-    const unsigned sidx = lane >> 4;
+// A wave of the table scan. Its four streams take the workgroup's regions as they come: a stream that finishes a region
+// claims the next unclaimed one from `counter` (LDS; set to the first region before the table's barriers), up to `rend`.
+// The SIMD favours its oldest wave, so waves that were given equal shares would finish 5-20 % apart; which stream scans a
+// region does not change a bit of its result.
+template <int G, int MODE>
+__device__ __forceinline__ void table_scan(const char* __restrict__ lds, unsigned F, unsigned f0, const uint8_t* __restrict__ K,
+                                           const uint32_t* __restrict__ R, unsigned* counter, unsigned rend,
+                                           float* __restrict__ pooled, uint32_t* __restrict__ argmax)
+{
+    constexpr int STEPS = 3 * G;
+    constexpr unsigned KSTRIDE = G * ROWB;                     // bytes per triple: G/2 lines of 256 B
+    const unsigned P = rend;
+    const unsigned lane = threadIdx.x & 63;
     const unsigned lanebase = (lane & 15u) * 16u;
-    const unsigned nstream = nsplit * nwave * 4u;
     constexpr unsigned TAIL = 3 * (G - 1);                       // steps between a position's start and its completion
+    auto claim = [&]() -> unsigned {
+        unsigned v = 0u;
+        if ((lane & 15u) == 0u) v = atomicAdd(counter, 1u);
+        return row_share<0>(v);
+    };
 
-    unsigned r = (split * nwave + wave) * 4u + sidx;
+    unsigned r = claim(), rn = claim();                          // the region in work, the one after it
     unsigned a = 0, rows = 0, a_next = 0, rows_next = 0;
     if (r < P) { a = R[2 * (size_t)r]; rows = R[2 * (size_t)r + 1] - a; }
-    if (r < P && r + nstream < P) { a_next = R[2 * (size_t)(r + nstream)]; rows_next = R[2 * (size_t)(r + nstream) + 1] - a_next; }
+    if (rn < P) { a_next = R[2 * (size_t)rn]; rows_next = R[2 * (size_t)rn + 1] - a_next; }
     unsigned nblk = (rows + TAIL + STEPS - 1) / STEPS;
     if (nblk < 1) nblk = 1;
 
@@ -281,7 +309,8 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
     uint2 best = make_uint2(0u, 0u);
     float2 sum = make_float2(0.f, 0.f);
     unsigned blk = 0;
-    const char* lds = reinterpret_cast<const char*>(smem);
+    float4 cur[G / 2];                                           // the lines of the coming block's first step
+    read_step<G, 0>(lds, k0, k1, lanebase, cur);
 
     while (true) {
         const bool active = r < P;
@@ -289,9 +318,9 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
         const bool last = blk + 1 >= nblk;
         // the next block's indices travel while this block computes
         unsigned n0, n1;
-        if (last) fetch(a_next, (r < P && r + nstream < P) ? rows_next + TAIL : 0u, 0u, n0, n1);
+        if (last) fetch(a_next, rn < P ? rows_next + TAIL : 0u, 0u, n0, n1);
         else fetch(a + (blk + 1) * STEPS, rows + TAIL, (blk + 1) * STEPS, n0, n1);
-        scan_block<G, MODE>(lds, k0, k1, acc, mx, best, sum, lanebase, blk * (unsigned)G);
+        scan_block<G, MODE>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, blk * (unsigned)G, cur);
         k0 = n0;
         k1 = n1;
         if (last) {
@@ -343,16 +372,38 @@ __global__ __launch_bounds__(MAXT) void scanpool_kmer_kernel(const float* __rest
             for (int c = 0; c < 3; ++c)
 #pragma unroll
                 for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
-            r = r < P ? r + nstream : r;
+            r = rn;
+            rn = claim();
             a = a_next; rows = rows_next; blk = 0;
             nblk = (rows + TAIL + STEPS - 1) / STEPS;
             if (nblk < 1) nblk = 1;
             a_next = 0; rows_next = 0;
-            if (r < P && r + nstream < P) { a_next = R[2 * (size_t)(r + nstream)]; rows_next = R[2 * (size_t)(r + nstream) + 1] - a_next; }
+            if (rn < P) { a_next = R[2 * (size_t)rn]; rows_next = R[2 * (size_t)rn + 1] - a_next; }
         } else {
             ++blk;
         }
     }
+}
+
+template <int G, int MAXT, int MODE>
+__global__ __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(3, 3))) void scanpool_kmer_kernel(const float* __restrict__ W, const float* __restrict__ bias,
+                                                            unsigned m, unsigned F, const uint8_t* __restrict__ K, size_t N,
+                                                            const uint32_t* __restrict__ R, unsigned P, unsigned nsplit,
+                                                            const unsigned* __restrict__ flag, float* __restrict__ pooled,
+                                                            uint32_t* __restrict__ argmax)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (flag[0] != 0) return;                                   // the general kernel takes this call
+    float* lut = reinterpret_cast<float*>(smem);
+    float* w5 = lut + (size_t)(NKMER + 1) * G * FTILE;         // [3G taps][5 letters][32 filters]
+    unsigned* counter = reinterpret_cast<unsigned*>(w5 + (size_t)3 * G * 5 * FTILE);
+    const unsigned split = blockIdx.x % nsplit, tile = blockIdx.x / nsplit;
+    const unsigned f0 = tile * FTILE;
+    // this workgroup's regions
+    const unsigned lo = (unsigned)((unsigned long long)P * split / nsplit), hi = (unsigned)((unsigned long long)P * (split + 1) / nsplit);
+    if (threadIdx.x == 0) counter[0] = lo;
+    build_table<G>(lut, w5, W, bias, m, F, f0);
+    table_scan<G, MODE>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled, argmax);
 }
 
 template <int G, int MODE>
@@ -371,7 +422,7 @@ template <int G>
 int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F, const uint8_t* K, size_t N,
            const uint32_t* R, size_t P, const unsigned* flag, int ptype, float* pooled, uint32_t* argmax)
 {
-    size_t smem = ((size_t)(NKMER + 1) * G * FTILE + (size_t)3 * G * 5 * FTILE) * sizeof(float);
+    size_t smem = ((size_t)(NKMER + 1) * G * FTILE + (size_t)3 * G * 5 * FTILE) * sizeof(float) + 16;   // table, letter weights, region counter
     if (smem > dbk_scan::lds_limit()) return -1;
     const unsigned ntile = dbk::divup(F, FTILE);
     unsigned nsplit = 256u / ntile;
