@@ -15,6 +15,60 @@ using dbk_rng::uniform_at;
 
 #define GRID_STRIDE(i, n) for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (n); i += (size_t)gridDim.x * blockDim.x)
 
+// Z[i] = f(X[i]) and Z[i] = f(X[i], Y[i]) over flat arrays, launched through EWV: ONE access of 16 bytes per lane (four
+// floats, two doubles) where every pointer is 16-byte aligned, thread t taking pack t; the threads after the last whole
+// pack take the remaining elements one each. (A 1 GB map streams at 6.2 TB/s this way; grid-stride loops, whatever their
+// grid and however many accesses they keep in flight, reached 4.6-5.5: the workgroups of a one-shot grid sweep the
+// arrays in launch order.) Arrays that are not aligned go element by element in a grid-stride loop.
+// Z may be X or Y itself: a lane writes only what it has read.
+template <typename T> struct pack16 {
+    static constexpr int V = 16 / sizeof(T);
+    typedef T type __attribute__((ext_vector_type(16 / sizeof(T))));
+};
+template <typename T> __device__ __forceinline__ bool aligned16(const void* a, const void* b, const void* c = nullptr)
+{
+    return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15u) == 0;
+}
+template <typename T, typename F> __device__ __forceinline__ void map1(const T* X, T* Z, size_t n, F f)
+{
+    using P = typename pack16<T>::type;
+    constexpr int V = pack16<T>::V;
+    if (aligned16<T>(X, Z)) {
+        const size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x, np = n / V;
+        if (p < np) {
+            const P a = reinterpret_cast<const P*>(X)[p];
+            P z;
+#pragma unroll
+            for (int k = 0; k < V; ++k) z[k] = f(a[k]);
+            reinterpret_cast<P*>(Z)[p] = z;
+        } else if (np * V + (p - np) < n) {
+            const size_t i = np * V + (p - np);
+            Z[i] = f(X[i]);
+        }
+        return;
+    }
+    GRID_STRIDE(i, n) Z[i] = f(X[i]);
+}
+template <typename T, typename F> __device__ __forceinline__ void map2(const T* X, const T* Y, T* Z, size_t n, F f)
+{
+    using P = typename pack16<T>::type;
+    constexpr int V = pack16<T>::V;
+    if (aligned16<T>(X, Y, Z)) {
+        const size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x, np = n / V;
+        if (p < np) {
+            const P a = reinterpret_cast<const P*>(X)[p], c = reinterpret_cast<const P*>(Y)[p];
+            P z;
+#pragma unroll
+            for (int k = 0; k < V; ++k) z[k] = f(a[k], c[k]);
+            reinterpret_cast<P*>(Z)[p] = z;
+        } else if (np * V + (p - np) < n) {
+            const size_t i = np * V + (p - np);
+            Z[i] = f(X[i], Y[i]);
+        }
+        return;
+    }
+    GRID_STRIDE(i, n) Z[i] = f(X[i], Y[i]);
+}
 template <typename T> __global__ void k_gradstep(T* P, const T* dP, const T* drate, T* mP, const T* mrate, size_t n)
 {
     GRID_STRIDE(i, n) {
@@ -226,9 +280,20 @@ template <typename T> __global__ void k_pair_max(const T* Z, T* out, size_t npai
         out[i] = a >= b ? a : b;
     }
 }
+// Z (n x m) = X + b, b added to every row. One pack of 16 bytes per thread (launched through EWV) when the rows are
+// whole packs (then a pack never straddles two rows and b's pack is aligned too) and the array has fewer than 2^32
+// elements (32-bit index arithmetic).
 template <typename T> __global__ void k_add_rowvec(const T* X, const T* b, T* Z, size_t n, size_t m)
 {
-    GRID_STRIDE(i, n * m) Z[i] = X[i] + b[i % m];
+    using P = typename pack16<T>::type;
+    constexpr int V = pack16<T>::V;
+    const size_t total = n * m;
+    if (m % V == 0 && aligned16<T>(X, b, Z) && total < 0xffffffffull) {
+        const size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (p < total / V) reinterpret_cast<P*>(Z)[p] = reinterpret_cast<const P*>(X)[p] + reinterpret_cast<const P*>(b)[(unsigned)p % (unsigned)(m / V)];
+        return;
+    }
+    GRID_STRIDE(i, total) Z[i] = X[i] + b[i % m];
 }
 // Column sums in a fixed order. Workgroup (x, y) takes 64 columns and row slice y; wave w sums rows
 // w, w+4, ... of the slice in ascending order (four rows in flight), the four waves are combined in
@@ -269,23 +334,19 @@ template <typename T> __global__ void k_colsum_fold(const T* __restrict__ partia
 }
 template <typename T> __global__ void k_relu(const T* X, T* Z, size_t n)
 {
-    GRID_STRIDE(i, n) Z[i] = X[i] > (T)0 ? X[i] : (T)0;   // NaN -> 0, as fmax(0, x)
+    map1(X, Z, n, [](T x) { return x > (T)0 ? x : (T)0; });   // NaN -> 0, as fmax(0, x)
 }
 template <typename T> __global__ void k_mul_sign(const T* dZ, const T* Z, T* dX, size_t n)
 {
-    GRID_STRIDE(i, n) {
-        T z = Z[i];
-        T s = (T)(z > (T)0) - (T)(z < (T)0);
-        dX[i] = dZ[i] * s;
-    }
+    map2(dZ, Z, dX, n, [](T g, T z) { return g * ((T)(z > (T)0) - (T)(z < (T)0)); });
 }
 template <typename T> __global__ void k_sign(const T* X, T* Z, size_t n)
 {
-    GRID_STRIDE(i, n) Z[i] = (T)(X[i] > (T)0) - (T)(X[i] < (T)0);
+    map1(X, Z, n, [](T x) { return (T)(x > (T)0) - (T)(x < (T)0); });
 }
 template <typename T> __global__ void k_logistic(const T* X, T* Z, size_t n)
 {
-    GRID_STRIDE(i, n) Z[i] = (T)1 / ((T)1 + exp(-X[i]));
+    map1(X, Z, n, [](T x) { return (T)1 / ((T)1 + exp(-x)); });
 }
 template <typename T> __global__ void k_loss_terms(int kind, const T* Z, const T* Y, T* L, size_t n)
 {
@@ -365,7 +426,7 @@ template <typename T> __global__ void k_normal_fill(T* Z, size_t n, uint64_t see
 __global__ void k_counter_add(unsigned long long* ctr, unsigned long long delta) { if (threadIdx.x == 0 && blockIdx.x == 0) ctr[0] += delta; }
 template <typename T> __global__ void k_sub_scale(const T* Z, const T* Y, T scale, T* dZ, size_t n)
 {
-    GRID_STRIDE(i, n) dZ[i] = (Z[i] - Y[i]) * scale;
+    map2(Z, Y, dZ, n, [scale](T z, T y) { return (z - y) * scale; });
 }
 template <typename T> __global__ void k_hinge_grad(const T* Z, const T* Y, T scale, T* dZ, size_t n)
 {
@@ -421,6 +482,18 @@ template <typename T> __global__ void k_scan_constraint(T* W, size_t m, size_t F
         if ((n) == 0) { dbk::clear_error(); return 0; }                                                    \
         if (dtype == DBK_F32) hipLaunchKernelGGL(kernel<float>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), ARGS32); \
         else hipLaunchKernelGGL(kernel<double>, dim3(dbk::ew_grid(n)), dim3(256), 0, dbk::as_stream(stream), ARGS64);                  \
+        DBK_LAUNCH_OK();                                                                                   \
+    } while (0)
+// The launch of a kernel built on map1 / map2: one thread per pack of 16 bytes, plus the few that take the elements after
+// the last whole pack (at most 2^31 - 1 workgroups: 2^41 bytes per array).
+inline unsigned pack_grid(size_t n, size_t per_pack) { return (unsigned)dbk::divup(n / per_pack + per_pack, (size_t)256); }
+#define EWV(kernel, n, ARGS32, ARGS64)                                                                     \
+    do {                                                                                                   \
+        DBK_DTYPE_OK(dtype);                                                                               \
+        if ((n) == 0) { dbk::clear_error(); return 0; }                                                    \
+        DBK_CHECK((n) < ((size_t)1 << 39), "ValueError: %zu elements are more than one launch takes", (size_t)(n)); \
+        if (dtype == DBK_F32) hipLaunchKernelGGL(kernel<float>, dim3(pack_grid(n, 4)), dim3(256), 0, dbk::as_stream(stream), ARGS32); \
+        else hipLaunchKernelGGL(kernel<double>, dim3(pack_grid(n, 2)), dim3(256), 0, dbk::as_stream(stream), ARGS64);                  \
         DBK_LAUNCH_OK();                                                                                   \
     } while (0)
 #define A(...) __VA_ARGS__
@@ -558,7 +631,7 @@ int dbk_pair_max(dbk_stream_t stream, int dtype, const void* Z, void* out, size_
 int dbk_add_rowvec(dbk_stream_t stream, int dtype, const void* X, const void* b, void* Z, size_t n, size_t m)
 {
     size_t total = n * m;
-    EW2(k_add_rowvec, total, A(CF32(X), CF32(b), F32(Z), n, m), A(CF64(X), CF64(b), F64(Z), n, m));
+    EWV(k_add_rowvec, total, A(CF32(X), CF32(b), F32(Z), n, m), A(CF64(X), CF64(b), F64(Z), n, m));
 }
 int dbk_colsum(dbk_stream_t stream, int dtype, const void* X, void* out, size_t n, size_t m)
 {
@@ -579,19 +652,19 @@ int dbk_corr1ord_constraint(dbk_stream_t stream, int dtype, void* W, size_t m, s
 }
 int dbk_relu(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
 {
-    EW2(k_relu, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
+    EWV(k_relu, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
 }
 int dbk_mul_sign(dbk_stream_t stream, int dtype, const void* dZ, const void* Z, void* dX, size_t n)
 {
-    EW2(k_mul_sign, n, A(CF32(dZ), CF32(Z), F32(dX), n), A(CF64(dZ), CF64(Z), F64(dX), n));
+    EWV(k_mul_sign, n, A(CF32(dZ), CF32(Z), F32(dX), n), A(CF64(dZ), CF64(Z), F64(dX), n));
 }
 int dbk_sign(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
 {
-    EW2(k_sign, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
+    EWV(k_sign, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
 }
 int dbk_logistic(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n)
 {
-    EW2(k_logistic, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
+    EWV(k_logistic, n, A(CF32(X), F32(Z), n), A(CF64(X), F64(Z), n));
 }
 int dbk_loss_terms(dbk_stream_t stream, int dtype, int kind, const void* Z, const void* Y, void* L, size_t n)
 {
@@ -606,7 +679,7 @@ int dbk_softmax(dbk_stream_t stream, int dtype, const void* X, void* Z, size_t n
 }
 int dbk_sub_scale(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n)
 {
-    EW2(k_sub_scale, n, A(CF32(Z), CF32(Y), (float)scale, F32(dZ), n), A(CF64(Z), CF64(Y), scale, F64(dZ), n));
+    EWV(k_sub_scale, n, A(CF32(Z), CF32(Y), (float)scale, F32(dZ), n), A(CF64(Z), CF64(Y), scale, F64(dZ), n));
 }
 int dbk_hinge_grad(dbk_stream_t stream, int dtype, const void* Z, const void* Y, double scale, void* dZ, size_t n)
 {

@@ -849,7 +849,8 @@ def test_masks_dropout_and_loss_ops(ds, sm, ks):
 
 # ------------------------------------------------------------------------------------------ k-mer table fast path
 @pytest.mark.parametrize("B,lo,hi,m,F", [(64, 101, 101, 24, 16), (128, 38, 41, 16, 16), (300, 20, 40, 24, 144), (33, 1, 300, 11, 70),
-                                          (50, 500, 500, 24, 64), (17, 0, 9, 5, 33), (700, 30, 60, 20, 40), (40, 90, 110, 2, 8)])
+                                          (50, 500, 500, 24, 64), (17, 0, 9, 5, 33), (700, 30, 60, 20, 40), (40, 90, 110, 2, 8),
+                                          (1, 50, 50, 24, 32), (49, 10, 80, 24, 32)])
 def test_scanpool_kmer_path_matches_oracle(ks, B, lo, hi, m, F):
     rng, W, b, X, R = _fused_case(1000 + B + m + F, B, lo, hi, m, F, pn=0.04)
     A, Pr, Ir = _chain_oracle(W, b, X, R, "max")
@@ -859,6 +860,18 @@ def test_scanpool_kmer_path_matches_oracle(ks, B, lo, hi, m, F):
     # and it agrees with the general kernel to the same tolerance
     Pg, _ = ks.scanpool_fprop(dev(W), dev(b), dev(X), dev(R), "max", path="general")
     assert_close(host(P), host(Pg), ACT, "kmer vs general")
+
+
+def test_scanpool_kmer_path_repeats_its_bits(ks):
+    """The table kernel's streams take regions as they become free, so which stream scans a region differs from call to
+    call; every region's result must not (same additions in the same order whoever performs them)."""
+    rng, W, b, X, R = _fused_case(515, 3000, 5, 200, 24, 96, pn=0.03)
+    Wd, bd, Xd, Rd = dev(W), dev(b), dev(X), dev(R)
+    for ptype, want in (("max", False), ("max", True), ("all", True), ("avg", False)):
+        P0, I0 = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=want, path="kmer")
+        for _ in range(3):
+            P1, I1 = ks.scanpool_fprop(Wd, bd, Xd, Rd, ptype, want_argmax=want, path="kmer")
+            assert torch.equal(P0, P1) and (I0 is None or torch.equal(I0, I1)), ptype
 
 
 def test_scanpool_kmer_path_device_side_fallbacks(ks):
