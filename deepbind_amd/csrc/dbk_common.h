@@ -20,7 +20,8 @@ void clear_error();
 // passes to the new stream (after draining the device). Growing a buffer or recycling a slot synchronises
 // the device, which a stream under capture does not allow: null then, and when memory runs out, with the
 // reason in workspace_error(). A buffer handed out DURING a capture is in a graph from then on: its slot is never
-// recycled and its buffers neither freed nor grown (a later, larger call on that stream fails and says so).
+// recycled and the buffer never freed (a later, larger eager call on that stream sets it aside for the graph's replays
+// and allocates a new one for the stream).
 // `which` selects one of four independent buffers of the stream: 0 and 1 hold kernels' partial results (a call
 // that must keep one kernel's partial results while another kernel fills its own uses the second), 2 and 3 the
 // whole maps of the unfused scan + pool chain, whose kernels use buffer 0 themselves.

@@ -87,9 +87,10 @@ void* workspace(size_t bytes, hipStream_t stream, int which)
         return nullptr;
     }
     if (w->ptr[which] && w->pinned) {
-        snprintf(g_ws_why, sizeof(g_ws_why), "a captured graph refers to this stream's scratch, which therefore cannot grow (%zu -> %zu bytes): issue the larger call on another stream",
-                 w->bytes[which], bytes);
-        return nullptr;
+        // A captured graph refers to this buffer and may be replayed as long as the process lives: it is set aside, never
+        // freed, and the stream gets a larger one for its eager calls and later captures.
+        w->ptr[which] = nullptr;
+        w->bytes[which] = 0;
     }
     if (w->ptr[which]) {
         // earlier launches may still be reading the old buffer
