@@ -479,8 +479,8 @@ __global__ __launch_bounds__(256) void k_head(size_t n, int nblock, int k, int k
 }
 
 // Scoring head, coalesced variant for hidden % 4 == 0: a workgroup owns 16 consecutive models and a tile of
-// 16 rows per pass; lane = (row, model) with the model fastest, so a wave's reads of the feature matrix
-// cover four contiguous 16*k*4-byte row segments. The 16 models' first-layer weights sit in LDS as
+// 16 rows (x 4, 2 or 1 rows per lane) per pass; lane = (row, model) with the model fastest, so a wave's reads of the
+// feature matrix cover four contiguous 16*k*4-byte row segments. The 16 models' first-layer weights sit in LDS as
 // [input][hidden/4][model][4]: the 16 lanes of a row read one aligned 256-byte line per ds_read_b128,
 // and the four rows of a wave read the same line.
 constexpr int HG = 16;
@@ -519,42 +519,68 @@ __global__ __launch_bounds__(256) void k_head16(size_t n, int nblock, int k, int
     const float4* b1v = reinterpret_cast<const float4*>(b1s) + g;
     const float4* w2v = reinterpret_cast<const float4*>(w2s) + g;
     if (!live) return;                                   // (after the only barrier)
-    const size_t rstep = (size_t)gridDim.y * 16, rowlen = (size_t)k * nblock;
-    size_t r = (size_t)blockIdx.y * 16 + rl;
-    float xn[KMAX];                                      // next row's inputs, fetched while this row is computed
+    // A pass takes 16 * HR rows: this lane rows base + rl + 16 j, j < HR, of its model. Every weight read from LDS serves
+    // the HR rows (one ds_read_b128 per 4 * HR multiply-adds), each row's sums are formed as for a single row; a row's
+    // inputs arrive as 16-byte loads where a model's k inputs are whole packs.
+    constexpr int HR = KMAX <= 16 ? 4 : (KMAX <= 32 ? 2 : 1);      // (the rows' inputs stay in registers: 64 of them)
+    const size_t rowlen = (size_t)k * nblock;
+    const bool packs = k == KMAX && kf == 0 && (reinterpret_cast<uintptr_t>(pooled) & 15u) == 0;
+    for (size_t base = (size_t)blockIdx.y * (16 * HR); base < n; base += (size_t)gridDim.y * (16 * HR)) {
+        float xr[HR][KMAX];
 #pragma unroll
-    for (int kk = 0; kk < KMAX; ++kk)
-        xn[kk] = r < n ? (kk < k ? pooled[r * rowlen + (size_t)mdl * k + kk] : (kk < kt ? feats[r * (size_t)kf + (kk - k)] : 0.0f)) : 0.0f;
-    for (; r < n; r += rstep) {
-        float xr[KMAX];
+        for (int j = 0; j < HR; ++j) {
+            const size_t r = base + rl + 16 * j;
+            if (packs) {
+                const float4* src = reinterpret_cast<const float4*>(pooled + (r < n ? r : n - 1) * rowlen + (size_t)mdl * k);
 #pragma unroll
-        for (int kk = 0; kk < KMAX; ++kk) xr[kk] = kk < k ? xn[kk] * sc : xn[kk];
-        const size_t rn = r + rstep;
+                for (int q = 0; q < KMAX / 4; ++q) {
+                    const float4 v = src[q];
+                    xr[j][4 * q] = v.x * sc; xr[j][4 * q + 1] = v.y * sc; xr[j][4 * q + 2] = v.z * sc; xr[j][4 * q + 3] = v.w * sc;
+                }
+            } else {
 #pragma unroll
-        for (int kk = 0; kk < KMAX; ++kk)
-            xn[kk] = rn < n ? (kk < k ? pooled[rn * rowlen + (size_t)mdl * k + kk] : (kk < kt ? feats[rn * (size_t)kf + (kk - k)] : 0.0f)) : 0.0f;
-        float out = 0.0f;
+                for (int kk = 0; kk < KMAX; ++kk) {
+                    const float v = r < n ? (kk < k ? pooled[r * rowlen + (size_t)mdl * k + kk] : (kk < kt ? feats[r * (size_t)kf + (kk - k)] : 0.0f)) : 0.0f;
+                    xr[j][kk] = kk < k ? v * sc : v;
+                }
+            }
+        }
+        float out[HR];
+#pragma unroll
+        for (int j = 0; j < HR; ++j) out[j] = 0.0f;
         for (int h4 = 0; h4 < hq; ++h4) {
-            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+            float a[HR][4];
+#pragma unroll
+            for (int j = 0; j < HR; ++j) a[j][0] = a[j][1] = a[j][2] = a[j][3] = 0.0f;
 #pragma unroll
             for (int kk = 0; kk < KMAX; ++kk)
                 if (kk < kt) {
                     const float4 w = w1v[(kk * hq + h4) * HG];
-                    a0 = __builtin_fmaf(xr[kk], w.x, a0);
-                    a1 = __builtin_fmaf(xr[kk], w.y, a1);
-                    a2 = __builtin_fmaf(xr[kk], w.z, a2);
-                    a3 = __builtin_fmaf(xr[kk], w.w, a3);
+#pragma unroll
+                    for (int j = 0; j < HR; ++j) {
+                        a[j][0] = __builtin_fmaf(xr[j][kk], w.x, a[j][0]);
+                        a[j][1] = __builtin_fmaf(xr[j][kk], w.y, a[j][1]);
+                        a[j][2] = __builtin_fmaf(xr[j][kk], w.z, a[j][2]);
+                        a[j][3] = __builtin_fmaf(xr[j][kk], w.w, a[j][3]);
+                    }
                 }
             const float4 bb = b1v[h4 * HG], ww = w2v[h4 * HG];
-            a0 += bb.x; a1 += bb.y; a2 += bb.z; a3 += bb.w;
-            out += (a0 > 0.0f ? a0 : 0.0f) * ww.x;
-            out += (a1 > 0.0f ? a1 : 0.0f) * ww.y;
-            out += (a2 > 0.0f ? a2 : 0.0f) * ww.z;
-            out += (a3 > 0.0f ? a3 : 0.0f) * ww.w;
+#pragma unroll
+            for (int j = 0; j < HR; ++j) {
+                const float a0 = a[j][0] + bb.x, a1 = a[j][1] + bb.y, a2 = a[j][2] + bb.z, a3 = a[j][3] + bb.w;
+                out[j] += (a0 > 0.0f ? a0 : 0.0f) * ww.x;
+                out[j] += (a1 > 0.0f ? a1 : 0.0f) * ww.y;
+                out[j] += (a2 > 0.0f ? a2 : 0.0f) * ww.z;
+                out[j] += (a3 > 0.0f ? a3 : 0.0f) * ww.w;
+            }
         }
-        out += bias2;
-        if (apply_logistic) out = 1.0f / (1.0f + expf(-out));
-        scores[r * (size_t)nblock + mdl] = out;
+#pragma unroll
+        for (int j = 0; j < HR; ++j) {
+            const size_t r = base + rl + 16 * j;
+            float o = out[j] + bias2;
+            if (apply_logistic) o = 1.0f / (1.0f + expf(-o));
+            if (r < n) scores[r * (size_t)nblock + mdl] = o;
+        }
     }
 }
 
@@ -899,7 +925,7 @@ int dbk_head_fprop(dbk_stream_t stream, size_t n, int nblock, int k, int hidden,
     const size_t smem16 = ((size_t)kk_all * hidden + 2 * (size_t)hidden) * HG * sizeof(float);
     if (hidden > 0 && (hidden & 3) == 0 && smem16 <= 65536 && n >= 4096) {
         // bulk scoring: 16 models per workgroup, coalesced reads of the feature matrix
-        const unsigned gy = row_slices(n, 16, dbk::divup(nblock, HG));
+        const unsigned gy = row_slices(n, kk_all <= 16 ? 64 : (kk_all <= 32 ? 32 : 16), dbk::divup(nblock, HG));
         auto kern16 = kk_all <= 16 ? k_head16<16> : (kk_all <= 32 ? k_head16<32> : k_head16<64>);
         DBK_HIP(hipFuncSetAttribute((const void*)kern16, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem16));
         hipLaunchKernelGGL(kern16, dim3(dbk::divup(nblock, HG), gy), dim3(256), smem16, dbk::as_stream(stream), n, nblock, k, kf, kw, hidden, pooled,
