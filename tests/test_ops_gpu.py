@@ -1138,3 +1138,70 @@ def test_softmax_chunks_and_multiclass_loss_terms(dtype):
     got = host(sm.loss_terms(dev(Z), dev(Y), "nll_multiclass"))
     ref = orc.nll_multiclass_terms(Z.astype(np.float64), Y.astype(np.float64))
     assert np.abs(got - ref).max() <= (1e-5 if dtype == np.float32 else 1e-13) * np.abs(ref).max()
+
+# ------------------------------------------------------------------------------------------ 16-byte packs
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 4096, 70001])
+def test_elementwise_packs_tails_unaligned_and_in_place(sm, n, dtype):
+    """The elementwise kernels take 16 bytes per thread where the arrays allow it: every size (no pack, whole packs, a
+    tail), arrays that start off a 16-byte boundary (element by element) and a result written over its input give the
+    values of the plain formulas, bit for bit."""
+    from deepbind_amd import _lib
+    g = torch.Generator(device="cuda").manual_seed(n)
+    for off in (0, 1):
+        X = torch.randn(n + off, generator=g, device="cuda", dtype=torch.float64).to(dtype)[off:]
+        Y = torch.randn(n + off, generator=g, device="cuda", dtype=torch.float64).to(dtype)[off:]
+        X[::7] = 0.0                                                      # sign(0) = 0, relu(0) = 0
+        zero = torch.zeros((), device="cuda", dtype=dtype)
+        assert torch.equal(sm.relu(X), torch.where(X > 0, X, zero))
+        assert torch.equal(sm.sign(X), torch.sign(X))
+        assert torch.equal(sm.mul_sign(Y, X), Y * torch.sign(X))
+        assert torch.equal(sm.sub_scale(X, Y, 0.125), (X - Y) * 0.125)
+        assert torch.allclose(sm.logistic(X), torch.sigmoid(X), rtol=1e-6 if dtype == torch.float32 else 1e-14, atol=0)
+        # in place: the result over the input
+        Z = X.clone()
+        _lib.call("dbk_relu", _lib.stream(), _lib.dtype_code(Z), _lib.ptr(Z), _lib.ptr(Z), n)
+        assert torch.equal(Z, torch.where(X > 0, X, zero))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (5, 3), (7, 4), (33, 6), (129, 16), (1000, 68), (3, 2050)])
+def test_add_rowvec_packs_and_plain_rows(sm, rows, cols, dtype):
+    """Rows of whole 16-byte packs take the packed kernel, other widths and unaligned arrays the element-wise one: the
+    same sums either way."""
+    g = torch.Generator(device="cuda").manual_seed(rows * 131 + cols)
+    for off in (0, 1):
+        X = torch.randn(rows * cols + off, generator=g, device="cuda", dtype=torch.float64).to(dtype)[off:].reshape(rows, cols)
+        b = torch.randn(cols, generator=g, device="cuda", dtype=torch.float64).to(dtype)
+        assert torch.equal(sm.add_rowvec(X, b), X + b)
+
+
+@pytest.mark.parametrize("F", [4, 6, 8, 64, 100, 256])
+def test_poolrgn_packed_and_plain_columns_agree(ks, F):
+    """Maps whose rows are whole packs pool four columns per lane, others one: every column's maximum, first winning
+    row, sum and gradient must be what the one-column kernels give (F = 6 and an unaligned map go through them)."""
+    rng = np.random.default_rng(F)
+    P, lens = 37, rng.integers(1, 40, size=37)
+    starts = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    R = np.stack([starts, starts + lens], 1).astype(np.uint32)
+    N = int(lens.sum())
+    U = rng.standard_normal((N, F)).astype(np.float32)
+    U[rng.random((N, F)) < 0.2] = 0.5                                      # ties: the first row wins
+    Ud, Rd = dev(U), dev(R)
+    base = torch.empty(N * F + 1, dtype=torch.float32, device="cuda")
+    Uoff = base[1:].reshape(N, F)                                          # the same map off a 16-byte boundary
+    Uoff.copy_(Ud)
+    for ptype in ("max", "avg", "sum", "all"):
+        want = ptype in ("max", "all")
+        Pa, Ia = ks.poolrgn(Ud, Rd, ptype, want_argmax=want)
+        Pb, Ib = ks.poolrgn(Uoff, Rd, ptype, want_argmax=want)
+        assert torch.equal(Pa, Pb), ptype
+        if want:
+            assert torch.equal(Ia, Ib), ptype
+        dP = dev(rng.standard_normal(tuple(Pa.shape)).astype(np.float32))
+        dUa = torch.zeros_like(Ud) + 0.25
+        dUb = torch.empty_like(base)[1:].reshape(N, F)
+        dUb.fill_(0.25)
+        ks.poolrgn_bprop(dUa, Rd, dP, Ia if want else None, ptype)
+        ks.poolrgn_bprop(dUb, Rd, dP, Ib if want else None, ptype)
+        assert torch.equal(dUa, dUb), ptype
