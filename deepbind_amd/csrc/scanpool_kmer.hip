@@ -24,6 +24,10 @@
 //    16 lanes fetch a block's 3G indices cooperatively (one or two bytes per lane, one block ahead)
 //    and each step takes its index from the owning lane with a DPP row_share folded into the add
 //    that forms the LDS address: one VALU instruction of addressing per step.
+//  * A workgroup owns a contiguous range of regions; its streams claim them one at a time from a counter in LDS (the
+//    SIMD favours its oldest wave: equal static shares would finish 5 % apart). A step's table lines are asked for
+//    one step before they are added (scheduling barriers keep that order in the unrolled block): four to eight
+//    ds_read_b128 in flight per wave, one wait per step, the LDS pipe busy 99 % of the time.
 //  * Positions outside a region never need a test. At a region's start every ring slot is reset to
 //    a large negative "poison" (-1e30), so the partial sums in flight from before the region finish
 //    far below any real value; and the steps a region's last block runs past its final useful
