@@ -695,18 +695,28 @@ def _side_by_side(streams, jobs):
 
 def _graphed_step(jobs):
     """jobs: list of (net, X, R, Y, Ymask, F) with static device tensors. Returns step(): one replay of a
-    HIP graph holding one fused training step of every net (several nets share each launch)."""
+    HIP graph holding one fused training step of every net (several nets share each launch).
+    Two graphs are captured: one whose step forms the look-ahead parameters itself, and one that takes the look-ahead the
+    previous step's update left behind (as a natively issued step does). A replay uses the second whenever the step
+    before it was such a step and nothing has touched the parameters since (torch's version counters tell)."""
     for net, *_ in jobs:
         assert net.mode == "fused" and net.dtype == torch.float32 and net.loss is not None
-    state = {"graph": None, "decay": None}
+    state = {"graphs": None, "decay": None}
 
     def decay_flags():
         return tuple((net.weight_decay_start <= net.step_count, net.step_count < net.start_training) for net, *_ in jobs)
 
-    def body():
-        # the natively issued step on the capturing stream; the graph always forms its look-ahead itself
+    def versions(net):
+        return (net.P._version, net.mP._version, net.mrate._version)
+
+    def keeps_lookahead(net):
+        # (the filters' constraint rewrites the parameters after the update: the look-ahead beside them is stale then)
+        return bool(net.nesterov) and net.constraint is None
+
+    def body(ready):
+        # the natively issued step on the capturing stream, with or without a look-ahead to start from
         for net, *_ in jobs:
-            net._L_versions = None
+            net._L_versions = versions(net) if (ready and keeps_lookahead(net)) else None
         _native_steps(jobs)
 
     def capture():
@@ -720,28 +730,35 @@ def _graphed_step(jobs):
         host_off = [(net._rng_offset, net.step_count) for net, *_ in jobs]
         cap.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(cap):
-            body()
+            body(False)
         torch.cuda.synchronize()
         for t, s_ in zip(live, saved):
             t.copy_(s_)
         for (net, *_), (off, count) in zip(jobs, host_off):
             net._rng_offset, net.step_count = off, count        # the warm-up step must not count (decay / freeze switches are baked in)
         torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=cap):
-            body()
-        # capturing executes nothing on the device; only the host mirrors of the step moved
-        for (net, *_), (off, count) in zip(jobs, host_off):
-            net._rng_offset, net.step_count = off, count
-        state["graph"], state["decay"] = g, decay_flags()
+        graphs = {}
+        for ready in (False, True):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=cap):
+                body(ready)
+            # capturing executes nothing on the device; only the host mirrors of the step moved
+            for (net, *_), (off, count) in zip(jobs, host_off):
+                net._rng_offset, net.step_count = off, count
+            graphs[ready] = g
+        for net, *_ in jobs:
+            net._L_versions = None              # (the warm-up step's look-ahead belongs to parameters that were put back)
+        state["graphs"], state["decay"] = graphs, decay_flags()
         state["single"] = [(net, net._step_buf) for net, *_ in jobs if net._last_single]      # workspaces of single-launch steps in the graph
 
     def step():
-        if state["graph"] is None or state["decay"] != decay_flags():
+        if state["graphs"] is None or state["decay"] != decay_flags():
             capture()
-        state["graph"].replay()
+        ready = all(keeps_lookahead(net) and net._L_versions == versions(net) for net, *_ in jobs)
+        state["graphs"][ready].replay()
         for net, X, R, *_ in jobs:
-            net._L_versions = None              # (a step issued natively after this one forms its look-ahead afresh)
+            # the update left the look-ahead of the new parameters (written through raw pointers: the counters stand still)
+            net._L_versions = versions(net) if (keeps_lookahead(net) and not net._last_single) else None
             if net.input_dropout > 0:
                 net._rng_offset += (X.numel() + 3) // 4
             if net.use_dropout:
