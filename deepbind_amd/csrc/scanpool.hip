@@ -861,11 +861,12 @@ inline unsigned wide_grid_x(unsigned ftiles, size_t P)
     return gx;
 }
 inline size_t wide_smem(unsigned mt) { return (size_t)mt * NL * FT * sizeof(float) + 4 * (mt == 16 ? wide_shape<16>::xbytes : wide_shape<24>::xbytes); }
-// The bit-count backward: a wave per region, two workgroups per CU resident (its 5 x MT sums take ~170 registers);
+// The bit-count backward: a wave per region, three workgroups per CU resident (its 5 x MT sums and the rest take ~160
+// registers at 24 taps: three waves per SIMD);
 // the smallest grid that gives every wave the same number of regions as the resident grid would.
 inline unsigned bits_grid_x(unsigned ftiles, size_t P)
 {
-    unsigned gx = 512u / ftiles;
+    unsigned gx = 768u / ftiles;
     if (gx < 1) gx = 1;
     // at least two regions per wave: the fold of a workgroup's sums and its slab cost about as much as two regions
     // (measured on a calibration batch of 256 regions x 23 tiles: 26.7 us with two, 29.6 with three, 34.5 with five
