@@ -137,10 +137,16 @@ __device__ __forceinline__ void read_step(const char* __restrict__ lds, unsigned
     for (int i = 0; i < G / 2; ++i) v[i] = *reinterpret_cast<const float4*>(lds + addr + i * 256);
 }
 
-template <int G, int MODE, int T>
+// How a block's finished positions are kept apart when regions follow each other without a fresh start (plain max pooling):
+// NP parts of PP positions each, every part with a maximum of its own.
+template <int G> struct run_parts {
+    static constexpr int NP = (G % 4 == 0) ? 4 : 2, PP = 3 * G / NP;
+};
+
+template <int G, int MODE, int T, bool PARTS = false>
 __device__ __forceinline__ void scan_steps(const char* __restrict__ lds, unsigned k0, unsigned k1, unsigned n0, unsigned n1,
                                            float2 (&acc)[3][G], float2& mx, uint2& best, float2& sum, unsigned lanebase, unsigned triple0,
-                                           float4 (&cur)[G / 2])
+                                           float4 (&cur)[G / 2], float2 (&part)[run_parts<G>::NP])
 {
     constexpr int H = G / 2, q = T / 3, c = T % 3;
     // the next step's lines (the next block's first step after the last one) are asked for before this step's are added:
@@ -171,6 +177,10 @@ __device__ __forceinline__ void scan_steps(const char* __restrict__ lds, unsigne
             mx.y = uy ? m3y : mx.y;
             best.x = ux ? triple0 + q : best.x;
             best.y = uy ? triple0 + q : best.y;
+        } else if (PARTS) {
+            constexpr int h = 3 * q / run_parts<G>::PP;
+            part[h].x = fmaxf(fmaxf(part[h].x, acc[0][cs].x), acc[1][cs].x); part[h].y = fmaxf(fmaxf(part[h].y, acc[0][cs].y), acc[1][cs].y);
+            part[h].x = fmaxf(part[h].x, acc[2][cs].x); part[h].y = fmaxf(part[h].y, acc[2][cs].y);
         } else if (MODE & M_MAX) {
             mx.x = fmaxf(fmaxf(mx.x, acc[0][cs].x), acc[1][cs].x); mx.y = fmaxf(fmaxf(mx.y, acc[0][cs].y), acc[1][cs].y);
             mx.x = fmaxf(mx.x, acc[2][cs].x); mx.y = fmaxf(mx.y, acc[2][cs].y);
@@ -187,7 +197,7 @@ __device__ __forceinline__ void scan_steps(const char* __restrict__ lds, unsigne
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < H; ++i) cur[i] = nxt[i];
-    if constexpr (T + 1 < 3 * G) scan_steps<G, MODE, T + 1>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, triple0, cur);
+    if constexpr (T + 1 < 3 * G) scan_steps<G, MODE, T + 1, PARTS>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, triple0, cur, part);
 }
 
 // One unrolled block of 3G text positions for one lane.
@@ -201,7 +211,8 @@ __device__ __forceinline__ void scan_block(const char* __restrict__ lds, unsigne
                                            float2 (&acc)[3][G], float2& mx, uint2& best, float2& sum, unsigned lanebase, unsigned triple0,
                                            float4 (&cur)[G / 2])
 {
-    scan_steps<G, MODE, 0>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, triple0, cur);
+    float2 none[run_parts<G>::NP];
+    scan_steps<G, MODE, 0>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, triple0, cur, none);
 }
 
 // The sum of one position's G table entries for this lane's two filters, groups in ascending order:
@@ -389,6 +400,185 @@ __device__ __forceinline__ void table_scan(const char* __restrict__ lds, unsigne
     }
 }
 
+// One position's sum for this lane's two filters from index bytes that lie spread over the stream's lanes (lane i holds
+// the table offsets of bytes i and 16 + i of a stretch of text in e0 / e1): position C of the stretch takes its group g
+// from byte C + 3g. The same additions, in the same order, as the ring performs.
+template <int G, int C, int GG>
+__device__ __forceinline__ void readd_group(const char* __restrict__ lds, unsigned e0, unsigned e1, unsigned lanebase, float2& z)
+{
+    const float2 v = *reinterpret_cast<const float2*>(lds + block_offset<C + 3 * GG>(e0, e1) + lanebase + (GG >> 1) * 256 + (GG & 1) * 8);
+    if constexpr (GG == 0) { z.x = v.x; z.y = v.y; }
+    else { z.x += v.x; z.y += v.y; }
+    if constexpr (GG + 1 < G) readd_group<G, C, GG + 1>(lds, e0, e1, lanebase, z);
+}
+// The PP positions of the part of a block that held the end of a region: the first `nold` go to the maximum of the region
+// that ended (o), the others to that of the region that followed it (n).
+template <int G, int C>
+__device__ __forceinline__ void readd_part(const char* __restrict__ lds, unsigned e0, unsigned e1, unsigned lanebase, unsigned nold,
+                                           float2& o, float2& n)
+{
+    float2 z;
+    readd_group<G, C, 0>(lds, e0, e1, lanebase, z);
+    const bool old = (unsigned)C < nold;
+    o.x = fmaxf(o.x, old ? z.x : POISON); o.y = fmaxf(o.y, old ? z.y : POISON);
+    n.x = fmaxf(n.x, old ? POISON : z.x); n.y = fmaxf(n.y, old ? POISON : z.y);
+    __builtin_amdgcn_sched_barrier(0);                           // (a position at a time: this path has no registers to spare)
+    if constexpr (C + 1 < run_parts<G>::PP) readd_part<G, C + 1>(lds, e0, e1, lanebase, nold, o, n);
+}
+
+// The table scan for plain max pooling. As table_scan, but a stream claims RUN consecutive regions at a time and, where
+// a region starts at the text position at which the one before it ended (sequences packed back to back) and is at
+// least three blocks long, walks on without a fresh start: the last positions of a region complete while the first of
+// the next are under way, which saves the TAIL steps of drain and the rounding to whole blocks that every region
+// otherwise costs (29 of 552 steps at 523 rows, 35 % at 101). A block keeps the maxima of its finished positions in NP
+// parts; where a region ends inside a block the parts before the boundary go to it, those after it to its follower, and
+// the part that holds the boundary is left out: its PP positions are added up again from the table one region later
+// (index bytes asked for at the boundary), just before the region that ended is written out. A region that does not
+// follow on ends the run: poison from its last step on, as in table_scan, and a fresh start.
+// Every position's sum is formed by the same additions in the same order either way.
+template <int G>
+__device__ __forceinline__ void table_scan_runs(const char* __restrict__ lds, unsigned F, unsigned f0, const uint8_t* __restrict__ K,
+                                                const uint32_t* __restrict__ R, unsigned* counter, unsigned rend, float* __restrict__ pooled)
+{
+    constexpr unsigned STEPS = 3 * G, NP = run_parts<G>::NP, PP = run_parts<G>::PP, RUN = 8, FOLLOW_ROWS = 3 * STEPS, NOLIMIT = 0xffffffffu;
+    constexpr unsigned KSTRIDE = G * ROWB;                     // bytes per triple: G/2 lines of 256 B
+    constexpr unsigned TAIL = 3 * (G - 1);                       // steps between a position's start and its completion
+    const unsigned P = rend;
+    const unsigned lane = threadIdx.x & 63;
+    const unsigned lanebase = (lane & 15u) * 16u;
+    // the stream's share of the workgroup's regions: RUN consecutive ones per claim
+    unsigned mine = 0u, mine_end = 0u;
+    bool dry = false;                                            // a claim came back past the last region
+    auto take = [&]() -> unsigned {
+        if (mine >= mine_end && !dry) {
+            unsigned v = 0u;
+            if ((lane & 15u) == 0u) v = atomicAdd(counter, RUN);
+            mine = row_share<0>(v);
+            mine_end = mine + RUN < P ? mine + RUN : P;
+            dry = mine >= P;
+        }
+        return dry ? P : mine++;
+    };
+    auto bounds = [&](unsigned rr, unsigned& a_, unsigned& rows_) {
+        a_ = 0u; rows_ = 0u;
+        if (rr < P) { a_ = R[2 * (size_t)rr]; rows_ = R[2 * (size_t)rr + 1] - a_; }
+    };
+    unsigned r = take(), r1 = take();                            // the region in work, the one after it
+    unsigned a, rows, a1, rows1;
+    bounds(r, a, rows); bounds(r1, a1, rows1);
+    unsigned base = a, end = rows, s0 = 0u;                      // the run's first text position; the region's end and the block's first step, relative to it
+    // the next region continues the run (a region that ends in the run's first block would need positions from before it)
+    bool follows = r1 == r + 1u && r1 < P && a1 == a + rows && rows1 >= FOLLOW_ROWS && rows >= STEPS;
+
+    const unsigned q16 = lane & 15;
+    const unsigned q16b = 16u + (STEPS > 16 ? (q16 < (unsigned)(STEPS - 16) ? q16 : (unsigned)(STEPS - 17)) : 0u);
+    auto fetch = [&](unsigned text, unsigned limit, unsigned pos0, unsigned& o0, unsigned& o1) {
+        // text: position of the block's first step, pos0: the same relative to the run's start; steps at or past `limit`
+        // read the poison entry
+        unsigned v0 = K[(size_t)text + q16];
+        unsigned v1 = STEPS > 16 ? (unsigned)K[(size_t)text + q16b] : 0u;
+        o0 = (pos0 + q16 < limit ? v0 : (unsigned)NKMER) * KSTRIDE;
+        o1 = (pos0 + q16b < limit ? v1 : (unsigned)NKMER) * KSTRIDE;
+    };
+    unsigned k0, k1;
+    fetch(base, r < P ? (follows ? NOLIMIT : end + TAIL) : 0u, 0u, k0, k1);
+
+    float2 acc[3][G];
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+        for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
+    float2 mx = make_float2(POISON, POISON);
+    uint2 best = make_uint2(0u, 0u);
+    float2 sum = make_float2(0.f, 0.f);
+    float4 cur[G / 2];                                           // the lines of the coming block's first step
+    read_step<G, 0>(lds, k0, k1, lanebase, cur);
+    // the region before the one in work, while the part that held its end waits to be added up again
+    bool pending = false;
+    float2 prev = make_float2(POISON, POISON);                   // its maximum without that part
+    unsigned e0 = 0u, e1 = 0u, pold = 0u;                        // the part's index bytes; how many of its positions are the region's
+
+    while (true) {
+        const bool active = r < P;
+        if (!__any(active)) break;
+        const unsigned fin = end + TAIL;                         // the first step at which nothing of the region completes any more
+        const bool closes = fin <= s0 + STEPS;                   // the region's last position completes in this block
+        const bool splits = closes && follows, stops = closes && !follows;
+        // the next block's indices travel while this block computes
+        unsigned n0, n1;
+        if (stops) fetch(a1, r1 < P ? rows1 + TAIL : 0u, 0u, n0, n1);
+        else fetch(base + s0 + STEPS, follows ? NOLIMIT : fin, s0 + STEPS, n0, n1);
+        float2 part[NP];
+#pragma unroll
+        for (unsigned h = 0; h < NP; ++h) part[h] = make_float2(POISON, POISON);
+        scan_steps<G, M_MAX, 0, true>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, 0u, cur, part);
+        k0 = n0;
+        k1 = n1;
+        float2 mx2 = make_float2(POISON, POISON);                // what completed of the region that follows
+        unsigned hb = NP, rem = 0u;                              // the part that holds the region's end; how many of its positions are the region's
+        // (the flag passes through an empty asm statement: knowing it ahead of the block, the compiler would make a second
+        // copy of the whole unrolled block for the rare case and run out of registers where the two meet)
+        unsigned split_at = splits ? fin - s0 : 0u;
+        asm volatile("" : "+v"(split_at));
+        if (__any(split_at != 0u)) {
+            if (split_at != 0u) { hb = split_at / PP; rem = split_at - hb * PP; }
+#pragma unroll
+            for (unsigned h = 0; h < NP; ++h) {
+                const bool before = h < hb, after = h > hb || (h == hb && rem == 0u);
+                mx.x = fmaxf(mx.x, before ? part[h].x : POISON); mx.y = fmaxf(mx.y, before ? part[h].y : POISON);
+                mx2.x = fmaxf(mx2.x, after ? part[h].x : POISON); mx2.y = fmaxf(mx2.y, after ? part[h].y : POISON);
+            }
+        } else {
+#pragma unroll
+            for (unsigned h = 0; h < NP; h += 2) { mx.x = fmaxf(fmaxf(mx.x, part[h].x), part[h + 1].x); mx.y = fmaxf(fmaxf(mx.y, part[h].y), part[h + 1].y); }
+        }
+        if (closes) {
+            const unsigned f = f0 + (lane & 15u) * 2;
+            if (pending) {
+                // the region before: the part that held its end, position by position, between it and this one; then out
+                if (pold != 0u) readd_part<G, 0>(lds, e0, e1, lanebase, pold, prev, mx);
+                float* out = pooled + (size_t)(r - 1u) * F + f;
+                if (f + 0 < F) out[0] = fmaxf(prev.x, 0.f);
+                if (f + 1 < F) out[1] = fmaxf(prev.y, 0.f);
+                pending = false;
+            }
+            if (splits) {
+                // the run goes on: this region waits for the part that holds its end; what completed of the next is its start
+                pending = true;
+                prev = mx;
+                pold = rem;
+                if (rem != 0u) {
+                    const size_t text = (size_t)base + s0 + hb * PP - TAIL;
+                    e0 = K[text + q16] * KSTRIDE;
+                    e1 = K[text + 16u + q16] * KSTRIDE;
+                }
+                mx = mx2;
+                end += rows1;
+                s0 += STEPS;
+            } else {
+                // ReLU and store this lane's two of the region's 32 pooled features; a fresh start
+                if (active) {
+                    float* out = pooled + (size_t)r * F + f;
+                    if (f + 0 < F) out[0] = fmaxf(mx.x, 0.f);
+                    if (f + 1 < F) out[1] = fmaxf(mx.y, 0.f);
+                }
+                mx = make_float2(POISON, POISON);
+#pragma unroll
+                for (int c = 0; c < 3; ++c)
+#pragma unroll
+                    for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
+                base = a1; end = rows1; s0 = 0u;
+            }
+            r = r1; rows = rows1;
+            r1 = take();
+            bounds(r1, a1, rows1);
+            follows = r1 == r + 1u && r1 < P && a1 == base + end && rows1 >= FOLLOW_ROWS && rows >= STEPS;
+        } else {
+            s0 += STEPS;
+        }
+    }
+}
+
 template <int G, int MAXT, int MODE>
 __global__ __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(3, 3))) void scanpool_kmer_kernel(const float* __restrict__ W, const float* __restrict__ bias,
                                                             unsigned m, unsigned F, const uint8_t* __restrict__ K, size_t N,
@@ -407,7 +597,12 @@ __global__ __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(3, 3))) vo
     const unsigned lo = (unsigned)((unsigned long long)P * split / nsplit), hi = (unsigned)((unsigned long long)P * (split + 1) / nsplit);
     if (threadIdx.x == 0) counter[0] = lo;
     build_table<G>(lut, w5, W, bias, m, F, f0);
-    table_scan<G, MODE>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled, argmax);
+    // Plain max pooling with filters of up to 18 taps walks through regions that follow each other (16 % faster at 101 nt
+    // x 16 taps, 7 % at 500 nt). At 19-24 taps the ring's 48 registers and the 32 of the read-ahead leave no room for the
+    // run's bookkeeping at three waves per SIMD (the compiler spills ~140 registers, the table lines it has just read
+    // among them), and the read-ahead is worth more there than the drain it would save.
+    if constexpr (MODE == M_MAX && G <= 6) table_scan_runs<G>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled);
+    else table_scan<G, MODE>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled, argmax);
 }
 
 template <int G, int MODE>
