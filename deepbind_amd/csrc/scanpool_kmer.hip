@@ -637,14 +637,15 @@ int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F
 #undef DBK_GO
 }
 
-// Whether a call of this size goes to the table kernel when the choice is left to the library: a filter tile's
-// table costs ~0.1 M position-equivalents to build, which only bulk work repays. From 9 taps on the general path
-// scans on the matrix cores and stays ahead for longer (measured at 1.0 M rows x 4 tiles, regions of 124 rows:
-// 0.147 ms against 0.164 ms for the table kernel, which is twice as fast per row once its tables are built).
+// Whether a call of this size goes to the table kernel when the choice is left to the library: building the tables and
+// the index pre-pass cost ~0.08 ms however small the call, which only bulk work repays. From 9 taps on the general path
+// scans on the matrix cores and stays ahead for longer: measured on 101 nt sequences x 8 tiles, 16 taps: 0.052 ms
+// against 0.095 ms at 3.8 M (rows x tiles), 0.097 against 0.107 at 7.6 M; 12 taps: 0.096 against 0.080 at 7.3 M;
+// 24 taps: level at 8 M. The table kernel is about twice as fast per row once its tables are built.
 bool takes(size_t m, size_t F, size_t N, size_t P)
 {
     if (m > 24 || N == 0 || N > 0x7fffff00u || P > 0x7fff0000u) return false;
-    return (double)N * dbk::divup(F, FTILE) >= (m > 8 ? 5.0e6 : 2.0e6);
+    return (double)N * dbk::divup(F, FTILE) >= (m > 8 ? 8.0e6 : 2.0e6);
 }
 
 // Bytes of device scratch a call over N sequence bytes needs: the flag word's 256-byte line, then the index bytes.
