@@ -426,7 +426,7 @@ __device__ __forceinline__ void readd_part(const char* __restrict__ lds, unsigne
     if constexpr (C + 1 < run_parts<G>::PP) readd_part<G, C + 1>(lds, e0, e1, lanebase, nold, o, n);
 }
 
-// The table scan for plain max pooling. As table_scan, but a stream claims RUN consecutive regions at a time and, where
+// The table scan for plain max pooling. As table_scan, but a stream claims `run` consecutive regions at a time and, where
 // a region starts at the text position at which the one before it ended (sequences packed back to back) and is at
 // least three blocks long, walks on without a fresh start: the last positions of a region complete while the first of
 // the next are under way, which saves the TAIL steps of drain and the rounding to whole blocks that every region
@@ -438,23 +438,23 @@ __device__ __forceinline__ void readd_part(const char* __restrict__ lds, unsigne
 // Every position's sum is formed by the same additions in the same order either way.
 template <int G>
 __device__ __forceinline__ void table_scan_runs(const char* __restrict__ lds, unsigned F, unsigned f0, const uint8_t* __restrict__ K,
-                                                const uint32_t* __restrict__ R, unsigned* counter, unsigned rend, float* __restrict__ pooled)
+                                                const uint32_t* __restrict__ R, unsigned* counter, unsigned run, unsigned rend, float* __restrict__ pooled)
 {
-    constexpr unsigned STEPS = 3 * G, NP = run_parts<G>::NP, PP = run_parts<G>::PP, RUN = 8, FOLLOW_ROWS = 3 * STEPS, NOLIMIT = 0xffffffffu;
+    constexpr unsigned STEPS = 3 * G, NP = run_parts<G>::NP, PP = run_parts<G>::PP, FOLLOW_ROWS = 3 * STEPS, NOLIMIT = 0xffffffffu;
     constexpr unsigned KSTRIDE = G * ROWB;                     // bytes per triple: G/2 lines of 256 B
     constexpr unsigned TAIL = 3 * (G - 1);                       // steps between a position's start and its completion
     const unsigned P = rend;
     const unsigned lane = threadIdx.x & 63;
     const unsigned lanebase = (lane & 15u) * 16u;
-    // the stream's share of the workgroup's regions: RUN consecutive ones per claim
+    // the stream's share of the workgroup's regions: `run` consecutive ones per claim
     unsigned mine = 0u, mine_end = 0u;
     bool dry = false;                                            // a claim came back past the last region
     auto take = [&]() -> unsigned {
         if (mine >= mine_end && !dry) {
             unsigned v = 0u;
-            if ((lane & 15u) == 0u) v = atomicAdd(counter, RUN);
+            if ((lane & 15u) == 0u) v = atomicAdd(counter, run);
             mine = row_share<0>(v);
-            mine_end = mine + RUN < P ? mine + RUN : P;
+            mine_end = mine + run < P ? mine + run : P;
             dry = mine >= P;
         }
         return dry ? P : mine++;
@@ -601,7 +601,9 @@ __global__ __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(3, 3))) vo
     // x 16 taps, 7 % at 500 nt). At 19-24 taps the ring's 48 registers and the 32 of the read-ahead leave no room for the
     // run's bookkeeping at three waves per SIMD (the compiler spills ~140 registers, the table lines it has just read
     // among them), and the read-ahead is worth more there than the drain it would save.
-    if constexpr (MODE == M_MAX && G <= 6) table_scan_runs<G>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled);
+    // (eight regions per claim where every stream gets at least four claims; fewer on small calls, so that no stream idles)
+    const unsigned per_stream = (hi - lo) / (blockDim.x >> 4), run = per_stream >= 32u ? 8u : (per_stream >= 4u ? per_stream / 4u : 1u);
+    if constexpr (MODE == M_MAX && G <= 6) table_scan_runs<G>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, run, hi, pooled);
     else table_scan<G, MODE>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled, argmax);
 }
 
@@ -638,14 +640,14 @@ int launch(hipStream_t st, const float* W, const float* bias, size_t m, size_t F
 }
 
 // Whether a call of this size goes to the table kernel when the choice is left to the library: building the tables and
-// the index pre-pass cost ~0.08 ms however small the call, which only bulk work repays. From 9 taps on the general path
-// scans on the matrix cores and stays ahead for longer: measured on 101 nt sequences x 8 tiles, 16 taps: 0.052 ms
-// against 0.095 ms at 3.8 M (rows x tiles), 0.097 against 0.107 at 7.6 M; 12 taps: 0.096 against 0.080 at 7.3 M;
-// 24 taps: level at 8 M. The table kernel is about twice as fast per row once its tables are built.
+// the index pre-pass make the smallest call ~36 us, which only bulk work repays. From 9 taps on the general path scans on
+// the matrix cores and stays ahead for longer. Measured break-even on 101 nt sequences x 8 tiles, in rows x tiles:
+// 9 and 12 taps ~2 M (0.028 ms either way), 16, 20 and 24 taps ~4 M (0.053-0.066 ms either way); at 8 M the table
+// kernel is 10-40 % ahead, and about twice as fast per row once its tables are built.
 bool takes(size_t m, size_t F, size_t N, size_t P)
 {
     if (m > 24 || N == 0 || N > 0x7fffff00u || P > 0x7fff0000u) return false;
-    return (double)N * dbk::divup(F, FTILE) >= (m > 8 ? 8.0e6 : 2.0e6);
+    return (double)N * dbk::divup(F, FTILE) >= (m > 12 ? 4.0e6 : 2.0e6);
 }
 
 // Bytes of device scratch a call over N sequence bytes needs: the flag word's 256-byte line, then the index bytes.
