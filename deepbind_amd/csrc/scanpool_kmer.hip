@@ -255,19 +255,31 @@ __device__ __forceinline__ void build_table(float* __restrict__ lut, float* __re
         row[0 * FTILE] = w0; row[1 * FTILE] = w1; row[2 * FTILE] = w2; row[3 * FTILE] = w3; row[4 * FTILE] = z * 0.25f;
     }
     __syncthreads();
-    //      element e -> (triple, line i, lane l, j): group 2i + j/2, filter 2l + j%2
-    for (unsigned e = threadIdx.x; e < (unsigned)(NKMER + 1) * G * FTILE; e += blockDim.x) {
-        const unsigned j = e & 3u, l = (e >> 2) & 15u, i = (e >> 6) % (unsigned)(G / 2), km = e / (unsigned)(G * FTILE);
-        const unsigned g = 2 * i + (j >> 1), fl = 2 * l + (j & 1u);
+    // a lane's 16 bytes of a line at a time: unit u -> (triple, line i, lane l) holds group 2i for filters 2l, 2l + 1, then
+    // group 2i + 1 for the same two (one decode of u, six 8-byte reads of the letter weights and one 16-byte write per unit)
+    const unsigned fmax = F > f0 ? F - f0 : 0u;                  // filters of this tile that exist
+    for (unsigned u = threadIdx.x; u < (unsigned)(NKMER + 1) * (G / 2) * 16u; u += blockDim.x) {
+        const unsigned l = u & 15u, i = (u >> 4) % (unsigned)(G / 2), km = u / (unsigned)(8 * G), fl = 2 * l;
         const unsigned l0 = km / 25u, l1 = (km / 5u) % 5u, l2 = km % 5u;
-        float s = POISON;
+        float4 v = make_float4(POISON, POISON, POISON, POISON);
         if (km < (unsigned)NKMER) {
-            s = (g == 0 && f0 + fl < F) ? bias[f0 + fl] : 0.0f;
-            s += w5[((size_t)(3 * g + 0) * 5 + l0) * FTILE + fl];
-            s += w5[((size_t)(3 * g + 1) * 5 + l1) * FTILE + fl];
-            s += w5[((size_t)(3 * g + 2) * 5 + l2) * FTILE + fl];
+            float2 sg[2];
+#pragma unroll
+            for (unsigned j = 0; j < 2; ++j) {
+                const unsigned g = 2 * i + j;
+                float2 t = make_float2(0.0f, 0.0f);
+                if (g == 0) { t.x = fl < fmax ? bias[f0 + fl] : 0.0f; t.y = fl + 1 < fmax ? bias[f0 + fl + 1] : 0.0f; }
+                const float2 a0 = *reinterpret_cast<const float2*>(w5 + ((size_t)(3 * g + 0) * 5 + l0) * FTILE + fl);
+                const float2 a1 = *reinterpret_cast<const float2*>(w5 + ((size_t)(3 * g + 1) * 5 + l1) * FTILE + fl);
+                const float2 a2 = *reinterpret_cast<const float2*>(w5 + ((size_t)(3 * g + 2) * 5 + l2) * FTILE + fl);
+                t.x += a0.x; t.y += a0.y;
+                t.x += a1.x; t.y += a1.y;
+                t.x += a2.x; t.y += a2.y;
+                sg[j] = t;
+            }
+            v = make_float4(sg[0].x, sg[0].y, sg[1].x, sg[1].y);
         }
-        lut[e] = s;
+        reinterpret_cast<float4*>(lut)[u] = v;
     }
     __syncthreads();
 }
