@@ -274,3 +274,59 @@ def test_drop_in_operators_against_the_oracle_over_random_shapes(ks):
         if not (ok and ok2):
             bad.append("%s: pooled err %.3e, gradient err %.3e" % (what, err, err2))
     assert not bad, "\n".join(bad)
+
+
+def test_dense_family_against_the_oracle_over_random_shapes():
+    """blockwise_dot, _nt, _tn and the scoring head: row counts on both sides of the bulk kernels' switch, block sizes
+    that are / are not multiples of 4 and 16, one to 70 models, shared inputs, both float types."""
+    from deepbind_amd import deepity_smat as ds
+    bad = []
+    for case in range(120):
+        rng = np.random.default_rng(400000 + case)
+        f64 = bool(rng.random() < 0.15)
+        dt = np.float64 if f64 else np.float32
+        tol = 1e-12 if f64 else ACT
+        n = int(rng.choice([1, 3, 50, 300, 2047, 2049, 5001, 9000]))
+        k = int(rng.choice([1, 3, 4, 5, 12, 16, 17, 32, 48, 64]))
+        h = int(rng.choice([1, 2, 4, 7, 8, 16, 32, 33, 64]))
+        nb = int(rng.choice([1, 2, 3, 4, 5, 16, 17, 37, 70]))
+        X = rng.standard_normal((n, k * nb)).astype(dt)
+        W = rng.standard_normal((k * nb, h)).astype(dt)
+        dZ = rng.standard_normal((n, h * nb)).astype(dt)
+        X64, W64, dZ64 = X.astype(np.float64), W.astype(np.float64), dZ.astype(np.float64)
+        what = "case %d: n=%d k=%d h=%d models=%d %s" % (case, n, k, h, nb, dt.__name__)
+        print(what, flush=True)
+        fails = []
+        ok, err = _close(host(ds.blockwise_dot(dev(X), dev(W), nb)), orc.blockwise_dot(X64, W64, nb), tol)
+        if not ok: fails.append("dot %.3e" % err)
+        ok, err = _close(host(ds.blockwise_dot_nt(dev(dZ), dev(W), nb)), orc.blockwise_dot_nt(dZ64, W64, nb), tol * 10)
+        if not ok: fails.append("dot_nt %.3e" % err)
+        got = host(ds.blockwise_dot_tn(dev(X), dev(dZ), nb, dev(W)))
+        ok, err = _close(got, orc.blockwise_dot_tn(X64, dZ64, nb, W64), tol * 10)
+        if not ok: fails.append("dot_tn %.3e" % err)
+        if not np.array_equal(got, host(ds.blockwise_dot_tn(dev(X), dev(dZ), nb, dev(W)))): fails.append("dot_tn not repeatable")
+        Xs = rng.standard_normal((n, k)).astype(dt)                   # one input shared by all models
+        ok, err = _close(host(ds.blockwise_dot(dev(Xs), dev(W), nb)), orc.blockwise_dot(Xs.astype(np.float64), W64, nb), tol)
+        if not ok: fails.append("dot shared %.3e" % err)
+        ok, err = _close(host(ds.blockwise_dot_tn(dev(Xs), dev(dZ), nb, dev(W))), orc.blockwise_dot_tn(Xs.astype(np.float64), dZ64, nb, W64), tol * 10)
+        if not ok: fails.append("dot_tn shared %.3e" % err)
+        if not f64:
+            # the scoring head: rescale -> dense -> rectifier -> dense (-> logistic), or one dense layer
+            Pl = np.abs(X)
+            W1, b1 = (W * 0.3).astype(np.float32), (rng.standard_normal((1, h * nb)) * 0.1).astype(np.float32)
+            W2, b2 = (rng.standard_normal((h * nb, 1)) * 0.3).astype(np.float32), (rng.standard_normal((1, nb)) * 0.1).astype(np.float32)
+            rate = rng.choice([0.0, 0.25, 0.5], size=nb).astype(np.float32)
+            logistic = bool(rng.random() < 0.5)
+            Hd = orc.relu_fprop(orc.bias_fprop(orc.blockwise_dot(orc.dropout_fp_test(Pl.astype(np.float64), rate), W1.astype(np.float64), nb), b1))
+            ref = orc.bias_fprop(orc.blockwise_dot(Hd, W2.astype(np.float64), nb), b2)
+            ref = orc.logistic(ref) if logistic else ref
+            out = ds.head_fprop(dev(Pl), dev(W1), dev(b1), dev(W2), dev(b2), nblock=nb, in_scale=1 - rate, apply_logistic=logistic)
+            ok, err = _close(host(out), ref, ACT * 3)
+            if not ok: fails.append("head %.3e" % err)
+            W0, b0 = (rng.standard_normal((k * nb, 1)) * 0.3).astype(np.float32), (rng.standard_normal((1, nb)) * 0.1).astype(np.float32)
+            ref0 = orc.bias_fprop(orc.blockwise_dot(orc.dropout_fp_test(Pl.astype(np.float64), rate), W0.astype(np.float64), nb), b0)
+            ok, err = _close(host(ds.head_fprop(dev(Pl), dev(W0), dev(b0), nblock=nb, in_scale=1 - rate)), ref0, ACT * 3)
+            if not ok: fails.append("head without hidden layer %.3e" % err)
+        if fails:
+            bad.append(what + ": " + "; ".join(fails))
+    assert not bad, "\n".join(bad)
