@@ -325,6 +325,20 @@ def ops_throughput(reps=5):
     rec("scanpool_fprop table[all, argmax]", timed(lambda: ks.scanpool_fprop(W, b, X, R, "all", want_argmax=True, path="kmer")),
         N + 3 * B * F * 4, adds)
     del X, R, W, b, dW, db, dX, P, I, dP
+    # shorter filters at bulk-scoring size (65 536 sequences x 101 nt): up to 18 taps the table kernel walks through
+    # regions that follow each other without a fresh start
+    B2 = 65536
+    codes = rng.integers(0, 4, (B2, L), dtype=np.uint8)
+    codes[rng.random((B2, L)) < 0.01] = 255
+    for m2 in (16, 11, 24):
+        Xh, Rh = data.pack_uniform_ordinals(codes, m2 - 1)
+        X, R = torch.from_numpy(Xh).cuda(), torch.from_numpy(Rh).cuda()
+        W = torch.randn(4 * m2, F, device="cuda") * 0.1
+        b = torch.randn(1, F, device="cuda") * 0.1
+        for path in ("kmer", "mfma"):
+            rec("scanpool_fprop %s[max] %d x %d nt, %d taps" % ("table" if path == "kmer" else "matrix cores", B2, L, m2),
+                timed(lambda: ks.scanpool_fprop(W, b, X, R, "max", path=path)), X.numel() + B2 * F * 4, float(X.numel()) * F * m2)
+        del X, R, W, b
     # per-model dense layer at bulk-scoring size: 100 000 rows, 64 models, 16 -> 32
     from deepbind_amd import deepity_smat as ds
     n, nb, k, h = 100000, 64, 16, 32
