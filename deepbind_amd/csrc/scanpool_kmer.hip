@@ -28,6 +28,8 @@
 //    SIMD favours its oldest wave: equal static shares would finish 5 % apart). A step's table lines are asked for
 //    one step before they are added (scheduling barriers keep that order in the unrolled block): four to eight
 //    ds_read_b128 in flight per wave, one wait per step, the LDS pipe busy 99 % of the time.
+//  * Plain max pooling goes on from one region into the next where they follow each other in the text: with filters of up
+//    to 18 taps through whole runs of regions (table_scan_runs), with 19-24 taps through pairs (table_scan_pairs).
 //  * Positions outside a region never need a test. At a region's start every ring slot is reset to
 //    a large negative "poison" (-1e30), so the partial sums in flight from before the region finish
 //    far below any real value; and the steps a region's last block runs past its final useful
@@ -412,6 +414,125 @@ __device__ __forceinline__ void table_scan(const char* __restrict__ lds, unsigne
     }
 }
 
+// table_scan for plain max pooling with filters of 19-24 taps: two regions that follow each other in the text are scanned
+// as one stretch, so the fill of the ring (TAIL steps) and the rounding to whole blocks are paid once per pair. The block
+// grid starts `lead` steps before the first region, chosen so that the first region's last position completes exactly at a
+// block's end: there its maximum is written out and the running maximum starts again, and nothing else changes - the ring
+// goes on, since what is in flight belongs to the second region. Steps before the first region read the poison entry
+// like those past the end, which sinks every position that does not belong to the pair. A stream claims two regions at
+// a time (`nclaim` = 2; with 1 - calls too small to give every stream a few pairs - regions are taken singly, as in
+// table_scan); two that do not follow each other are scanned one after the other.
+template <int G>
+__device__ __forceinline__ void table_scan_pairs(const char* __restrict__ lds, unsigned F, unsigned f0, const uint8_t* __restrict__ K,
+                                                 const uint32_t* __restrict__ R, unsigned* counter, unsigned nclaim, unsigned rend, float* __restrict__ pooled)
+{
+    constexpr unsigned STEPS = 3 * G, KSTRIDE = G * ROWB, TAIL = 3 * (G - 1), NONE = 0xffffffffu;
+    const unsigned P = rend;
+    const unsigned lane = threadIdx.x & 63;
+    const unsigned lanebase = (lane & 15u) * 16u;
+    const unsigned q16 = lane & 15;
+    const unsigned q16b = 16u + (STEPS > 16 ? (q16 < (unsigned)(STEPS - 16) ? q16 : (unsigned)(STEPS - 17)) : 0u);
+    unsigned carry = NONE;                                       // the second region of a claim whose two do not follow each other
+    // The next item: its first region (P: none left), the text position of its block grid, the steps that are real
+    // ([lead, lead + span)), and the number of blocks after which the first region of a pair is complete (0: a single).
+    auto take = [&](unsigned& rr, unsigned& grid, unsigned& lead, unsigned& span, unsigned& bnd) {
+        bool fresh = carry == NONE;
+        if (fresh) {
+            unsigned v = 0u;
+            if (q16 == 0u) v = atomicAdd(counter, nclaim);
+            rr = row_share<0>(v);
+        } else {
+            rr = carry;
+            carry = NONE;
+        }
+        grid = 0u; lead = 0u; span = 0u; bnd = 0u;
+        if (rr >= P) { rr = P; return; }
+        const unsigned a_ = R[2 * (size_t)rr], rows_ = R[2 * (size_t)rr + 1] - a_;
+        grid = a_; span = rows_ + TAIL;
+        if (fresh && nclaim == 2u && rr + 1u < P) {
+            const unsigned a2 = R[2 * (size_t)rr + 2], rows2 = R[2 * (size_t)rr + 3] - a2;
+            const unsigned ld = (STEPS - (rows_ + TAIL) % STEPS) % STEPS;
+            if (a2 == a_ + rows_ && a_ >= ld) {
+                grid = a_ - ld; lead = ld; span = rows_ + rows2 + TAIL; bnd = (ld + rows_ + TAIL) / STEPS;
+            } else {
+                carry = rr + 1u;
+            }
+        }
+    };
+    auto fetch = [&](unsigned text, unsigned pos0, unsigned lead, unsigned span, unsigned& o0, unsigned& o1) {
+        // text: position of the block's first step, pos0: the same counted from the grid's start
+        unsigned v0 = K[(size_t)text + q16];
+        unsigned v1 = STEPS > 16 ? (unsigned)K[(size_t)text + q16b] : 0u;
+        o0 = (pos0 + q16 - lead < span ? v0 : (unsigned)NKMER) * KSTRIDE;
+        o1 = (pos0 + q16b - lead < span ? v1 : (unsigned)NKMER) * KSTRIDE;
+    };
+    unsigned r, grid, lead, span, bnd, rn, grid_n, lead_n, span_n, bnd_n;
+    take(r, grid, lead, span, bnd);
+    take(rn, grid_n, lead_n, span_n, bnd_n);
+    unsigned nblk = (lead + span + STEPS - 1) / STEPS;
+    if (nblk < 1) nblk = 1;
+    unsigned k0, k1;
+    fetch(grid, 0u, lead, r < P ? span : 0u, k0, k1);
+
+    float2 acc[3][G];
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+        for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
+    float2 mx = make_float2(POISON, POISON);
+    uint2 best = make_uint2(0u, 0u);
+    float2 sum = make_float2(0.f, 0.f);
+    float2 mx1 = make_float2(POISON, POISON);                    // the first region's maximum while the second is scanned
+    unsigned blk = 0;
+    float4 cur[G / 2];                                           // the lines of the coming block's first step
+    read_step<G, 0>(lds, k0, k1, lanebase, cur);
+    const unsigned f = f0 + q16 * 2;
+
+    while (true) {
+        const bool active = r < P;
+        if (!__any(active)) break;
+        const bool last = blk + 1 >= nblk;
+        // the next block's indices travel while this block computes
+        unsigned n0, n1;
+        if (last) fetch(grid_n, 0u, lead_n, rn < P ? span_n : 0u, n0, n1);
+        else fetch(grid + (blk + 1) * STEPS, (blk + 1) * STEPS, lead, span, n0, n1);
+        scan_block<G, M_MAX>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, 0u, cur);
+        k0 = n0;
+        k1 = n1;
+        // where the first region of a pair is complete (and nothing of the second is) its maximum is put aside and the
+        // running maximum starts again; the ring goes on. (Selects, not a branch: any control flow between the unrolled
+        // block and the loop's end that leaves the ring alive costs the compiler its register allocation.)
+        const bool first_done = blk + 1 == bnd;
+        mx1.x = first_done ? mx.x : mx1.x; mx1.y = first_done ? mx.y : mx1.y;
+        mx.x = first_done ? POISON : mx.x; mx.y = first_done ? POISON : mx.y;
+        if (last) {
+            // ReLU and store this lane's two of each region's 32 pooled features
+            if (active) {
+                if (bnd != 0u) {
+                    float* out1 = pooled + (size_t)r * F + f;
+                    if (f + 0 < F) out1[0] = fmaxf(mx1.x, 0.f);
+                    if (f + 1 < F) out1[1] = fmaxf(mx1.y, 0.f);
+                }
+                float* out = pooled + (size_t)(r + (bnd != 0u ? 1u : 0u)) * F + f;
+                if (f + 0 < F) out[0] = fmaxf(mx.x, 0.f);
+                if (f + 1 < F) out[1] = fmaxf(mx.y, 0.f);
+            }
+            // a new item: everything still in the ring belongs to the old one
+            mx = make_float2(POISON, POISON);
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+#pragma unroll
+                for (int s = 0; s < G; ++s) acc[c][s] = make_float2(POISON, POISON);
+            r = rn; grid = grid_n; lead = lead_n; span = span_n; bnd = bnd_n; blk = 0;
+            nblk = (lead + span + STEPS - 1) / STEPS;
+            if (nblk < 1) nblk = 1;
+            take(rn, grid_n, lead_n, span_n, bnd_n);
+        } else {
+            ++blk;
+        }
+    }
+}
+
 // One position's sum for this lane's two filters from index bytes that lie spread over the stream's lanes (lane i holds
 // the table offsets of bytes i and 16 + i of a stretch of text in e0 / e1): position C of the stretch takes its group g
 // from byte C + 3g. The same additions, in the same order, as the ring performs.
@@ -612,10 +733,13 @@ __global__ __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(3, 3))) vo
     // Plain max pooling with filters of up to 18 taps walks through regions that follow each other (16 % faster at 101 nt
     // x 16 taps, 7 % at 500 nt). At 19-24 taps the ring's 48 registers and the 32 of the read-ahead leave no room for the
     // run's bookkeeping at three waves per SIMD (the compiler spills ~140 registers, the table lines it has just read
-    // among them), and the read-ahead is worth more there than the drain it would save.
-    // (eight regions per claim where every stream gets at least four claims; fewer on small calls, so that no stream idles)
+    // among them), and the read-ahead is worth more there than the drain it would save; there two regions that follow each
+    // other are scanned as one stretch, which needs no branch beside the block (1.3 % at 500 nt, 5 % at 101 nt).
+    // (eight regions per claim where every stream gets at least four claims; fewer on small calls, so that no stream idles;
+    // pairs where every stream gets at least two)
     const unsigned per_stream = (hi - lo) / (blockDim.x >> 4), run = per_stream >= 32u ? 8u : (per_stream >= 4u ? per_stream / 4u : 1u);
     if constexpr (MODE == M_MAX && G <= 6) table_scan_runs<G>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, run, hi, pooled);
+    else if constexpr (MODE == M_MAX) table_scan_pairs<G>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, per_stream >= 4u ? 2u : 1u, hi, pooled);
     else table_scan<G, MODE>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled, argmax);
 }
 

@@ -972,6 +972,40 @@ def test_scanpool_kmer_regions_in_any_order(ks, B, lo, hi, m, F):
     assert np.array_equal(host(P2), host(P)[perm]), "a region's result depends on its neighbours in the region table"
 
 
+@pytest.mark.parametrize("B,lo,hi,m", [(4000, 20, 60, 16), (13000, 5, 30, 11), (4000, 20, 60, 24), (13000, 1, 40, 20), (5000, 30, 30, 24),
+                                        (4500, 101, 101, 18)])
+def test_scanpool_kmer_walks_on_through_regions_at_bulk_sizes(ks, B, lo, hi, m):
+    """Enough regions per workgroup (1 024 filters: eight workgroups per tile) that every stream of the table kernel
+    claims several regions at a time and goes on from one into the next where they follow each other in the text (runs
+    of up to eight with at most 18 taps, pairs with 19-24): the packed table, the same with a third of the regions
+    dropped (runs and pairs break off, second halves of claims are scanned alone), with regions cut in two that touch,
+    and shuffled (no region follows another) - against the general kernel, against the C oracle on a sample, and the
+    shuffled call against the packed one bit for bit."""
+    from oracle import oracle_c
+    F = 1024
+    rng, W, b, X, R = _fused_case(77 + B + m, B, lo, hi, m, F, pn=0.02)
+    Wd, bd, Xd = dev(W), dev(b), dev(X)
+    cut = []
+    for a_, b_ in R:
+        if b_ - a_ >= 2 and rng.random() < 0.5:
+            c_ = int(rng.integers(a_ + 1, b_))
+            cut += [(a_, c_), (c_, b_)]
+        else:
+            cut.append((a_, b_))
+    tables = {"packed": R, "some dropped": np.ascontiguousarray(R[rng.random(B) < 0.67]),
+              "cut in two": np.array(cut, dtype=R.dtype).reshape(-1, 2)}
+    for name, Rt in tables.items():
+        P, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(Rt), "max", path="kmer")
+        Pg, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(Rt), "max", path="general")
+        assert_close(host(P), host(Pg), ACT, "table vs general kernel, %s" % name)
+        pick = np.sort(rng.choice(len(Rt), 40, replace=False))
+        Pr, _ = oracle_c.scanpool(W, b, X, np.ascontiguousarray(Rt[pick]), 0)
+        assert_close(host(P)[pick], Pr, ACT, "table kernel vs C oracle, %s" % name)
+        perm = rng.permutation(len(Rt))
+        P2, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(np.ascontiguousarray(Rt[perm])), "max", path="kmer")
+        assert np.array_equal(host(P2), host(P)[perm]), "a region's result depends on its neighbours in the region table (%s)" % name
+
+
 @pytest.mark.parametrize("n,m,dtype", [(1, 5, np.float32), (255, 64, np.float32), (13591, 720, np.float32), (100000, 70, np.float32),
                                        (4097, 1, np.float64), (0, 9, np.float32)])
 def test_column_sums(sm, n, m, dtype):
