@@ -422,7 +422,7 @@ __device__ __forceinline__ void table_scan(const char* __restrict__ lds, unsigne
 // like those past the end, which sinks every position that does not belong to the pair. A stream claims two regions at
 // a time (`nclaim` = 2; with 1 - calls too small to give every stream a few pairs - regions are taken singly, as in
 // table_scan); two that do not follow each other are scanned one after the other.
-template <int G>
+template <int G, int MODE>
 __device__ __forceinline__ void table_scan_pairs(const char* __restrict__ lds, unsigned F, unsigned f0, const uint8_t* __restrict__ K,
                                                  const uint32_t* __restrict__ R, unsigned* counter, unsigned nclaim, unsigned rend, float* __restrict__ pooled)
 {
@@ -482,7 +482,7 @@ __device__ __forceinline__ void table_scan_pairs(const char* __restrict__ lds, u
     float2 mx = make_float2(POISON, POISON);
     uint2 best = make_uint2(0u, 0u);
     float2 sum = make_float2(0.f, 0.f);
-    float2 mx1 = make_float2(POISON, POISON);                    // the first region's maximum while the second is scanned
+    float2 mx1 = make_float2(POISON, POISON), sum1 = make_float2(0.f, 0.f);   // the first region's maximum and sum while the second is scanned
     unsigned blk = 0;
     float4 cur[G / 2];                                           // the lines of the coming block's first step
     read_step<G, 0>(lds, k0, k1, lanebase, cur);
@@ -496,29 +496,48 @@ __device__ __forceinline__ void table_scan_pairs(const char* __restrict__ lds, u
         unsigned n0, n1;
         if (last) fetch(grid_n, 0u, lead_n, rn < P ? span_n : 0u, n0, n1);
         else fetch(grid + (blk + 1) * STEPS, (blk + 1) * STEPS, lead, span, n0, n1);
-        scan_block<G, M_MAX>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, 0u, cur);
+        scan_block<G, MODE>(lds, k0, k1, n0, n1, acc, mx, best, sum, lanebase, 0u, cur);
         k0 = n0;
         k1 = n1;
         // where the first region of a pair is complete (and nothing of the second is) its maximum is put aside and the
         // running maximum starts again; the ring goes on. (Selects, not a branch: any control flow between the unrolled
         // block and the loop's end that leaves the ring alive costs the compiler its register allocation.)
         const bool first_done = blk + 1 == bnd;
-        mx1.x = first_done ? mx.x : mx1.x; mx1.y = first_done ? mx.y : mx1.y;
-        mx.x = first_done ? POISON : mx.x; mx.y = first_done ? POISON : mx.y;
+        if (MODE & M_MAX) {
+            mx1.x = first_done ? mx.x : mx1.x; mx1.y = first_done ? mx.y : mx1.y;
+            mx.x = first_done ? POISON : mx.x; mx.y = first_done ? POISON : mx.y;
+        }
+        if (MODE & M_SUM) {
+            sum1.x = first_done ? sum.x : sum1.x; sum1.y = first_done ? sum.y : sum1.y;
+            sum.x = first_done ? 0.f : sum.x; sum.y = first_done ? 0.f : sum.y;
+        }
         if (last) {
             // ReLU and store this lane's two of each region's 32 pooled features
             if (active) {
-                if (bnd != 0u) {
-                    float* out1 = pooled + (size_t)r * F + f;
-                    if (f + 0 < F) out1[0] = fmaxf(mx1.x, 0.f);
-                    if (f + 1 < F) out1[1] = fmaxf(mx1.y, 0.f);
-                }
-                float* out = pooled + (size_t)(r + (bnd != 0u ? 1u : 0u)) * F + f;
-                if (f + 0 < F) out[0] = fmaxf(mx.x, 0.f);
-                if (f + 1 < F) out[1] = fmaxf(mx.y, 0.f);
+                // (the first region's rows from where its last position completed; the second's are the rest)
+                const unsigned rows1 = bnd * STEPS - lead - TAIL, rows2 = span - TAIL - (bnd != 0u ? rows1 : 0u);
+                auto put = [&](unsigned rr, float2 vmax, float2 vsum, unsigned nrow) {
+                    const float inv = 1.0f / (float)nrow;
+                    if (MODE == M_SUM) {
+                        float* out = pooled + (size_t)rr * F + f;
+                        if (f + 0 < F) out[0] = vsum.x * inv;
+                        if (f + 1 < F) out[1] = vsum.y * inv;
+                    } else if (MODE & M_SUM) {
+                        float* out = pooled + ((size_t)rr * F + f) * 2;          // (max, avg) interleaved per filter
+                        if (f + 0 < F) { out[0] = fmaxf(vmax.x, 0.f); out[1] = vsum.x * inv; }
+                        if (f + 1 < F) { out[2] = fmaxf(vmax.y, 0.f); out[3] = vsum.y * inv; }
+                    } else {
+                        float* out = pooled + (size_t)rr * F + f;
+                        if (f + 0 < F) out[0] = fmaxf(vmax.x, 0.f);
+                        if (f + 1 < F) out[1] = fmaxf(vmax.y, 0.f);
+                    }
+                };
+                if (bnd != 0u) put(r, mx1, sum1, rows1);
+                put(r + (bnd != 0u ? 1u : 0u), mx, sum, rows2);
             }
             // a new item: everything still in the ring belongs to the old one
             mx = make_float2(POISON, POISON);
+            sum = make_float2(0.f, 0.f);
 #pragma unroll
             for (int c = 0; c < 3; ++c)
 #pragma unroll
@@ -739,7 +758,7 @@ __global__ __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(3, 3))) vo
     // pairs where every stream gets at least two)
     const unsigned per_stream = (hi - lo) / (blockDim.x >> 4), run = per_stream >= 32u ? 8u : (per_stream >= 4u ? per_stream / 4u : 1u);
     if constexpr (MODE == M_MAX && G <= 6) table_scan_runs<G>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, run, hi, pooled);
-    else if constexpr (MODE == M_MAX) table_scan_pairs<G>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, per_stream >= 4u ? 2u : 1u, hi, pooled);
+    else if constexpr (!(MODE & M_ARG)) table_scan_pairs<G, MODE>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, per_stream >= 4u ? 2u : 1u, hi, pooled);
     else table_scan<G, MODE>(reinterpret_cast<const char*>(smem), F, f0, K, R, counter, hi, pooled, argmax);
 }
 

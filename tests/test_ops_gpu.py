@@ -977,7 +977,7 @@ def test_scanpool_kmer_regions_in_any_order(ks, B, lo, hi, m, F):
 def test_scanpool_kmer_walks_on_through_regions_at_bulk_sizes(ks, B, lo, hi, m):
     """Enough regions per workgroup (1 024 filters: eight workgroups per tile) that every stream of the table kernel
     claims several regions at a time and goes on from one into the next where they follow each other in the text (runs
-    of up to eight with at most 18 taps, pairs with 19-24): the packed table, the same with a third of the regions
+    of up to eight with at most 18 taps, pairs with 19-24 and for average pooling): the packed table, the same with a third of the regions
     dropped (runs and pairs break off, second halves of claims are scanned alone), with regions cut in two that touch,
     and shuffled (no region follows another) - against the general kernel, against the C oracle on a sample, and the
     shuffled call against the packed one bit for bit."""
@@ -1004,6 +1004,13 @@ def test_scanpool_kmer_walks_on_through_regions_at_bulk_sizes(ks, B, lo, hi, m):
         perm = rng.permutation(len(Rt))
         P2, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(np.ascontiguousarray(Rt[perm])), "max", path="kmer")
         assert np.array_equal(host(P2), host(P)[perm]), "a region's result depends on its neighbours in the region table (%s)" % name
+        # average and max + average pooling go through pairs at every filter length
+        for ptype in ("avg", "all"):
+            Pa, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(Rt), ptype, path="kmer")
+            Pag, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(Rt), ptype, path="general")
+            assert_close(host(Pa), host(Pag), ACT, "table vs general kernel, %s, %s" % (ptype, name))
+            Pa2, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(np.ascontiguousarray(Rt[perm])), ptype, path="kmer")
+            assert np.array_equal(host(Pa2), host(Pa)[perm]), "%s pooling: a region's result depends on its neighbours (%s)" % (ptype, name)
 
 
 @pytest.mark.parametrize("n,m,dtype", [(1, 5, np.float32), (255, 64, np.float32), (13591, 720, np.float32), (100000, 70, np.float32),
