@@ -998,6 +998,9 @@ def test_scanpool_kmer_walks_on_through_regions_at_bulk_sizes(ks, B, lo, hi, m):
         P, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(Rt), "max", path="kmer")
         Pg, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(Rt), "max", path="general")
         assert_close(host(P), host(Pg), ACT, "table vs general kernel, %s" % name)
+        for _ in range(2):                                             # which stream takes which regions differs from call to call
+            Pagain, _ = ks.scanpool_fprop(Wd, bd, Xd, dev(Rt), "max", path="kmer")
+            assert torch.equal(P, Pagain), "two calls, different bits (%s)" % name
         pick = np.sort(rng.choice(len(Rt), 40, replace=False))
         Pr, _ = oracle_c.scanpool(W, b, X, np.ascontiguousarray(Rt[pick]), 0)
         assert_close(host(P)[pick], Pr, ACT, "table kernel vs C oracle, %s" % name)
